@@ -1,0 +1,72 @@
+"""Loader of the native library.  There is no fallback: every op in this package runs in
+libhccl_amd.so (HIP kernels for gfx950 behind a C ABI) or raises."""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libhccl_amd.so")
+
+MAX_FAN = 16
+
+
+class Seg(ctypes.Structure):
+    """hcclx_seg_t of include/hcclx.h."""
+    _fields_ = [
+        ("count", ctypes.c_uint64),
+        ("nsrc", ctypes.c_uint32),
+        ("ndst", ctypes.c_uint32),
+        ("src", ctypes.c_void_p * MAX_FAN),
+        ("dst", ctypes.c_void_p * MAX_FAN),
+    ]
+
+
+_lib = None
+
+
+def load():
+    """Returns the ctypes handle of libhccl_amd.so, loading it on first use."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+            "or `make -C hccl_amd/csrc`; there is no CPU fallback")
+    lib = ctypes.CDLL(LIB_PATH)
+    u64p = ctypes.POINTER(ctypes.c_uint64)
+    vpp = ctypes.POINTER(ctypes.c_void_p)
+    lib.hcclx_init.restype = ctypes.c_int
+    lib.hcclx_last_error.restype = ctypes.c_char_p
+    lib.hcclx_dtype_size.restype = ctypes.c_uint32
+    lib.hcclx_dtype_size.argtypes = [ctypes.c_int]
+    lib.hcclx_fold.restype = ctypes.c_int
+    lib.hcclx_fold.argtypes = [ctypes.POINTER(Seg), ctypes.c_uint32, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                               ctypes.c_void_p]
+    lib.hcclx_plan_create.restype = ctypes.c_int
+    lib.hcclx_plan_create.argtypes = [ctypes.POINTER(Seg), ctypes.c_uint32, ctypes.c_int, ctypes.c_int,
+                                      ctypes.c_int, ctypes.POINTER(ctypes.c_void_p)]
+    lib.hcclx_plan_launch.restype = ctypes.c_int
+    lib.hcclx_plan_launch.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+    lib.hcclx_plan_destroy.restype = ctypes.c_int
+    lib.hcclx_plan_destroy.argtypes = [ctypes.c_void_p]
+    lib.hcclx_plan_bytes.restype = ctypes.c_uint64
+    lib.hcclx_plan_bytes.argtypes = [ctypes.c_void_p]
+    lib.hcclx_alltoallv.restype = ctypes.c_int
+    lib.hcclx_alltoallv.argtypes = [vpp, vpp, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32,
+                                    ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    lib.hcclx_allgatherv.restype = ctypes.c_int
+    lib.hcclx_allgatherv.argtypes = [vpp, vpp, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_int,
+                                     ctypes.c_int, ctypes.c_void_p]
+    _lib = lib
+    return lib
+
+
+class HcclError(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__(f"HcclResult {code}: {text}")
+        self.code = code
+
+
+def check(rc):
+    if rc != 0:
+        raise HcclError(rc, load().hcclx_last_error().decode())

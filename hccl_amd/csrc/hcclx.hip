@@ -1,0 +1,412 @@
+// C-ABI launcher of the fold kernels (see include/hcclx.h): table building, descriptor ring, plans.
+#include "hcclx.h"
+#include "hcclx_internal.h"
+#include "kernels/fold.h"
+
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <vector>
+
+namespace hcclx {
+
+static thread_local std::string g_err;
+
+void set_error(const std::string &msg) { g_err = msg; }
+int fail(int code, const std::string &msg)
+{
+    g_err = msg;
+    return code;
+}
+int fail_hip(hipError_t e, const char *what)
+{
+    g_err = std::string(what) + ": " + hipGetErrorString(e);
+    return (e == hipErrorOutOfMemory) ? HCCL_E_MEMORY : HCCL_E_RUNTIME;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// device context + descriptor ring
+// ---------------------------------------------------------------------------------------------------
+namespace {
+
+constexpr int kMaxDevices = 32;
+constexpr size_t kSliceBytes = 1u << 20;
+constexpr int kSlices = 8;
+
+struct Ring {
+    std::mutex mu;
+    int cur = 0;
+    size_t off = 0;
+    struct Pending {
+        hipStream_t stream;
+        hipEvent_t event;
+    };
+    std::vector<hipStream_t> used[kSlices];   // streams that launched from the slice since it was opened
+    std::vector<Pending> pending[kSlices];    // events recorded when the slice was closed
+    std::vector<hipEvent_t> pool;
+};
+
+struct DeviceSlot {
+    std::once_flag once;
+    bool ok = false;
+    std::string err;
+    DeviceCtx ctx;
+    Ring ring;
+};
+
+DeviceSlot g_slots[kMaxDevices];
+
+void init_slot(DeviceSlot *s, int dev)
+{
+    DeviceCtx &c = s->ctx;
+    c.device = dev;
+    hipError_t e = hipDeviceGetAttribute(&c.num_cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess || c.num_cus <= 0) {
+        s->err = std::string("hipDeviceGetAttribute(MultiprocessorCount): ") + hipGetErrorString(e);
+        return;
+    }
+    if (const char *v = std::getenv("HCCLX_BLOCKS_PER_CU")) {
+        c.blocks_per_cu = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
+    }
+    c.ring_bytes = kSliceBytes * kSlices;
+    e = hipHostMalloc(reinterpret_cast<void **>(&c.h_ring), c.ring_bytes, hipHostMallocDefault);
+    if (e != hipSuccess) {
+        s->err = std::string("hipHostMalloc(descriptor ring): ") + hipGetErrorString(e);
+        return;
+    }
+    e = hipMalloc(reinterpret_cast<void **>(&c.d_ring), c.ring_bytes);
+    if (e != hipSuccess) {
+        s->err = std::string("hipMalloc(descriptor ring): ") + hipGetErrorString(e);
+        return;
+    }
+    s->ok = true;
+}
+
+}  // namespace
+
+DeviceCtx *device_ctx()
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        fail_hip(e, "hipGetDevice");
+        return nullptr;
+    }
+    if (dev < 0 || dev >= kMaxDevices) {
+        fail(HCCL_E_PARA, "device index out of range");
+        return nullptr;
+    }
+    DeviceSlot *s = &g_slots[dev];
+    std::call_once(s->once, init_slot, s, dev);
+    if (!s->ok) {
+        set_error(s->err);
+        return nullptr;
+    }
+    return &s->ctx;
+}
+
+int ring_reserve(DeviceCtx *ctx, size_t bytes, hipStream_t stream, char **h, char **d)
+{
+    bytes = (bytes + 255) & ~static_cast<size_t>(255);
+    if (bytes > kSliceBytes) {
+        return fail(HCCL_E_PARA, "descriptor table larger than one ring slice");
+    }
+    Ring &r = g_slots[ctx->device].ring;
+    std::lock_guard<std::mutex> lock(r.mu);
+    if (r.off + bytes > kSliceBytes) {
+        // close the current slice: one event per stream that read from it
+        for (hipStream_t s : r.used[r.cur]) {
+            hipEvent_t ev;
+            if (!r.pool.empty()) {
+                ev = r.pool.back();
+                r.pool.pop_back();
+            } else {
+                HCCLX_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+            }
+            HCCLX_HIP(hipEventRecord(ev, s));
+            r.pending[r.cur].push_back({s, ev});
+        }
+        r.used[r.cur].clear();
+        r.cur = (r.cur + 1) % kSlices;
+        r.off = 0;
+        // open the next one: everything that still reads it must have finished
+        for (auto &p : r.pending[r.cur]) {
+            HCCLX_HIP(hipEventSynchronize(p.event));
+            r.pool.push_back(p.event);
+        }
+        r.pending[r.cur].clear();
+    }
+    bool seen = false;
+    for (hipStream_t s : r.used[r.cur]) seen = seen || (s == stream);
+    if (!seen) r.used[r.cur].push_back(stream);
+    const size_t at = static_cast<size_t>(r.cur) * kSliceBytes + r.off;
+    r.off += bytes;
+    *h = ctx->h_ring + at;
+    *d = ctx->d_ring + at;
+    return HCCL_SUCCESS;
+}
+
+uint32_t grid_for(const DeviceCtx *ctx, uint64_t total_tiles)
+{
+    uint64_t cap = static_cast<uint64_t>(ctx->num_cus) * ctx->blocks_per_cu;
+    if (ctx->blocks_per_cu == 0 || total_tiles < cap) cap = total_tiles;
+    if (cap > 0x7fffffffu) cap = 0x7fffffffu;
+    return static_cast<uint32_t>(cap);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// fold tables
+// ---------------------------------------------------------------------------------------------------
+namespace {
+
+bool is_reduce_dtype(int dt)
+{
+    switch (dt) {
+        case HCCL_DATA_TYPE_INT8:
+        case HCCL_DATA_TYPE_INT16:
+        case HCCL_DATA_TYPE_INT32:
+        case HCCL_DATA_TYPE_INT64:
+        case HCCL_DATA_TYPE_UINT64:
+        case HCCL_DATA_TYPE_FP16:
+        case HCCL_DATA_TYPE_FP32:
+        case HCCL_DATA_TYPE_FP64:
+        case HCCL_DATA_TYPE_BFP16:
+            return true;
+        default:
+            return false;
+    }
+}
+
+bool is_float_dtype(int dt)
+{
+    return dt == HCCL_DATA_TYPE_FP16 || dt == HCCL_DATA_TYPE_FP32 || dt == HCCL_DATA_TYPE_FP64 ||
+           dt == HCCL_DATA_TYPE_BFP16;
+}
+
+// What one kernel launch needs, before it is placed in device memory.
+struct Batch {
+    bool copy = false;
+    int dtype = 0;
+    int op = 0;
+    int mode = 0;
+    int maxn = 1;
+    uint64_t total_tiles = 0;
+    std::vector<uint64_t> tile_end;
+    std::vector<SegDev> segs;
+    size_t bytes() const { return align256(tile_end.size() * 8) + segs.size() * sizeof(SegDev); }
+    static size_t align256(size_t x) { return (x + 255) & ~static_cast<size_t>(255); }
+};
+
+struct Built {
+    std::vector<Batch> batches;
+    uint64_t algo_bytes = 0;
+};
+
+int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, Built *out)
+{
+    if (nseg != 0 && segs == nullptr) return fail(HCCL_E_PTR, "segs is null");
+    const int esz = dtype_size(dtype);
+    if (esz == 0) return fail(HCCL_E_NOT_SUPPORT, "unknown data type " + std::to_string(dtype));
+    if (mode != HCCLX_FOLD_CHAIN && mode != HCCLX_FOLD_SELF_FIRST) return fail(HCCL_E_PARA, "unknown fold mode");
+
+    uint32_t max_src = 0;
+    for (uint32_t i = 0; i < nseg; ++i) {
+        const hcclx_seg_t &s = segs[i];
+        if (s.nsrc == 0 || s.nsrc > HCCLX_MAX_FAN || s.ndst == 0 || s.ndst > HCCLX_MAX_FAN) {
+            return fail(HCCL_E_PARA, "segment " + std::to_string(i) + ": nsrc/ndst outside 1.." +
+                                         std::to_string(HCCLX_MAX_FAN));
+        }
+        if (mode == HCCLX_FOLD_SELF_FIRST && s.nsrc != s.ndst) {
+            return fail(HCCL_E_PARA, "self-first fold needs nsrc == ndst");
+        }
+        if (s.count != 0) {
+            for (uint32_t k = 0; k < s.nsrc; ++k) {
+                if (s.src[k] == nullptr) return fail(HCCL_E_PTR, "segment " + std::to_string(i) + ": null source");
+            }
+            for (uint32_t k = 0; k < s.ndst; ++k) {
+                if (s.dst[k] == nullptr) return fail(HCCL_E_PTR, "segment " + std::to_string(i) + ": null destination");
+            }
+        }
+        if (s.nsrc > max_src) max_src = s.nsrc;
+    }
+
+    Batch proto;
+    proto.copy = (max_src <= 1);
+    proto.dtype = dtype;
+    proto.op = op;
+    proto.mode = mode;
+    if (!proto.copy) {
+        if (!is_reduce_dtype(dtype)) return fail(HCCL_E_NOT_SUPPORT, "data type cannot be reduced");
+        if (op < HCCL_REDUCE_SUM || op > HCCL_REDUCE_MIN) return fail(HCCL_E_NOT_SUPPORT, "unknown reduce op");
+        proto.maxn = max_src <= 2 ? 2 : max_src <= 4 ? 4 : max_src <= 8 ? 8 : 16;
+        // Integer folds are association-free: the self-first order gives the bits of the plain chain.
+        // The kernel for it exists only for floating types, so integers take the chain kernel with the
+        // self-first segment rewritten below.
+    } else {
+        proto.maxn = 1;
+        proto.mode = HCCLX_FOLD_CHAIN;
+    }
+    const bool rewrite_self = (!proto.copy && mode == HCCLX_FOLD_SELF_FIRST && !is_float_dtype(dtype));
+    if (rewrite_self) proto.mode = HCCLX_FOLD_CHAIN;
+
+    const int ne = proto.copy ? 16 : 16 / esz;
+    Batch cur = proto;
+    for (uint32_t i = 0; i < nseg; ++i) {
+        const hcclx_seg_t &s = segs[i];
+        if (s.count == 0) continue;
+        SegDev sd;
+        std::memset(&sd, 0, sizeof(sd));
+        sd.count = proto.copy ? s.count * esz : s.count;  // the copy kernel counts bytes
+        sd.nsrc = s.nsrc;
+        sd.ndst = s.ndst;
+        for (uint32_t k = 0; k < s.nsrc; ++k) sd.src[k] = static_cast<const char *>(s.src[k]);
+        for (uint32_t k = 0; k < s.ndst; ++k) sd.dst[k] = static_cast<char *>(s.dst[k]);
+        const uint64_t tiles = fold_tiles_of(sd.count, ne, proto.maxn);
+        if (static_cast<int>(cur.segs.size()) == kMaxSegsPerLaunch) {
+            out->batches.push_back(std::move(cur));
+            cur = proto;
+        }
+        cur.total_tiles += tiles;
+        cur.tile_end.push_back(cur.total_tiles);
+        cur.segs.push_back(sd);
+        out->algo_bytes += static_cast<uint64_t>(s.nsrc + s.ndst) * s.count * esz;
+    }
+    if (!cur.segs.empty()) out->batches.push_back(std::move(cur));
+    return HCCL_SUCCESS;
+}
+
+void fill_table(const Batch &b, char *h)
+{
+    std::memcpy(h, b.tile_end.data(), b.tile_end.size() * 8);
+    std::memcpy(h + Batch::align256(b.tile_end.size() * 8), b.segs.data(), b.segs.size() * sizeof(SegDev));
+}
+
+int launch_batch(const DeviceCtx *ctx, const Batch &b, const char *d_table, hipStream_t stream)
+{
+    FoldLaunch l;
+    l.tile_end = reinterpret_cast<const uint64_t *>(d_table);
+    l.segs = reinterpret_cast<const SegDev *>(d_table + Batch::align256(b.tile_end.size() * 8));
+    l.nseg = static_cast<uint32_t>(b.segs.size());
+    l.total_tiles = b.total_tiles;
+    l.grid = grid_for(ctx, b.total_tiles);
+    l.stream = stream;
+    hipError_t e;
+    if (b.copy) {
+        e = fold_dispatch_copy(l);
+    } else {
+        switch (b.dtype) {
+            case HCCL_DATA_TYPE_INT8: e = fold_dispatch_i8(b.op, b.maxn, b.mode, l); break;
+            case HCCL_DATA_TYPE_INT16: e = fold_dispatch_i16(b.op, b.maxn, b.mode, l); break;
+            case HCCL_DATA_TYPE_INT32: e = fold_dispatch_i32(b.op, b.maxn, b.mode, l); break;
+            case HCCL_DATA_TYPE_INT64: e = fold_dispatch_i64(b.op, b.maxn, b.mode, l); break;
+            case HCCL_DATA_TYPE_UINT64: e = fold_dispatch_u64(b.op, b.maxn, b.mode, l); break;
+            case HCCL_DATA_TYPE_FP16: e = fold_dispatch_f16(b.op, b.maxn, b.mode, l); break;
+            case HCCL_DATA_TYPE_FP32: e = fold_dispatch_f32(b.op, b.maxn, b.mode, l); break;
+            case HCCL_DATA_TYPE_FP64: e = fold_dispatch_f64(b.op, b.maxn, b.mode, l); break;
+            case HCCL_DATA_TYPE_BFP16: e = fold_dispatch_bf16(b.op, b.maxn, b.mode, l); break;
+            default: e = hipErrorInvalidValue; break;
+        }
+    }
+    if (e != hipSuccess) return fail_hip(e, "fold kernel launch");
+    return HCCL_SUCCESS;
+}
+
+}  // namespace
+}  // namespace hcclx
+
+using namespace hcclx;
+
+struct hcclx_plan {
+    int device = -1;
+    char *d_table = nullptr;
+    uint64_t algo_bytes = 0;
+    std::vector<Batch> batches;
+    std::vector<size_t> offsets;
+};
+
+extern "C" {
+
+int hcclx_init(void) { return device_ctx() ? HCCL_SUCCESS : HCCL_E_RUNTIME; }
+
+const char *hcclx_last_error(void) { return g_err.c_str(); }
+
+uint32_t hcclx_dtype_size(int dtype) { return static_cast<uint32_t>(dtype_size(dtype)); }
+
+int hcclx_fold(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, void *stream)
+{
+    DeviceCtx *ctx = device_ctx();
+    if (!ctx) return HCCL_E_RUNTIME;
+    Built built;
+    int rc = build_batches(segs, nseg, dtype, op, mode, &built);
+    if (rc != HCCL_SUCCESS) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    for (const Batch &b : built.batches) {
+        char *h = nullptr;
+        char *d = nullptr;
+        rc = ring_reserve(ctx, b.bytes(), st, &h, &d);
+        if (rc != HCCL_SUCCESS) return rc;
+        fill_table(b, h);
+        HCCLX_HIP(hipMemcpyAsync(d, h, b.bytes(), hipMemcpyHostToDevice, st));
+        rc = launch_batch(ctx, b, d, st);
+        if (rc != HCCL_SUCCESS) return rc;
+    }
+    return HCCL_SUCCESS;
+}
+
+int hcclx_plan_create(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, hcclx_plan_t **plan)
+{
+    if (plan == nullptr) return fail(HCCL_E_PTR, "plan is null");
+    *plan = nullptr;
+    DeviceCtx *ctx = device_ctx();
+    if (!ctx) return HCCL_E_RUNTIME;
+    Built built;
+    int rc = build_batches(segs, nseg, dtype, op, mode, &built);
+    if (rc != HCCL_SUCCESS) return rc;
+    hcclx_plan *p = new hcclx_plan;
+    p->device = ctx->device;
+    p->algo_bytes = built.algo_bytes;
+    p->batches = std::move(built.batches);
+    size_t total = 0;
+    for (const Batch &b : p->batches) {
+        p->offsets.push_back(total);
+        total += b.bytes();
+    }
+    if (total != 0) {
+        std::vector<char> host(total);
+        for (size_t i = 0; i < p->batches.size(); ++i) fill_table(p->batches[i], host.data() + p->offsets[i]);
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&p->d_table), total);
+        if (e == hipSuccess) e = hipMemcpy(p->d_table, host.data(), total, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            if (p->d_table) (void)hipFree(p->d_table);
+            delete p;
+            return fail_hip(e, "plan table upload");
+        }
+    }
+    *plan = p;
+    return HCCL_SUCCESS;
+}
+
+int hcclx_plan_launch(const hcclx_plan_t *plan, void *stream)
+{
+    if (plan == nullptr) return fail(HCCL_E_PTR, "plan is null");
+    DeviceCtx *ctx = device_ctx();
+    if (!ctx) return HCCL_E_RUNTIME;
+    if (ctx->device != plan->device) return fail(HCCL_E_PARA, "plan belongs to another device");
+    for (size_t i = 0; i < plan->batches.size(); ++i) {
+        int rc = launch_batch(ctx, plan->batches[i], plan->d_table + plan->offsets[i], static_cast<hipStream_t>(stream));
+        if (rc != HCCL_SUCCESS) return rc;
+    }
+    return HCCL_SUCCESS;
+}
+
+int hcclx_plan_destroy(hcclx_plan_t *plan)
+{
+    if (plan == nullptr) return HCCL_SUCCESS;
+    if (plan->d_table) (void)hipFree(plan->d_table);
+    delete plan;
+    return HCCL_SUCCESS;
+}
+
+uint64_t hcclx_plan_bytes(const hcclx_plan_t *plan) { return plan ? plan->algo_bytes : 0; }
+
+}  // extern "C"

@@ -1,0 +1,42 @@
+// Host-side helpers shared by the C-ABI translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <string>
+#include "hccl_types.h"
+
+namespace hcclx {
+
+// Thread-local text of the last failure; returned by hcclx_last_error().
+void set_error(const std::string &msg);
+int fail(int code, const std::string &msg);  // records msg, returns code
+int fail_hip(hipError_t e, const char *what);
+
+#define HCCLX_HIP(expr)                                          \
+    do {                                                         \
+        hipError_t e_ = (expr);                                  \
+        if (e_ != hipSuccess) return ::hcclx::fail_hip(e_, #expr); \
+    } while (0)
+
+// Per-device launch resources.
+struct DeviceCtx {
+    int device = -1;
+    int num_cus = 0;
+    uint32_t blocks_per_cu = 8;  // persistent-grid cap; 0 = one workgroup per tile
+    // Descriptor ring: tables of one-shot launches are written to pinned host memory and copied to the
+    // device ring on the launch stream just before the kernel.
+    char *h_ring = nullptr;
+    char *d_ring = nullptr;
+    size_t ring_bytes = 0;
+};
+
+// Returns the context of the current device, creating it on first use (nullptr + error set on failure).
+DeviceCtx *device_ctx();
+
+// Reserves `bytes` (multiple of 256) in the descriptor ring.  Blocks the host only when the ring wraps
+// onto a slice whose earlier launches have not finished.
+int ring_reserve(DeviceCtx *ctx, size_t bytes, hipStream_t stream, char **h, char **d);
+
+uint32_t grid_for(const DeviceCtx *ctx, uint64_t total_tiles);
+
+}  // namespace hcclx

@@ -1,0 +1,95 @@
+// C-ABI entry points of the V collectives (see include/hcclx.h).
+#include "hcclx.h"
+#include "hcclx_internal.h"
+#include "kernels/elem.h"
+#include "kernels/vops.h"
+
+#include <cstring>
+
+using namespace hcclx;
+
+namespace {
+
+// Host tables are staged through the descriptor ring; device tables are used where they are.
+int stage_tables(DeviceCtx *ctx, const uint64_t *const *tabs, int ntabs, size_t entries, int on_device,
+                 hipStream_t st, const uint64_t **out)
+{
+    if (on_device) {
+        for (int i = 0; i < ntabs; ++i) out[i] = tabs[i];
+        return HCCL_SUCCESS;
+    }
+    const size_t one = (entries * sizeof(uint64_t) + 255) & ~static_cast<size_t>(255);
+    char *h = nullptr;
+    char *d = nullptr;
+    int rc = ring_reserve(ctx, one * ntabs, st, &h, &d);
+    if (rc != HCCL_SUCCESS) return rc;
+    for (int i = 0; i < ntabs; ++i) {
+        std::memcpy(h + one * i, tabs[i], entries * sizeof(uint64_t));
+        out[i] = reinterpret_cast<const uint64_t *>(d + one * i);
+    }
+    HCCLX_HIP(hipMemcpyAsync(d, h, one * ntabs, hipMemcpyHostToDevice, st));
+    return HCCL_SUCCESS;
+}
+
+int fill_ptrs(const void *const *send, void *const *recv, uint32_t n, VRankPtrs *p)
+{
+    if (send == nullptr || recv == nullptr) return fail(HCCL_E_PTR, "send/recv pointer array is null");
+    if (n == 0 || n > kMaxVRanks) return fail(HCCL_E_PARA, "rank count outside 1.." + std::to_string(kMaxVRanks));
+    std::memset(p, 0, sizeof(*p));
+    for (uint32_t i = 0; i < n; ++i) {
+        p->send[i] = static_cast<const char *>(send[i]);
+        p->recv[i] = static_cast<char *>(recv[i]);
+    }
+    return HCCL_SUCCESS;
+}
+
+}  // namespace
+
+extern "C" {
+
+int hcclx_alltoallv(const void *const *send, void *const *recv, const uint64_t *send_counts,
+                    const uint64_t *sdispls, const uint64_t *rdispls, uint32_t n, int dtype,
+                    int tables_on_device, void *stream)
+{
+    DeviceCtx *ctx = device_ctx();
+    if (!ctx) return HCCL_E_RUNTIME;
+    const int esz = dtype_size(dtype);
+    if (esz == 0) return fail(HCCL_E_NOT_SUPPORT, "unknown data type " + std::to_string(dtype));
+    if (!send_counts || !sdispls || !rdispls) return fail(HCCL_E_PTR, "count/displacement table is null");
+    VRankPtrs ptrs;
+    int rc = fill_ptrs(send, recv, n, &ptrs);
+    if (rc != HCCL_SUCCESS) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint64_t *tabs[3] = {send_counts, sdispls, rdispls};
+    const uint64_t *dev[3];
+    rc = stage_tables(ctx, tabs, 3, static_cast<size_t>(n) * n, tables_on_device, st, dev);
+    if (rc != HCCL_SUCCESS) return rc;
+    const uint32_t grid = grid_for(ctx, ~0ull);
+    hipError_t e = launch_alltoallv(ptrs, dev[0], dev[1], dev[2], n, static_cast<uint32_t>(esz), grid, st);
+    if (e != hipSuccess) return fail_hip(e, "alltoallv kernel launch");
+    return HCCL_SUCCESS;
+}
+
+int hcclx_allgatherv(const void *const *send, void *const *recv, const uint64_t *counts,
+                     const uint64_t *displs, uint32_t n, int dtype, int tables_on_device, void *stream)
+{
+    DeviceCtx *ctx = device_ctx();
+    if (!ctx) return HCCL_E_RUNTIME;
+    const int esz = dtype_size(dtype);
+    if (esz == 0) return fail(HCCL_E_NOT_SUPPORT, "unknown data type " + std::to_string(dtype));
+    if (!counts || !displs) return fail(HCCL_E_PTR, "count/displacement table is null");
+    VRankPtrs ptrs;
+    int rc = fill_ptrs(send, recv, n, &ptrs);
+    if (rc != HCCL_SUCCESS) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint64_t *tabs[2] = {counts, displs};
+    const uint64_t *dev[2];
+    rc = stage_tables(ctx, tabs, 2, n, tables_on_device, st, dev);
+    if (rc != HCCL_SUCCESS) return rc;
+    const uint32_t grid = grid_for(ctx, ~0ull);
+    hipError_t e = launch_allgatherv(ptrs, dev[0], dev[1], n, static_cast<uint32_t>(esz), grid, st);
+    if (e != hipSuccess) return fail_hip(e, "allgatherv kernel launch");
+    return HCCL_SUCCESS;
+}
+
+}  // extern "C"

@@ -1,0 +1,222 @@
+// The fused fold kernel: every segment reads each of its sources once and writes each of its
+// destinations once, in a single pass over HBM.
+//
+// It replaces the reference's per-step primitives HcommLocalCopyOnThread / HcommLocalReduceOnThread /
+// Hcomm{Write,Read}[Reduce]OnThread (ABI visible in test/st/algorithm/utils/src/hccl_proxy/hccl_stub.cc:467,
+// :633, :664, :705) and, when a whole template is fused, the chains of them that the templates emit, e.g.
+// PostLocalReduce of the one-shot AllReduce (src/ops/all_reduce/template/aicpu/
+// ins_temp_all_reduce_mesh_1D_one_shot.cc:182-197) and PostCopy of the mesh ReduceScatter
+// (src/ops/reduce_scatter/template/aicpu/ins_temp_reduce_scatter_mesh_1D.cc:147-154).
+//
+// Bound: HBM bandwidth.  Algorithmic bytes per element: (nsrc + ndst) * sizeof(element).
+#pragma once
+#include "elem.h"
+#include "segtab.h"
+
+namespace hcclx {
+
+// 16-byte vectors each thread keeps in flight per source.  More sources -> fewer vectors per source, so
+// the loads outstanding per thread stay near 16 and the register file still holds several wavefronts.
+__host__ __device__ constexpr int fold_unroll(int maxn)
+{
+    return maxn <= 1 ? 8 : maxn <= 4 ? 4 : maxn <= 8 ? 2 : 1;
+}
+__host__ __device__ constexpr uint64_t fold_tile_vecs(int maxn)
+{
+    return static_cast<uint64_t>(kThreads) * fold_unroll(maxn);
+}
+
+__device__ __forceinline__ u32x4 ld16(const char *p)
+{
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4_u *>(p));
+}
+__device__ __forceinline__ void st16(char *p, u32x4 v)
+{
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4_u *>(p));
+}
+__device__ __forceinline__ uint64_t uniform64(uint64_t x)
+{
+    uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(x));
+    uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(x >> 32));
+    return (static_cast<uint64_t>(hi) << 32) | lo;
+}
+
+template <int DT, int OP, int MAXN, int MODE, bool CHECK>
+__device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint32_t ndst, uint64_t v0, uint64_t nvec)
+{
+    constexpr int UNROLL = fold_unroll(MAXN);
+    using V = Vec16<DT>;
+    using C = typename V::C;
+    constexpr int NE = V::NE;
+    using Op = Combine<DT, OP>;
+
+    u32x4 raw[UNROLL][MAXN];
+#pragma unroll
+    for (int k = 0; k < MAXN; ++k) {
+        if (k < static_cast<int>(nsrc)) {
+            const char *p = sd.src[k] + v0 * 16;
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                if (!CHECK || v0 + static_cast<uint64_t>(u) * kThreads < nvec) {
+                    raw[u][k] = ld16(p + static_cast<uint64_t>(u) * kThreads * 16);
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const uint64_t vi = v0 + static_cast<uint64_t>(u) * kThreads;
+        if (CHECK && vi >= nvec) {
+            continue;
+        }
+        if constexpr (MODE == kFoldChain) {
+            C acc[NE];
+            V::unpack(raw[u][0], acc);
+#pragma unroll
+            for (int k = 1; k < MAXN; ++k) {
+                if (k < static_cast<int>(nsrc)) {
+                    C x[NE];
+                    V::unpack(raw[u][k], x);
+#pragma unroll
+                    for (int e = 0; e < NE; ++e) acc[e] = Op::run(x[e], acc[e]);
+                }
+            }
+            const u32x4 out = V::pack(acc);
+            for (uint32_t d = 0; d < ndst; ++d) {
+                st16(sd.dst[d] + vi * 16, out);
+            }
+        } else {
+            C val[MAXN][NE];
+#pragma unroll
+            for (int k = 0; k < MAXN; ++k) {
+                if (k < static_cast<int>(nsrc)) V::unpack(raw[u][k], val[k]);
+            }
+#pragma unroll
+            for (int j = 0; j < MAXN; ++j) {
+                if (j < static_cast<int>(nsrc)) {
+                    C acc[NE];
+#pragma unroll
+                    for (int e = 0; e < NE; ++e) acc[e] = val[j][e];
+#pragma unroll
+                    for (int k = 0; k < MAXN; ++k) {
+                        if (k != j && k < static_cast<int>(nsrc)) {
+#pragma unroll
+                            for (int e = 0; e < NE; ++e) acc[e] = Op::run(val[k][e], acc[e]);
+                        }
+                    }
+                    st16(sd.dst[j] + vi * 16, V::pack(acc));
+                }
+            }
+        }
+    }
+}
+
+// The last (count % NE) elements of a segment, one per thread.
+template <int DT, int OP, int MODE>
+__device__ __forceinline__ void fold_tail(const SegDev &sd, uint32_t nsrc, uint32_t ndst, uint64_t idx)
+{
+    using D = DTypeOf<DT>;
+    using S = typename D::S;
+    using C = typename D::C;
+    using Op = Combine<DT, OP>;
+    if constexpr (MODE == kFoldChain) {
+        C acc = D::widen(reinterpret_cast<const S *>(sd.src[0])[idx]);
+        for (uint32_t k = 1; k < nsrc; ++k) {
+            acc = Op::run(D::widen(reinterpret_cast<const S *>(sd.src[k])[idx]), acc);
+        }
+        const S out = D::narrow(acc);
+        for (uint32_t d = 0; d < ndst; ++d) reinterpret_cast<S *>(sd.dst[d])[idx] = out;
+    } else {
+        // Every source is read before the first destination is written: a destination may alias a source.
+        C val[kMaxFan];
+        for (uint32_t k = 0; k < nsrc; ++k) val[k] = D::widen(reinterpret_cast<const S *>(sd.src[k])[idx]);
+        for (uint32_t j = 0; j < nsrc; ++j) {
+            C acc = val[j];
+            for (uint32_t k = 0; k < nsrc; ++k) {
+                if (k != j) acc = Op::run(val[k], acc);
+            }
+            reinterpret_cast<S *>(sd.dst[j])[idx] = D::narrow(acc);
+        }
+    }
+}
+
+template <int DT, int OP, int MAXN, int MODE>
+__global__ void __launch_bounds__(kThreads)
+k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, uint32_t nseg, uint64_t total_tiles)
+{
+    constexpr int NE = Vec16<DT>::NE;
+    constexpr uint64_t TV = fold_tile_vecs(MAXN);
+    extern __shared__ uint64_t s_end[];  // nseg entries, sized by the launcher
+    for (uint32_t i = threadIdx.x; i < nseg; i += kThreads) {
+        s_end[i] = tile_end[i];
+    }
+    __syncthreads();
+
+    for (uint64_t t = blockIdx.x; t < total_tiles; t += gridDim.x) {
+        // first segment whose inclusive tile prefix exceeds t
+        uint32_t lo = 0;
+        uint32_t hi = nseg - 1;
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (s_end[mid] > t) {
+                hi = mid;
+            } else {
+                lo = mid + 1;
+            }
+        }
+        const uint32_t s = __builtin_amdgcn_readfirstlane(lo);
+        const uint64_t tl = uniform64(t - (s ? s_end[s - 1] : 0));
+        const SegDev &sd = segs[s];
+        const uint32_t nsrc = sd.nsrc;
+        const uint32_t ndst = sd.ndst;
+        const uint64_t count = sd.count;
+        const uint64_t nvec = count / NE;
+        const uint32_t rem = static_cast<uint32_t>(count % NE);
+        const uint64_t v0 = tl * TV + threadIdx.x;
+        if ((tl + 1) * TV <= nvec) {
+            fold_tile<DT, OP, MAXN, MODE, false>(sd, nsrc, ndst, v0, nvec);
+        } else {
+            fold_tile<DT, OP, MAXN, MODE, true>(sd, nsrc, ndst, v0, nvec);
+            if (rem != 0 && tl == nvec / TV && threadIdx.x < rem) {
+                fold_tail<DT, OP, MODE>(sd, nsrc, ndst, nvec * NE + threadIdx.x);
+            }
+        }
+    }
+}
+
+// Host-side geometry, used by the launcher to build tile_end[].
+inline uint64_t fold_tiles_of(uint64_t count, int ne, int maxn)
+{
+    if (count == 0) {
+        return 0;
+    }
+    const uint64_t nvec = count / ne;
+    const uint64_t units = nvec + ((count % ne) ? 1 : 0);
+    const uint64_t tv = fold_tile_vecs(maxn);
+    return (units + tv - 1) / tv;
+}
+
+struct FoldLaunch {
+    const uint64_t *tile_end;  // device
+    const SegDev *segs;        // device
+    uint32_t nseg;
+    uint64_t total_tiles;
+    uint32_t grid;
+    hipStream_t stream;
+};
+
+// One translation unit per data type defines these (fold_inst.hip).
+#define HCCLX_DECLARE_FOLD(NAME) hipError_t fold_dispatch_##NAME(int op, int maxn, int mode, const FoldLaunch &l);
+HCCLX_DECLARE_FOLD(i8)
+HCCLX_DECLARE_FOLD(i16)
+HCCLX_DECLARE_FOLD(i32)
+HCCLX_DECLARE_FOLD(i64)
+HCCLX_DECLARE_FOLD(u64)
+HCCLX_DECLARE_FOLD(f16)
+HCCLX_DECLARE_FOLD(f32)
+HCCLX_DECLARE_FOLD(f64)
+HCCLX_DECLARE_FOLD(bf16)
+hipError_t fold_dispatch_copy(const FoldLaunch &l);
+
+}  // namespace hcclx

@@ -1,0 +1,69 @@
+// One data type's instantiations of the fold kernel.  Built once per type with
+//   -DHCCLX_DT=<HcclDataType enumerator> -DHCCLX_NAME=<suffix> -DHCCLX_ORDERED=<0|1>
+// HCCLX_ORDERED=1 (floating types) also builds the self-first mode; for integers every fold order gives
+// the same bits, so the launcher maps that mode onto the chain kernel.
+// With -DHCCLX_COPY the unit holds the byte copy kernel instead (one source, many destinations).
+#include "fold.h"
+
+namespace hcclx {
+
+template <int DT, int OP, int MAXN, int MODE>
+static hipError_t launch_one(const FoldLaunch &l)
+{
+    hipLaunchKernelGGL((k_fold<DT, OP, MAXN, MODE>), dim3(l.grid), dim3(kThreads), l.nseg * sizeof(uint64_t), l.stream,
+                       l.tile_end, l.segs, l.nseg, l.total_tiles);
+    return hipGetLastError();
+}
+
+#ifdef HCCLX_COPY
+
+hipError_t fold_dispatch_copy(const FoldLaunch &l)
+{
+    return launch_one<HCCL_DATA_TYPE_INT8, HCCL_REDUCE_SUM, 1, kFoldChain>(l);
+}
+
+#else
+
+template <int OP, int MODE>
+static hipError_t by_fan(int maxn, const FoldLaunch &l)
+{
+    switch (maxn) {
+        case 2: return launch_one<HCCLX_DT, OP, 2, MODE>(l);
+        case 4: return launch_one<HCCLX_DT, OP, 4, MODE>(l);
+        case 8: return launch_one<HCCLX_DT, OP, 8, MODE>(l);
+        case 16: return launch_one<HCCLX_DT, OP, 16, MODE>(l);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+template <int MODE>
+static hipError_t by_op(int op, int maxn, const FoldLaunch &l)
+{
+    switch (op) {
+        case HCCL_REDUCE_SUM: return by_fan<HCCL_REDUCE_SUM, MODE>(maxn, l);
+        case HCCL_REDUCE_PROD: return by_fan<HCCL_REDUCE_PROD, MODE>(maxn, l);
+        case HCCL_REDUCE_MAX: return by_fan<HCCL_REDUCE_MAX, MODE>(maxn, l);
+        case HCCL_REDUCE_MIN: return by_fan<HCCL_REDUCE_MIN, MODE>(maxn, l);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+#define HCCLX_CAT_(a, b) a##b
+#define HCCLX_CAT(a, b) HCCLX_CAT_(a, b)
+
+hipError_t HCCLX_CAT(fold_dispatch_, HCCLX_NAME)(int op, int maxn, int mode, const FoldLaunch &l)
+{
+    if (mode == kFoldChain) {
+        return by_op<kFoldChain>(op, maxn, l);
+    }
+#if HCCLX_ORDERED
+    if (mode == kFoldSelfFirst) {
+        return by_op<kFoldSelfFirst>(op, maxn, l);
+    }
+#endif
+    return hipErrorInvalidValue;
+}
+
+#endif
+
+}  // namespace hcclx

@@ -1,0 +1,32 @@
+// Device-side work tables shared by the host launcher and the kernels.
+//
+// A launch processes a list of segments.  A segment is one contiguous run of elements with up to
+// kMaxFan sources and up to kMaxFan destinations; it is cut into tiles of 256 threads x UNROLL x 16 B
+// (per source).  tile_end[] is the inclusive prefix sum of tiles per segment, staged into LDS by every
+// workgroup and binary-searched to map a tile number to its segment.
+#pragma once
+#include <stdint.h>
+
+namespace hcclx {
+
+constexpr int kMaxFan = 16;        // sources fused in one pass / destinations written in one pass
+constexpr int kThreads = 256;      // workgroup size: 4 wavefronts of 64
+constexpr int kMaxSegsPerLaunch = 2048;  // tile_end[] must fit the LDS staging array (16 KiB)
+
+struct SegDev {
+    uint64_t count;            // elements (bytes for the copy kernel)
+    uint32_t nsrc;
+    uint32_t ndst;
+    const char *src[kMaxFan];  // in fold order
+    char *dst[kMaxFan];
+};
+
+// How the sources of a segment are folded.
+enum FoldMode : int {
+    // acc = src[0]; for k = 1..nsrc-1: acc = src[k] (+) acc; the one value goes to every dst.
+    kFoldChain = 0,
+    // nsrc == ndst; dst[j] = fold starting from src[j], then src[k] for k ascending, k != j.
+    kFoldSelfFirst = 1,
+};
+
+}  // namespace hcclx

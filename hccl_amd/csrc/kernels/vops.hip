@@ -1,0 +1,213 @@
+// Ragged data movement of the V collectives: AlltoAllV pack/unpack and AllGatherV, for n virtual ranks
+// whose buffers live in one GPU.
+//
+// Reference behaviour restated (one copy instead of the reference's pack -> CCL slot -> unpack pair):
+//   AlltoAllV  in_i[sdispls_i[j] .. +sendCounts_i[j])  ->  out_j[rdispls_j[i] .. )
+//              src/ops/all_to_all_v/template/aicpu/ins_temp_all_to_all_v_mesh_1D.cc:304-308 (pack into the
+//              peer's CCL slot), :431-438 (unpack), :161-170 (self block)
+//   AllGatherV out_j[displs[i] .. +counts[i]) = in_i[0 .. counts[i])   for all i, j
+//              src/ops/all_gather_v/template/aicpu/ins_temp_all_gather_v_mesh_1D.cc:97-242;
+//              contract include/hccl.h:120-135
+//
+// The count/displacement tables stay on the device.  Each workgroup stages the per-block tile counts in
+// LDS, turns them into an inclusive prefix with a wavefront scan, and then walks tile numbers in a
+// grid-stride loop, locating a tile's (source, destination) block by binary search in LDS.  No host
+// round trip is needed when the tables come from an on-device router.
+//
+// Bound: HBM bandwidth.  Algorithmic bytes: AlltoAllV 2 x payload; AllGatherV (1 + n) x payload moved,
+// 2n x payload delivered.
+#include "fold.h"
+#include "vops.h"
+
+namespace hcclx {
+
+namespace {
+
+constexpr int kCopyUnroll = 8;
+constexpr uint32_t kTileVecs = kThreads * kCopyUnroll;  // 16-byte vectors per tile
+constexpr uint32_t kTileBytes = kTileVecs * 16;         // 32 KiB
+
+// Tiles of a block of `bytes` bytes whose first destination byte sits at address `dst`.
+// Stores are aligned: the bytes before the first 16-byte boundary of dst (head) and after the last
+// whole vector (tail) are moved one byte per thread by the block's last tile.
+__device__ __forceinline__ uint64_t tiles_of(uint64_t bytes, uint64_t dst)
+{
+    if (bytes == 0) return 0;
+    uint64_t head = (16 - (dst & 15)) & 15;
+    if (head > bytes) head = bytes;
+    return (bytes - head) / 16 / kTileVecs + 1;
+}
+
+__device__ __forceinline__ uint64_t wave_inclusive_scan(uint64_t v)
+{
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t lo = __shfl_up(static_cast<uint32_t>(v), d, 64);
+        const uint32_t hi = __shfl_up(static_cast<uint32_t>(v >> 32), d, 64);
+        if (lane >= d) v += (static_cast<uint64_t>(hi) << 32) | lo;
+    }
+    return v;
+}
+
+// In place: s_tab[0..m) (per-block tile counts) becomes its inclusive prefix sum.  m <= 4096.
+// Each thread sums a contiguous run, a wavefront scan orders the 64 runs of a wave, and the four wave
+// totals are combined through LDS.
+__device__ void block_inclusive_scan(uint64_t *s_tab, uint32_t m, uint64_t *s_wave)
+{
+    const uint32_t per = (m + kThreads - 1) / kThreads;
+    const uint32_t b = threadIdx.x * per;
+    const uint32_t e = (b + per < m) ? b + per : m;
+    uint64_t sum = 0;
+    for (uint32_t i = b; i < e; ++i) sum += s_tab[i];
+    const uint64_t incl = wave_inclusive_scan(sum);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 63) s_wave[wave] = incl;
+    __syncthreads();
+    uint64_t base = incl - sum;
+    for (int w = 0; w < wave; ++w) base += s_wave[w];
+    for (uint32_t i = b; i < e; ++i) {
+        base += s_tab[i];
+        s_tab[i] = base;
+    }
+    __syncthreads();
+}
+
+__device__ __forceinline__ uint32_t find_block(const uint64_t *s_end, uint32_t m, uint64_t t)
+{
+    uint32_t lo = 0;
+    uint32_t hi = m - 1;
+    while (lo < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (s_end[mid] > t) {
+            hi = mid;
+        } else {
+            lo = mid + 1;
+        }
+    }
+    return __builtin_amdgcn_readfirstlane(lo);
+}
+
+// One tile of a block copy: tile `tl` of a block of `bytes` bytes from src to dst[0..ndst) (all
+// destinations share dst[0]'s alignment modulo 16, or lose only speed if they do not).
+template <typename DstFn>
+__device__ __forceinline__ void copy_tile(const char *src, uint64_t dst0, uint64_t bytes, uint64_t tl, uint32_t ndst,
+                                          DstFn dst_of)
+{
+    uint64_t head = (16 - (dst0 & 15)) & 15;
+    if (head > bytes) head = bytes;
+    const uint64_t body = bytes - head;
+    const uint64_t nvec = body / 16;
+    const uint64_t v0 = tl * kTileVecs + threadIdx.x;
+    const char *sb = src + head;
+    if ((tl + 1) * kTileVecs <= nvec) {
+        u32x4 r[kCopyUnroll];
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u) r[u] = ld16(sb + (v0 + static_cast<uint64_t>(u) * kThreads) * 16);
+        for (uint32_t d = 0; d < ndst; ++d) {
+            char *db = dst_of(d) + head;
+#pragma unroll
+            for (int u = 0; u < kCopyUnroll; ++u) st16(db + (v0 + static_cast<uint64_t>(u) * kThreads) * 16, r[u]);
+        }
+        return;
+    }
+    // last tile of the block: remaining vectors, then head and tail bytes
+    u32x4 r[kCopyUnroll];
+#pragma unroll
+    for (int u = 0; u < kCopyUnroll; ++u) {
+        const uint64_t vi = v0 + static_cast<uint64_t>(u) * kThreads;
+        if (vi < nvec) r[u] = ld16(sb + vi * 16);
+    }
+    const uint64_t tail = body - nvec * 16;
+    char edge = 0;
+    uint64_t edge_off = 0;
+    const bool has_edge = threadIdx.x < head + tail;
+    if (has_edge) {
+        edge_off = (threadIdx.x < head) ? threadIdx.x : head + nvec * 16 + (threadIdx.x - head);
+        edge = src[edge_off];
+    }
+    for (uint32_t d = 0; d < ndst; ++d) {
+        char *dp = dst_of(d);
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u) {
+            const uint64_t vi = v0 + static_cast<uint64_t>(u) * kThreads;
+            if (vi < nvec) st16(dp + head + vi * 16, r[u]);
+        }
+        if (has_edge) dp[edge_off] = edge;
+    }
+}
+
+__global__ void __launch_bounds__(kThreads)
+k_alltoallv(VRankPtrs ptrs, const uint64_t *__restrict__ send_counts, const uint64_t *__restrict__ sdispls,
+            const uint64_t *__restrict__ rdispls, uint32_t n, uint32_t esz)
+{
+    extern __shared__ uint64_t s_end[];  // n*n entries, then 4 wave totals
+    const uint32_t m = n * n;
+    uint64_t *s_wave = s_end + m;
+    for (uint32_t p = threadIdx.x; p < m; p += kThreads) {
+        const uint32_t i = p / n;
+        const uint32_t j = p - i * n;
+        const uint64_t dst = reinterpret_cast<uint64_t>(ptrs.recv[j]) + rdispls[j * n + i] * esz;
+        s_end[p] = tiles_of(send_counts[p] * esz, dst);
+    }
+    __syncthreads();
+    block_inclusive_scan(s_end, m, s_wave);
+    const uint64_t total = s_end[m - 1];
+
+    for (uint64_t t = blockIdx.x; t < total; t += gridDim.x) {
+        const uint32_t p = find_block(s_end, m, t);
+        const uint64_t tl = uniform64(t - (p ? s_end[p - 1] : 0));
+        const uint32_t i = p / n;
+        const uint32_t j = p - i * n;
+        const uint64_t bytes = send_counts[p] * esz;
+        const char *src = ptrs.send[i] + sdispls[p] * esz;
+        char *dst = ptrs.recv[j] + rdispls[j * n + i] * esz;
+        copy_tile(src, reinterpret_cast<uint64_t>(dst), bytes, tl, 1, [=](uint32_t) { return dst; });
+    }
+}
+
+__global__ void __launch_bounds__(kThreads)
+k_allgatherv(VRankPtrs ptrs, const uint64_t *__restrict__ counts, const uint64_t *__restrict__ displs, uint32_t n,
+             uint32_t esz)
+{
+    extern __shared__ uint64_t s_end[];  // n entries, then 4 wave totals
+    uint64_t *s_wave = s_end + n;
+    for (uint32_t i = threadIdx.x; i < n; i += kThreads) {
+        const uint64_t dst = reinterpret_cast<uint64_t>(ptrs.recv[0]) + displs[i] * esz;
+        s_end[i] = tiles_of(counts[i] * esz, dst);
+    }
+    __syncthreads();
+    block_inclusive_scan(s_end, n, s_wave);
+    const uint64_t total = s_end[n - 1];
+
+    for (uint64_t t = blockIdx.x; t < total; t += gridDim.x) {
+        const uint32_t i = find_block(s_end, n, t);
+        const uint64_t tl = uniform64(t - (i ? s_end[i - 1] : 0));
+        const uint64_t bytes = counts[i] * esz;
+        const uint64_t off = displs[i] * esz;
+        const char *src = ptrs.send[i];
+        copy_tile(src, reinterpret_cast<uint64_t>(ptrs.recv[0]) + off, bytes, tl, n,
+                  [&](uint32_t d) { return ptrs.recv[d] + off; });
+    }
+}
+
+}  // namespace
+
+hipError_t launch_alltoallv(const VRankPtrs &ptrs, const uint64_t *send_counts, const uint64_t *sdispls,
+                            const uint64_t *rdispls, uint32_t n, uint32_t esz, uint32_t grid, hipStream_t stream)
+{
+    const size_t lds = (static_cast<size_t>(n) * n + 4) * sizeof(uint64_t);
+    hipLaunchKernelGGL(k_alltoallv, dim3(grid), dim3(kThreads), lds, stream, ptrs, send_counts, sdispls, rdispls, n,
+                       esz);
+    return hipGetLastError();
+}
+
+hipError_t launch_allgatherv(const VRankPtrs &ptrs, const uint64_t *counts, const uint64_t *displs, uint32_t n,
+                             uint32_t esz, uint32_t grid, hipStream_t stream)
+{
+    const size_t lds = (static_cast<size_t>(n) + 4) * sizeof(uint64_t);
+    hipLaunchKernelGGL(k_allgatherv, dim3(grid), dim3(kThreads), lds, stream, ptrs, counts, displs, n, esz);
+    return hipGetLastError();
+}
+
+}  // namespace hcclx

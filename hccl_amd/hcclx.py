@@ -1,0 +1,89 @@
+"""Python face of the hcclx C ABI (include/hcclx.h).  Pointers are plain integers (device addresses)."""
+import ctypes
+
+from . import _lib
+from ._lib import Seg, check
+
+FOLD_CHAIN = 0
+FOLD_SELF_FIRST = 1
+
+
+def make_segs(segs):
+    """segs: iterable of (count, [src addresses], [dst addresses]) -> ctypes array of hcclx_seg_t."""
+    segs = list(segs)
+    arr = (Seg * max(1, len(segs)))()
+    for i, (count, srcs, dsts) in enumerate(segs):
+        arr[i].count = count
+        arr[i].nsrc = len(srcs)
+        arr[i].ndst = len(dsts)
+        for k, p in enumerate(srcs):
+            arr[i].src[k] = p
+        for k, p in enumerate(dsts):
+            arr[i].dst[k] = p
+    return arr, len(segs)
+
+
+def init():
+    check(_lib.load().hcclx_init())
+
+
+def fold(segs, dtype, op=0, mode=FOLD_CHAIN, stream=0):
+    arr, n = make_segs(segs)
+    check(_lib.load().hcclx_fold(arr, n, int(dtype), int(op), int(mode), ctypes.c_void_p(stream)))
+
+
+class Plan:
+    """A fold whose table already sits in device memory: launch() is one kernel launch."""
+
+    def __init__(self, segs, dtype, op=0, mode=FOLD_CHAIN):
+        arr, n = make_segs(segs)
+        h = ctypes.c_void_p()
+        check(_lib.load().hcclx_plan_create(arr, n, int(dtype), int(op), int(mode), ctypes.byref(h)))
+        self._h = h
+
+    @property
+    def bytes(self):
+        return _lib.load().hcclx_plan_bytes(self._h)
+
+    def launch(self, stream=0):
+        check(_lib.load().hcclx_plan_launch(self._h, ctypes.c_void_p(stream)))
+
+    def close(self):
+        if self._h:
+            _lib.load().hcclx_plan_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def _ptr_array(ptrs):
+    return (ctypes.c_void_p * len(ptrs))(*ptrs)
+
+
+def _table(t):
+    """Host table (sequence of ints / numpy uint64 array) or device address (int)."""
+    if isinstance(t, int):
+        return ctypes.c_void_p(t), None
+    arr = (ctypes.c_uint64 * len(t))(*[int(x) for x in t])
+    return ctypes.cast(arr, ctypes.c_void_p), arr
+
+
+def alltoallv(send, recv, send_counts, sdispls, rdispls, dtype, on_device=False, stream=0):
+    n = len(send)
+    a, ka = _table(send_counts)
+    b, kb = _table(sdispls)
+    c, kc = _table(rdispls)
+    check(_lib.load().hcclx_alltoallv(_ptr_array(send), _ptr_array(recv), a, b, c, n, int(dtype),
+                                      1 if on_device else 0, ctypes.c_void_p(stream)))
+
+
+def allgatherv(send, recv, counts, displs, dtype, on_device=False, stream=0):
+    n = len(send)
+    a, ka = _table(counts)
+    b, kb = _table(displs)
+    check(_lib.load().hcclx_allgatherv(_ptr_array(send), _ptr_array(recv), a, b, n, int(dtype),
+                                       1 if on_device else 0, ctypes.c_void_p(stream)))

@@ -1,0 +1,102 @@
+/*
+ * hcclx.h -- the thin C ABI over the HIP kernels of the virtual-rank backend.
+ *
+ * This is the boundary a host runtime binds (C++, cgo, JNI, ctypes ...): plain pointers and sizes, no
+ * C++ or torch types.  All data pointers are device pointers in one GPU's HBM; tables (segment lists,
+ * host count arrays) are host pointers unless stated otherwise.  `stream` is a hipStream_t (NULL = the
+ * default stream).  Work is enqueued, not completed, when a call returns.  Every function returns an
+ * HcclResult value (0 = HCCL_SUCCESS); hcclx_last_error() gives the text of the last failure on the
+ * calling thread.
+ *
+ * What each entry point replaces in the reference (paths relative to the reference tree):
+ *   hcclx_fold / hcclx_plan_*   the Hcomm data primitives the templates enqueue -- HcommLocalCopyOnThread,
+ *                               HcommLocalReduceOnThread, HcommWriteOnThread, HcommReadOnThread,
+ *                               HcommWriteReduceOnThread, HcommReadReduceOnThread
+ *                               (test/st/algorithm/utils/src/hccl_proxy/hccl_stub.cc:467, :633, :495, :534,
+ *                               :664, :705) and the CPU reduce AicpuReduce
+ *                               (src/ops/op_common/template/wrapper/alg_data_trans_wrapper.cc:1165-1252);
+ *   hcclx_alltoallv             pack/unpack of InsTempAlltoAllVMesh1D
+ *                               (src/ops/all_to_all_v/template/aicpu/ins_temp_all_to_all_v_mesh_1D.cc:275-339,
+ *                               :412-440);
+ *   hcclx_allgatherv            InsTempAllGatherVMesh1D
+ *                               (src/ops/all_gather_v/template/aicpu/ins_temp_all_gather_v_mesh_1D.cc:97-242).
+ */
+#ifndef HCCL_AMD_HCCLX_H_
+#define HCCL_AMD_HCCLX_H_
+
+#include <stdint.h>
+#include "hccl_types.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HCCLX_MAX_FAN 16
+
+/* How the sources of a segment are folded; every step is  acc = src (+) acc  (operand order of
+ * AicpuReduceTemplate, alg_data_trans_wrapper.cc:1226-1243). */
+typedef enum {
+    /* acc = src[0]; for k = 1 .. nsrc-1: acc = src[k] (+) acc; the result goes to dst[0 .. ndst-1]. */
+    HCCLX_FOLD_CHAIN = 0,
+    /* nsrc == ndst; dst[j] = fold that starts from src[j] and then takes src[k], k ascending, k != j:
+     * the per-rank order of the one-shot AllReduce and of the CPU-reduce NHR AllReduce
+     * (ins_temp_all_reduce_mesh_1D_one_shot.cc:182-197, ins_temp_all_reduce_aicpu_reduce_nhr.cc:226-233). */
+    HCCLX_FOLD_SELF_FIRST = 1
+} hcclx_fold_mode_t;
+
+/* One contiguous run of `count` elements: nsrc sources (fold order), ndst destinations.
+ * nsrc == 1 is a copy (to ndst places).  A destination may be the same run as one of the sources (an
+ * in-place step); any other overlap between a destination and a source of the same launch is a race. */
+typedef struct {
+    uint64_t count;
+    uint32_t nsrc;
+    uint32_t ndst;
+    const void *src[HCCLX_MAX_FAN];
+    void *dst[HCCLX_MAX_FAN];
+} hcclx_seg_t;
+
+/* Library set-up for the current device: creates the descriptor arena.  Idempotent.  Called lazily by the
+ * other entry points; call it yourself to keep allocation out of the first timed call. */
+int hcclx_init(void);
+
+/* Text of the last error raised on this thread ("" if none). */
+const char *hcclx_last_error(void);
+
+/* Size in bytes of an HcclDataType (0 if unknown).  DATATYPE_SIZE_TABLE, alg_param.h:43-45. */
+uint32_t hcclx_dtype_size(int dtype);
+
+/* Fold (reduce and/or copy) a list of segments in one pass over HBM.
+ * dtype: HcclDataType of the elements; reduce types are int8 int16 int32 int64 uint64 fp16 fp32 fp64 bf16.
+ * For nsrc == 1 everywhere any dtype with a known size is accepted (pure copy).  op: HcclReduceOp.
+ * All segments of a call share nsrc's upper bound HCCLX_MAX_FAN.  segs is a host array, copied before
+ * return. */
+int hcclx_fold(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, void *stream);
+
+/* The same, split in two so that a repeated collective uploads its table once. */
+typedef struct hcclx_plan hcclx_plan_t;
+int hcclx_plan_create(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, hcclx_plan_t **plan);
+int hcclx_plan_launch(const hcclx_plan_t *plan, void *stream);
+int hcclx_plan_destroy(hcclx_plan_t *plan);
+/* Algorithmic bytes one launch of the plan moves: sum over segments of (nsrc + ndst) * count * size. */
+uint64_t hcclx_plan_bytes(const hcclx_plan_t *plan);
+
+/* AlltoAllV among n virtual ranks whose buffers live in this GPU.
+ *   send[i], recv[i]      device base pointers of rank i                               (host arrays, n)
+ *   send_counts[i*n + j]  elements rank i sends to rank j, taken at sdispls[i*n + j]
+ *   rdispls[j*n + i]      element offset in recv[j] where the block from rank i lands
+ * counts/displacements are uint64 in elements, row-major n x n.  If tables_on_device is non-zero the
+ * three tables are device pointers (e.g. produced by an on-device router) and no host copy of them is
+ * read; the kernel stages them into LDS and derives its tile map with a wavefront prefix sum. */
+int hcclx_alltoallv(const void *const *send, void *const *recv, const uint64_t *send_counts,
+                    const uint64_t *sdispls, const uint64_t *rdispls, uint32_t n, int dtype,
+                    int tables_on_device, void *stream);
+
+/* AllGatherV among n virtual ranks: recv[j][displs[i] .. displs[i]+counts[i]) = send[i][0 .. counts[i])
+ * for every i and j; each source element is read once and written n times.  counts/displs as above. */
+int hcclx_allgatherv(const void *const *send, void *const *recv, const uint64_t *counts,
+                     const uint64_t *displs, uint32_t n, int dtype, int tables_on_device, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HCCL_AMD_HCCLX_H_ */
