@@ -1,0 +1,231 @@
+"""Pins oracle/templates.py: the schedules must satisfy what the reference's semantics checkers demand
+(every output element reduced from each rank exactly once, at the right offset), agree with plain numpy
+folds wherever the operator is associative, reduce to a single pairwise op for two ranks, and show the
+association orders the step formulas imply."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+
+from oracle import templates as T
+
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "st_cases.json")))
+AR_ALGS = list(T.ALLREDUCE_TEMPLATES)
+RS_ALGS = list(T.REDUCE_SCATTER_TEMPLATES)
+
+
+def sym_inputs(n, count, tag_index=False):
+    out = []
+    for r in range(n):
+        a = np.empty(count, dtype=object)
+        a[:] = [f"x{r}[{i}]" if tag_index else f"x{r}" for i in range(count)]
+        out.append(a)
+    return out
+
+
+def leaves(expr):
+    return sorted(expr.replace("(", "").replace(")", "").split("+"))
+
+
+@pytest.mark.parametrize("alg", AR_ALGS)
+@pytest.mark.parametrize("n", [2, 3, 4, 5, 7, 8, 12, 13, 16])
+def test_allreduce_every_element_reduces_every_rank_once_at_its_own_offset(alg, n):
+    for count in (1, n - 1, n, 3 * n + 2):
+        outs = T.run_allreduce(T.SymbolicElems(), sym_inputs(n, count, True), count, 4, alg)
+        for r in range(n):
+            for i in range(count):
+                assert leaves(outs[r][i]) == sorted(f"x{k}[{i}]" for k in range(n)), (alg, n, count, r, i)
+
+
+@pytest.mark.parametrize("alg", RS_ALGS)
+@pytest.mark.parametrize("n", [2, 3, 5, 8, 12])
+def test_reduce_scatter_shard_offsets(alg, n):
+    rc = 5
+    outs = T.run_reduce_scatter(T.SymbolicElems(), sym_inputs(n, n * rc, True), rc, 2, alg)
+    for r in range(n):
+        for i in range(rc):
+            assert leaves(outs[r][i]) == sorted(f"x{k}[{r * rc + i}]" for k in range(n))
+
+
+@pytest.mark.parametrize("alg", AR_ALGS + RS_ALGS)
+def test_two_ranks_is_one_pairwise_op(alg):
+    if alg in T.ALLREDUCE_TEMPLATES:
+        outs = T.run_allreduce(T.SymbolicElems(), sym_inputs(2, 2), 2, 4, alg)
+    else:
+        outs = T.run_reduce_scatter(T.SymbolicElems(), sym_inputs(2, 2), 1, 4, alg)
+    for o in outs:
+        assert o[0] in ("(x0+x1)", "(x1+x0)")
+
+
+def test_nhr_association_order_matches_hand_worked_shapes():
+    for n_str, want in GOLD["nhr"]["slice0"].items():
+        n = int(n_str)
+        outs = T.run_allreduce(T.SymbolicElems(), sym_inputs(n, n), n, 4, "InsAllReduceNHR")
+        assert all(o[0] == want for o in outs)
+        # other slices rotate the rank indices by the slice number
+        for k in range(1, n):
+            rot = want
+            for r in reversed(range(n)):
+                rot = rot.replace(f"x{r}+", f"y{(r + k) % n}+").replace(f"x{r})", f"y{(r + k) % n})")
+            assert outs[0][k] == rot.replace("y", "x")
+        rs = T.run_reduce_scatter(T.SymbolicElems(), sym_inputs(n, n), 1, 4, "InsReduceScatterNHR")
+        assert rs[0][0] == want
+
+
+def test_nhr_step_table_rank0_of_12():
+    steps = T.nhr_rs_steps(12, 0)
+    assert [{"to": s[0], "tx": s[2]} for s in steps] == GOLD["nhr"]["rank0_of_12_steps"]
+
+
+@pytest.mark.parametrize("n", range(2, 65))
+def test_nhr_closed_forms(n):
+    ns = T.nhr_step_num(n)
+    assert ns == math.ceil(math.log2(n))
+    total = 0
+    for s in range(ns):
+        for r in range(n):
+            to, frm, tx, rx = T.nhr_rs_steps(n, r)[s]
+            assert to == (r - (1 << s)) % n and frm == (r + (1 << s)) % n
+            assert not set(tx) & set(rx)                      # a step never sends what it receives
+            assert T.nhr_rs_steps(n, to)[s][3] == tx          # the peer expects exactly these slices
+            for k in tx:                                       # sender rule on d = (rank - slice) mod n
+                d = (r - k) % n
+                assert d % (1 << (s + 1)) == (1 << s)
+            if r == 0:
+                total += len(tx)
+    assert total == n - 1
+    have = {r: {r} for r in range(n)}                        # all-gather completeness
+    for s in range(ns):
+        new = {r: set(have[r]) for r in range(n)}
+        for r in range(n):
+            to, _, tx, _ = T.nhr_ag_steps(n, r)[s]
+            assert set(tx) <= have[r]
+            new[to] |= set(tx)
+        have = new
+    assert all(have[r] == set(range(n)) for r in range(n))
+
+
+def test_self_first_orders():
+    n = 5
+    for alg in ("InsAllReduceMesh1DOneShot", "InsAllReduceAicpuReduceNHR"):
+        outs = T.run_allreduce(T.SymbolicElems(), sym_inputs(n, 1), 1, 4, alg)
+        for r in range(n):
+            want = f"x{r}"
+            for k in range(n):
+                if k != r:
+                    want = f"(x{k}+{want})"
+            assert outs[r][0] == want
+    outs = T.run_reduce_scatter(T.SymbolicElems(), sym_inputs(n, n), 1, 4, "InsReduceScatterMesh1D")
+    assert outs[2][0] == "(x4+(x3+(x1+(x0+x2))))"
+    outs = T.run_allreduce(T.SymbolicElems(), sym_inputs(n, 1), 1, 4, "InsAllReduceMesh1DTwoShot")
+    assert all(o[0] == "(x4+(x3+(x2+(x1+x0))))" for o in outs)
+
+
+@pytest.mark.parametrize("count,n", [(0, 4), (1, 4), (3, 4), (4, 4), (5, 4), (17, 8), (1048576, 8), (100, 12)])
+def test_split_data_tiles_the_range(count, n):
+    sl = T.split_data(count, n)
+    assert len(sl) == n
+    off = 0
+    short_seen = False
+    full = -(-count // n)
+    for o, c in sl:
+        assert o == off
+        off += c
+        if short_seen:
+            assert c == 0
+        elif c < full:
+            short_seen = True
+    assert off == count
+
+
+def test_chunk_sizes_of_the_default_scratch_buffer():
+    ccl = T.CCL_BYTES_DEFAULT
+    ch = T.chunk_counts(1 << 40, ccl - (1 << 20), 8, 1, ccl - (1 << 20))
+    assert ch[0][1] == GOLD["chunks"]["reduce_scatter_mesh_n8"]
+    ch = T.chunk_counts(1 << 30, ccl, 12, 1, ccl)
+    assert ch[0][1] == GOLD["chunks"]["allreduce_aicpu_nhr_n12"] and len(ch) == 62
+    assert len(T.chunk_counts(1 << 30, ccl, 1, 1, ccl)) == 6
+    assert T.chunk_counts(1, ccl, 7, 1, ccl) == [(0, 1)]
+    assert ccl // 7 // 128 * 128 == GOLD["chunks"]["alltoallv_mult7"]
+
+
+@pytest.mark.parametrize("alg", AR_ALGS)
+@pytest.mark.parametrize("dtype,op", [(T.INT32, T.SUM), (T.INT32, T.MAX), (T.INT64, T.MIN), (T.INT8, T.PROD),
+                                      (T.UINT64, T.SUM), (T.INT16, T.SUM)])
+def test_allreduce_integers_equal_numpy_fold_with_chunking(alg, dtype, op):
+    rng = np.random.default_rng(1)
+    npd = T.NP_STORAGE[dtype]
+    ii = np.iinfo(npd)
+    for n, count in ((3, 1000), (8, 777), (12, 4099)):
+        xs = [rng.integers(ii.min, ii.max, size=count, dtype=npd, endpoint=True) for _ in range(n)]
+        # a 4 KiB scratch buffer forces many executor chunks
+        outs = T.run_allreduce(T.NumericElems(dtype, op), xs, count, T.DTYPE_SIZE[dtype], alg, ccl_bytes=4096)
+        stack = np.stack(xs)
+        with np.errstate(over="ignore"):
+            want = {T.SUM: lambda: np.add.reduce(stack, 0, dtype=npd), T.PROD: lambda: np.multiply.reduce(stack, 0, dtype=npd),
+                    T.MAX: lambda: stack.max(0), T.MIN: lambda: stack.min(0)}[op]()
+        for o in outs:
+            assert np.array_equal(o, want)
+
+
+@pytest.mark.parametrize("alg", RS_ALGS)
+def test_reduce_scatter_integers_equal_numpy_fold_with_chunking(alg):
+    rng = np.random.default_rng(2)
+    n, rc = 6, 1111
+    xs = [rng.integers(-2**31, 2**31 - 1, size=n * rc, dtype=np.int32) for _ in range(n)]
+    outs = T.run_reduce_scatter(T.NumericElems(T.INT32, T.SUM), xs, rc, 4, alg, ccl_bytes=(1 << 20) + 6 * 512)
+    want = np.add.reduce(np.stack(xs), 0, dtype=np.int32)
+    for r in range(n):
+        assert np.array_equal(outs[r], want[r * rc:(r + 1) * rc])
+
+
+def test_fp32_orders_differ_between_templates_and_between_ranks():
+    rng = np.random.default_rng(3)
+    n, count = 8, 4096
+    xs = [(rng.random(count, dtype=np.float32) * 2 - 1) for _ in range(n)]
+    one = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs, count, 4, "InsAllReduceMesh1DOneShot")
+    two = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs, count, 4, "InsAllReduceMesh1DTwoShot")
+    assert not np.array_equal(one[2].view(np.uint32), one[5].view(np.uint32))      # rank-dependent order
+    assert all(np.array_equal(two[0].view(np.uint32), t.view(np.uint32)) for t in two)
+    acc = xs[3].copy()                                                               # one-shot, rank 3, by hand
+    for k in range(n):
+        if k != 3:
+            acc = xs[k] + acc
+    assert np.array_equal(acc.view(np.uint32), one[3].view(np.uint32))
+
+
+def scaled(matrix, div):
+    return [[-(-c // div) for c in row] for row in matrix]
+
+
+@pytest.mark.parametrize("case", GOLD["alltoallv"], ids=lambda c: c["name"])
+def test_alltoallv_contract_on_reference_matrices(case):
+    n = case["ranks"]
+    m = scaled(case["matrix"], 1 << 19)      # counts divided by 2^19, rounded up: zeros stay zero
+    rng = np.random.default_rng(n)
+    ins = [rng.integers(0, 65535, size=sum(m[i]), dtype=np.uint16) for i in range(n)]
+    v = [T.alltoallvc_to_v(m, r) for r in range(n)]
+    outs = T.run_alltoallv(ins, [x[0] for x in v], [x[1] for x in v], [x[2] for x in v], [x[3] for x in v],
+                           [sum(x[2]) for x in v])
+    for j in range(n):                          # element by element, straight from the API text
+        pos = 0
+        for i in range(n):
+            start = sum(m[i][:j])
+            for e in range(m[i][j]):
+                assert outs[j][pos] == ins[i][start + e]
+                pos += 1
+        assert pos == len(outs[j])
+
+
+@pytest.mark.parametrize("case", GOLD["allgatherv"], ids=lambda c: c["name"])
+def test_allgatherv_contract_on_reference_lists(case):
+    div = 1 << 12 if max(case["counts"]) > 100000 else 1
+    counts = [-(-c // div) for c in case["counts"]]
+    displs = [sum(counts[:i]) for i in range(len(counts))] if div > 1 else case["displs"]
+    rng = np.random.default_rng(len(counts))
+    ins = [rng.integers(0, 65535, size=c, dtype=np.uint16) for c in counts]
+    outs = T.run_allgatherv(ins, counts, displs, displs[-1] + counts[-1], 0)
+    for o in outs:
+        assert np.array_equal(o, np.concatenate(ins))
