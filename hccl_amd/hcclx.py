@@ -16,9 +16,9 @@ def make_segs(segs):
         arr[i].count = count
         arr[i].nsrc = len(srcs)
         arr[i].ndst = len(dsts)
-        for k, p in enumerate(srcs):
+        for k, p in enumerate(srcs[:_lib.MAX_FAN]):   # the library rejects nsrc/ndst beyond MAX_FAN
             arr[i].src[k] = p
-        for k, p in enumerate(dsts):
+        for k, p in enumerate(dsts[:_lib.MAX_FAN]):
             arr[i].dst[k] = p
     return arr, len(segs)
 

@@ -1,0 +1,173 @@
+"""GPU parity of the fold kernels through the C ABI (hcclx_fold / hcclx_plan_*), against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import templates as T
+from hccl_amd import hcclx
+from hccl_amd._lib import HcclError
+
+from gpu_util import DevBuf, assert_same_bits, fold_oracle, fused_is_wide, payload
+
+pytestmark = pytest.mark.gpu
+
+REDUCE_DTYPES = [T.INT8, T.INT16, T.INT32, T.INT64, T.UINT64, T.FP16, T.FP32, T.FP64, T.BFP16]
+OPS = [T.SUM, T.PROD, T.MAX, T.MIN]
+
+
+def sync():
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("dtype", REDUCE_DTYPES)
+@pytest.mark.parametrize("op", OPS)
+def test_pairwise_step_in_place_matches_reference_loop(dtype, op):
+    """dst = src (+) dst, the LocalReduce step, in place, with a ragged count and a misaligned source."""
+    rng = np.random.default_rng(100 + dtype * 4 + op)
+    n = 70001
+    kind = "bits" if dtype in (T.FP16, T.BFP16) and op != T.PROD else ("prod" if op == T.PROD else "normal")
+    a, b = payload(rng, dtype, n, kind), payload(rng, dtype, n, kind)
+    esz = T.DTYPE_SIZE[dtype]
+    src, dst = DevBuf(a, offset=esz), DevBuf(b, offset=256)
+    hcclx.fold([(n, [dst.ptr, src.ptr], [dst.ptr])], dtype, op)
+    sync()
+    want = fold_oracle([b, a], dtype, op, [0, 1], wide=False)
+    assert_same_bits(dst.get(T.NP_STORAGE[dtype]), want, dtype, f"dtype {dtype} op {op}")
+    assert dst.guard_intact() and src.guard_intact()
+
+
+@pytest.mark.parametrize("nsrc", [3, 4, 5, 8, 9, 12, 16])
+@pytest.mark.parametrize("dtype,op", [(T.FP32, T.SUM), (T.FP32, T.PROD), (T.BFP16, T.SUM), (T.FP16, T.SUM),
+                                      (T.FP16, T.PROD), (T.FP64, T.SUM), (T.INT32, T.MAX), (T.FP32, T.MAX)])
+def test_chain_fold_reproduces_the_fold_order(nsrc, dtype, op):
+    rng = np.random.default_rng(nsrc * 100 + dtype)
+    n = 2 * 4096 + 13
+    kind = "prod" if op == T.PROD else "uniform" if dtype in (T.FP32, T.FP64) else "normal"
+    xs = [payload(rng, dtype, n, kind) for _ in range(nsrc)]
+    order = list(rng.permutation(nsrc))
+    bufs = [DevBuf(x) for x in xs]
+    outs = [DevBuf(nbytes=xs[0].nbytes) for _ in range(3)]
+    hcclx.fold([(n, [bufs[k].ptr for k in order], [o.ptr for o in outs])], dtype, op)
+    sync()
+    want = fold_oracle(xs, dtype, op, order, wide=fused_is_wide(dtype, op))
+    for o in outs:
+        assert_same_bits(o.get(T.NP_STORAGE[dtype]), want, dtype)
+        assert o.guard_intact()
+
+
+@pytest.mark.parametrize("nsrc", [2, 3, 8, 12, 16])
+@pytest.mark.parametrize("dtype,op", [(T.FP32, T.SUM), (T.FP32, T.PROD), (T.BFP16, T.SUM), (T.FP16, T.PROD),
+                                      (T.INT32, T.SUM), (T.INT64, T.MIN), (T.FP64, T.PROD)])
+def test_self_first_fold_gives_every_rank_its_own_order(nsrc, dtype, op):
+    rng = np.random.default_rng(nsrc * 10 + dtype + op)
+    n = 4096 + 3
+    xs = [payload(rng, dtype, n, "prod" if op == T.PROD else "normal") for _ in range(nsrc)]
+    bufs = [DevBuf(x) for x in xs]
+    outs = [DevBuf(nbytes=xs[0].nbytes) for _ in range(nsrc)]
+    hcclx.fold([(n, [b.ptr for b in bufs], [o.ptr for o in outs])], dtype, op, hcclx.FOLD_SELF_FIRST)
+    sync()
+    for r in range(nsrc):
+        order = [r] + [k for k in range(nsrc) if k != r]
+        want = fold_oracle(xs, dtype, op, order, wide=fused_is_wide(dtype, op))
+        assert_same_bits(outs[r].get(T.NP_STORAGE[dtype]), want, dtype, f"rank {r}")
+
+
+def test_self_first_in_place_allreduce():
+    """sendBuf == recvBuf on every rank: each destination aliases one source."""
+    rng = np.random.default_rng(5)
+    n, nsrc = 10007, 8
+    xs = [payload(rng, T.FP32, n, "uniform") for _ in range(nsrc)]
+    bufs = [DevBuf(x) for x in xs]
+    hcclx.fold([(n, [b.ptr for b in bufs], [b.ptr for b in bufs])], T.FP32, T.SUM, hcclx.FOLD_SELF_FIRST)
+    sync()
+    for r in range(nsrc):
+        order = [r] + [k for k in range(nsrc) if k != r]
+        assert_same_bits(bufs[r].get(np.float32), fold_oracle(xs, T.FP32, T.SUM, order, False), T.FP32)
+
+
+def test_fp32_subnormals_and_signed_zeros_survive():
+    a = np.array([1e-45, -1e-45, 1e-39, 0.0, -0.0, 3e-39, 1.17549435e-38] * 37, dtype=np.float32)
+    b = np.array([1e-45, 1e-45, -2e-39, -0.0, -0.0, 3e-39, -1e-45] * 37, dtype=np.float32)
+    for op in OPS:
+        da, db = DevBuf(a), DevBuf(b)
+        hcclx.fold([(a.size, [db.ptr, da.ptr], [db.ptr])], T.FP32, op)
+        sync()
+        assert_same_bits(db.get(np.float32), fold_oracle([b, a], T.FP32, op, [0, 1], False), T.FP32, f"op {op}")
+
+
+def test_float_max_min_nan_and_zero_operand_order():
+    src = np.array([np.nan, 1.0, 0.0, -0.0, np.inf, -np.inf] * 11, dtype=np.float32)
+    dst = np.array([1.0, np.nan, -0.0, 0.0, np.nan, 2.0] * 11, dtype=np.float32)
+    for op in (T.MAX, T.MIN):
+        ds, dd = DevBuf(src), DevBuf(dst)
+        hcclx.fold([(src.size, [dd.ptr, ds.ptr], [dd.ptr])], T.FP32, op)
+        sync()
+        assert_same_bits(dd.get(np.float32), fold_oracle([dst, src], T.FP32, op, [0, 1], False), T.FP32)
+
+
+def test_many_ragged_segments_and_empty_ones():
+    rng = np.random.default_rng(8)
+    counts = [0, 1, 3, 4, 5, 255, 256, 257, 1023, 1024, 4099, 0, 8191, 65537] + list(rng.integers(0, 3000, 2200))
+    segs, checks = [], []
+    big_a = payload(rng, T.INT32, int(sum(counts)) + 8)
+    big_b = payload(rng, T.INT32, int(sum(counts)) + 8)
+    da, db = DevBuf(big_a), DevBuf(big_b)
+    out = DevBuf(nbytes=big_a.nbytes)
+    off = 0
+    for c in counts:
+        c = int(c)
+        segs.append((c, [da.ptr + off * 4, db.ptr + off * 4], [out.ptr + off * 4]))
+        off += c
+    hcclx.fold(segs, T.INT32, T.SUM)      # more segments than one launch holds: the launcher splits
+    sync()
+    want = fold_oracle([big_a, big_b], T.INT32, T.SUM, [0, 1], False)
+    assert np.array_equal(out.get(np.int32)[:off], want[:off])
+    assert (out.get(np.uint8)[off * 4:] == 0xA5).all()
+
+
+@pytest.mark.parametrize("soff,doff", [(0, 0), (1, 0), (0, 3), (5, 9), (16, 2), (7, 7)])
+def test_copy_any_alignment_to_several_destinations(soff, doff):
+    rng = np.random.default_rng(soff * 16 + doff)
+    n = 300003
+    x = rng.integers(0, 256, size=n, dtype=np.uint8)
+    src = DevBuf(x, offset=soff)
+    dsts = [DevBuf(nbytes=n, offset=doff) for _ in range(3)]
+    hcclx.fold([(n, [src.ptr], [d.ptr for d in dsts])], T.UINT8)
+    sync()
+    for d in dsts:
+        assert np.array_equal(d.get(np.uint8), x) and d.guard_intact()
+
+
+def test_plan_relaunch_and_algorithmic_bytes():
+    rng = np.random.default_rng(1)
+    n = 50000
+    xs = [payload(rng, T.FP32, n, "uniform") for _ in range(4)]
+    bufs = [DevBuf(x) for x in xs]
+    out = DevBuf(nbytes=n * 4)
+    plan = hcclx.Plan([(n, [b.ptr for b in bufs], [out.ptr])], T.FP32, T.SUM)
+    assert plan.bytes == 5 * n * 4
+    for _ in range(3):
+        out.t.zero_()
+        plan.launch()
+        sync()
+        assert_same_bits(out.get(np.float32), fold_oracle(xs, T.FP32, T.SUM, [0, 1, 2, 3], False), T.FP32)
+    plan.close()
+
+
+def test_errors_are_reported_not_launched():
+    b = DevBuf(nbytes=64)
+    with pytest.raises(HcclError) as e:
+        hcclx.fold([(4, [b.ptr] * 17, [b.ptr])], T.FP32, T.SUM)
+    assert e.value.code == 1      # HCCL_E_PARA
+    with pytest.raises(HcclError) as e:
+        hcclx.fold([(4, [b.ptr, 0], [b.ptr])], T.FP32, T.SUM)
+    assert e.value.code == 2      # HCCL_E_PTR
+    with pytest.raises(HcclError) as e:
+        hcclx.fold([(4, [b.ptr, b.ptr], [b.ptr])], T.UINT8, T.SUM)
+    assert e.value.code == 5      # HCCL_E_NOT_SUPPORT: uint8 is not a reduce type
+    with pytest.raises(HcclError) as e:
+        hcclx.fold([(4, [b.ptr, b.ptr], [b.ptr, b.ptr, b.ptr])], T.FP32, T.SUM, hcclx.FOLD_SELF_FIRST)
+    assert e.value.code == 1
+    hcclx.fold([], T.FP32, T.SUM)           # nothing to do is fine
+    hcclx.fold([(0, [0, 0], [0])], T.FP32)  # zero-size slices are skipped (LocalCopy/LocalReduce do the same)
+    sync()
