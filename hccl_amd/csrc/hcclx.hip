@@ -68,6 +68,10 @@ void init_slot(DeviceSlot *s, int dev)
     if (const char *v = std::getenv("HCCLX_BLOCKS_PER_CU")) {
         c.blocks_per_cu = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
     }
+    if (const char *v = std::getenv("HCCLX_V_BLOCKS_PER_CU")) {
+        const uint32_t b = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
+        if (b != 0) c.v_blocks_per_cu = b;
+    }
     c.ring_bytes = kSliceBytes * kSlices;
     e = hipHostMalloc(reinterpret_cast<void **>(&c.h_ring), c.ring_bytes, hipHostMallocDefault);
     if (e != hipSuccess) {

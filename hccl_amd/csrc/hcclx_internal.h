@@ -22,7 +22,13 @@ int fail_hip(hipError_t e, const char *what);
 struct DeviceCtx {
     int device = -1;
     int num_cus = 0;
-    uint32_t blocks_per_cu = 8;  // persistent-grid cap; 0 = one workgroup per tile
+    // Fold launches use one workgroup per tile (measured faster than a persistent grid on MI355X: the
+    // hardware staggers workgroups, a grid-stride loop runs them in lock step).  A non-zero value caps
+    // the grid at blocks_per_cu x CUs instead.
+    uint32_t blocks_per_cu = 0;
+    // V kernels whose tables live on the device cannot know their tile count on the host and run as a
+    // persistent grid of this many workgroups per CU.
+    uint32_t v_blocks_per_cu = 2;
     // Descriptor ring: tables of one-shot launches are written to pinned host memory and copied to the
     // device ring on the launch stream just before the kernel.
     char *h_ring = nullptr;

@@ -64,8 +64,21 @@ int hcclx_alltoallv(const void *const *send, void *const *recv, const uint64_t *
     const uint64_t *dev[3];
     rc = stage_tables(ctx, tabs, 3, static_cast<size_t>(n) * n, tables_on_device, st, dev);
     if (rc != HCCL_SUCCESS) return rc;
-    const uint32_t grid = grid_for(ctx, ~0ull);
-    hipError_t e = launch_alltoallv(ptrs, dev[0], dev[1], dev[2], n, static_cast<uint32_t>(esz), grid, st);
+    uint64_t grid = static_cast<uint64_t>(ctx->num_cus) * ctx->v_blocks_per_cu;
+    if (!tables_on_device) {
+        // host tables: the tile count is known here, so launch exactly one workgroup per tile
+        uint64_t total = 0;
+        for (uint32_t i = 0; i < n; ++i) {
+            for (uint32_t j = 0; j < n; ++j) {
+                const uint64_t dst = reinterpret_cast<uint64_t>(ptrs.recv[j]) + rdispls[j * n + i] * esz;
+                total += v_tiles_of(send_counts[i * n + j] * esz, dst);
+            }
+        }
+        if (total == 0) return HCCL_SUCCESS;
+        grid = total < 0x7fffffffull ? total : 0x7fffffffull;
+    }
+    hipError_t e = launch_alltoallv(ptrs, dev[0], dev[1], dev[2], n, static_cast<uint32_t>(esz),
+                                    static_cast<uint32_t>(grid), st);
     if (e != hipSuccess) return fail_hip(e, "alltoallv kernel launch");
     return HCCL_SUCCESS;
 }
@@ -86,8 +99,16 @@ int hcclx_allgatherv(const void *const *send, void *const *recv, const uint64_t 
     const uint64_t *dev[2];
     rc = stage_tables(ctx, tabs, 2, n, tables_on_device, st, dev);
     if (rc != HCCL_SUCCESS) return rc;
-    const uint32_t grid = grid_for(ctx, ~0ull);
-    hipError_t e = launch_allgatherv(ptrs, dev[0], dev[1], n, static_cast<uint32_t>(esz), grid, st);
+    uint64_t grid = static_cast<uint64_t>(ctx->num_cus) * ctx->v_blocks_per_cu;
+    if (!tables_on_device) {
+        uint64_t total = 0;
+        for (uint32_t i = 0; i < n; ++i) {
+            total += v_tiles_of(counts[i] * esz, reinterpret_cast<uint64_t>(ptrs.recv[0]) + displs[i] * esz);
+        }
+        if (total == 0) return HCCL_SUCCESS;
+        grid = total < 0x7fffffffull ? total : 0x7fffffffull;
+    }
+    hipError_t e = launch_allgatherv(ptrs, dev[0], dev[1], n, static_cast<uint32_t>(esz), static_cast<uint32_t>(grid), st);
     if (e != hipSuccess) return fail_hip(e, "allgatherv kernel launch");
     return HCCL_SUCCESS;
 }

@@ -1,0 +1,248 @@
+#include "alg_data_trans_wrapper.h"
+
+#include "hcomm_primitives.h"
+
+namespace ops_hccl {
+
+namespace {
+constexpr u32 kTimeout = CUSTOM_TIMEOUT;
+
+HcclResult R(int32_t rc) { return static_cast<HcclResult>(rc); }
+
+// LocalReduce routes 64-bit types and PROD to the CPU loop AicpuReduce, everything else to the inline
+// reduce of the transport (wrapper.cc:837-841).  Both are the same fold kernel here, so the two routes
+// only differ in the checks they make.
+bool NeedsAicpuReduce(HcclDataType dt, HcclReduceOp op)
+{
+    return dt == HCCL_DATA_TYPE_INT64 || dt == HCCL_DATA_TYPE_UINT64 || dt == HCCL_DATA_TYPE_FP64 ||
+           op == HCCL_REDUCE_PROD;
+}
+
+bool AicpuReduceSupports(HcclDataType dt)
+{
+    switch (dt) {  // wrapper.cc:1176-1207
+        case HCCL_DATA_TYPE_INT8:
+        case HCCL_DATA_TYPE_INT32:
+        case HCCL_DATA_TYPE_FP16:
+        case HCCL_DATA_TYPE_FP32:
+        case HCCL_DATA_TYPE_INT64:
+        case HCCL_DATA_TYPE_UINT64:
+        case HCCL_DATA_TYPE_FP64:
+            return true;
+        default:
+            return false;
+    }
+}
+
+HcclResult CheckReduceSlices(const DataSlice &src, const DataSlice &dst, HcclDataType dt)
+{
+    CHK_PRT_RET(src.count_ * DATATYPE_SIZE_TABLE[dt] != src.size_,
+                HCCL_ERROR("reduce: src slice count does not match its size"), HCCL_E_INTERNAL);
+    CHK_PRT_RET(dst.count_ * DATATYPE_SIZE_TABLE[dt] != dst.size_,
+                HCCL_ERROR("reduce: dst slice count does not match its size"), HCCL_E_INTERNAL);
+    return HCCL_SUCCESS;
+}
+}  // namespace
+
+HcclResult LocalCopy(const ThreadHandle &thread, const DataSlice &srcSlice, const DataSlice &dstSlice)
+{
+    if (srcSlice.size_ == 0) return HCCL_SUCCESS;  // zero-size copy is a no-op success (wrapper.cc:817-819)
+    CHK_PRT_RET(srcSlice.size_ != dstSlice.size_, HCCL_ERROR("LocalCopy: slice sizes differ"), HCCL_E_INTERNAL);
+    return R(HcommLocalCopyOnThread(thread, GetSliceAddr(dstSlice), GetSliceAddr(srcSlice), srcSlice.size_));
+}
+
+HcclResult LocalReduce(const ThreadHandle &thread, const DataSlice &srcSlice, const DataSlice &dstSlice,
+                       HcclDataType dataType, HcclReduceOp reduceOp)
+{
+    if (NeedsAicpuReduce(dataType, reduceOp)) {
+        CHK_PRT_RET(srcSlice.size_ != dstSlice.size_, HCCL_ERROR("AicpuReduce: slice sizes differ"), HCCL_E_INTERNAL);
+        CHK_PRT_RET(!AicpuReduceSupports(dataType), HCCL_ERROR("AicpuReduce: DataType[%d] not support", dataType),
+                    HCCL_E_INTERNAL);
+        const u64 count = srcSlice.size_ / DATATYPE_SIZE_TABLE[dataType];
+        return R(HcommLocalReduceOnThread(thread, GetSliceAddr(dstSlice), GetSliceAddr(srcSlice), count, dataType,
+                                          reduceOp));
+    }
+    if (srcSlice.size_ == 0) return HCCL_SUCCESS;
+    CHK_PRT_RET(srcSlice.size_ != dstSlice.size_, HCCL_ERROR("LocalReduce: slice sizes differ"), HCCL_E_INTERNAL);
+    return R(HcommLocalReduceOnThread(thread, GetSliceAddr(dstSlice), GetSliceAddr(srcSlice), srcSlice.count_,
+                                      dataType, reduceOp));
+}
+
+bool IsContinuousSlice(const DataSlice &nxtSlice, const DataSlice &currSlice)
+{
+    return nxtSlice.addr_ == currSlice.addr_ && nxtSlice.offset_ == currSlice.offset_ + currSlice.size_;
+}
+
+HcclResult LocalCopySlices(const ThreadHandle &thread, const std::vector<DataSlice> &srcSlices,
+                           const std::vector<DataSlice> &dstSlices)
+{
+    CHK_PRT_RET(srcSlices.size() != dstSlices.size(), HCCL_ERROR("LocalCopySlices: slice counts differ"),
+                HCCL_E_INTERNAL);
+    // Address-contiguous neighbours are merged into one copy (wrapper.cc:864-924).
+    bool open = false;
+    DataSlice runSrc, runDst;
+    for (size_t i = 0; i < srcSlices.size(); ++i) {
+        if (srcSlices[i].size_ == 0) continue;
+        CHK_PRT_RET(srcSlices[i].size_ != dstSlices[i].size_, HCCL_ERROR("LocalCopySlices: slice sizes differ"),
+                    HCCL_E_INTERNAL);
+        if (open && IsContinuousSlice(srcSlices[i], runSrc) && IsContinuousSlice(dstSlices[i], runDst)) {
+            runSrc.size_ += srcSlices[i].size_;
+            runDst.size_ += dstSlices[i].size_;
+            continue;
+        }
+        if (open) CHK_RET(LocalCopy(thread, runSrc, runDst));
+        runSrc = DataSlice(srcSlices[i].addr_, srcSlices[i].offset_, srcSlices[i].size_);
+        runDst = DataSlice(dstSlices[i].addr_, dstSlices[i].offset_, dstSlices[i].size_);
+        open = true;
+    }
+    if (open) CHK_RET(LocalCopy(thread, runSrc, runDst));
+    return HCCL_SUCCESS;
+}
+
+// ---- write family: the receiver says "my buffer is free" (ACK), the sender writes and says "data is there"
+
+HcclResult SendWrite(const DataInfo &sendInfo, const ThreadHandle &thread)
+{
+    const ChannelInfo &ch = sendInfo.channel_;
+    CHK_RET(HcommChannelNotifyWaitOnThread(thread, ch.handle, NOTIFY_IDX_ACK, kTimeout));
+    for (size_t i = 0; i < sendInfo.slices_.srcSlices_.size(); ++i) {
+        const DataSlice &s = sendInfo.slices_.srcSlices_[i];
+        const DataSlice &d = sendInfo.slices_.dstSlices_[i];
+        if (s.size_ == 0) continue;
+        CHK_RET(HcommWriteOnThread(thread, ch.handle, GetSliceAddr(d), GetSliceAddr(s), s.size_));
+    }
+    return R(HcommChannelNotifyRecordOnThread(thread, ch.handle, NOTIFY_IDX_DATA_SIGNAL));
+}
+
+HcclResult RecvWrite(const DataInfo &recvInfo, const ThreadHandle &thread)
+{
+    const ChannelInfo &ch = recvInfo.channel_;
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, ch.handle, NOTIFY_IDX_ACK));
+    return R(HcommChannelNotifyWaitOnThread(thread, ch.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+}
+
+HcclResult SendRecvWrite(const SendRecvInfo &info, const ThreadHandle &thread)
+{
+    const auto &src = info.sendRecvSlices_.txSlicesList_.srcSlices_;
+    const auto &dst = info.sendRecvSlices_.txSlicesList_.dstSlices_;
+    const ChannelInfo &tx = info.sendRecvChannels_.txChannel_;
+    const ChannelInfo &rx = info.sendRecvChannels_.rxChannel_;
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, rx.handle, NOTIFY_IDX_ACK));
+    CHK_RET(HcommChannelNotifyWaitOnThread(thread, tx.handle, NOTIFY_IDX_ACK, kTimeout));
+    for (size_t i = 0; i < src.size(); ++i) {
+        if (src[i].size_ == 0) continue;
+        CHK_RET(HcommWriteOnThread(thread, tx.handle, GetSliceAddr(dst[i]), GetSliceAddr(src[i]), src[i].size_));
+    }
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, tx.handle, NOTIFY_IDX_DATA_SIGNAL));
+    return R(HcommChannelNotifyWaitOnThread(thread, rx.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+}
+
+HcclResult SendRecvWriteReduce(const SendRecvReduceInfo &info, const ThreadHandle &thread)
+{
+    const auto &src = info.sendRecvSlices_.txSlicesList_.srcSlices_;
+    const auto &dst = info.sendRecvSlices_.txSlicesList_.dstSlices_;
+    const ChannelInfo &tx = info.sendRecvChannels_.txChannel_;
+    const ChannelInfo &rx = info.sendRecvChannels_.rxChannel_;
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, rx.handle, NOTIFY_IDX_ACK));
+    CHK_RET(HcommChannelNotifyWaitOnThread(thread, tx.handle, NOTIFY_IDX_ACK, kTimeout));
+    for (size_t i = 0; i < src.size(); ++i) {
+        if (src[i].size_ == 0) continue;
+        CHK_RET(CheckReduceSlices(src[i], dst[i], info.dataType_));
+        CHK_RET(HcommWriteReduceOnThread(thread, tx.handle, GetSliceAddr(dst[i]), GetSliceAddr(src[i]), src[i].count_,
+                                         info.dataType_, info.reduceType_));
+    }
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, tx.handle, NOTIFY_IDX_DATA_SIGNAL));
+    return R(HcommChannelNotifyWaitOnThread(thread, rx.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+}
+
+// ---- read family: the owner says "my data is ready" (ACK), the reader reads and says "I am done"
+
+HcclResult SendRead(const DataInfo &sendInfo, const ThreadHandle &thread)
+{
+    const ChannelInfo &ch = sendInfo.channel_;
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, ch.handle, NOTIFY_IDX_ACK));
+    return R(HcommChannelNotifyWaitOnThread(thread, ch.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+}
+
+HcclResult RecvRead(const DataInfo &recvInfo, const ThreadHandle &thread)
+{
+    const ChannelInfo &ch = recvInfo.channel_;
+    CHK_RET(HcommChannelNotifyWaitOnThread(thread, ch.handle, NOTIFY_IDX_ACK, kTimeout));
+    for (size_t i = 0; i < recvInfo.slices_.srcSlices_.size(); ++i) {
+        const DataSlice &s = recvInfo.slices_.srcSlices_[i];
+        const DataSlice &d = recvInfo.slices_.dstSlices_[i];
+        if (s.size_ == 0) continue;
+        CHK_RET(HcommReadOnThread(thread, ch.handle, GetSliceAddr(d), GetSliceAddr(s), s.size_));
+    }
+    return R(HcommChannelNotifyRecordOnThread(thread, ch.handle, NOTIFY_IDX_DATA_SIGNAL));
+}
+
+HcclResult SendRecvRead(const SendRecvInfo &info, const ThreadHandle &thread)
+{
+    const auto &src = info.sendRecvSlices_.rxSlicesList_.srcSlices_;
+    const auto &dst = info.sendRecvSlices_.rxSlicesList_.dstSlices_;
+    const ChannelInfo &tx = info.sendRecvChannels_.txChannel_;
+    const ChannelInfo &rx = info.sendRecvChannels_.rxChannel_;
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, tx.handle, NOTIFY_IDX_ACK));
+    CHK_RET(HcommChannelNotifyWaitOnThread(thread, rx.handle, NOTIFY_IDX_ACK, kTimeout));
+    for (size_t i = 0; i < src.size(); ++i) {
+        if (src[i].size_ == 0) continue;
+        CHK_RET(HcommReadOnThread(thread, rx.handle, GetSliceAddr(dst[i]), GetSliceAddr(src[i]), src[i].size_));
+    }
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, rx.handle, NOTIFY_IDX_DATA_SIGNAL));
+    return R(HcommChannelNotifyWaitOnThread(thread, tx.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+}
+
+HcclResult SendRecvReadReduce(const SendRecvReduceInfo &info, const ThreadHandle &thread)
+{
+    const auto &src = info.sendRecvSlices_.rxSlicesList_.srcSlices_;
+    const auto &dst = info.sendRecvSlices_.rxSlicesList_.dstSlices_;
+    const ChannelInfo &tx = info.sendRecvChannels_.txChannel_;
+    const ChannelInfo &rx = info.sendRecvChannels_.rxChannel_;
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, tx.handle, NOTIFY_IDX_ACK));
+    CHK_RET(HcommChannelNotifyWaitOnThread(thread, rx.handle, NOTIFY_IDX_ACK, kTimeout));
+    for (size_t i = 0; i < src.size(); ++i) {
+        if (src[i].size_ == 0) continue;
+        CHK_RET(CheckReduceSlices(src[i], dst[i], info.dataType_));
+        CHK_RET(HcommReadReduceOnThread(thread, rx.handle, GetSliceAddr(dst[i]), GetSliceAddr(src[i]), src[i].count_,
+                                        info.dataType_, info.reduceType_));
+    }
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, rx.handle, NOTIFY_IDX_DATA_SIGNAL));
+    return R(HcommChannelNotifyWaitOnThread(thread, tx.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+}
+
+// ---- main thread <-> sub threads
+
+HcclResult PreSyncInterThreads(const ThreadHandle &mainThread, const std::vector<ThreadHandle> &subThreads,
+                               const std::vector<u32> &notifyIdxMainToSub)
+{
+    CHK_PRT_RET(subThreads.empty() || notifyIdxMainToSub.empty(), HCCL_ERROR("PreSyncInterThreads: empty"),
+                HCCL_E_INTERNAL);
+    CHK_PRT_RET(subThreads.size() != notifyIdxMainToSub.size(), HCCL_ERROR("PreSyncInterThreads: size mismatch"),
+                HCCL_E_INTERNAL);
+    for (size_t i = 0; i < subThreads.size(); ++i) {
+        CHK_RET(HcommThreadNotifyRecordOnThread(mainThread, subThreads[i], notifyIdxMainToSub[i]));
+    }
+    for (size_t i = 0; i < subThreads.size(); ++i) {
+        CHK_RET(HcommThreadNotifyWaitOnThread(subThreads[i], notifyIdxMainToSub[i], kTimeout));
+    }
+    return HCCL_SUCCESS;
+}
+
+HcclResult PostSyncInterThreads(const ThreadHandle &mainThread, const std::vector<ThreadHandle> &subThreads,
+                                const std::vector<u32> &notifyIdxSubToMain)
+{
+    CHK_PRT_RET(subThreads.empty() || notifyIdxSubToMain.empty(), HCCL_ERROR("PostSyncInterThreads: empty"),
+                HCCL_E_INTERNAL);
+    CHK_PRT_RET(subThreads.size() != notifyIdxSubToMain.size(), HCCL_ERROR("PostSyncInterThreads: size mismatch"),
+                HCCL_E_INTERNAL);
+    for (size_t i = 0; i < subThreads.size(); ++i) {
+        CHK_RET(HcommThreadNotifyWaitOnThread(mainThread, notifyIdxSubToMain[i], kTimeout));
+    }
+    for (size_t i = 0; i < subThreads.size(); ++i) {
+        CHK_RET(HcommThreadNotifyRecordOnThread(subThreads[i], mainThread, notifyIdxSubToMain[i]));
+    }
+    return HCCL_SUCCESS;
+}
+
+}  // namespace ops_hccl

@@ -1,0 +1,41 @@
+// ReduceScatter, AllGather, AllGatherV and AlltoAllV templates: see the .cc files for what each restates.
+#pragma once
+#include "all_reduce_templates.h"
+
+namespace ops_hccl {
+
+// scratch multiples: reduce_scatter mesh_1D.cc:59-63 (N), nhr.cc:369-377 (N); all_gather mesh/NHR (N);
+// all_gather_v mesh_1D.cc:48-57 (N in single-op mode); all_to_all_v mesh_1D.cc:66-73 (min(16, N-1)).
+HCCL_DECLARE_TEMPLATE(InsTempReduceScatterMesh1D, "ReduceScatter mesh 1D",
+                      (templateRankSize_ > 1 ? templateRankSize_ : 1), templateRankSize_);
+HCCL_DECLARE_TEMPLATE(InsTempReduceScatterNHR, "ReduceScatter NHR", 1, templateRankSize_);
+HCCL_DECLARE_TEMPLATE(InsTempAllGatherMesh1D, "AllGather mesh 1D",
+                      (templateRankSize_ > 1 ? templateRankSize_ - 1 : 1), templateRankSize_);
+HCCL_DECLARE_TEMPLATE(InsTempAllGatherNHR, "AllGather NHR", 1, templateRankSize_);
+HCCL_DECLARE_TEMPLATE(InsTempAllGatherVMesh1D, "AllGatherV mesh 1D",
+                      (templateRankSize_ > 1 ? templateRankSize_ - 1 : 1), templateRankSize_);
+
+constexpr u32 ALLTOALLV_DIRECT_FULLMESH_CONCURRENT_SIZE = 16;
+
+class InsTempAlltoAllVMesh1D : public InsAlgTemplateBase {
+public:
+    using InsAlgTemplateBase::InsAlgTemplateBase;
+    std::string Describe() const override { return "AlltoAllV mesh 1D"; }
+    u64 GetThreadNum() const override { return Concurrent() + 1; }
+    u64 CalcScratchMultiple(BufferType, BufferType) override { return Concurrent(); }
+    HcclResult KernelRun(const OpParam &param, const TemplateDataParams &tempAlgParams,
+                         TemplateResource &templateResource) override;
+    // peers of one round: left and right neighbours at growing distance (mesh_1D.cc:75-93)
+    void CalcCommRankSetForOneLoop(u32 roundIdx, u32 remainRankSize, std::vector<u32> &commRanks) const;
+    // which scratch slot each side of a pair uses (mesh_1D.cc:101-126)
+    void CalcCclBuffIdx(u32 remoteRank, u32 &myRankCclBuffIdx, u32 &remoteCclBuffIdx) const;
+
+private:
+    u32 Concurrent() const
+    {
+        const u32 peers = templateRankSize_ > 0 ? templateRankSize_ - 1 : 0;
+        return peers < ALLTOALLV_DIRECT_FULLMESH_CONCURRENT_SIZE ? peers : ALLTOALLV_DIRECT_FULLMESH_CONCURRENT_SIZE;
+    }
+};
+
+}  // namespace ops_hccl

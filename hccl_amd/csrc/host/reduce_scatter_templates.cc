@@ -1,0 +1,145 @@
+// ReduceScatter algorithm templates, restated from the reference
+// (src/ops/reduce_scatter/template/aicpu/):
+//   InsTempReduceScatterMesh1D   ins_temp_reduce_scatter_mesh_1D.cc:65-227
+//   InsTempReduceScatterNHR      ins_temp_reduce_scatter_nhr.cc:77-425
+#include "data_move_templates.h"
+
+namespace ops_hccl {
+
+namespace {
+bool NeedsCpuReduce(HcclDataType dt, HcclReduceOp op)
+{
+    return dt == HCCL_DATA_TYPE_INT64 || dt == HCCL_DATA_TYPE_UINT64 || dt == HCCL_DATA_TYPE_FP64 ||
+           op == HCCL_REDUCE_PROD;
+}
+}  // namespace
+
+// Every rank writes its slice k into slot <own rank> of rank k's scratch; rank k then copies its own
+// slice to the output and folds the other slots in, ranks ascending.
+HcclResult InsTempReduceScatterMesh1D::KernelRun(const OpParam &param, const TemplateDataParams &p,
+                                                 TemplateResource &res)
+{
+    if (p.sliceSize == 0 && p.tailSize == 0) return HCCL_SUCCESS;
+    threadNum_ = static_cast<u32>(GetThreadNum());
+    CHK_PRT_RET(res.threads.size() < threadNum_, HCCL_ERROR("[RS mesh] thread num is invalid"), HCCL_E_INTERNAL);
+    dataType_ = param.DataDes.dataType;
+    const u64 esz = DATATYPE_SIZE_TABLE[dataType_];
+    u32 me = 0;
+    CHK_RET(GetAlgRank(myRank_, subCommRanks_[0], me));
+    const u32 n = templateRankSize_;
+    std::vector<ThreadHandle> threads(res.threads.begin(), res.threads.begin() + threadNum_);
+    auto sliceOf = [&](u32 algRank) { return (algRank == n - 1 && p.tailSize > 0) ? p.tailSize : p.sliceSize; };
+
+    CHK_RET(PreSync(threads));
+    u32 que = 1;
+    for (u32 i = 1; i < n; ++i) {
+        const u32 next = (me + i) % n;
+        const u64 size = sliceOf(next);
+        const u64 slotStride = size;  // slots are laid out with the slice size of this chunk
+        const ChannelInfo &link = res.channels.at(subCommRanks_[0][next])[0];
+        std::vector<DataSlice> txSrc, txDst, rxSrc, rxDst;
+        for (u64 rpt = 0; rpt < p.repeatNum; ++rpt) {
+            txSrc.emplace_back(p.buffInfo.inputPtr,
+                               p.buffInfo.inBuffBaseOff + rpt * p.inputRepeatStride + next * p.inputSliceStride, size,
+                               size / esz);
+            txDst.emplace_back(link.remoteCclMem.addr,
+                               p.buffInfo.hcclBuffBaseOff + rpt * p.outputRepeatStride + me * slotStride, size,
+                               size / esz);
+            rxSrc.emplace_back(link.remoteCclMem.addr,
+                               p.buffInfo.inBuffBaseOff + rpt * p.inputRepeatStride + me * p.inputSliceStride, size,
+                               size / esz);
+            rxDst.emplace_back(p.buffInfo.hcclBuff.addr,
+                               p.buffInfo.hcclBuffBaseOff + rpt * p.outputRepeatStride + next * slotStride, size,
+                               size / esz);
+        }
+        SendRecvInfo info{{link, link}, {{txSrc, txDst}, {rxSrc, rxDst}}, dataType_};
+        CHK_RET(SendRecvBatchWrite(info, threads[que]));
+        que++;
+    }
+    CHK_RET(PostSync(threads));
+    const bool cpu = NeedsCpuReduce(dataType_, reduceOp_);
+    if (cpu) {
+        CHK_RET(HcommBatchModeEnd(param.algTag.c_str()));
+        CHK_RET(HcommBatchModeStart(param.algTag.c_str()));
+        for (ThreadHandle t : threads) CHK_RET(HcommThreadJoin(t, CUSTOM_TIMEOUT));
+    }
+
+    // PostCopy: own slice input -> output, then fold the scratch slots of the other ranks into it
+    const u64 size = sliceOf(me);
+    const u64 count = size / esz;
+    for (u64 rpt = 0; rpt < p.repeatNum; ++rpt) {
+        DataSlice dst(p.buffInfo.outputPtr,
+                      p.buffInfo.outBuffBaseOff + rpt * p.outputRepeatStride + me * p.outputSliceStride, size, count);
+        if (p.buffInfo.inBuffType != p.buffInfo.outBuffType || p.buffInfo.inBuffBaseOff != p.buffInfo.outBuffBaseOff) {
+            DataSlice src(p.buffInfo.inputPtr,
+                          p.buffInfo.inBuffBaseOff + rpt * p.inputRepeatStride + me * p.inputSliceStride, size, count);
+            CHK_RET(LocalCopy(threads[0], src, dst));
+        }
+        for (u32 k = 0; k < n; ++k) {
+            if (k == me) continue;
+            DataSlice src(p.buffInfo.hcclBuff.addr, p.buffInfo.hcclBuffBaseOff + rpt * p.outputRepeatStride + k * size,
+                          size, count);
+            CHK_RET(LocalReduce(threads[0], src, dst, dataType_, reduceOp_));
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
+// Shards are copied into scratch slots (slot k = shard k), the NHR reduce-scatter steps fold them across
+// ranks, and the own slot is copied out.  The slices a rank sends in step 0 go straight from its input
+// (ins_temp_reduce_scatter_nhr.cc:98-101, :329-332), so they are not pre-copied.
+HcclResult InsTempReduceScatterNHR::KernelRun(const OpParam &param, const TemplateDataParams &p,
+                                              TemplateResource &res)
+{
+    if (p.sliceSize == 0 && p.tailSize == 0) return HCCL_SUCCESS;
+    CHK_PRT_RET(res.threads.empty(), HCCL_ERROR("[RS NHR] no thread"), HCCL_E_INTERNAL);
+    dataType_ = param.DataDes.dataType;
+    const u64 esz = DATATYPE_SIZE_TABLE[dataType_];
+    const u32 n = templateRankSize_;
+    u32 me = 0;
+    CHK_RET(GetAlgRank(myRank_, subCommRanks_[0], me));
+    const ThreadHandle th = res.threads[0];
+    void *ccl = p.buffInfo.hcclBuff.addr;
+    auto sizeOf = [&](u32 idx) { return (idx == n - 1 && p.tailSize > 0) ? p.tailSize : p.sliceSize; };
+
+    std::vector<NHRStepInfo> steps;
+    if (n > 1) GetNHRReduceScatterSteps(n, me, steps);
+    std::vector<bool> sentInStep0(n, false);
+    if (!steps.empty()) {
+        for (u32 idx : steps[0].txSliceIdxs) sentInStep0[idx] = true;
+    }
+    for (u32 k = 0; k < n; ++k) {
+        if (sentInStep0[k]) continue;
+        const u64 size = sizeOf(k);
+        CHK_RET(LocalCopy(th, DataSlice(p.buffInfo.inputPtr, p.buffInfo.inBuffBaseOff + k * p.inputSliceStride, size),
+                          DataSlice(ccl, p.buffInfo.hcclBuffBaseOff + k * p.sliceSize, size)));
+    }
+    for (u32 s = 0; s < steps.size(); ++s) {
+        const NHRStepInfo &st = steps[s];
+        const ChannelInfo &recv = res.channels.at(subCommRanks_[0][st.fromRank]).at(0);
+        const ChannelInfo &send = res.channels.at(subCommRanks_[0][st.toRank]).at(0);
+        std::vector<DataSlice> txSrc, txDst, rxSrc, rxDst;
+        for (u32 i = 0; i < st.nSlices; ++i) {
+            const u32 tx = st.txSliceIdxs[i];
+            const u32 rx = st.rxSliceIdxs[i];
+            const u64 txOff = p.buffInfo.hcclBuffBaseOff + p.sliceSize * tx;
+            const u64 rxOff = p.buffInfo.hcclBuffBaseOff + p.sliceSize * rx;
+            if (s == 0) {
+                txSrc.emplace_back(p.buffInfo.inputPtr, p.buffInfo.inBuffBaseOff + p.inputSliceStride * tx, sizeOf(tx),
+                                   sizeOf(tx) / esz);
+            } else {
+                txSrc.emplace_back(ccl, txOff, sizeOf(tx), sizeOf(tx) / esz);
+            }
+            txDst.emplace_back(send.remoteCclMem.addr, txOff, sizeOf(tx), sizeOf(tx) / esz);
+            rxSrc.emplace_back(recv.remoteCclMem.addr, rxOff, sizeOf(rx), sizeOf(rx) / esz);
+            rxDst.emplace_back(ccl, rxOff, sizeOf(rx), sizeOf(rx) / esz);
+        }
+        SendRecvReduceInfo info{{send, recv}, {{txSrc, txDst}, {rxSrc, rxDst}}, dataType_, reduceOp_};
+        CHK_RET(SendRecvBatchWriteReduce(info, th));
+    }
+    const u64 size = sizeOf(me);
+    return LocalCopy(th, DataSlice(ccl, p.buffInfo.hcclBuffBaseOff + p.sliceSize * me, size),
+                     DataSlice(p.buffInfo.outputPtr, p.buffInfo.outBuffBaseOff + me * p.outputSliceStride, size));
+}
+
+}  // namespace ops_hccl

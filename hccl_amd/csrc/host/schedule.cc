@@ -1,0 +1,791 @@
+#include "schedule.h"
+
+#include <algorithm>
+#include <cstring>
+#include <map>
+#include <sstream>
+#include <unordered_map>
+
+#include "executor.h"
+#include "hcclx.h"
+#include "selector.h"
+
+namespace ops_hccl {
+
+void SetForcedAlgorithm(World *w, HcclCMDType type, const std::string &algName)
+{
+    std::lock_guard<std::mutex> lock(w->mu);
+    w->forcedAlg[static_cast<int>(type)] = algName;
+}
+
+std::string GetForcedAlgorithm(World *w, HcclCMDType type)
+{
+    auto it = w->forcedAlg.find(static_cast<int>(type));
+    return it == w->forcedAlg.end() ? std::string() : it->second;
+}
+
+void SetWorldTopo(World *w, u32 levels, Level0Shape shape, u32 devicesPerServer)
+{
+    std::lock_guard<std::mutex> lock(w->mu);
+    w->topoLevels = levels;
+    w->topoShape = shape;
+    w->devicesPerServer = devicesPerServer;
+}
+
+namespace {
+
+bool IsDataOp(const TaskItem &it) { return it.kind == ItemKind::COPY || it.kind == ItemKind::REDUCE; }
+
+// ---------------------------------------------------------------------------------------------------
+// dependency order of the recorded steps
+// ---------------------------------------------------------------------------------------------------
+struct Node {
+    const TaskItem *item = nullptr;
+    u32 level = 0;
+};
+
+// Flattens every thread's items into `order` (a topological order) and gives each data step a level:
+// steps of one level do not depend on each other.  Fails when a wait has no matching record (the
+// schedule would hang) or the dependencies form a cycle.
+HcclResult BuildOrder(World *w, std::vector<Node> &order, u32 &numLevels)
+{
+    struct Flat {
+        const TaskItem *item;
+        int prev;   // previous item of the same thread
+        int match;  // for a wait: the record that releases it
+        u32 level;
+        u32 indeg;
+    };
+    std::vector<Flat> flat;
+    std::map<std::pair<u64, u32>, int> records;
+    for (auto &perRank : w->threads) {
+        for (auto &t : perRank) {
+            int prev = -1;
+            for (const TaskItem &it : t->items) {
+                const int id = static_cast<int>(flat.size());
+                flat.push_back({&it, prev, -1, 0, 0});
+                if (it.kind == ItemKind::NOTIFY_RECORD) records[{it.key, it.seq}] = id;
+                prev = id;
+            }
+        }
+    }
+    std::vector<std::vector<int>> succ(flat.size());
+    for (int id = 0; id < static_cast<int>(flat.size()); ++id) {
+        Flat &f = flat[id];
+        if (f.prev >= 0) {
+            succ[f.prev].push_back(id);
+            f.indeg++;
+        }
+        if (f.item->kind == ItemKind::NOTIFY_WAIT) {
+            auto it = records.find({f.item->key, f.item->seq});
+            CHK_PRT_RET(it == records.end(), HCCL_ERROR("[schedule] a notify wait has no matching record"),
+                        HCCL_E_INTERNAL);
+            f.match = it->second;
+            succ[f.match].push_back(id);
+            f.indeg++;
+        }
+    }
+    std::vector<int> ready;
+    for (int id = 0; id < static_cast<int>(flat.size()); ++id) {
+        if (flat[id].indeg == 0) ready.push_back(id);
+    }
+    order.clear();
+    numLevels = 0;
+    size_t head = 0;
+    while (head < ready.size()) {
+        const int id = ready[head++];
+        const Flat &f = flat[id];
+        if (IsDataOp(*f.item)) {
+            order.push_back({f.item, f.level});
+            numLevels = std::max(numLevels, f.level + 1);
+        }
+        const u32 out = f.level + (IsDataOp(*f.item) ? 1 : 0);
+        for (int s : succ[id]) {
+            flat[s].level = std::max(flat[s].level, out);
+            if (--flat[s].indeg == 0) ready.push_back(s);
+        }
+    }
+    CHK_PRT_RET(head != flat.size(), HCCL_ERROR("[schedule] the recorded handshakes deadlock"), HCCL_E_INTERNAL);
+    std::stable_sort(order.begin(), order.end(), [](const Node &a, const Node &b) { return a.level < b.level; });
+    return HCCL_SUCCESS;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// STEP mode: every recorded copy / reduce is launched, one fold launch per level and kind
+// ---------------------------------------------------------------------------------------------------
+HcclResult LaunchSteps(World *w, const std::vector<Node> &order, u32 numLevels, int dtype, int op, void *stream)
+{
+    size_t i = 0;
+    w->lastLaunches = 0;
+    for (u32 level = 0; level < numLevels; ++level) {
+        std::vector<hcclx_seg_t> copies;
+        std::vector<hcclx_seg_t> reduces;
+        for (; i < order.size() && order[i].level == level; ++i) {
+            const TaskItem &it = *order[i].item;
+            hcclx_seg_t s;
+            std::memset(&s, 0, sizeof(s));
+            if (it.kind == ItemKind::COPY) {
+                s.count = it.bytes;
+                s.nsrc = 1;
+                s.ndst = 1;
+                s.src[0] = it.src;
+                s.dst[0] = it.dst;
+                copies.push_back(s);
+            } else {
+                s.count = it.count;
+                s.nsrc = 2;  // dst = src (+) dst: the accumulator comes first in fold order
+                s.ndst = 1;
+                s.src[0] = it.dst;
+                s.src[1] = it.src;
+                s.dst[0] = it.dst;
+                reduces.push_back(s);
+            }
+        }
+        if (!copies.empty()) {
+            const int rc = hcclx_fold(copies.data(), static_cast<uint32_t>(copies.size()), HCCL_DATA_TYPE_INT8, 0,
+                                      HCCLX_FOLD_CHAIN, stream);
+            if (rc != HCCL_SUCCESS) return static_cast<HcclResult>(rc);
+            w->lastLaunches++;
+        }
+        if (!reduces.empty()) {
+            const int rc = hcclx_fold(reduces.data(), static_cast<uint32_t>(reduces.size()), dtype, op,
+                                      HCCLX_FOLD_CHAIN, stream);
+            if (rc != HCCL_SUCCESS) return static_cast<HcclResult>(rc);
+            w->lastLaunches++;
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// FUSED mode: symbolic execution
+// ---------------------------------------------------------------------------------------------------
+// An expression gives a byte stream: value(e, off).  Expression 0 is memory as it was when the collective
+// started: value(0, off) = mem[off] (off is an absolute address).  Any other expression is one reduce
+// step: value(e, off) = value(src, off + srcShift) (+) value(dst, off + dstShift).
+struct Expr {
+    int src = -1;
+    int dst = -1;
+    u64 srcShift = 0;
+    u64 dstShift = 0;
+};
+
+struct Piece {
+    u64 len = 0;
+    int expr = 0;
+    u64 shift = 0;  // value at address a of the piece = value(expr, a - start + shift)
+};
+
+struct Sub {
+    u64 start;
+    u64 len;
+    int expr;
+    u64 shift;
+};
+
+class Tracer {
+public:
+    Tracer() { exprs_.push_back(Expr()); }
+
+    void Copy(u64 dst, u64 src, u64 len)
+    {
+        const std::vector<Sub> from = Lookup(src, len);
+        Erase(dst, len);
+        for (const Sub &s : from) {
+            Piece p;
+            p.len = s.len;
+            p.expr = s.expr;
+            p.shift = s.shift;
+            mem_[dst + (s.start - src)] = p;
+        }
+    }
+
+    void Reduce(u64 dst, u64 src, u64 len)
+    {
+        const std::vector<Sub> a = Lookup(src, len);
+        const std::vector<Sub> b = Lookup(dst, len);
+        Erase(dst, len);
+        size_t ia = 0;
+        size_t ib = 0;
+        u64 off = 0;
+        while (off < len) {
+            const Sub &sa = a[ia];
+            const Sub &sb = b[ib];
+            const u64 endA = sa.start - src + sa.len;
+            const u64 endB = sb.start - dst + sb.len;
+            const u64 end = std::min(endA, endB);
+            Expr e;
+            e.src = sa.expr;
+            e.srcShift = sa.shift + (off - (sa.start - src));
+            e.dst = sb.expr;
+            e.dstShift = sb.shift + (off - (sb.start - dst));
+            exprs_.push_back(e);
+            Piece p;
+            p.len = end - off;
+            p.expr = static_cast<int>(exprs_.size()) - 1;
+            p.shift = 0;
+            mem_[dst + off] = p;
+            off = end;
+            if (off == endA) ++ia;
+            if (off == endB) ++ib;
+        }
+    }
+
+    // The pieces that cover [addr, addr + len): written ranges as recorded, untouched ranges as memory.
+    std::vector<Sub> Lookup(u64 addr, u64 len) const
+    {
+        std::vector<Sub> out;
+        u64 cur = addr;
+        const u64 end = addr + len;
+        auto it = mem_.upper_bound(addr);
+        if (it != mem_.begin()) {
+            auto pv = std::prev(it);
+            if (pv->first + pv->second.len > addr) it = pv;
+        }
+        while (cur < end) {
+            if (it == mem_.end() || it->first >= end) {
+                out.push_back({cur, end - cur, 0, cur});
+                break;
+            }
+            if (it->first > cur) {
+                out.push_back({cur, it->first - cur, 0, cur});
+                cur = it->first;
+            }
+            const u64 pEnd = std::min(end, it->first + it->second.len);
+            out.push_back({cur, pEnd - cur, it->second.expr, it->second.shift + (cur - it->first)});
+            cur = pEnd;
+            ++it;
+        }
+        return out;
+    }
+
+    const Expr &At(int e) const { return exprs_[e]; }
+
+private:
+    void Split(u64 addr)
+    {
+        auto it = mem_.upper_bound(addr);
+        if (it == mem_.begin()) return;
+        --it;
+        if (it->first < addr && it->first + it->second.len > addr) {
+            Piece tail = it->second;
+            const u64 cut = addr - it->first;
+            tail.len -= cut;
+            tail.shift += cut;
+            it->second.len = cut;
+            mem_[addr] = tail;
+        }
+    }
+
+    void Erase(u64 addr, u64 len)
+    {
+        Split(addr);
+        Split(addr + len);
+        mem_.erase(mem_.lower_bound(addr), mem_.lower_bound(addr + len));
+    }
+
+    std::map<u64, Piece> mem_;
+    std::vector<Expr> exprs_;
+};
+
+// One output piece flattened to a fold: source addresses in fold order.
+struct Fold {
+    std::vector<u64> src;
+    u64 dst = 0;
+    u64 bytes = 0;
+    bool chain = true;  // false: a tree that no chain reproduces
+};
+
+bool IsFloatType(int dt)
+{
+    return dt == HCCL_DATA_TYPE_FP16 || dt == HCCL_DATA_TYPE_FP32 || dt == HCCL_DATA_TYPE_FP64 ||
+           dt == HCCL_DATA_TYPE_BFP16;
+}
+
+void CollectLeaves(const Tracer &tr, int e, u64 shift, std::vector<u64> &out)
+{
+    if (e == 0) {
+        out.push_back(shift);
+        return;
+    }
+    const Expr &x = tr.At(e);
+    CollectLeaves(tr, x.dst, shift + x.dstShift, out);
+    CollectLeaves(tr, x.src, shift + x.srcShift, out);
+}
+
+std::string ExprText(const Tracer &tr, int e, u64 shift, const std::vector<OpParam> &params)
+{
+    if (e == 0) {
+        for (size_t r = 0; r < params.size(); ++r) {
+            const u64 base = reinterpret_cast<u64>(params[r].inputPtr);
+            if (shift >= base && shift < base + std::max<u64>(params[r].inputSize, 1)) {
+                std::ostringstream os;
+                os << "x" << r << "@" << (shift - base);
+                return os.str();
+            }
+        }
+        return "?";
+    }
+    const Expr &x = tr.At(e);
+    return "(" + ExprText(tr, x.src, shift + x.srcShift, params) + "+" + ExprText(tr, x.dst, shift + x.dstShift, params) +
+           ")";
+}
+
+// Turns the expression of a piece into a fold.  A left-deep spine "leaf (+) acc" is a chain as it
+// stands.  Integer arithmetic (wrap-around sum and product, max, min) is associative and commutative, so
+// any tree equals the chain of its leaves.  For floating types IEEE addition and multiplication are
+// commutative but not associative: "acc (+) leaf" still equals "leaf (+) acc" bit for bit (NaN payloads
+// aside), other tree shapes do not flatten; max/min additionally depend on operand order for NaN and
+// signed zeros, so only the exact spine is taken.
+Fold Flatten(const Tracer &tr, int e, u64 shift, int dtype, int op)
+{
+    Fold f;
+    if (!IsFloatType(dtype)) {
+        CollectLeaves(tr, e, shift, f.src);
+        return f;
+    }
+    const bool commutes = (op == HCCL_REDUCE_SUM || op == HCCL_REDUCE_PROD);
+    std::vector<u64> rev;  // leaves from the outermost step inwards
+    int cur = e;
+    u64 sh = shift;
+    while (cur != 0) {
+        const Expr &x = tr.At(cur);
+        if (x.src == 0) {
+            rev.push_back(sh + x.srcShift);
+            sh += x.dstShift;
+            cur = x.dst;
+        } else if (x.dst == 0 && commutes) {
+            rev.push_back(sh + x.dstShift);
+            sh += x.srcShift;
+            cur = x.src;
+        } else {
+            f.chain = false;
+            return f;
+        }
+    }
+    f.src.push_back(sh);
+    for (auto it = rev.rbegin(); it != rev.rend(); ++it) f.src.push_back(*it);
+    return f;
+}
+
+struct FusedPlan {
+    std::vector<hcclx_seg_t> chainSegs;
+    std::vector<hcclx_seg_t> selfSegs;
+    std::vector<hcclx_seg_t> copySegs;
+};
+
+bool Overlaps(u64 a, u64 alen, u64 b, u64 blen) { return a < b + blen && b < a + alen; }
+
+// Builds the fused launch plan from the traced outputs.  Returns false when the schedule cannot be fused
+// (a floating-point tree, a source that is not an input, or an output that overlaps another fold's
+// source); the caller then runs the steps one by one.
+bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &params, int dtype, int op, u32 esz,
+                    FusedPlan &plan, std::string *text)
+{
+    std::vector<Fold> folds;
+    bool allChains = true;
+    for (size_t r = 0; r < params.size(); ++r) {
+        const u64 out = reinterpret_cast<u64>(params[r].outputPtr);
+        if (params[r].outputSize == 0) continue;
+        for (const Sub &s : tr.Lookup(out, params[r].outputSize)) {
+            if (s.expr == 0 && s.shift == s.start) continue;  // never written: stays as it is
+            Fold f = Flatten(tr, s.expr, s.shift, dtype, op);
+            f.dst = s.start;
+            f.bytes = s.len;
+            if (text) {
+                std::ostringstream os;
+                os << "rank " << r << " out[" << (s.start - out) << "," << s.len << ") = "
+                   << ExprText(tr, s.expr, s.shift, params) << "\n";
+                *text += os.str();
+            }
+            if (!f.chain) allChains = false;
+            folds.push_back(std::move(f));
+        }
+    }
+    if (!allChains) return false;
+    // every source must be input data (or an output that the same fold overwrites in place)
+    for (const Fold &f : folds) {
+        for (u64 a : f.src) {
+            bool ok = false;
+            for (const OpParam &p : params) {
+                const u64 in = reinterpret_cast<u64>(p.inputPtr);
+                if (a >= in && a + f.bytes <= in + p.inputSize) ok = true;
+            }
+            if (!ok) return false;
+        }
+    }
+    if (folds.size() > 100000) return false;
+
+    // group folds with the same sources in the same order: one segment, several destinations
+    std::map<std::vector<u64>, std::vector<size_t>> bySrc;
+    for (size_t i = 0; i < folds.size(); ++i) {
+        std::vector<u64> key = folds[i].src;
+        key.push_back(folds[i].bytes);
+        bySrc[key].push_back(i);
+    }
+    // and find groups of N folds over the same N sources where fold j starts from source j and then takes
+    // the others in a common order: the per-rank order of the one-shot templates, computed in one pass
+    std::map<std::vector<u64>, std::vector<size_t>> bySet;
+    for (auto &kv : bySrc) {
+        if (kv.second.size() != 1) continue;
+        const Fold &f = folds[kv.second[0]];
+        if (f.src.size() < 2 || f.src.size() > HCCLX_MAX_FAN) continue;
+        std::vector<u64> key = f.src;
+        std::sort(key.begin(), key.end());
+        key.push_back(f.bytes);
+        bySet[key].push_back(kv.second[0]);
+    }
+    std::vector<bool> taken(folds.size(), false);
+    std::vector<int> group(folds.size(), -1);
+    for (auto &kv : bySet) {
+        const std::vector<size_t> &grp = kv.second;
+        const size_t n = folds[grp[0]].src.size();
+        if (grp.size() != n || n < 2) continue;
+        for (size_t cand : grp) {  // the fold whose own source comes first in the common order
+            const std::vector<u64> &base = folds[cand].src;
+            std::vector<int> owner(n, -1);
+            bool ok = true;
+            for (size_t g : grp) {
+                const std::vector<u64> &s = folds[g].src;
+                size_t j = 0;
+                while (j < n && base[j] != s[0]) ++j;
+                if (j == n || owner[j] != -1) {
+                    ok = false;
+                    break;
+                }
+                size_t pos = 1;
+                for (size_t k = 0; k < n && ok; ++k) {
+                    if (k == j) continue;
+                    if (s[pos++] != base[k]) ok = false;
+                }
+                if (!ok) break;
+                owner[j] = static_cast<int>(g);
+            }
+            if (!ok) continue;
+            hcclx_seg_t seg;
+            std::memset(&seg, 0, sizeof(seg));
+            seg.count = folds[cand].bytes / esz;
+            seg.nsrc = static_cast<uint32_t>(n);
+            seg.ndst = static_cast<uint32_t>(n);
+            for (size_t j = 0; j < n; ++j) {
+                seg.src[j] = reinterpret_cast<const void *>(base[j]);
+                seg.dst[j] = reinterpret_cast<void *>(folds[owner[j]].dst);
+                taken[owner[j]] = true;
+                group[owner[j]] = static_cast<int>(plan.selfSegs.size());
+            }
+            plan.selfSegs.push_back(seg);
+            break;
+        }
+    }
+    // A destination may coincide exactly with a source of its own fold, or of a fold of the same
+    // self-first group (every thread reads all sources of an element before it writes any destination):
+    // that is an in-place collective.  Any other overlap between what one fold writes and what another
+    // reads would be a race inside a single pass.
+    for (size_t i = 0; i < folds.size(); ++i) {
+        for (size_t j = 0; j < folds.size(); ++j) {
+            for (u64 a : folds[j].src) {
+                if (!Overlaps(folds[i].dst, folds[i].bytes, a, folds[j].bytes)) continue;
+                const bool sameUnit = (i == j) || (group[i] != -1 && group[i] == group[j]);
+                if (sameUnit && a == folds[i].dst) continue;
+                return false;
+            }
+        }
+    }
+    for (auto &kv : bySrc) {
+        std::vector<size_t> rest;
+        for (size_t i : kv.second) {
+            if (!taken[i]) rest.push_back(i);
+        }
+        for (size_t at = 0; at < rest.size(); at += HCCLX_MAX_FAN) {
+            const Fold &f = folds[rest[at]];
+            if (f.src.size() > HCCLX_MAX_FAN) return false;
+            hcclx_seg_t seg;
+            std::memset(&seg, 0, sizeof(seg));
+            seg.nsrc = static_cast<uint32_t>(f.src.size());
+            for (size_t k = 0; k < f.src.size(); ++k) seg.src[k] = reinterpret_cast<const void *>(f.src[k]);
+            for (size_t d = at; d < rest.size() && d < at + HCCLX_MAX_FAN; ++d) {
+                seg.dst[seg.ndst++] = reinterpret_cast<void *>(folds[rest[d]].dst);
+            }
+            if (f.src.size() == 1) {
+                seg.count = f.bytes;  // a copy: counted in bytes
+                plan.copySegs.push_back(seg);
+            } else {
+                seg.count = f.bytes / esz;
+                plan.chainSegs.push_back(seg);
+            }
+        }
+    }
+    (void)w;
+    return true;
+}
+
+std::string PlanKey(const std::vector<OpParam> &params, const std::string &alg, u64 cclBytes)
+{
+    std::ostringstream os;
+    const OpParam &p0 = params[0];
+    os << static_cast<int>(p0.opType) << "|" << alg << "|" << p0.DataDes.dataType << "|" << p0.reduceType << "|"
+       << p0.DataDes.count << "|" << cclBytes;
+    for (const OpParam &p : params) os << "|" << p.inputPtr << "," << p.outputPtr << "," << p.inputSize;
+    return os.str();
+}
+
+HcclResult LaunchPlans(World *w, const std::vector<hcclx_plan *> &plans, void *stream)
+{
+    w->lastLaunches = 0;
+    for (hcclx_plan *p : plans) {
+        const int rc = hcclx_plan_launch(p, stream);
+        if (rc != HCCL_SUCCESS) return static_cast<HcclResult>(rc);
+        w->lastLaunches++;
+    }
+    return HCCL_SUCCESS;
+}
+
+bool SameOperands(const OpParam &a, const OpParam &b)
+{
+    if (a.opType != b.opType) return false;
+    switch (a.opType) {
+        case HcclCMDType::HCCL_CMD_ALLREDUCE:
+        case HcclCMDType::HCCL_CMD_REDUCE_SCATTER:
+            return a.DataDes.count == b.DataDes.count && a.DataDes.dataType == b.DataDes.dataType &&
+                   a.reduceType == b.reduceType;
+        case HcclCMDType::HCCL_CMD_ALLGATHER:
+            return a.DataDes.count == b.DataDes.count && a.DataDes.dataType == b.DataDes.dataType;
+        case HcclCMDType::HCCL_CMD_ALLGATHER_V:
+            return a.vDataDes.dataType == b.vDataDes.dataType && a.vDataDes.counts == b.vDataDes.counts &&
+                   a.vDataDes.displs == b.vDataDes.displs;
+        default:
+            return a.all2AllVDataDes.sendType == b.all2AllVDataDes.sendType;
+    }
+}
+
+bool IsDataMove(HcclCMDType t)
+{
+    return t == HcclCMDType::HCCL_CMD_ALLGATHER || t == HcclCMDType::HCCL_CMD_ALLGATHER_V ||
+           t == HcclCMDType::HCCL_CMD_ALLTOALL || t == HcclCMDType::HCCL_CMD_ALLTOALLV ||
+           t == HcclCMDType::HCCL_CMD_ALLTOALLVC;
+}
+
+// Pure data movement has no fold order to preserve: in FUSED mode the contract itself is launched on the
+// ragged-copy kernels (one read and one write per delivered byte), with the tables of all ranks.
+HcclResult LaunchDataMove(World *w, const std::vector<OpParam> &params, void *stream)
+{
+    const u32 n = w->rankSize;
+    std::vector<const void *> send(n);
+    std::vector<void *> recv(n);
+    for (u32 r = 0; r < n; ++r) {
+        send[r] = params[r].inputPtr;
+        recv[r] = params[r].outputPtr;
+    }
+    const HcclCMDType t = params[0].opType;
+    w->lastLaunches = 1;
+    if (t == HcclCMDType::HCCL_CMD_ALLGATHER || t == HcclCMDType::HCCL_CMD_ALLGATHER_V) {
+        std::vector<u64> counts(n);
+        std::vector<u64> displs(n);
+        for (u32 r = 0; r < n; ++r) {
+            if (t == HcclCMDType::HCCL_CMD_ALLGATHER) {
+                counts[r] = params[0].DataDes.count;
+                displs[r] = r * params[0].DataDes.count;
+            } else {
+                counts[r] = params[0].vDataDes.counts[r];
+                displs[r] = params[0].vDataDes.displs[r];
+            }
+        }
+        const int dt = (t == HcclCMDType::HCCL_CMD_ALLGATHER) ? params[0].DataDes.dataType : params[0].vDataDes.dataType;
+        return static_cast<HcclResult>(
+            hcclx_allgatherv(send.data(), recv.data(), counts.data(), displs.data(), n, dt, 0, stream));
+    }
+    std::vector<u64> sc(static_cast<size_t>(n) * n);
+    std::vector<u64> sd(static_cast<size_t>(n) * n);
+    std::vector<u64> rd(static_cast<size_t>(n) * n);
+    for (u32 i = 0; i < n; ++i) {
+        for (u32 j = 0; j < n; ++j) {
+            sc[i * n + j] = params[i].all2AllVDataDes.sendCounts[j];
+            sd[i * n + j] = params[i].all2AllVDataDes.sdispls[j];
+            rd[i * n + j] = params[i].all2AllVDataDes.rdispls[j];
+        }
+    }
+    return static_cast<HcclResult>(hcclx_alltoallv(send.data(), recv.data(), sc.data(), sd.data(), rd.data(), n,
+                                                   params[0].all2AllVDataDes.sendType, 0, stream));
+}
+
+}  // namespace
+
+namespace {
+HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params);
+
+// Ranks may pass different streams.  The collective runs on the stream of the last rank; it first waits
+// for everything the other ranks' streams hold so far (their inputs), and those streams then wait for it.
+HcclResult JoinStreams(const std::vector<OpParam> &params, hipStream_t launch, bool before)
+{
+    std::vector<hipStream_t> others;
+    for (const OpParam &p : params) {
+        hipStream_t s = static_cast<hipStream_t>(p.stream);
+        if (s != launch && std::find(others.begin(), others.end(), s) == others.end()) others.push_back(s);
+    }
+    for (hipStream_t s : others) {
+        hipEvent_t ev;
+        if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) return HCCL_E_RUNTIME;
+        const hipError_t e1 = hipEventRecord(ev, before ? s : launch);
+        const hipError_t e2 = hipStreamWaitEvent(before ? launch : s, ev, 0);
+        (void)hipEventDestroy(ev);  // released once the recorded work has passed it
+        if (e1 != hipSuccess || e2 != hipSuccess) return HCCL_E_RUNTIME;
+    }
+    return HCCL_SUCCESS;
+}
+}  // namespace
+
+HcclResult RunCollective(World *w, std::vector<OpParam> &params)
+{
+    if (w->dryRun) return RunCollectiveOnStream(w, params);
+    hipStream_t launch = static_cast<hipStream_t>(params[w->rankSize - 1].stream);
+    CHK_RET(JoinStreams(params, launch, true));
+    const HcclResult res = RunCollectiveOnStream(w, params);
+    CHK_RET(JoinStreams(params, launch, false));
+    return res;
+}
+
+namespace {
+HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
+{
+    const u32 n = w->rankSize;
+    // every rank must have issued the same collective with the same operands
+    for (u32 r = 1; r < n; ++r) {
+        CHK_PRT_RET(!SameOperands(params[0], params[r]),
+                    HCCL_ERROR("[RunCollective] rank %u issued a different collective than rank 0", r), HCCL_E_PARA);
+    }
+    const HcclCMDType type = params[0].opType;
+    if (IsDataMove(type)) {
+        // what i sends to j must be what j expects from i
+        for (u32 i = 0; i < n && type != HcclCMDType::HCCL_CMD_ALLGATHER && type != HcclCMDType::HCCL_CMD_ALLGATHER_V;
+             ++i) {
+            for (u32 j = 0; j < n; ++j) {
+                CHK_PRT_RET(params[i].all2AllVDataDes.sendCounts[j] != params[j].all2AllVDataDes.recvCounts[i],
+                            HCCL_ERROR("[RunCollective] sendCounts[%u][%u] != recvCounts[%u][%u]", i, j, j, i),
+                            HCCL_E_PARA);
+            }
+        }
+    }
+
+    // algorithm: forced for this world, or the selector's choice
+    std::string algName = GetForcedAlgorithm(w, type);
+    if (algName.empty()) {
+        TopoInfoWithNetLayerDetails topo;
+        topo.userRankSize = n;
+        topo.topoLevelNums = w->topoLevels;
+        topo.level0Topo = w->topoShape;
+        topo.localNetInsSizeOfLayer0 = w->devicesPerServer ? w->devicesPerServer : n;
+        CHK_RET(ExecuteSelector().Run(params[0], &topo, algName));
+    }
+    w->lastAlgName = algName;
+    w->lastWasFused = false;
+    w->lastPlanCacheHit = false;
+    w->lastFusedSegments = 0;
+    w->lastLevels = 0;
+    void *stream = params[n - 1].stream;
+
+    const int dtype = params[0].DataDes.dataType;
+    const int op = params[0].reduceType;
+    const bool fused = (w->mode == ExecMode::FUSED);
+    if (fused && !w->dryRun && !w->traceText && IsDataMove(type)) {
+        w->lastWasFused = true;
+        return LaunchDataMove(w, params, stream);
+    }
+    std::string key;
+    if (fused && !w->dryRun && !w->traceText) {
+        key = PlanKey(params, algName, w->cclBytes);
+        for (CachedPlan &c : w->planCache) {
+            if (c.key == key) {
+                c.lastUse = ++w->useCounter;
+                w->lastWasFused = true;
+                w->lastPlanCacheHit = true;
+                return LaunchPlans(w, c.plans, stream);
+            }
+        }
+    }
+
+    // expand: every rank's executor + template records its steps
+    CHK_RET(w->EnsureScratch());
+    w->ResetRecording();
+    for (u32 r = 0; r < n; ++r) {
+        params[r].algName = algName;
+        std::unique_ptr<InsCollAlgBase> exec = CollAlgExecRegistryV2::Instance().GetAlgExec(type, algName);
+        CHK_PRT_RET(exec == nullptr, HCCL_ERROR("[RunCollective] no executor named %s", algName.c_str()),
+                    HCCL_E_NOT_SUPPORT);
+        AlgResourceCtxSerializable resCtx;
+        const u64 threadNum = exec->CalcThreadNum(params[r], r, n);
+        FillResources(w, r, static_cast<u32>(threadNum), resCtx);
+        CHK_RET(exec->Orchestrate(params[r], resCtx));
+    }
+    std::vector<Node> order;
+    u32 numLevels = 0;
+    CHK_RET(BuildOrder(w, order, numLevels));
+    w->lastLevels = numLevels;
+
+    const u32 esz = IsDataMove(type) ? 1 : DATATYPE_SIZE_TABLE[dtype];
+    const int foldType = IsDataMove(type) ? HCCL_DATA_TYPE_INT8 : dtype;
+    if (fused || w->dryRun || w->traceText) {
+        Tracer tr;
+        for (const Node &nd : order) {
+            const TaskItem &it = *nd.item;
+            if (it.kind == ItemKind::COPY) {
+                tr.Copy(reinterpret_cast<u64>(it.dst), reinterpret_cast<u64>(it.src), it.bytes);
+            } else {
+                tr.Reduce(reinterpret_cast<u64>(it.dst), reinterpret_cast<u64>(it.src), it.bytes);
+            }
+        }
+        FusedPlan plan;
+        w->lastTrace.clear();
+        const bool ok = BuildFusedPlan(w, tr, params, foldType, op, esz, plan,
+                                       (w->traceText || w->dryRun) ? &w->lastTrace : nullptr);
+        w->lastFusedSegments =
+            static_cast<u32>(plan.chainSegs.size() + plan.selfSegs.size() + plan.copySegs.size());
+        if (w->dryRun) {
+            w->lastWasFused = ok;
+            return HCCL_SUCCESS;
+        }
+        if (ok && fused) {
+            CachedPlan c;
+            c.key = key;
+            const std::pair<std::vector<hcclx_seg_t> *, int> parts[3] = {
+                {&plan.selfSegs, HCCLX_FOLD_SELF_FIRST}, {&plan.chainSegs, HCCLX_FOLD_CHAIN},
+                {&plan.copySegs, HCCLX_FOLD_CHAIN}};
+            for (int i = 0; i < 3; ++i) {
+                if (parts[i].first->empty()) continue;
+                hcclx_plan *hp = nullptr;
+                const int dt = (i == 2) ? HCCL_DATA_TYPE_INT8 : foldType;
+                const int rc = hcclx_plan_create(parts[i].first->data(), static_cast<uint32_t>(parts[i].first->size()),
+                                                 dt, op, parts[i].second, &hp);
+                if (rc != HCCL_SUCCESS) {
+                    for (hcclx_plan *q : c.plans) (void)hcclx_plan_destroy(q);
+                    return static_cast<HcclResult>(rc);
+                }
+                c.plans.push_back(hp);
+            }
+            w->lastWasFused = true;
+            const HcclResult res = LaunchPlans(w, c.plans, stream);
+            if (!key.empty() && res == HCCL_SUCCESS) {
+                c.lastUse = ++w->useCounter;
+                if (w->planCache.size() >= 32) {  // evict the least recently used plan
+                    size_t victim = 0;
+                    for (size_t i = 1; i < w->planCache.size(); ++i) {
+                        if (w->planCache[i].lastUse < w->planCache[victim].lastUse) victim = i;
+                    }
+                    // its kernels may still be queued: wait for the device before the tables are freed
+                    (void)hipDeviceSynchronize();
+                    for (hcclx_plan *q : w->planCache[victim].plans) (void)hcclx_plan_destroy(q);
+                    w->planCache.erase(w->planCache.begin() + victim);
+                }
+                w->planCache.push_back(std::move(c));
+            } else {
+                (void)hipDeviceSynchronize();
+                for (hcclx_plan *q : c.plans) (void)hcclx_plan_destroy(q);
+            }
+            return res;
+        }
+    }
+    return LaunchSteps(w, order, numLevels, foldType, op, stream);
+}
+
+}  // namespace
+
+}  // namespace ops_hccl

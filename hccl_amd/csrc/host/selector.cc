@@ -1,0 +1,161 @@
+#include "selector.h"
+
+namespace ops_hccl {
+
+SelectorRegistry *SelectorRegistry::Global()
+{
+    static SelectorRegistry *inst = new SelectorRegistry;
+    return inst;
+}
+
+HcclResult SelectorRegistry::RegisterByOpType(HcclCMDType opType, u32 priority, AutoSelectorBase *selector)
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    if (opTypeImpls_[opType].count(priority)) return HCCL_E_INTERNAL;
+    opTypeImpls_[opType][priority] = selector;
+    return HCCL_SUCCESS;
+}
+
+std::map<u32, AutoSelectorBase *> SelectorRegistry::GetSelectorsByOpType(HcclCMDType opType)
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    return opTypeImpls_[opType];
+}
+
+HcclResult ExecuteSelector::Run(OpParam &opParam, TopoInfoWithNetLayerDetails *topoInfo,
+                                std::string &selectAlgName) const
+{
+    for (auto &kv : SelectorRegistry::Global()->GetSelectorsByOpType(opParam.opType)) {
+        if (kv.second->Select(opParam, topoInfo, selectAlgName) == SelectorStatus::MATCH) return HCCL_SUCCESS;
+    }
+    HCCL_ERROR("[Algo][Selector] No selector is matched.");
+    return HCCL_E_NOT_SUPPORT;
+}
+
+namespace {
+
+bool IsSpecial(HcclDataType dt, HcclReduceOp op)
+{
+    return dt == HCCL_DATA_TYPE_INT64 || dt == HCCL_DATA_TYPE_UINT64 || dt == HCCL_DATA_TYPE_FP64 ||
+           op == HCCL_REDUCE_PROD;
+}
+
+// ---- AllReduce (src/ops/all_reduce/selector/all_reduce_auto_selector.cc:351-529) -----------------------
+constexpr u64 AR_AICPU_1D_SMALL_DATA_SIZE = 8ull * 1024 * 1024;
+constexpr u64 AR_AICPU_1D_MAX_DATA_SIZE = 32ull * 1024 * 1024;
+constexpr u64 AR_AICPU_1D_64DATATYPE_DATA_SIZE = 8ull * 1024 * 1024;
+
+class AllReduceAutoSelector : public AutoSelectorBase {
+protected:
+    SelectorStatus SelectAicpuAlgo(const TopoInfoWithNetLayerDetails *topo, const OpParam &p,
+                                   std::string &name) const override
+    {
+        const u64 dataSize = p.DataDes.count * DATATYPE_SIZE_TABLE[p.DataDes.dataType];
+        const bool special = IsSpecial(p.DataDes.dataType, p.reduceType);
+        if (topo->topoLevelNums > 1) {
+            // several levels: the flat log-step algorithm; the reference's hierarchical mesh+NHR
+            // combinations (:396-409) need real link tiers and are not built
+            name = special ? "InsAllReduceAicpuReduceNHR" : "InsAllReduceNHR";
+            return SelectorStatus::MATCH;
+        }
+        if (topo->level0Topo == Level0Shape::MESH_1D) {
+            if (special) {
+                name = dataSize <= AR_AICPU_1D_64DATATYPE_DATA_SIZE ? "InsAllReduceMesh1DOneShot"
+                                                                    : "InsAllReduceMesh1DTwoShot";
+            } else if (dataSize <= AR_AICPU_1D_SMALL_DATA_SIZE) {
+                name = "InsAllReduceMesh1DOneShot";
+            } else {
+                // Above size * 8 / N^2 > 32 MiB the reference moves on to its mesh-chunk template
+                // (:485-487), which is not built; the two-shot template takes those sizes too.
+                name = "InsAllReduceMesh1DTwoShot";
+            }
+            return SelectorStatus::MATCH;
+        }
+        if (topo->level0Topo == Level0Shape::CLOS) {
+            name = special ? "InsAllReduceAicpuReduceNHR" : "InsAllReduceNHR";
+            return SelectorStatus::MATCH;
+        }
+        return SelectorStatus::NOT_MATCH;  // MESH_1D_CLOS machines: not modelled
+    }
+};
+
+// ---- ReduceScatter (src/ops/reduce_scatter/selector/reduce_scatter_auto_selector.cc:328-446) ---------------
+class ReduceScatterAutoSelector : public AutoSelectorBase {
+protected:
+    SelectorStatus SelectAicpuAlgo(const TopoInfoWithNetLayerDetails *topo, const OpParam &p,
+                                   std::string &name) const override
+    {
+        if (topo->topoLevelNums > 1 || topo->level0Topo == Level0Shape::CLOS) {
+            // The reference picks InsReduceScatterAicpuReduceNHR for PROD / 64-bit here (:350, :430);
+            // its fold order is the NHR gather followed by the own-data-first fold, which is what
+            // InsReduceScatterMesh1D computes, so that template serves those types.
+            name = IsSpecial(p.DataDes.dataType, p.reduceType) ? "InsReduceScatterMesh1D" : "InsReduceScatterNHR";
+            return SelectorStatus::MATCH;
+        }
+        if (topo->level0Topo == Level0Shape::MESH_1D) {
+            // dataSize * (8/N)^2 > 16 MiB selects the mesh-chunk template in the reference (:404-408);
+            // it is not built, the mesh template takes those sizes too.
+            name = "InsReduceScatterMesh1D";
+            return SelectorStatus::MATCH;
+        }
+        return SelectorStatus::NOT_MATCH;
+    }
+};
+
+// ---- AllGather (src/ops/all_gather/selector/all_gather_auto_selector.cc:258-340) ---------------------------
+class AllGatherAutoSelector : public AutoSelectorBase {
+protected:
+    SelectorStatus SelectAicpuAlgo(const TopoInfoWithNetLayerDetails *topo, const OpParam &p,
+                                   std::string &name) const override
+    {
+        (void)p;
+        if (topo->topoLevelNums > 1 || topo->level0Topo == Level0Shape::CLOS) {
+            name = "InsAllGatherNHR";
+            return SelectorStatus::MATCH;
+        }
+        if (topo->level0Topo == Level0Shape::MESH_1D) {
+            name = "InsAllGatherMesh1D";
+            return SelectorStatus::MATCH;
+        }
+        return SelectorStatus::NOT_MATCH;
+    }
+};
+
+// ---- AllGatherV: always the mesh template (src/ops/all_gather_v/selector/all_gather_v_auto_selector.cc:63-77)
+class AllGatherVAutoSelector : public AutoSelectorBase {
+protected:
+    SelectorStatus SelectAicpuAlgo(const TopoInfoWithNetLayerDetails *, const OpParam &, std::string &name) const override
+    {
+        name = "InsAllGatherVMesh1D";
+        return SelectorStatus::MATCH;
+    }
+};
+
+// ---- AlltoAll family (src/ops/all_to_all_v/selector/alltoallv_auto_selector.cc:94-128,
+//      alltoall_auto_selector.cc:111-154, alltoallvc_auto_selector.cc:53-62) -------------------------------
+template <int KIND> class AlltoAllFamilySelector : public AutoSelectorBase {
+protected:
+    SelectorStatus SelectAicpuAlgo(const TopoInfoWithNetLayerDetails *topo, const OpParam &, std::string &name) const override
+    {
+        if (topo->level0Topo != Level0Shape::MESH_1D && topo->level0Topo != Level0Shape::CLOS) {
+            return SelectorStatus::NOT_MATCH;
+        }
+        name = KIND == 0 ? "InsAlltoAllMesh1D" : KIND == 1 ? "InsAlltoAllVMesh1D" : "InsAlltoAllVCMesh1D";
+        return SelectorStatus::MATCH;
+    }
+};
+using AlltoAllAutoSelector = AlltoAllFamilySelector<0>;
+using AlltoAllVAutoSelector = AlltoAllFamilySelector<1>;
+using AlltoAllVCAutoSelector = AlltoAllFamilySelector<2>;
+
+}  // namespace
+
+REGISTER_SELECTOR_BY_OPTYPE(HcclCMDType::HCCL_CMD_ALLREDUCE, SELECTOR_PRIORITY_BUILTIN, AllReduceAutoSelector);
+REGISTER_SELECTOR_BY_OPTYPE(HcclCMDType::HCCL_CMD_REDUCE_SCATTER, SELECTOR_PRIORITY_BUILTIN, ReduceScatterAutoSelector);
+REGISTER_SELECTOR_BY_OPTYPE(HcclCMDType::HCCL_CMD_ALLGATHER, SELECTOR_PRIORITY_BUILTIN, AllGatherAutoSelector);
+REGISTER_SELECTOR_BY_OPTYPE(HcclCMDType::HCCL_CMD_ALLGATHER_V, SELECTOR_PRIORITY_BUILTIN, AllGatherVAutoSelector);
+REGISTER_SELECTOR_BY_OPTYPE(HcclCMDType::HCCL_CMD_ALLTOALL, SELECTOR_PRIORITY_BUILTIN, AlltoAllAutoSelector);
+REGISTER_SELECTOR_BY_OPTYPE(HcclCMDType::HCCL_CMD_ALLTOALLV, SELECTOR_PRIORITY_BUILTIN, AlltoAllVAutoSelector);
+REGISTER_SELECTOR_BY_OPTYPE(HcclCMDType::HCCL_CMD_ALLTOALLVC, SELECTOR_PRIORITY_BUILTIN, AlltoAllVCAutoSelector);
+
+}  // namespace ops_hccl

@@ -1,0 +1,80 @@
+// Base class of the algorithm templates (reference: src/ops/op_common/template/common_alg_template_base.h:19-56,
+// alg_v2_template_base.h:18-76, alg_v2_template_base.cc:15-26).  A template turns one executor chunk into
+// copy / reduce / send / receive steps by calling the verbs of alg_data_trans_wrapper.h.
+//
+// Left out on purpose: CalcRes / GetRes / FastLaunch / DPUKernelRun -- resource plumbing for real links,
+// CCU fast launch and DPU offload, none of which exists for virtual ranks in one GPU.
+#pragma once
+#include <string>
+#include <vector>
+
+#include "alg_data_trans_wrapper.h"
+#include "alg_param.h"
+
+namespace ops_hccl {
+
+class InsAlgTemplateBase {
+public:
+    InsAlgTemplateBase(const OpParam &param, u32 rankId, const std::vector<std::vector<u32>> &subCommRanks)
+        : opMode_(param.opMode), myRank_(rankId), subCommRanks_(subCommRanks), reduceOp_(param.reduceType)
+    {
+        templateRankSize_ = subCommRanks.empty() ? 0 : static_cast<u32>(subCommRanks[0].size());
+    }
+    virtual ~InsAlgTemplateBase() = default;
+
+    virtual std::string Describe() const = 0;
+    // Threads (task queues) of this rank the template spreads its steps over.
+    virtual u64 GetThreadNum() const = 0;
+    // How many chunk-sized slots of the scratch buffer one KernelRun needs.
+    virtual u64 CalcScratchMultiple(BufferType inBuffType, BufferType outBuffType) = 0;
+    virtual HcclResult KernelRun(const OpParam &param, const TemplateDataParams &tempAlgParams,
+                                 TemplateResource &templateResource) = 0;
+
+    virtual void GetNotifyIdxMainToSub(std::vector<u32> &notifyIdxMainToSub)
+    {
+        // every sub thread is woken on its own notify 0
+        notifyIdxMainToSub.assign(GetThreadNum() > 0 ? GetThreadNum() - 1 : 0, 0);
+    }
+    virtual void GetNotifyIdxSubToMain(std::vector<u32> &notifyIdxSubToMain)
+    {
+        // the main thread has one notify per sub thread
+        notifyIdxSubToMain.clear();
+        for (u32 i = 0; i + 1 < GetThreadNum(); ++i) notifyIdxSubToMain.push_back(i);
+    }
+
+protected:
+    HcclResult PreSync(const std::vector<ThreadHandle> &threads)
+    {
+        if (threads.size() <= 1) return HCCL_SUCCESS;
+        std::vector<ThreadHandle> subs(threads.begin() + 1, threads.end());
+        std::vector<u32> idx(subs.size(), 0);
+        return PreSyncInterThreads(threads[0], subs, idx);
+    }
+    HcclResult PostSync(const std::vector<ThreadHandle> &threads)
+    {
+        if (threads.size() <= 1) return HCCL_SUCCESS;
+        std::vector<ThreadHandle> subs(threads.begin() + 1, threads.end());
+        std::vector<u32> idx;
+        for (u32 i = 0; i < subs.size(); ++i) idx.push_back(i);
+        return PostSyncInterThreads(threads[0], subs, idx);
+    }
+
+    OpMode opMode_;
+    u32 myRank_ = INVALID_VALUE_RANKID;
+    u32 templateRankSize_ = 0;
+    std::vector<std::vector<u32>> subCommRanks_;
+    u32 threadNum_ = 0;
+    HcclReduceOp reduceOp_;
+    HcclDataType dataType_ = HCCL_DATA_TYPE_RESERVED;
+};
+
+// ceil(count / n) elements per slice, the remainder short or empty
+// (SplitData, src/ops/all_reduce/template/aicpu/ins_temp_all_reduce_nhr.cc:137-163).
+std::vector<SliceInfo> SplitDataByRank(u64 count, u32 sliceNum, u64 dataTypeSize);
+
+// Step tables of the NHR (nonuniform hierarchical ring) algorithm
+// (ins_temp_all_reduce_nhr.cc:325-404).
+void GetNHRReduceScatterSteps(u32 rankSize, u32 myRankIdx, std::vector<NHRStepInfo> &steps);
+void GetNHRAllGatherSteps(u32 rankSize, u32 myRankIdx, std::vector<NHRStepInfo> &steps);
+
+}  // namespace ops_hccl

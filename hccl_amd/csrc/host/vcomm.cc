@@ -1,0 +1,343 @@
+// Virtual-rank world: creation, the recording primitive backend and the rank rendezvous.
+#include "vcomm.h"
+
+#include <cstring>
+
+#include "hcclx.h"
+#include "hcomm_primitives.h"
+#include "schedule.h"
+
+namespace ops_hccl {
+
+namespace {
+
+std::mutex g_worldsMu;
+std::vector<World *> g_worlds;
+
+u64 ChannelKey(u32 sender, u32 receiver, u32 idx)
+{
+    return (1ull << 63) | (static_cast<u64>(sender) << 40) | (static_cast<u64>(receiver) << 16) | idx;
+}
+
+u64 ThreadKey(const VThread *t, u32 idx)
+{
+    return (static_cast<u64>(t->rank) << 40) | (static_cast<u64>(t->index) << 16) | idx;
+}
+
+VThread *AsThread(ThreadHandle h) { return reinterpret_cast<VThread *>(h); }
+VChannel *AsChannel(ChannelHandle h) { return reinterpret_cast<VChannel *>(h); }
+
+int32_t RecordData(ThreadHandle thread, ItemKind kind, void *dst, const void *src, u64 bytes, u64 count, int dtype,
+                   int op)
+{
+    VThread *t = AsThread(thread);
+    if (t == nullptr) return HCCL_E_PTR;
+    if (bytes == 0) return HCCL_SUCCESS;
+    if (dst == nullptr || src == nullptr) return HCCL_E_PTR;
+    TaskItem it;
+    it.kind = kind;
+    it.dst = static_cast<char *>(dst);
+    it.src = static_cast<const char *>(src);
+    it.bytes = bytes;
+    it.count = count;
+    it.dtype = static_cast<u8>(dtype);
+    it.op = static_cast<u8>(op);
+    t->items.push_back(it);
+    return HCCL_SUCCESS;
+}
+
+int32_t RecordNotify(VThread *t, ItemKind kind, u64 key)
+{
+    World *w = t->world;
+    TaskItem it;
+    it.kind = kind;
+    it.key = key;
+    it.seq = (kind == ItemKind::NOTIFY_RECORD) ? w->recordSeq[key]++ : w->waitSeq[key]++;
+    t->items.push_back(it);
+    return HCCL_SUCCESS;
+}
+
+int32_t ReduceArgsOk(HcommDataType dt, HcommReduceOp op)
+{
+    if (dt < 0 || dt >= HCCL_DATA_TYPE_RESERVED) return HCCL_E_PARA;
+    if (op < HCCL_REDUCE_SUM || op > HCCL_REDUCE_MIN) return HCCL_E_PARA;
+    return HCCL_SUCCESS;
+}
+
+}  // namespace
+
+World::~World()
+{
+    for (char *p : cclBuf) {
+        if (p && !dryRun) (void)hipFree(p);
+    }
+    for (CachedPlan &c : planCache) {
+        for (hcclx_plan *p : c.plans) (void)hcclx_plan_destroy(p);
+    }
+}
+
+HcclResult World::EnsureScratch()
+{
+    for (u32 r = 0; r < rankSize; ++r) {
+        if (cclBuf[r] == nullptr && dryRun) {
+            // never dereferenced: a distinct, non-overlapping address range per rank
+            cclBuf[r] = reinterpret_cast<char *>(0x7000000000000000ull + static_cast<u64>(r) * (1ull << 40));
+        }
+        if (cclBuf[r] == nullptr) {
+            hipError_t e = hipMalloc(reinterpret_cast<void **>(&cclBuf[r]), cclBytes);
+            if (e != hipSuccess) {
+                HCCL_ERROR("scratch buffer of rank %u: %s", r, hipGetErrorString(e));
+                return HCCL_E_MEMORY;
+            }
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
+void World::ResetRecording()
+{
+    recordSeq.clear();
+    waitSeq.clear();
+    for (auto &perRank : threads) {
+        for (auto &t : perRank) t->items.clear();
+    }
+}
+
+HcclResult WorldCreate(u32 rankSize, u64 cclBytes, bool dryRun, std::vector<HcclComm> &comms)
+{
+    if (rankSize == 0 || rankSize > 64) return HCCL_E_PARA;
+    // the ReduceScatter executor keeps 1 MiB of the buffer back; leave room for at least one aligned slot per rank
+    if (cclBytes < 1024 * 1024 + 128ull * 64) return HCCL_E_PARA;
+    World *w = new World;
+    w->rankSize = rankSize;
+    w->cclBytes = cclBytes;
+    w->dryRun = dryRun;
+    if (hipGetDevice(&w->device) != hipSuccess) w->device = -1;  // a host-only process can still record
+    if (const char *m = std::getenv("HCCL_VRANK_EXEC_MODE")) {
+        if (std::strcmp(m, "step") == 0) w->mode = ExecMode::STEP;
+    }
+    if (const char *b = std::getenv("HCCL_VRANK_BLOCKING")) w->blocking = (std::atoi(b) != 0);
+    w->cclBuf.assign(rankSize, nullptr);
+    w->queue.resize(rankSize);
+    w->launched.assign(rankSize, 0);
+    w->lastResult.assign(rankSize, HCCL_SUCCESS);
+    w->threads.resize(rankSize);
+    w->channels.resize(rankSize);
+    comms.clear();
+    for (u32 r = 0; r < rankSize; ++r) {
+        w->ranks.emplace_back(new RankComm{w, r});
+        for (u32 t = 0; t < rankSize + 1; ++t) {  // mesh templates use one thread per rank
+            w->threads[r].emplace_back(new VThread);
+            VThread *vt = w->threads[r].back().get();
+            vt->world = w;
+            vt->rank = r;
+            vt->index = t;
+        }
+        for (u32 p = 0; p < rankSize; ++p) {
+            w->channels[r].emplace_back(new VChannel{w, r, p});
+        }
+        comms.push_back(w->ranks.back().get());
+    }
+    std::lock_guard<std::mutex> lock(g_worldsMu);
+    g_worlds.push_back(w);
+    return HCCL_SUCCESS;
+}
+
+RankComm *AsRankComm(HcclComm comm)
+{
+    RankComm *rc = static_cast<RankComm *>(comm);
+    if (rc == nullptr) return nullptr;
+    std::lock_guard<std::mutex> lock(g_worldsMu);
+    for (World *w : g_worlds) {
+        if (rc->world == w && rc->rank < w->rankSize && w->ranks[rc->rank].get() == rc) return rc;
+    }
+    return nullptr;
+}
+
+HcclResult WorldDestroyRank(HcclComm comm)
+{
+    RankComm *rc = AsRankComm(comm);
+    if (rc == nullptr) return HCCL_E_PTR;
+    World *w = rc->world;
+    {
+        std::lock_guard<std::mutex> lock(w->mu);
+        w->launched[rc->rank] = ~0ull;  // marks the rank handle as destroyed
+        for (u64 v : w->launched) {
+            if (v != ~0ull) return HCCL_SUCCESS;
+        }
+    }
+    {
+        std::lock_guard<std::mutex> lock(g_worldsMu);
+        for (size_t i = 0; i < g_worlds.size(); ++i) {
+            if (g_worlds[i] == w) {
+                g_worlds.erase(g_worlds.begin() + i);
+                break;
+            }
+        }
+    }
+    delete w;
+    return HCCL_SUCCESS;
+}
+
+void FillResources(World *w, u32 rank, u32 threadNum, AlgResourceCtxSerializable &resCtx)
+{
+    resCtx.topoInfo.userRank = rank;
+    resCtx.topoInfo.userRankSize = w->rankSize;
+    resCtx.subCommRanks.assign(1, std::vector<u32>());
+    for (u32 r = 0; r < w->rankSize; ++r) resCtx.subCommRanks[0].push_back(r);  // TopoMatch1D: ranks 0..N-1
+    resCtx.cclMem.addr = w->cclBuf[rank];
+    resCtx.cclMem.size = w->cclBytes;
+    resCtx.threads.clear();
+    for (u32 t = 0; t < threadNum && t < w->threads[rank].size(); ++t) {
+        resCtx.threads.push_back(reinterpret_cast<ThreadHandle>(w->threads[rank][t].get()));
+    }
+    resCtx.channels.clear();
+    for (u32 p = 0; p < w->rankSize; ++p) {
+        if (p == rank) continue;
+        ChannelInfo ch;
+        ch.isValid = true;
+        ch.remoteRank = p;
+        ch.notifyNum = 3;
+        ch.portGroupSize = 1;
+        ch.handle = reinterpret_cast<ChannelHandle>(w->channels[rank][p].get());
+        ch.remoteCclMem.addr = w->cclBuf[p];
+        ch.remoteCclMem.size = w->cclBytes;
+        resCtx.channels[p].push_back(ch);
+    }
+}
+
+HcclResult SubmitOp(RankComm *rc, const OpParam &param)
+{
+    World *w = rc->world;
+    std::unique_lock<std::mutex> lock(w->mu);
+    QueuedOp q;
+    q.param = param;
+    w->queue[rc->rank].push_back(std::move(q));
+    const u64 myTicket = w->launched[rc->rank] + w->queue[rc->rank].size();  // collective number of this call
+
+    bool all = true;
+    for (u32 r = 0; r < w->rankSize; ++r) all = all && !w->queue[r].empty();
+    while (all) {
+        std::vector<OpParam> params;
+        for (u32 r = 0; r < w->rankSize; ++r) {
+            params.push_back(std::move(w->queue[r].front().param));
+            w->queue[r].pop_front();
+        }
+        const HcclResult res = RunCollective(w, params);
+        for (u32 r = 0; r < w->rankSize; ++r) {
+            w->launched[r]++;
+            w->lastResult[r] = res;
+        }
+        w->cv.notify_all();
+        all = true;
+        for (u32 r = 0; r < w->rankSize; ++r) all = all && !w->queue[r].empty();
+    }
+    if (w->launched[rc->rank] >= myTicket) return w->lastResult[rc->rank];
+    if (!w->blocking) return HCCL_SUCCESS;  // queued; the last rank to arrive launches
+    w->cv.wait(lock, [&] { return w->launched[rc->rank] >= myTicket; });
+    return w->lastResult[rc->rank];
+}
+
+}  // namespace ops_hccl
+
+// ---------------------------------------------------------------------------------------------------
+// the primitive ABI: every call is recorded on its thread
+// ---------------------------------------------------------------------------------------------------
+using namespace ops_hccl;
+
+extern "C" {
+
+int32_t HcommLocalCopyOnThread(ThreadHandle thread, void *dst, const void *src, uint64_t len)
+{
+    return RecordData(thread, ItemKind::COPY, dst, src, len, len, HCCL_DATA_TYPE_INT8, 0);
+}
+
+int32_t HcommLocalReduceOnThread(ThreadHandle thread, void *dst, const void *src, uint64_t count,
+                                 HcommDataType dataType, HcommReduceOp reduceOp)
+{
+    if (ReduceArgsOk(dataType, reduceOp) != HCCL_SUCCESS) return HCCL_E_PARA;
+    return RecordData(thread, ItemKind::REDUCE, dst, src, count * DATATYPE_SIZE_TABLE[dataType], count, dataType,
+                      reduceOp);
+}
+
+int32_t HcommWriteOnThread(ThreadHandle thread, ChannelHandle channel, void *dst, const void *src, uint64_t len)
+{
+    if (AsChannel(channel) == nullptr) return HCCL_E_PTR;
+    return RecordData(thread, ItemKind::COPY, dst, src, len, len, HCCL_DATA_TYPE_INT8, 0);
+}
+
+int32_t HcommReadOnThread(ThreadHandle thread, ChannelHandle channel, void *dst, const void *src, uint64_t len)
+{
+    if (AsChannel(channel) == nullptr) return HCCL_E_PTR;
+    return RecordData(thread, ItemKind::COPY, dst, src, len, len, HCCL_DATA_TYPE_INT8, 0);
+}
+
+int32_t HcommWriteReduceOnThread(ThreadHandle thread, ChannelHandle channel, void *dst, const void *src,
+                                 uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp)
+{
+    if (AsChannel(channel) == nullptr) return HCCL_E_PTR;
+    if (ReduceArgsOk(dataType, reduceOp) != HCCL_SUCCESS) return HCCL_E_PARA;
+    return RecordData(thread, ItemKind::REDUCE, dst, src, count * DATATYPE_SIZE_TABLE[dataType], count, dataType,
+                      reduceOp);
+}
+
+int32_t HcommReadReduceOnThread(ThreadHandle thread, ChannelHandle channel, void *dst, const void *src,
+                                uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp)
+{
+    return HcommWriteReduceOnThread(thread, channel, dst, src, count, dataType, reduceOp);
+}
+
+int32_t HcommChannelNotifyRecordOnThread(ThreadHandle thread, ChannelHandle channel, uint32_t remoteNotifyIdx)
+{
+    VThread *t = AsThread(thread);
+    VChannel *c = AsChannel(channel);
+    if (t == nullptr || c == nullptr) return HCCL_E_PTR;
+    return RecordNotify(t, ItemKind::NOTIFY_RECORD, ChannelKey(c->localRank, c->remoteRank, remoteNotifyIdx));
+}
+
+int32_t HcommChannelNotifyWaitOnThread(ThreadHandle thread, ChannelHandle channel, uint32_t localNotifyIdx,
+                                       uint32_t timeout)
+{
+    (void)timeout;
+    VThread *t = AsThread(thread);
+    VChannel *c = AsChannel(channel);
+    if (t == nullptr || c == nullptr) return HCCL_E_PTR;
+    return RecordNotify(t, ItemKind::NOTIFY_WAIT, ChannelKey(c->remoteRank, c->localRank, localNotifyIdx));
+}
+
+int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThread, uint32_t dstNotifyIdx)
+{
+    VThread *t = AsThread(thread);
+    VThread *d = AsThread(dstThread);
+    if (t == nullptr || d == nullptr) return HCCL_E_PTR;
+    return RecordNotify(t, ItemKind::NOTIFY_RECORD, ThreadKey(d, dstNotifyIdx));
+}
+
+int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, uint32_t timeout)
+{
+    (void)timeout;
+    VThread *t = AsThread(thread);
+    if (t == nullptr) return HCCL_E_PTR;
+    return RecordNotify(t, ItemKind::NOTIFY_WAIT, ThreadKey(t, notifyIdx));
+}
+
+int32_t HcommBatchModeStart(const char *batchTag)
+{
+    (void)batchTag;
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommBatchModeEnd(const char *batchTag)
+{
+    (void)batchTag;
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommThreadJoin(ThreadHandle thread, uint32_t timeout)
+{
+    (void)thread;
+    (void)timeout;
+    return HCCL_SUCCESS;
+}
+
+}  // extern "C"

@@ -1,0 +1,134 @@
+// The virtual-rank world: N ranks of one communicator whose buffers all live in one GPU's HBM.
+//
+// It stands where the reference has HCOMM (communicator, threads, channels, transport).  A rank's
+// collective call is queued; when every rank of the world has a call at the head of its queue, the
+// calls are checked for consistency, each rank's executor + template is run with a recording backend,
+// and the recorded steps are launched on the GPU (schedule.h).
+#pragma once
+#include <condition_variable>
+#include <map>
+#include <deque>
+#include <memory>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include <hip/hip_runtime.h>
+
+#include "alg_param.h"
+
+struct hcclx_plan;
+
+namespace ops_hccl {
+
+enum class ItemKind : u8 { COPY, REDUCE, NOTIFY_RECORD, NOTIFY_WAIT };
+
+// One primitive call, as recorded on a thread.
+struct TaskItem {
+    ItemKind kind = ItemKind::COPY;
+    u8 dtype = 0;
+    u8 op = 0;
+    char *dst = nullptr;
+    const char *src = nullptr;
+    u64 bytes = 0;
+    u64 count = 0;
+    u64 key = 0;  // notify identity: who signals whom on which index
+    u32 seq = 0;  // n-th record / n-th wait on that identity: they pair up in order
+};
+
+struct World;
+
+struct VThread {
+    World *world = nullptr;
+    u32 rank = 0;
+    u32 index = 0;
+    std::vector<TaskItem> items;
+};
+
+struct VChannel {
+    World *world = nullptr;
+    u32 localRank = 0;
+    u32 remoteRank = 0;
+};
+
+enum class ExecMode {
+    FUSED = 0,  // trace the recorded schedule symbolically and launch one fused pass per output
+    STEP = 1,   // launch the recorded copy / reduce steps level by level, as the reference's engines would
+};
+
+struct RankComm {
+    World *world = nullptr;
+    u32 rank = 0;
+};
+
+struct QueuedOp {
+    OpParam param;
+    hipEvent_t ready = nullptr;  // recorded on the caller's stream when it differs from the launch stream
+};
+
+struct CachedPlan {
+    std::string key;
+    std::vector<hcclx_plan *> plans;
+    u64 lastUse = 0;
+};
+
+struct World {
+    u32 rankSize = 0;
+    int device = 0;
+    u64 cclBytes = HCCL_CCL_BUFFER_DEFAULT;
+    ExecMode mode = ExecMode::FUSED;
+    bool blocking = false;  // a rank's call returns only after the collective was launched
+    std::vector<std::unique_ptr<RankComm>> ranks;
+    std::vector<char *> cclBuf;  // per rank, allocated on first use
+    std::vector<std::vector<std::unique_ptr<VThread>>> threads;    // [rank][thread]
+    std::vector<std::vector<std::unique_ptr<VChannel>>> channels;  // [rank][peer]
+
+    std::mutex mu;
+    std::condition_variable cv;
+    std::vector<std::deque<QueuedOp>> queue;  // per rank
+    std::vector<u64> launched;                // per rank: collectives completed so far
+    std::vector<HcclResult> lastResult;
+
+    // recording state of the collective being expanded
+    std::unordered_map<u64, u32> recordSeq;
+    std::unordered_map<u64, u32> waitSeq;
+
+    // statistics of the last launched collective, for tests and the benchmark
+    std::string lastAlgName;
+    u32 lastLevels = 0;
+    u32 lastLaunches = 0;
+    u32 lastFusedSegments = 0;
+    bool lastWasFused = false;
+    bool lastPlanCacheHit = false;
+    std::string lastTrace;  // expression of every output piece, filled when traceText is set
+    bool traceText = false;
+
+    std::vector<CachedPlan> planCache;
+    u64 useCounter = 0;
+
+    // configuration
+    std::map<int, std::string> forcedAlg;  // per HcclCMDType; empty = selector decides
+    u32 topoLevels = 1;
+    Level0Shape topoShape = Level0Shape::MESH_1D;
+    u32 devicesPerServer = 0;
+    // A dry world has no GPU behind it: scratch buffers are address ranges that are never touched, and a
+    // collective stops after its schedule has been recorded, ordered and traced.  Used to check schedules
+    // on a machine without a GPU.
+    bool dryRun = false;
+
+    ~World();
+    HcclResult EnsureScratch();
+    void ResetRecording();
+};
+
+HcclResult WorldCreate(u32 rankSize, u64 cclBytes, bool dryRun, std::vector<HcclComm> &comms);
+HcclResult WorldDestroyRank(HcclComm comm);
+RankComm *AsRankComm(HcclComm comm);
+
+// Resources a template asks for: `threadNum` threads of this rank and one channel per peer.
+void FillResources(World *w, u32 rank, u32 threadNum, AlgResourceCtxSerializable &resCtx);
+
+// Queues one rank's call; launches the collective when all ranks have one queued.
+HcclResult SubmitOp(RankComm *rc, const OpParam &param);
+
+}  // namespace ops_hccl

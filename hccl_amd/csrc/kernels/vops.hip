@@ -23,20 +23,9 @@ namespace hcclx {
 
 namespace {
 
-constexpr int kCopyUnroll = 8;
-constexpr uint32_t kTileVecs = kThreads * kCopyUnroll;  // 16-byte vectors per tile
-constexpr uint32_t kTileBytes = kTileVecs * 16;         // 32 KiB
+constexpr uint32_t kTileBytes = kTileVecs * 16;  // 32 KiB
 
-// Tiles of a block of `bytes` bytes whose first destination byte sits at address `dst`.
-// Stores are aligned: the bytes before the first 16-byte boundary of dst (head) and after the last
-// whole vector (tail) are moved one byte per thread by the block's last tile.
-__device__ __forceinline__ uint64_t tiles_of(uint64_t bytes, uint64_t dst)
-{
-    if (bytes == 0) return 0;
-    uint64_t head = (16 - (dst & 15)) & 15;
-    if (head > bytes) head = bytes;
-    return (bytes - head) / 16 / kTileVecs + 1;
-}
+__device__ __forceinline__ uint64_t tiles_of(uint64_t bytes, uint64_t dst) { return v_tiles_of(bytes, dst); }
 
 __device__ __forceinline__ uint64_t wave_inclusive_scan(uint64_t v)
 {

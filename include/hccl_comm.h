@@ -1,0 +1,73 @@
+/*
+ * hccl_comm.h -- communicators of virtual ranks.
+ *
+ * In the reference the communicator API lives in HCOMM (<hccl/hccl_comm.h>, included at include/hccl.h:15)
+ * and one rank is one device.  Here all ranks of a communicator share one GPU; HcclCommInitAll keeps the
+ * HCOMM signature (ndev handles at once), the hcclx* functions are additions for what has no counterpart
+ * in the reference: the size of the per-rank scratch ("CCL") buffer, how the recorded schedule is run,
+ * which algorithm and topology the selector sees, and what the last collective did.
+ *
+ * Calling convention of the collectives: each rank's call is queued and returns; when the last rank has
+ * called, the collective is launched on that rank's stream (streams of the other ranks are joined with
+ * events).  With one host thread driving all ranks the calls behave like a group: use the outputs after
+ * the last rank's call.  With one host thread per rank set blocking mode, so that a call returns only
+ * after the launch and the caller's later work on its stream is ordered after the collective.
+ */
+#ifndef HCCL_AMD_HCCL_COMM_H_
+#define HCCL_AMD_HCCL_COMM_H_
+
+#include "hccl_types.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ndev communicator handles, rank i = comms[i], all on the current GPU.  devices may be NULL. */
+HcclResult HcclCommInitAll(uint32_t ndev, int32_t *devices, HcclComm *comms);
+HcclResult HcclCommDestroy(HcclComm comm);
+HcclResult HcclGetRankSize(HcclComm comm, uint32_t *rankSize);
+HcclResult HcclGetRankId(HcclComm comm, uint32_t *rank);
+
+/* The same with an explicit scratch-buffer size per rank (bytes, > 1 MiB + 8 KiB; the default is 200 MiB, or
+ * HCCL_BUFFSIZE megabytes).  dry != 0 creates a world without a GPU behind it: collectives record, order
+ * and trace their schedule and launch nothing. */
+HcclResult hcclxCommInitAll(uint32_t nranks, uint64_t cclBytes, int dry, HcclComm *comms);
+
+typedef enum { HCCLX_EXEC_FUSED = 0, HCCLX_EXEC_STEP = 1 } hcclxExecMode;
+/* FUSED (default): one pass per output, inputs read once, the template's fold order kept.
+ * STEP: every copy / reduce step of the template is launched, through the scratch buffers. */
+HcclResult hcclxCommSetExecMode(HcclComm comm, hcclxExecMode mode);
+HcclResult hcclxCommSetBlocking(HcclComm comm, int blocking);
+
+/* HcclCMDType values used by hcclxCommSetAlgorithm. */
+typedef enum {
+    HCCLX_CMD_ALLREDUCE = 2, HCCLX_CMD_ALLGATHER = 6, HCCLX_CMD_REDUCE_SCATTER = 7, HCCLX_CMD_ALLTOALLV = 8,
+    HCCLX_CMD_ALLTOALLVC = 9, HCCLX_CMD_ALLTOALL = 10, HCCLX_CMD_ALLGATHER_V = 16
+} hcclxCmdType;
+/* Forces the algorithm (executor name, e.g. "InsAllReduceRing") of an op type; NULL or "" = selector. */
+HcclResult hcclxCommSetAlgorithm(HcclComm comm, int cmdType, const char *algName);
+/* Topology the selectors see: levels (1 = one flat level), shape 0 = CLOS, 1 = 1-D mesh,
+ * devicesPerServer (0 = all ranks in one server; 1 = single-device servers, which selects the NHR family). */
+HcclResult hcclxCommSetTopo(HcclComm comm, uint32_t levels, int level0Shape, uint32_t devicesPerServer);
+
+typedef struct {
+    char algName[64];
+    uint32_t levels;        /* dependency levels of the recorded schedule */
+    uint32_t launches;      /* kernel launches made */
+    uint32_t fusedSegments; /* segments of the fused plan */
+    int fused;              /* 1 = ran as fused passes, 0 = step by step */
+    int planCacheHit;
+} hcclxLastOpInfo;
+HcclResult hcclxCommGetLastOpInfo(HcclComm comm, hcclxLastOpInfo *info);
+
+/* When tracing is on, every collective also produces the expression of each output piece as text, e.g.
+ * "rank 2 out[0,4096) = (x3@0+(x1@0+(x0@0+x2@0)))": "(a+b)" means dst = b, src = a; "xK@B" is byte B of
+ * rank K's send buffer.  hcclxCommGetLastTrace copies it (NUL-terminated, truncated to size) and returns
+ * the full length. */
+HcclResult hcclxCommSetTrace(HcclComm comm, int on);
+uint64_t hcclxCommGetLastTrace(HcclComm comm, char *buf, uint64_t size);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HCCL_AMD_HCCL_COMM_H_ */

@@ -1,0 +1,55 @@
+/*
+ * hcomm_primitives.h -- the data-plane primitive ABI the algorithm templates call.
+ *
+ * In the reference these symbols come from libhcomm.so, loaded with dlopen/dlsym
+ * (src/common/hcomm_dlsym/hcomm_dlsym.cc:62-82); their signatures are visible in the system-test stubs
+ * (test/st/algorithm/utils/src/hccl_proxy/hccl_stub.cc, line given per function).  Here they are the
+ * entry of the virtual-rank backend: every call is recorded on its thread; when all ranks of the
+ * communicator have issued their collective, the recorded steps are ordered by their notify
+ * dependencies and launched as HIP kernels over buffers that all live in one GPU's HBM.
+ * Return value: 0 = success, otherwise an HcclResult.
+ */
+#ifndef HCCL_AMD_HCOMM_PRIMITIVES_H_
+#define HCCL_AMD_HCOMM_PRIMITIVES_H_
+
+#include <stdint.h>
+#include "hccl_types.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint64_t ThreadHandle;   /* sim_common.h:40 */
+typedef uint64_t ChannelHandle;  /* sim_common.h:41 */
+typedef HcclDataType HcommDataType;
+typedef HcclReduceOp HcommReduceOp;
+
+/* dst[0..len) = src[0..len), both local to the calling rank.            hccl_stub.cc:467 */
+int32_t HcommLocalCopyOnThread(ThreadHandle thread, void *dst, const void *src, uint64_t len);
+/* dst[i] = src[i] (+) dst[i] for count elements.                        hccl_stub.cc:633 */
+int32_t HcommLocalReduceOnThread(ThreadHandle thread, void *dst, const void *src, uint64_t count,
+                                 HcommDataType dataType, HcommReduceOp reduceOp);
+/* Write local src into the peer's dst / read the peer's src into local dst.   hccl_stub.cc:495, :534 */
+int32_t HcommWriteOnThread(ThreadHandle thread, ChannelHandle channel, void *dst, const void *src, uint64_t len);
+int32_t HcommReadOnThread(ThreadHandle thread, ChannelHandle channel, void *dst, const void *src, uint64_t len);
+/* The same with dst = src (+) dst at the destination.                   hccl_stub.cc:664, :705 */
+int32_t HcommWriteReduceOnThread(ThreadHandle thread, ChannelHandle channel, void *dst, const void *src,
+                                 uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp);
+int32_t HcommReadReduceOnThread(ThreadHandle thread, ChannelHandle channel, void *dst, const void *src,
+                                uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp);
+/* Inter-rank handshake over a channel.                                  hccl_stub.cc:573, :601 */
+int32_t HcommChannelNotifyRecordOnThread(ThreadHandle thread, ChannelHandle channel, uint32_t remoteNotifyIdx);
+int32_t HcommChannelNotifyWaitOnThread(ThreadHandle thread, ChannelHandle channel, uint32_t localNotifyIdx,
+                                       uint32_t timeout);
+/* Main thread <-> sub thread fan-out / fan-in inside one rank.          hccl_stub.cc:449, :397 */
+int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThread, uint32_t dstNotifyIdx);
+int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, uint32_t timeout);
+/* Flush / join before CPU-side work.  Stream order already gives that here.   hccl_stub.cc:799, :805, :937 */
+int32_t HcommBatchModeStart(const char *batchTag);
+int32_t HcommBatchModeEnd(const char *batchTag);
+int32_t HcommThreadJoin(ThreadHandle thread, uint32_t timeout);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HCCL_AMD_HCOMM_PRIMITIVES_H_ */

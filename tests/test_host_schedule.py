@@ -1,0 +1,224 @@
+"""The host runtime without a GPU: op entry -> selector -> executor -> template -> recorded steps ->
+dependency order -> symbolic trace.  The trace of every output is evaluated with the oracle's element
+arithmetic and compared, bit for bit, with the oracle's own restatement of the same template."""
+import numpy as np
+import pytest
+
+from oracle import templates as T
+from hccl_amd import api
+
+from host_util import (FAKE_STREAM, eval_trace, expr_to_oracle_string, fake_ptrs, parse_expr, parse_trace)
+
+SMALL_CCL = 1024 * 1024 + 64 * 1024     # forces several executor chunks at a few thousand elements
+AR_ALGS = list(T.ALLREDUCE_TEMPLATES)
+RS_ALGS = list(T.REDUCE_SCATTER_TEMPLATES)
+
+
+def sym_inputs(n, count):
+    out = []
+    for r in range(n):
+        a = np.empty(count, dtype=object)
+        a[:] = [f"x{r}[{i}]" for i in range(count)]
+        out.append(a)
+    return out
+
+
+def dry_allreduce(n, count, dtype, op, alg, ccl=SMALL_CCL):
+    w = api.World(n, ccl_bytes=ccl, dry=True)
+    try:
+        w.set_algorithm(api.CMD_ALLREDUCE, alg)
+        ins, outs = fake_ptrs(n)
+        for r in range(n):
+            assert w.all_reduce(r, ins[r], outs[r], count, dtype, op, FAKE_STREAM) == 0
+        return w.last_trace(), w.last_info()
+    finally:
+        w.close()
+
+
+def dry_reduce_scatter(n, recv_count, dtype, op, alg, ccl=SMALL_CCL):
+    w = api.World(n, ccl_bytes=ccl, dry=True)
+    try:
+        w.set_algorithm(api.CMD_REDUCE_SCATTER, alg)
+        ins, outs = fake_ptrs(n)
+        for r in range(n):
+            assert w.reduce_scatter(r, ins[r], outs[r], recv_count, dtype, op, FAKE_STREAM) == 0
+        return w.last_trace(), w.last_info()
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("alg", AR_ALGS)
+@pytest.mark.parametrize("n", [2, 3, 4, 5, 8, 12, 13])
+def test_allreduce_association_order_equals_oracle(alg, n):
+    for count in (1, n - 1, n, 2 * n + 3):
+        text, _ = dry_allreduce(n, count, T.FP32, T.SUM, alg)
+        want = T.run_allreduce(T.SymbolicElems(), sym_inputs(n, count), count, 4, alg)
+        seen = [set() for _ in range(n)]
+        for rank, off, nbytes, expr in parse_trace(text):
+            tree = parse_expr(expr)
+            for e in range(nbytes // 4):
+                idx = off // 4 + e
+                assert expr_to_oracle_string(tree, e, 4, off) == want[rank][idx], (alg, n, count, rank, idx)
+                seen[rank].add(idx)
+        assert all(s == set(range(count)) for s in seen)      # every output element is produced
+
+
+@pytest.mark.parametrize("alg", RS_ALGS)
+@pytest.mark.parametrize("n", [2, 3, 5, 8, 12])
+def test_reduce_scatter_association_order_equals_oracle(alg, n):
+    rc = 7
+    text, _ = dry_reduce_scatter(n, rc, T.BFP16, T.SUM, alg)
+    want = T.run_reduce_scatter(T.SymbolicElems(), sym_inputs(n, n * rc), rc, 2, alg)
+    seen = [set() for _ in range(n)]
+    for rank, off, nbytes, expr in parse_trace(text):
+        tree = parse_expr(expr)
+        for e in range(nbytes // 2):
+            assert expr_to_oracle_string(tree, e, 2, off) == want[rank][off // 2 + e]
+            seen[rank].add(off // 2 + e)
+    assert all(s == set(range(rc)) for s in seen)
+
+
+@pytest.mark.parametrize("alg", AR_ALGS)
+@pytest.mark.parametrize("dtype,op,n,count", [(T.FP32, T.SUM, 8, 70001), (T.FP32, T.PROD, 12, 30011),
+                                             (T.FP64, T.SUM, 5, 40000), (T.INT32, T.MAX, 12, 50000),
+                                             (T.FP16, T.PROD, 3, 190001)])
+def test_allreduce_values_with_executor_chunks(alg, dtype, op, n, count):
+    """Several chunks of the small scratch buffer: slice boundaries move with the chunk, and so does the
+    association tree an element sees."""
+    rng = np.random.default_rng(n * 1000 + count)
+    npd = T.NP_STORAGE[dtype]
+    if dtype == T.INT32:
+        xs = [rng.integers(-2**31, 2**31 - 1, size=count, dtype=np.int32) for _ in range(n)]
+    elif dtype == T.FP16:
+        xs = [T.narrow16((0.9 + 0.2 * rng.random(count)).astype(np.float32), T.FP16) for _ in range(n)]
+    else:
+        lo, hi = (0.9, 1.1) if op == T.PROD else (-1.0, 1.0)
+        xs = [(lo + (hi - lo) * rng.random(count)).astype(npd) for _ in range(n)]
+    esz = T.DTYPE_SIZE[dtype]
+    text, _ = dry_allreduce(n, count, dtype, op, alg)
+    got = eval_trace(text, xs, count, dtype, op, 0)
+    want = T.run_allreduce(T.NumericElems(dtype, op), xs, count, esz, alg, ccl_bytes=SMALL_CCL)
+    mult = T.ALLREDUCE_TEMPLATES[alg][1](n)
+    if mult >= n:      # the slot-per-rank templates run several chunks at these sizes
+        assert len(T.chunk_counts(count, SMALL_CCL, mult, esz, SMALL_CCL)) >= 2
+    for r in range(n):
+        assert np.array_equal(got[r].view(np.uint8), want[r].view(np.uint8)), (alg, r)
+
+
+@pytest.mark.parametrize("alg", RS_ALGS)
+def test_reduce_scatter_values_with_executor_chunks(alg):
+    rng = np.random.default_rng(5)
+    n, rc = 8, 9000          # (64 KiB usable scratch) / 8 slots = 8 KiB = 2048 fp32 per chunk
+    xs = [(rng.random(n * rc) * 2 - 1).astype(np.float32) for _ in range(n)]
+    text, _ = dry_reduce_scatter(n, rc, T.FP32, T.SUM, alg)
+    got = eval_trace(text, xs, rc, T.FP32, T.SUM, 0)
+    want = T.run_reduce_scatter(T.NumericElems(T.FP32, T.SUM), xs, rc, 4, alg, ccl_bytes=SMALL_CCL)
+    assert len(T.chunk_counts(rc, SMALL_CCL - (1 << 20), n, 4, SMALL_CCL - (1 << 20))) == 5
+    for r in range(n):
+        assert np.array_equal(got[r].view(np.uint32), want[r].view(np.uint32))
+
+
+def test_which_templates_fuse():
+    """Chains (and every integer schedule) become fused passes; floating-point trees do not."""
+    for alg, dtype, fused in [("InsAllReduceMesh1DOneShot", T.FP32, 1), ("InsAllReduceMesh1DTwoShot", T.FP32, 1),
+                              ("InsAllReduceAicpuReduceNHR", T.FP32, 1), ("InsAllReduceRing", T.FP32, 1),
+                              ("InsAllReduceNHR", T.FP32, 0), ("InsAllReduceRHD", T.FP32, 0),
+                              ("InsAllReduceNHR", T.INT32, 1), ("InsAllReduceRHD", T.INT32, 1)]:
+        _, info = dry_allreduce(12, 1200, dtype, T.SUM, alg)
+        assert info.fused == fused, alg
+        assert info.algName.decode() == alg
+    # the one-shot order of all 12 ranks is one segment: 12 sources read once, 12 outputs
+    _, info = dry_allreduce(12, 1200, T.FP32, T.SUM, "InsAllReduceMesh1DOneShot")
+    assert info.fusedSegments == 1
+    # float max keeps operand order: the ring's "acc (+) leaf" steps are not swapped into a chain
+    _, info = dry_allreduce(4, 64, T.FP32, T.MAX, "InsAllReduceRing")
+    assert info.fused == 0
+
+
+def test_selector_choices_follow_the_reference_thresholds():
+    def pick(n, count, dtype, op, topo=None, cmd="ar"):
+        w = api.World(n, ccl_bytes=SMALL_CCL, dry=True)
+        try:
+            if topo:
+                w.set_topo(*topo)
+            ins, outs = fake_ptrs(n)
+            for r in range(n):
+                if cmd == "ar":
+                    assert w.all_reduce(r, ins[r], outs[r], count, dtype, op, FAKE_STREAM) == 0
+                elif cmd == "rs":
+                    assert w.reduce_scatter(r, ins[r], outs[r], count, dtype, op, FAKE_STREAM) == 0
+                else:
+                    assert w.all_gather(r, ins[r], outs[r], count, dtype, FAKE_STREAM) == 0
+            return w.last_info().algName.decode()
+        finally:
+            w.close()
+
+    mib = 1 << 20
+    assert pick(8, 8 * mib // 4, T.FP32, T.SUM) == "InsAllReduceMesh1DOneShot"          # <= 8 MiB
+    assert pick(8, 8 * mib // 4 + 1, T.FP32, T.SUM) == "InsAllReduceMesh1DTwoShot"
+    assert pick(8, 1024, T.FP32, T.PROD) == "InsAllReduceMesh1DOneShot"
+    assert pick(8, 8 * mib // 8 + 1, T.FP64, T.SUM) == "InsAllReduceMesh1DTwoShot"
+    # 12 single-device servers: the log-step family; PROD / 64-bit types reduce after an NHR gather
+    assert pick(12, 4096, T.INT32, T.MAX, topo=(2, api.SHAPE_MESH_1D, 1)) == "InsAllReduceNHR"
+    assert pick(12, 4096, T.FP32, T.PROD, topo=(2, api.SHAPE_MESH_1D, 1)) == "InsAllReduceAicpuReduceNHR"
+    assert pick(12, 4096, T.FP32, T.SUM, topo=(1, api.SHAPE_CLOS, 0)) == "InsAllReduceNHR"
+    assert pick(8, 4096, T.BFP16, T.SUM, cmd="rs") == "InsReduceScatterMesh1D"
+    assert pick(8, 4096, T.BFP16, T.SUM, topo=(2, api.SHAPE_MESH_1D, 1), cmd="rs") == "InsReduceScatterNHR"
+    assert pick(8, 4096, T.FP16, None, cmd="ag") == "InsAllGatherMesh1D"
+    assert pick(8, 4096, T.FP16, None, topo=(1, api.SHAPE_CLOS, 0), cmd="ag") == "InsAllGatherNHR"
+
+
+def test_parameter_checks_and_early_returns():
+    w = api.World(4, ccl_bytes=SMALL_CCL, dry=True)
+    ins, outs = fake_ptrs(4)
+    try:
+        assert w.all_reduce(0, ins[0], outs[0], 0, T.FP32, T.SUM, FAKE_STREAM) == 0          # count 0: success, nothing queued
+        assert w.all_reduce(0, ins[0], outs[0], 8, T.FP32, T.SUM, None) == 2                 # null stream: HCCL_E_PTR
+        assert w.all_reduce(0, None, outs[0], 8, T.FP32, T.SUM, FAKE_STREAM) == 2
+        assert w.all_reduce(0, ins[0], outs[0], 0x800000000, T.FP32, T.SUM, FAKE_STREAM) == 1   # > SYS_MAX_COUNT
+        assert w.all_reduce(0, ins[0], outs[0], 8, T.UINT8, T.SUM, FAKE_STREAM) == 5         # not a reduce type
+        assert w.all_reduce(0, ins[0], outs[0], 8, T.BFP16, T.PROD, FAKE_STREAM) == 5        # PROD excludes bf16
+        assert w.all_reduce(0, ins[0], outs[0], 8, T.INT16, T.PROD, FAKE_STREAM) == 5
+        assert w.reduce_scatter(0, ins[0], outs[0], 8, T.UINT32, T.SUM, FAKE_STREAM) == 5
+        assert w.all_gather(0, ins[0], outs[0], 8, 12, FAKE_STREAM) == 5                     # int128
+        assert w.all_to_all_v(0, ins[0], [1] * 4, [0] * 4, ins[0], [1] * 4, [0] * 4, T.INT8, FAKE_STREAM) == 1  # in place
+        assert w.all_to_all_v(0, None, [1] * 4, [0] * 4, outs[0], [1] * 4, [0] * 4, T.INT8, FAKE_STREAM) == 2
+        assert w.all_gather_v(0, ins[0], 3, outs[0], [0] * 4, [0] * 4, T.FP16, FAKE_STREAM) == 0   # all counts 0
+        assert w.all_gather_v(0, ins[0], 3, None, [3, 1, 1, 1], [0, 3, 4, 5], T.FP16, FAKE_STREAM) == 2
+    finally:
+        w.close()
+
+
+def test_ranks_that_disagree_are_rejected():
+    w = api.World(2, ccl_bytes=SMALL_CCL, dry=True)
+    ins, outs = fake_ptrs(2)
+    try:
+        assert w.all_reduce(0, ins[0], outs[0], 8, T.FP32, T.SUM, FAKE_STREAM) == 0
+        assert w.all_reduce(1, ins[1], outs[1], 9, T.FP32, T.SUM, FAKE_STREAM) == 1   # HCCL_E_PARA
+    finally:
+        w.close()
+
+
+def test_single_rank_world_is_a_local_copy():
+    w = api.World(1, ccl_bytes=SMALL_CCL, dry=True)
+    ins, outs = fake_ptrs(1)
+    try:
+        assert w.all_reduce(0, ins[0], outs[0], 8, T.FP32, T.SUM, FAKE_STREAM) == 0
+        assert w.all_reduce(0, ins[0], ins[0], 8, T.FP32, T.SUM, FAKE_STREAM) == 0    # in place: nothing to do
+    finally:
+        w.close()
+
+
+def test_calls_queue_per_rank_and_pair_up_in_order():
+    """Rank 0 may run ahead: its second call waits in its queue until rank 1 has made both calls."""
+    w = api.World(2, ccl_bytes=SMALL_CCL, dry=True)
+    ins, outs = fake_ptrs(2)
+    try:
+        assert w.all_reduce(0, ins[0], outs[0], 8, T.FP32, T.SUM, FAKE_STREAM) == 0
+        assert w.all_reduce(0, ins[0], outs[0], 16, T.INT32, T.MAX, FAKE_STREAM) == 0
+        assert w.all_reduce(1, ins[1], outs[1], 8, T.FP32, T.SUM, FAKE_STREAM) == 0
+        assert "out[0,32)" in w.last_trace()
+        assert w.all_reduce(1, ins[1], outs[1], 16, T.INT32, T.MAX, FAKE_STREAM) == 0
+        assert "out[0,64)" in w.last_trace()
+    finally:
+        w.close()
