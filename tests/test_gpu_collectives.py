@@ -1,0 +1,303 @@
+"""GPU parity of the collectives through the HCCL entry points (HcclAllReduce ... HcclAlltoAllVC) for
+virtual ranks, in both execution modes, against the CPU oracle's restatement of the same template."""
+import threading
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import templates as T
+from hccl_amd import api
+
+from gpu_util import DevBuf, assert_same_bits, payload
+
+pytestmark = pytest.mark.gpu
+
+SMALL_CCL = 1024 * 1024 + 64 * 1024
+AR_ALGS = list(T.ALLREDUCE_TEMPLATES)
+MODES = [api.EXEC_FUSED, api.EXEC_STEP]
+
+
+@pytest.fixture(scope="module")
+def stream():
+    s = torch.cuda.Stream()
+    yield s
+    s.synchronize()
+
+
+def wide_oracle_allreduce(xs, count, dtype, alg, ccl):
+    """16-bit float SUM as a fused pass computes it: the template's order in fp32, one narrowing."""
+    wide = [T.widen16(x, dtype) for x in xs]
+    outs = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), wide, count, T.DTYPE_SIZE[dtype], alg, ccl_bytes=ccl)
+    return [T.narrow16(o, dtype) for o in outs]
+
+
+def run_allreduce(world, stream, xs, count, dtype, op, in_place=False):
+    n = len(xs)
+    send = [DevBuf(x) for x in xs]
+    recv = send if in_place else [DevBuf(nbytes=xs[0].nbytes) for _ in range(n)]
+    torch.cuda.synchronize()
+    for r in range(n):
+        assert world.all_reduce(r, send[r].ptr, recv[r].ptr, count, dtype, op, stream.cuda_stream) == 0
+    stream.synchronize()
+    return [b.get(T.NP_STORAGE[dtype]) for b in recv], recv
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("alg", AR_ALGS)
+@pytest.mark.parametrize("dtype,op,n,count", [(T.FP32, T.SUM, 8, 131072 + 5), (T.FP32, T.PROD, 12, 40000),
+                                             (T.INT32, T.MAX, 12, 70001), (T.BFP16, T.SUM, 8, 100003),
+                                             (T.FP16, T.PROD, 5, 50001), (T.FP64, T.MIN, 3, 30000),
+                                             (T.INT8, T.SUM, 16, 200001)])
+def test_allreduce_every_template_both_modes(stream, mode, alg, dtype, op, n, count):
+    rng = np.random.default_rng(n * 7 + count)
+    kind = "prod" if op == T.PROD else "uniform" if dtype == T.FP32 else "normal"
+    xs = [payload(rng, dtype, count, kind) for _ in range(n)]
+    w = api.World(n, ccl_bytes=SMALL_CCL)
+    try:
+        w.set_mode(mode)
+        w.set_algorithm(api.CMD_ALLREDUCE, alg)
+        got, bufs = run_allreduce(w, stream, xs, count, dtype, op)
+        info = w.last_info()
+        if info.fused and dtype in (T.FP16, T.BFP16) and op == T.SUM:
+            want = wide_oracle_allreduce(xs, count, dtype, alg, SMALL_CCL)
+        else:
+            want = T.run_allreduce(T.NumericElems(dtype, op), xs, count, T.DTYPE_SIZE[dtype], alg, ccl_bytes=SMALL_CCL)
+        for r in range(n):
+            assert_same_bits(got[r], want[r], dtype, f"{alg} rank {r} fused={info.fused}")
+            assert bufs[r].guard_intact()
+        if mode == api.EXEC_STEP:
+            assert info.fused == 0 and info.launches >= info.levels
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_allreduce_in_place(stream, mode):
+    rng = np.random.default_rng(3)
+    n, count = 8, 65536 + 1
+    xs = [payload(rng, T.FP32, count, "uniform") for _ in range(n)]
+    w = api.World(n, ccl_bytes=4 << 20)
+    try:
+        w.set_mode(mode)
+        got, _ = run_allreduce(w, stream, xs, count, T.FP32, T.SUM, in_place=True)
+        alg = w.last_info().algName.decode()
+        assert alg == "InsAllReduceMesh1DOneShot"
+        want = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs, count, 4, alg, ccl_bytes=4 << 20)
+        for r in range(n):
+            assert_same_bits(got[r], want[r], T.FP32, f"rank {r}")
+    finally:
+        w.close()
+
+
+def test_allreduce_default_selector_and_plan_cache(stream):
+    """Config 1 of the baseline: AllReduce SUM fp32, 8 ranks x 1,048,576 elements, uniform[-1,1): the
+    selector takes the one-shot mesh template at this size; the ring template is forced next."""
+    rng = np.random.default_rng(11)
+    n, count = 8, 1048576
+    xs = [payload(rng, T.FP32, count, "uniform") for _ in range(n)]
+    w = api.World(n)
+    try:
+        send = [DevBuf(x) for x in xs]
+        recv = [DevBuf(nbytes=count * 4) for _ in range(n)]
+        torch.cuda.synchronize()
+        for rep in range(2):
+            for r in range(n):
+                assert w.all_reduce(r, send[r].ptr, recv[r].ptr, count, T.FP32, T.SUM, stream.cuda_stream) == 0
+            stream.synchronize()
+            info = w.last_info()
+            assert info.algName.decode() == "InsAllReduceMesh1DOneShot" and info.fused == 1
+            assert info.planCacheHit == rep and info.launches == 1
+        want = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs, count, 4, "InsAllReduceMesh1DOneShot")
+        for r in range(n):
+            assert_same_bits(recv[r].get(np.float32), want[r], T.FP32, f"one-shot rank {r}")
+        w.set_algorithm(api.CMD_ALLREDUCE, "InsAllReduceRing")
+        for r in range(n):
+            assert w.all_reduce(r, send[r].ptr, recv[r].ptr, count, T.FP32, T.SUM, stream.cuda_stream) == 0
+        stream.synchronize()
+        assert w.last_info().fused == 1 and w.last_info().planCacheHit == 0
+        want = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs, count, 4, "InsAllReduceRing")
+        for r in range(n):
+            assert_same_bits(recv[r].get(np.float32), want[r], T.FP32, f"ring rank {r}")
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("alg", list(T.REDUCE_SCATTER_TEMPLATES))
+@pytest.mark.parametrize("dtype,op,n,rc", [(T.BFP16, T.SUM, 8, 65536 + 3), (T.FP32, T.SUM, 5, 30001),
+                                          (T.INT64, T.MAX, 12, 10007), (T.FP16, T.SUM, 3, 50000)])
+def test_reduce_scatter_both_templates_both_modes(stream, mode, alg, dtype, op, n, rc):
+    rng = np.random.default_rng(rc)
+    xs = [payload(rng, dtype, n * rc, "normal") for _ in range(n)]
+    w = api.World(n, ccl_bytes=SMALL_CCL)
+    try:
+        w.set_mode(mode)
+        w.set_algorithm(api.CMD_REDUCE_SCATTER, alg)
+        send = [DevBuf(x) for x in xs]
+        recv = [DevBuf(nbytes=rc * T.DTYPE_SIZE[dtype]) for _ in range(n)]
+        torch.cuda.synchronize()
+        for r in range(n):
+            assert w.reduce_scatter(r, send[r].ptr, recv[r].ptr, rc, dtype, op, stream.cuda_stream) == 0
+        stream.synchronize()
+        info = w.last_info()
+        esz = T.DTYPE_SIZE[dtype]
+        if info.fused and dtype in (T.FP16, T.BFP16) and op == T.SUM:
+            wide = [T.widen16(x, dtype) for x in xs]
+            want = [T.narrow16(o, dtype) for o in
+                    T.run_reduce_scatter(T.NumericElems(T.FP32, T.SUM), wide, rc, esz, alg, ccl_bytes=SMALL_CCL)]
+        else:
+            want = T.run_reduce_scatter(T.NumericElems(dtype, op), xs, rc, esz, alg, ccl_bytes=SMALL_CCL)
+        for r in range(n):
+            assert_same_bits(recv[r].get(T.NP_STORAGE[dtype]), want[r], dtype, f"{alg} rank {r} fused={info.fused}")
+            assert recv[r].guard_intact()
+    finally:
+        w.close()
+
+
+def test_reduce_scatter_bf16_within_one_ulp_of_fp32_accumulation(stream):
+    """The tolerance the baseline states for 16-bit floats: every output within 1 bf16 ULP of the sum
+    accumulated in fp32 (here: in float64, then compared on the bf16 grid)."""
+    rng = np.random.default_rng(2)
+    n, rc = 8, 1 << 16
+    xs = [payload(rng, T.BFP16, n * rc, "normal") for _ in range(n)]
+    w = api.World(n)
+    try:
+        send = [DevBuf(x) for x in xs]
+        recv = [DevBuf(nbytes=rc * 2) for _ in range(n)]
+        torch.cuda.synchronize()
+        for r in range(n):
+            assert w.reduce_scatter(r, send[r].ptr, recv[r].ptr, rc, T.BFP16, T.SUM, stream.cuda_stream) == 0
+        stream.synchronize()
+        assert w.last_info().algName.decode() == "InsReduceScatterMesh1D"
+        exact = np.sum([T.widen16(x, T.BFP16).astype(np.float64) for x in xs], axis=0)
+        for r in range(n):
+            got = T.widen16(recv[r].get(np.uint16), T.BFP16).astype(np.float64)
+            ref = exact[r * rc:(r + 1) * rc]
+            ulp = np.maximum(np.abs(ref), 2.0 ** -126) * 2.0 ** -7      # spacing of bf16 at that magnitude
+            assert np.all(np.abs(got - ref) <= ulp), f"rank {r}"         # tolerance: 1 bf16 ULP
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("alg", ["InsAllGatherMesh1D", "InsAllGatherNHR"])
+def test_allgather(stream, mode, alg):
+    rng = np.random.default_rng(4)
+    for n, count in ((2, 5), (8, 70001), (12, 4097)):
+        xs = [rng.integers(0, 65535, size=count, dtype=np.uint16) for _ in range(n)]
+        w = api.World(n, ccl_bytes=SMALL_CCL)
+        try:
+            w.set_mode(mode)
+            w.set_algorithm(api.CMD_ALLGATHER, alg)
+            send = [DevBuf(x) for x in xs]
+            recv = [DevBuf(nbytes=n * count * 2) for _ in range(n)]
+            torch.cuda.synchronize()
+            for r in range(n):
+                assert w.all_gather(r, send[r].ptr, recv[r].ptr, count, T.FP16, stream.cuda_stream) == 0
+            stream.synchronize()
+            for r in range(n):
+                assert np.array_equal(recv[r].get(np.uint16), np.concatenate(xs)) and recv[r].guard_intact()
+        finally:
+            w.close()
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_allgatherv_ragged(stream, mode):
+    rng = np.random.default_rng(9)
+    for counts in ([3, 0, 70001, 1, 4096, 0, 33, 12345], [0, 0, 9], list(rng.integers(0, 30000, 16))):
+        counts = [int(c) for c in counts]
+        n = len(counts)
+        displs = [sum(counts[:i]) for i in range(n)]
+        total = sum(counts)
+        xs = [rng.integers(0, 65535, size=c, dtype=np.uint16) for c in counts]
+        w = api.World(n, ccl_bytes=SMALL_CCL)
+        try:
+            w.set_mode(mode)
+            send = [DevBuf(x) for x in xs]
+            recv = [DevBuf(nbytes=total * 2) for _ in range(n)]
+            torch.cuda.synchronize()
+            for r in range(n):
+                sp = send[r].ptr if counts[r] else None
+                assert w.all_gather_v(r, sp, counts[r], recv[r].ptr, counts, displs, T.FP16, stream.cuda_stream) == 0
+            stream.synchronize()
+            for r in range(n):
+                assert np.array_equal(recv[r].get(np.uint16), np.concatenate(xs)) and recv[r].guard_intact()
+        finally:
+            w.close()
+
+
+def a2a_run(w, stream, m, dtype, npd, rng, kind="v"):
+    n = len(m)
+    v = [T.alltoallvc_to_v(m, r) for r in range(n)]
+    xs = [rng.integers(0, np.iinfo(npd).max, size=sum(m[i]), dtype=npd, endpoint=True) for i in range(n)]
+    send = [DevBuf(x) for x in xs]
+    recv = [DevBuf(nbytes=sum(x[2]) * np.dtype(npd).itemsize) for x in v]
+    torch.cuda.synchronize()
+    for r in range(n):
+        sc, sd, rc, rd = v[r]
+        sp = send[r].ptr if sum(sc) else None
+        rp = recv[r].ptr if sum(rc) else None
+        if kind == "v":
+            assert w.all_to_all_v(r, sp, sc, sd, rp, rc, rd, dtype, stream.cuda_stream) == 0
+        elif kind == "vc":
+            assert w.all_to_all_vc(r, sp, [x for row in m for x in row], rp, dtype, stream.cuda_stream) == 0
+        else:
+            assert w.all_to_all(r, sp, m[0][0], rp, dtype, stream.cuda_stream) == 0
+    stream.synchronize()
+    want = T.run_alltoallv(xs, [x[0] for x in v], [x[1] for x in v], [x[2] for x in v], [x[3] for x in v],
+                           [sum(x[2]) for x in v])
+    for r in range(n):
+        assert np.array_equal(recv[r].get(npd), want[r]), f"rank {r}"
+        assert recv[r].guard_intact()
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_alltoall_family(stream, mode):
+    rng = np.random.default_rng(21)
+    for n in (2, 5, 8, 18):
+        m = rng.integers(0, 3000, size=(n, n)).tolist()
+        m[0][1] = 0
+        if n == 8:
+            m[2][6] = 120000          # larger than one scratch slot: the executor loops
+        w = api.World(n, ccl_bytes=SMALL_CCL)
+        try:
+            w.set_mode(mode)
+            a2a_run(w, stream, m, T.BFP16, np.uint16, rng, "v")
+            a2a_run(w, stream, m, T.INT8, np.uint8, rng, "vc")
+            a2a_run(w, stream, [[777] * n for _ in range(n)], T.FP32, np.uint32, rng, "uniform")
+        finally:
+            w.close()
+
+
+def test_ranks_on_different_streams_and_threads():
+    """One host thread and one stream per rank, blocking rendezvous: the reference's calling pattern."""
+    n, count = 4, 50000
+    rng = np.random.default_rng(8)
+    xs = [payload(rng, T.FP32, count, "uniform") for _ in range(n)]
+    w = api.World(n, ccl_bytes=4 << 20)
+    try:
+        w.set_blocking(True)
+        send = [DevBuf(x) for x in xs]
+        recv = [DevBuf(nbytes=count * 4) for _ in range(n)]
+        streams = [torch.cuda.Stream() for _ in range(n)]
+        torch.cuda.synchronize()
+        rcs = [None] * n
+
+        def body(r):
+            for _ in range(3):
+                rcs[r] = w.all_reduce(r, send[r].ptr, recv[r].ptr, count, T.FP32, T.SUM, streams[r].cuda_stream)
+            streams[r].synchronize()
+
+        ts = [threading.Thread(target=body, args=(r,)) for r in range(n)]
+        for t in ts:
+            t.start()
+        for t in ts:
+            t.join(timeout=60)
+        assert all(not t.is_alive() for t in ts) and rcs == [0] * n
+        torch.cuda.synchronize()
+        want = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs, count, 4, "InsAllReduceMesh1DOneShot")
+        for r in range(n):
+            assert_same_bits(recv[r].get(np.float32), want[r], T.FP32, f"rank {r}")
+    finally:
+        w.close()

@@ -222,3 +222,127 @@ def test_calls_queue_per_rank_and_pair_up_in_order():
         assert "out[0,64)" in w.last_trace()
     finally:
         w.close()
+
+
+# ---- data movement: the traced schedule must be the API contract ---------------------------------
+
+def copy_trace_outputs(text, inputs, out_lens, esz):
+    fill = 0xA5A5 & int(np.iinfo(inputs[0].dtype).max)
+    outs = [np.full(l, fill, dtype=inputs[0].dtype) for l in out_lens]
+    for rank, off, nbytes, expr in parse_trace(text):
+        tree = parse_expr(expr)
+        assert tree[0] == "x", "a data-movement collective must not reduce"
+        _, k, b = tree
+        outs[rank][off // esz:(off + nbytes) // esz] = inputs[k][b // esz:(b + nbytes) // esz]
+    return outs
+
+
+@pytest.mark.parametrize("alg", ["InsAllGatherMesh1D", "InsAllGatherNHR"])
+@pytest.mark.parametrize("n,count", [(2, 5), (3, 1000), (8, 33), (12, 70000), (16, 9)])
+def test_allgather_templates_deliver_the_concatenation(alg, n, count):
+    w = api.World(n, ccl_bytes=SMALL_CCL, dry=True)
+    try:
+        w.set_algorithm(api.CMD_ALLGATHER, alg)
+        ins, outs = fake_ptrs(n)
+        for r in range(n):
+            assert w.all_gather(r, ins[r], outs[r], count, T.FP16, FAKE_STREAM) == 0
+        rng = np.random.default_rng(n)
+        xs = [rng.integers(0, 65535, size=count, dtype=np.uint16) for _ in range(n)]
+        got = copy_trace_outputs(w.last_trace(), xs, [n * count] * n, 2)
+        for r in range(n):
+            assert np.array_equal(got[r], np.concatenate(xs))
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("counts", [[3, 0, 7, 1], [100, 100, 100, 100], [0, 0, 5], [70000, 1, 0, 33000, 12, 9, 400, 8],
+                                    [700, 700, 600, 600, 500, 500, 400, 400, 300, 300, 200, 200, 100, 100]])
+def test_allgatherv_template_with_ragged_counts_and_chunks(counts):
+    n = len(counts)
+    displs, off = [], 2
+    for c in counts:
+        displs.append(off)
+        off += c + 1                      # one element of slack between blocks: it must stay untouched
+    w = api.World(n, ccl_bytes=SMALL_CCL, dry=True)
+    try:
+        ins, outs = fake_ptrs(n)
+        for r in range(n):
+            assert w.all_gather_v(r, ins[r], counts[r], outs[r], counts, displs, T.FP16, FAKE_STREAM) == 0
+        assert w.last_info().algName.decode() == "InsAllGatherVMesh1D"
+        rng = np.random.default_rng(n)
+        xs = [rng.integers(0, 65535, size=max(c, 1), dtype=np.uint16) for c in counts]
+        got = copy_trace_outputs(w.last_trace(), xs, [off] * n, 2)
+        want = T.run_allgatherv(xs, counts, displs, off, 0xA5A5)
+        for r in range(n):
+            assert np.array_equal(got[r], want[r]), r
+    finally:
+        w.close()
+
+
+def a2a_tables(m):
+    n = len(m)
+    return [T.alltoallvc_to_v(m, r) for r in range(n)]
+
+
+@pytest.mark.parametrize("n", [2, 3, 5, 8, 17, 20])
+def test_alltoallv_template_permutes_as_the_contract_says(n):
+    rng = np.random.default_rng(n)
+    m = rng.integers(0, 40, size=(n, n)).tolist()
+    m[0][n - 1] = 0
+    m[n - 1][0] = 0
+    if n == 8:
+        m[3][5] = 90000                   # one block larger than a scratch slot: several executor loops
+    v = a2a_tables(m)
+    w = api.World(n, ccl_bytes=SMALL_CCL, dry=True)
+    try:
+        ins, outs = fake_ptrs(n)
+        for r in range(n):
+            sc, sd, rc, rd = v[r]
+            assert w.all_to_all_v(r, ins[r], sc, sd, outs[r], rc, rd, T.FP32, FAKE_STREAM) == 0
+        xs = [rng.integers(0, 2**32 - 1, size=max(1, sum(m[i])), dtype=np.uint32) for i in range(n)]
+        got = copy_trace_outputs(w.last_trace(), xs, [max(1, sum(x[2])) for x in v], 4)
+        want = T.run_alltoallv(xs, [x[0] for x in v], [x[1] for x in v], [x[2] for x in v], [x[3] for x in v],
+                               [max(1, sum(x[2])) for x in v], fill=0xA5A5)
+        for r in range(n):
+            assert np.array_equal(got[r][:sum(v[r][2])], want[r][:sum(v[r][2])]), r
+    finally:
+        w.close()
+
+
+def test_alltoall_and_alltoallvc_reduce_to_alltoallv():
+    n, c = 4, 6
+    rng = np.random.default_rng(1)
+    xs = [rng.integers(0, 255, size=n * c, dtype=np.uint8) for _ in range(n)]
+    w = api.World(n, ccl_bytes=SMALL_CCL, dry=True)
+    try:
+        ins, outs = fake_ptrs(n)
+        for r in range(n):
+            assert w.all_to_all(r, ins[r], c, outs[r], T.UINT8, FAKE_STREAM) == 0
+        assert w.last_info().algName.decode() == "InsAlltoAllMesh1D"
+        got = copy_trace_outputs(w.last_trace(), xs, [n * c] * n, 1)
+        for j in range(n):
+            assert np.array_equal(got[j], np.concatenate([xs[i][j * c:(j + 1) * c] for i in range(n)]))
+        m = [[1, 2, 0, 3], [4, 0, 1, 1], [2, 2, 2, 0], [0, 5, 1, 1]]
+        flat = [x for row in m for x in row]
+        for r in range(n):
+            assert w.all_to_all_vc(r, ins[r], flat, outs[r], T.UINT8, FAKE_STREAM) == 0
+        assert w.last_info().algName.decode() == "InsAlltoAllVCMesh1D"
+        v = a2a_tables(m)
+        got = copy_trace_outputs(w.last_trace(), xs, [sum(x[2]) for x in v], 1)
+        want = T.run_alltoallv(xs, [x[0] for x in v], [x[1] for x in v], [x[2] for x in v], [x[3] for x in v],
+                               [sum(x[2]) for x in v])
+        for r in range(n):
+            assert np.array_equal(got[r], want[r])
+    finally:
+        w.close()
+
+
+def test_alltoallv_count_mismatch_between_ranks_is_rejected():
+    w = api.World(2, ccl_bytes=SMALL_CCL, dry=True)
+    ins, outs = fake_ptrs(2)
+    try:
+        assert w.all_to_all_v(0, ins[0], [1, 2], [0, 1], outs[0], [1, 3], [0, 1], T.INT8, FAKE_STREAM) == 0
+        # rank 1 expects 4 elements from rank 0, which sends 2
+        assert w.all_to_all_v(1, ins[1], [3, 1], [0, 3], outs[1], [4, 1], [0, 4], T.INT8, FAKE_STREAM) == 1
+    finally:
+        w.close()
