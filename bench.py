@@ -34,7 +34,8 @@ def parse():
 
 
 # ----------------------------------------------------------------------------------------------------
-# workloads: each builds device buffers once and exposes step() = one launch of the hot path
+# workloads: each builds device buffers once; step() = one collective through the HCCL entry points
+# (one call per virtual rank; the last call launches)
 # ----------------------------------------------------------------------------------------------------
 
 class Workload:
@@ -42,15 +43,22 @@ class Workload:
     dtype = ""
     kernel = ""          # name of the dominant kernel as rocprofv3 prints it (prefix)
 
-    def __init__(self, torch, hcclx, T):
-        self.torch, self.hcclx, self.T = torch, hcclx, T
-        self.stream = torch.cuda.current_stream().cuda_stream
+    def __init__(self, torch, api, T, n):
+        self.torch, self.api, self.T, self.n = torch, api, T, n
+        self.stream_obj = torch.cuda.Stream()
+        self.stream = self.stream_obj.cuda_stream
+        self.world = api.World(n)
 
     def step(self):
         raise NotImplementedError
 
     def algo_bytes(self):
         raise NotImplementedError
+
+    def info(self):
+        i = self.world.last_info()
+        return {"algorithm": i.algName.decode(), "fused": bool(i.fused), "launches": i.launches,
+                "plan_cache_hit": bool(i.planCacheHit)}
 
 
 def _randn_bits16(torch, n, seed, dt):
@@ -60,26 +68,26 @@ def _randn_bits16(torch, n, seed, dt):
 
 
 class ReduceScatterMesh(Workload):
-    """BASELINE config 2: ReduceScatter SUM bf16, mesh template, N ranks x (N * recv) elements in.
-    Output shard r folds slice r of every rank starting from rank r's own data, then ranks ascending
-    (ins_temp_reduce_scatter_mesh_1D.cc:132-154), fused into one pass."""
+    """BASELINE config 2: HcclReduceScatter SUM bf16, 8 ranks x 33,554,432 elements in (64 MiB per rank).
+    The selector picks the mesh template; output shard r folds slice r of every rank starting from rank
+    r's own data, then ranks ascending (ins_temp_reduce_scatter_mesh_1D.cc:132-154), as one fused pass."""
     dtype = "bf16"
     kernel = "hcclx::k_fold<11, 0, 8, 0>"
 
-    def __init__(self, torch, hcclx, T, n=8, recv=4 * 1024 * 1024):
-        super().__init__(torch, hcclx, T)
+    def __init__(self, torch, api, T, n=8, recv=4 * 1024 * 1024):
+        super().__init__(torch, api, T, n)
         self.name = "reduce_scatter_sum_bf16_mesh_%dx%dMiB" % (n, n * recv * 2 >> 20)
-        self.n, self.recv = n, recv
+        self.recv = recv
         self.x = [_randn_bits16(torch, n * recv, 1000 + r, torch.bfloat16) for r in range(n)]
         self.out = [torch.empty(recv, device="cuda:0", dtype=torch.bfloat16) for _ in range(n)]
-        segs = []
-        for r in range(n):
-            order = [r] + [k for k in range(n) if k != r]
-            segs.append((recv, [self.x[k].data_ptr() + r * recv * 2 for k in order], [self.out[r].data_ptr()]))
-        self.plan = hcclx.Plan(segs, T.BFP16, T.SUM)
+        self.sp = [t.data_ptr() for t in self.x]
+        self.rp = [t.data_ptr() for t in self.out]
 
     def step(self):
-        self.plan.launch(self.stream)
+        w, T = self.world, self.T
+        for r in range(self.n):
+            rc = w.reduce_scatter(r, self.sp[r], self.rp[r], self.recv, T.BFP16, T.SUM, self.stream)
+            assert rc == 0, rc
 
     def algo_bytes(self):
         return (self.n + 1) * self.n * self.recv * 2
@@ -100,81 +108,88 @@ class ReduceScatterMesh(Workload):
         return self.algo_bytes() / best / 1e9, "full workload (8 ranks x 64 MiB bf16), best of 2 runs"
 
 
-class AllReduceOneShotOrder(Workload):
-    """AllReduce SUM fp32, N ranks: every rank's output is the fold that starts from its own data
-    (one-shot mesh order, ins_temp_all_reduce_mesh_1D_one_shot.cc:182-197); inputs read once."""
+class AllReduce(Workload):
+    """HcclAllReduce SUM fp32, 8 ranks x 16,777,216 elements (64 MiB per rank).  At this size the selector
+    takes the two-shot mesh template: every slice is the fold x7 (+) (... (x1 (+) x0)), the same on all
+    ranks, so each input is read once and the result is written to the eight outputs."""
     dtype = "f32"
+    kernel = "hcclx::k_fold<4, 0, 8, 0>"
 
-    def __init__(self, torch, hcclx, T, n=8, count=16 * 1024 * 1024):
-        super().__init__(torch, hcclx, T)
+    def __init__(self, torch, api, T, n=8, count=16 * 1024 * 1024):
+        super().__init__(torch, api, T, n)
         self.name = "all_reduce_sum_fp32_%dx%dMiB" % (n, count * 4 >> 20)
-        self.n, self.count = n, count
+        self.count = count
         g = torch.Generator(device="cuda:0")
         g.manual_seed(7)
         self.x = [torch.rand(count, device="cuda:0", generator=g) * 2 - 1 for _ in range(n)]
         self.out = [torch.empty(count, device="cuda:0") for _ in range(n)]
-        self.plan = hcclx.Plan([(count, [t.data_ptr() for t in self.x], [t.data_ptr() for t in self.out])],
-                               T.FP32, T.SUM, hcclx.FOLD_SELF_FIRST)
+        self.sp = [t.data_ptr() for t in self.x]
+        self.rp = [t.data_ptr() for t in self.out]
 
     def step(self):
-        self.plan.launch(self.stream)
+        w, T = self.world, self.T
+        for r in range(self.n):
+            rc = w.all_reduce(r, self.sp[r], self.rp[r], self.count, T.FP32, T.SUM, self.stream)
+            assert rc == 0, rc
 
     def algo_bytes(self):
         return 2 * self.n * self.count * 4
 
 
 class AllGather(Workload):
-    """AllGather fp16: every rank's block lands in every output; read once, written N times."""
+    """HcclAllGather fp16, 8 ranks x 33,554,432 elements (64 MiB per rank): every block lands in every
+    output; each source byte is read once and written eight times."""
     dtype = "u8"
+    kernel = "hcclx::(anonymous namespace)::k_allgatherv"
 
-    def __init__(self, torch, hcclx, T, n=8, count=32 * 1024 * 1024):
-        super().__init__(torch, hcclx, T)
+    def __init__(self, torch, api, T, n=8, count=32 * 1024 * 1024):
+        super().__init__(torch, api, T, n)
         self.name = "all_gather_fp16_%dx%dMiB" % (n, count * 2 >> 20)
-        self.n, self.count = n, count
+        self.count = count
         self.x = [torch.randint(-32768, 32767, (count,), device="cuda:0", dtype=torch.int16) for _ in range(n)]
         self.out = [torch.empty(n * count, device="cuda:0", dtype=torch.int16) for _ in range(n)]
-        segs = [(count, [self.x[i].data_ptr()], [o.data_ptr() + i * count * 2 for o in self.out]) for i in range(n)]
-        self.plan = hcclx.Plan(segs, T.FP16)
+        self.sp = [t.data_ptr() for t in self.x]
+        self.rp = [t.data_ptr() for t in self.out]
 
     def step(self):
-        self.plan.launch(self.stream)
+        w, T = self.world, self.T
+        for r in range(self.n):
+            rc = w.all_gather(r, self.sp[r], self.rp[r], self.count, T.FP16, self.stream)
+            assert rc == 0, rc
 
     def algo_bytes(self):
         return 2 * self.n * self.n * self.count * 2
 
 
 class AllToAllV(Workload):
-    """BASELINE config 4 shape: MoE dispatch, N ranks x tokens x hidden bf16, destinations Zipf(1.2),
-    tokens grouped by destination; count/displacement tables resident on the device."""
+    """BASELINE config 4: HcclAlltoAllV bf16, MoE dispatch: 8 ranks x 4096 tokens x hidden 7168,
+    destination rank per token Zipf(s=1.2), tokens grouped by destination."""
     dtype = "u8"
+    kernel = "hcclx::(anonymous namespace)::k_alltoallv"
 
-    def __init__(self, torch, hcclx, T, n=8, tokens=4096, hidden=7168, seed=0):
+    def __init__(self, torch, api, T, n=8, tokens=4096, hidden=7168, seed=0):
         import numpy as np
-        super().__init__(torch, hcclx, T)
+        super().__init__(torch, api, T, n)
         self.name = "all_to_all_v_bf16_moe_%dx%dx%d" % (n, tokens, hidden)
         rng = np.random.default_rng(seed)
         w = 1.0 / np.arange(1, n + 1) ** 1.2
         w /= w.sum()
         tok = np.stack([np.bincount(rng.choice(n, size=tokens, p=w), minlength=n) for _ in range(n)])
-        sc = (tok * hidden).astype(np.uint64)
-        sd = np.zeros_like(sc)
-        sd[:, 1:] = np.cumsum(sc, 1)[:, :-1]
-        rc = sc.T.copy()
-        rd = np.zeros_like(rc)
-        rd[:, 1:] = np.cumsum(rc, 1)[:, :-1]
-        self.n = n
-        self.payload = int(sc.sum()) * 2
+        m = (tok * hidden).tolist()
+        self.v = [T.alltoallvc_to_v(m, r) for r in range(n)]
+        self.payload = int(sum(sum(row) for row in m)) * 2
         self.send = [torch.randint(-32768, 32767, (tokens * hidden,), device="cuda:0", dtype=torch.int16)
                      for _ in range(n)]
-        self.recv = [torch.empty(max(1, int(rc[j].sum())), device="cuda:0", dtype=torch.int16) for j in range(n)]
-        self.tab = torch.from_numpy(np.concatenate([sc.ravel(), sd.ravel(), rd.ravel()]).astype(np.int64)).to("cuda:0")
+        self.recv = [torch.empty(max(1, sum(self.v[j][2])), device="cuda:0", dtype=torch.int16) for j in range(n)]
         self.sp = [t.data_ptr() for t in self.send]
         self.rp = [t.data_ptr() for t in self.recv]
 
     def step(self):
-        p, nn = self.tab.data_ptr(), self.n * self.n * 8
-        self.hcclx.alltoallv(self.sp, self.rp, p, p + nn, p + 2 * nn, self.T.BFP16, on_device=True,
-                             stream=self.stream)
+        w, T = self.world, self.T
+        for r in range(self.n):
+            sc, sd, rc_, rd = self.v[r]
+            rc = w.all_to_all_v(r, self.sp[r], sc, sd, self.rp[r], rc_, rd, T.BFP16, self.stream)
+            assert rc == 0, rc
 
     def algo_bytes(self):
         return 2 * self.payload
@@ -182,23 +197,25 @@ class AllToAllV(Workload):
 
 WORKLOADS = {
     "reduce_scatter_sum_bf16_mesh_8x64MiB": lambda *a: ReduceScatterMesh(*a),
-    "all_reduce_sum_fp32_8x64MiB": lambda *a: AllReduceOneShotOrder(*a),
+    "all_reduce_sum_fp32_8x64MiB": lambda *a: AllReduce(*a),
     "all_gather_fp16_8x64MiB": lambda *a: AllGather(*a),
     "all_to_all_v_bf16_moe_8x4096x7168": lambda *a: AllToAllV(*a),
 }
 
 
 def time_steps(torch, wl, steps, warmup):
+    """W untimed steps, then K steps bracketed by synchronisation; events sit on the launch stream."""
+    torch.cuda.synchronize()
     for _ in range(warmup):
         wl.step()
     torch.cuda.synchronize()
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
-    e0.record()
+    e0.record(wl.stream_obj)
     for _ in range(steps):
         wl.step()
-    e1.record()
+    e1.record(wl.stream_obj)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     ev_ms = e0.elapsed_time(e1) / steps
@@ -212,7 +229,7 @@ def main():
               "run it with --gpus 1 (no multi-GPU figure exists for this build)", file=sys.stderr)
         sys.exit(2)
     import torch
-    from hccl_amd import hcclx
+    from hccl_amd import api, hcclx
     from oracle import templates as T   # cpu_baseline leg only
 
     if not torch.cuda.is_available():
@@ -223,7 +240,7 @@ def main():
         print("unknown workload; choose one of: " + ", ".join(WORKLOADS), file=sys.stderr)
         sys.exit(2)
 
-    wl = WORKLOADS[args.workload](torch, hcclx, T)
+    wl = WORKLOADS[args.workload](torch, api, T)
     wall_ms, ev_ms = time_steps(torch, wl, args.steps, args.warmup)
     gbs = wl.algo_bytes() / (ev_ms * 1e-3) / 1e9
     line = {
@@ -239,8 +256,9 @@ def main():
         "vs_baseline": None,
         "dtype": wl.dtype,
         "data": "synthetic",
-        "config": {"workload": wl.name, "virtual_ranks": 8, "algorithmic_bytes": wl.algo_bytes(),
-                   "pct_of_hbm_peak": round(gbs / HBM_PEAK_GBS * 100, 1)},
+        "config": dict({"workload": wl.name, "virtual_ranks": 8, "algorithmic_bytes": wl.algo_bytes(),
+                        "pct_of_hbm_peak": round(gbs / HBM_PEAK_GBS * 100, 1), "entry": "HcclReduceScatter"
+                        if "reduce_scatter" in wl.name else "Hccl* entry points"}, **wl.info()),
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": wl.kernel,
                      "kernel_us": round(ev_ms * 1e3, 2)},
@@ -252,11 +270,13 @@ def main():
             if name == args.workload:
                 w2, ms = wl, ev_ms
             else:
-                w2 = make(torch, hcclx, T)
+                w2 = make(torch, api, T)
                 _, ms = time_steps(torch, w2, max(5, args.steps // 2), args.warmup)
             g = w2.algo_bytes() / (ms * 1e-3) / 1e9
-            ops[name] = {"GB/s": round(g, 1), "pct_of_peak": round(g / HBM_PEAK_GBS * 100, 1), "us": round(ms * 1e3, 1)}
+            ops[name] = dict({"GB/s": round(g, 1), "pct_of_peak": round(g / HBM_PEAK_GBS * 100, 1),
+                              "us": round(ms * 1e3, 1)}, **w2.info())
             if w2 is not wl:
+                w2.world.close()
                 del w2
                 torch.cuda.empty_cache()
         line["ops"] = ops
