@@ -177,6 +177,7 @@ class AllToAllV(Workload):
         tok = np.stack([np.bincount(rng.choice(n, size=tokens, p=w), minlength=n) for _ in range(n)])
         m = (tok * hidden).tolist()
         self.v = [T.alltoallvc_to_v(m, r) for r in range(n)]
+        self.tabs = [[api.u64_table(t) for t in self.v[r]] for r in range(n)]   # converted once
         self.payload = int(sum(sum(row) for row in m)) * 2
         self.send = [torch.randint(-32768, 32767, (tokens * hidden,), device="cuda:0", dtype=torch.int16)
                      for _ in range(n)]
@@ -187,12 +188,40 @@ class AllToAllV(Workload):
     def step(self):
         w, T = self.world, self.T
         for r in range(self.n):
-            sc, sd, rc_, rd = self.v[r]
+            sc, sd, rc_, rd = self.tabs[r]
             rc = w.all_to_all_v(r, self.sp[r], sc, sd, self.rp[r], rc_, rd, T.BFP16, self.stream)
             assert rc == 0, rc
 
     def algo_bytes(self):
         return 2 * self.payload
+
+
+class CopyCalibration(Workload):
+    """A plain device copy of 1 GiB through the fold kernel's copy instantiation: a kernel of known size,
+    used to scale the HBM traffic counters of a profiler run.  Not part of the per-op table."""
+    dtype = "u8"
+    kernel = "hcclx::k_fold<0, 0, 1, 0>"
+
+    def __init__(self, torch, api, T, nbytes=1 << 30):
+        from hccl_amd import hcclx
+        self.torch, self.n = torch, 1
+        self.stream_obj = torch.cuda.Stream()
+        self.stream = self.stream_obj.cuda_stream
+        self.world = None
+        self.name = "copy_calibration_%dMiB" % (nbytes >> 20)
+        self.nbytes = nbytes
+        self.a = torch.empty(nbytes, device="cuda:0", dtype=torch.uint8).random_(0, 255)
+        self.b = torch.empty(nbytes, device="cuda:0", dtype=torch.uint8)
+        self.plan = hcclx.Plan([(nbytes, [self.a.data_ptr()], [self.b.data_ptr()])], T.UINT8)
+
+    def step(self):
+        self.plan.launch(self.stream)
+
+    def algo_bytes(self):
+        return 2 * self.nbytes
+
+    def info(self):
+        return {"algorithm": "copy", "fused": True, "launches": 1, "plan_cache_hit": True}
 
 
 WORKLOADS = {
@@ -201,14 +230,18 @@ WORKLOADS = {
     "all_gather_fp16_8x64MiB": lambda *a: AllGather(*a),
     "all_to_all_v_bf16_moe_8x4096x7168": lambda *a: AllToAllV(*a),
 }
+EXTRA_WORKLOADS = {"copy_calibration_1024MiB": lambda *a: CopyCalibration(*a)}
 
 
 def time_steps(torch, wl, steps, warmup):
     """W untimed steps, then K steps bracketed by synchronisation; events sit on the launch stream."""
+    import gc
     torch.cuda.synchronize()
     for _ in range(warmup):
         wl.step()
     torch.cuda.synchronize()
+    gc.collect()
+    gc.disable()   # a full collection of the interpreter's heap would show up as a 40 ms step
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
@@ -217,6 +250,7 @@ def time_steps(torch, wl, steps, warmup):
         wl.step()
     e1.record(wl.stream_obj)
     torch.cuda.synchronize()
+    gc.enable()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     ev_ms = e0.elapsed_time(e1) / steps
     return wall_ms, ev_ms
@@ -236,11 +270,12 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     hcclx.init()
-    if args.workload not in WORKLOADS:
-        print("unknown workload; choose one of: " + ", ".join(WORKLOADS), file=sys.stderr)
+    makers = dict(WORKLOADS, **EXTRA_WORKLOADS)
+    if args.workload not in makers:
+        print("unknown workload; choose one of: " + ", ".join(makers), file=sys.stderr)
         sys.exit(2)
 
-    wl = WORKLOADS[args.workload](torch, api, T)
+    wl = makers[args.workload](torch, api, T)
     wall_ms, ev_ms = time_steps(torch, wl, args.steps, args.warmup)
     gbs = wl.algo_bytes() / (ev_ms * 1e-3) / 1e9
     line = {

@@ -60,8 +60,15 @@ def check(rc):
         raise HcclError(rc, "collective call failed")
 
 
-def _u64(seq):
+def u64_table(seq):
+    """Host count / displacement table as the C entry points take it (uint64 array).  Tables that do not
+    change between calls can be converted once and passed again."""
+    if isinstance(seq, ctypes.Array):
+        return seq
     return (ctypes.c_uint64 * len(seq))(*[int(x) for x in seq])
+
+
+_u64 = u64_table
 
 
 class World:

@@ -72,6 +72,10 @@ void init_slot(DeviceSlot *s, int dev)
         const uint32_t b = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
         if (b != 0) c.v_blocks_per_cu = b;
     }
+    if (const char *v = std::getenv("HCCLX_V_TILES_PER_BLOCK")) {
+        const uint32_t b = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
+        if (b != 0) c.v_tiles_per_block = b;
+    }
     c.ring_bytes = kSliceBytes * kSlices;
     e = hipHostMalloc(reinterpret_cast<void **>(&c.h_ring), c.ring_bytes, hipHostMallocDefault);
     if (e != hipSuccess) {

@@ -29,6 +29,8 @@ struct DeviceCtx {
     // V kernels whose tables live on the device cannot know their tile count on the host and run as a
     // persistent grid of this many workgroups per CU.
     uint32_t v_blocks_per_cu = 2;
+    // With host tables the V kernels launch one workgroup per run of this many consecutive tiles.
+    uint32_t v_tiles_per_block = 1;
     // Descriptor ring: tables of one-shot launches are written to pinned host memory and copied to the
     // device ring on the launch stream just before the kernel.
     char *h_ring = nullptr;

@@ -60,11 +60,8 @@ int hcclx_alltoallv(const void *const *send, void *const *recv, const uint64_t *
     int rc = fill_ptrs(send, recv, n, &ptrs);
     if (rc != HCCL_SUCCESS) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const uint64_t *tabs[3] = {send_counts, sdispls, rdispls};
-    const uint64_t *dev[3];
-    rc = stage_tables(ctx, tabs, 3, static_cast<size_t>(n) * n, tables_on_device, st, dev);
-    if (rc != HCCL_SUCCESS) return rc;
     uint64_t grid = static_cast<uint64_t>(ctx->num_cus) * ctx->v_blocks_per_cu;
+    bool inline_ok = !tables_on_device && n <= kA2avInlineRanks;
     if (!tables_on_device) {
         // host tables: the tile count is known here, so launch exactly one workgroup per tile
         uint64_t total = 0;
@@ -75,10 +72,37 @@ int hcclx_alltoallv(const void *const *send, void *const *recv, const uint64_t *
             }
         }
         if (total == 0) return HCCL_SUCCESS;
-        grid = total < 0x7fffffffull ? total : 0x7fffffffull;
+        grid = (total + ctx->v_tiles_per_block - 1) / ctx->v_tiles_per_block;
+        if (grid > 0x7fffffffull) grid = 0x7fffffffull;
+        for (size_t k = 0; k < static_cast<size_t>(n) * n && inline_ok; ++k) {
+            inline_ok = send_counts[k] <= 0xffffffffull && sdispls[k] <= 0xffffffffull && rdispls[k] <= 0xffffffffull;
+        }
     }
+    if (inline_ok) {
+        // small host tables ride in the kernel arguments: nothing is copied in front of the kernel
+        VRankPtrs16 p16;
+        A2avTablesInline tabs;
+        std::memset(&p16, 0, sizeof(p16));
+        for (uint32_t i = 0; i < n; ++i) {
+            p16.send[i] = ptrs.send[i];
+            p16.recv[i] = ptrs.recv[i];
+        }
+        for (size_t k = 0; k < static_cast<size_t>(n) * n; ++k) {
+            tabs.send_counts[k] = static_cast<uint32_t>(send_counts[k]);
+            tabs.sdispls[k] = static_cast<uint32_t>(sdispls[k]);
+            tabs.rdispls[k] = static_cast<uint32_t>(rdispls[k]);
+        }
+        hipError_t e = launch_alltoallv_inline(p16, tabs, n, static_cast<uint32_t>(esz), static_cast<uint32_t>(grid),
+                                               ctx->v_tiles_per_block, st);
+        if (e != hipSuccess) return fail_hip(e, "alltoallv kernel launch");
+        return HCCL_SUCCESS;
+    }
+    const uint64_t *tabs[3] = {send_counts, sdispls, rdispls};
+    const uint64_t *dev[3];
+    rc = stage_tables(ctx, tabs, 3, static_cast<size_t>(n) * n, tables_on_device, st, dev);
+    if (rc != HCCL_SUCCESS) return rc;
     hipError_t e = launch_alltoallv(ptrs, dev[0], dev[1], dev[2], n, static_cast<uint32_t>(esz),
-                                    static_cast<uint32_t>(grid), st);
+                                    static_cast<uint32_t>(grid), tables_on_device ? 1u : ctx->v_tiles_per_block, st);
     if (e != hipSuccess) return fail_hip(e, "alltoallv kernel launch");
     return HCCL_SUCCESS;
 }
@@ -95,10 +119,6 @@ int hcclx_allgatherv(const void *const *send, void *const *recv, const uint64_t 
     int rc = fill_ptrs(send, recv, n, &ptrs);
     if (rc != HCCL_SUCCESS) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const uint64_t *tabs[2] = {counts, displs};
-    const uint64_t *dev[2];
-    rc = stage_tables(ctx, tabs, 2, n, tables_on_device, st, dev);
-    if (rc != HCCL_SUCCESS) return rc;
     uint64_t grid = static_cast<uint64_t>(ctx->num_cus) * ctx->v_blocks_per_cu;
     if (!tables_on_device) {
         uint64_t total = 0;
@@ -106,9 +126,21 @@ int hcclx_allgatherv(const void *const *send, void *const *recv, const uint64_t 
             total += v_tiles_of(counts[i] * esz, reinterpret_cast<uint64_t>(ptrs.recv[0]) + displs[i] * esz);
         }
         if (total == 0) return HCCL_SUCCESS;
-        grid = total < 0x7fffffffull ? total : 0x7fffffffull;
+        grid = (total + ctx->v_tiles_per_block - 1) / ctx->v_tiles_per_block;
+        if (grid > 0x7fffffffull) grid = 0x7fffffffull;
+        AgvTablesInline tabs;   // host tables of up to 64 ranks always fit the kernel arguments
+        std::memset(&tabs, 0, sizeof(tabs));
+        for (uint32_t i = 0; i < n; ++i) {
+            tabs.counts[i] = counts[i];
+            tabs.displs[i] = displs[i];
+        }
+        hipError_t e = launch_allgatherv_inline(ptrs, tabs, n, static_cast<uint32_t>(esz), static_cast<uint32_t>(grid),
+                                                ctx->v_tiles_per_block, st);
+        if (e != hipSuccess) return fail_hip(e, "allgatherv kernel launch");
+        return HCCL_SUCCESS;
     }
-    hipError_t e = launch_allgatherv(ptrs, dev[0], dev[1], n, static_cast<uint32_t>(esz), static_cast<uint32_t>(grid), st);
+    const uint64_t *dev[2] = {counts, displs};
+    hipError_t e = launch_allgatherv(ptrs, dev[0], dev[1], n, static_cast<uint32_t>(esz), static_cast<uint32_t>(grid), tables_on_device ? 1u : ctx->v_tiles_per_block, st);
     if (e != hipSuccess) return fail_hip(e, "allgatherv kernel launch");
     return HCCL_SUCCESS;
 }

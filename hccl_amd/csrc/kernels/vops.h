@@ -29,12 +29,56 @@ struct VRankPtrs {
     char *recv[kMaxVRanks];
 };
 
+// Count / displacement tables as the kernels read them.  Tables that arrive as host arrays and are small
+// enough travel inside the kernel arguments (no host-to-device copy is queued in front of the kernel);
+// larger ones, and tables that already live on the device, are read through pointers.
+struct A2avTablesPtr {
+    const uint64_t *send_counts;
+    const uint64_t *sdispls;
+    const uint64_t *rdispls;
+    __device__ uint64_t count(uint32_t p) const { return send_counts[p]; }
+    __device__ uint64_t sdispl(uint32_t p) const { return sdispls[p]; }
+    __device__ uint64_t rdispl(uint32_t p) const { return rdispls[p]; }
+};
+constexpr uint32_t kA2avInlineRanks = 16;  // 16 x 16 x 3 tables of uint32 = 3 KiB of kernel arguments
+struct A2avTablesInline {
+    uint32_t send_counts[kA2avInlineRanks * kA2avInlineRanks];
+    uint32_t sdispls[kA2avInlineRanks * kA2avInlineRanks];
+    uint32_t rdispls[kA2avInlineRanks * kA2avInlineRanks];
+    __device__ uint64_t count(uint32_t p) const { return send_counts[p]; }
+    __device__ uint64_t sdispl(uint32_t p) const { return sdispls[p]; }
+    __device__ uint64_t rdispl(uint32_t p) const { return rdispls[p]; }
+};
+// Base pointers for up to kA2avInlineRanks ranks, for the inline-table launch.
+struct VRankPtrs16 {
+    const char *send[kA2avInlineRanks];
+    char *recv[kA2avInlineRanks];
+};
+struct AgvTablesPtr {
+    const uint64_t *counts;
+    const uint64_t *displs;
+    __device__ uint64_t count(uint32_t i) const { return counts[i]; }
+    __device__ uint64_t displ(uint32_t i) const { return displs[i]; }
+};
+struct AgvTablesInline {
+    uint64_t counts[kMaxVRanks];
+    uint64_t displs[kMaxVRanks];
+    __device__ uint64_t count(uint32_t i) const { return counts[i]; }
+    __device__ uint64_t displ(uint32_t i) const { return displs[i]; }
+};
+
+hipError_t launch_alltoallv_inline(const VRankPtrs16 &ptrs, const A2avTablesInline &tabs, uint32_t n, uint32_t esz,
+                                   uint32_t grid, uint32_t tiles_per_block, hipStream_t stream);
+hipError_t launch_allgatherv_inline(const VRankPtrs &ptrs, const AgvTablesInline &tabs, uint32_t n, uint32_t esz,
+                                    uint32_t grid, uint32_t tiles_per_block, hipStream_t stream);
+
 // send_counts / sdispls / rdispls: device pointers, uint64 elements, row-major n x n.
 hipError_t launch_alltoallv(const VRankPtrs &ptrs, const uint64_t *send_counts, const uint64_t *sdispls,
-                            const uint64_t *rdispls, uint32_t n, uint32_t esz, uint32_t grid, hipStream_t stream);
+                            const uint64_t *rdispls, uint32_t n, uint32_t esz, uint32_t grid, uint32_t tiles_per_block,
+                            hipStream_t stream);
 
 // counts / displs: device pointers, uint64 elements, n entries.
 hipError_t launch_allgatherv(const VRankPtrs &ptrs, const uint64_t *counts, const uint64_t *displs, uint32_t n,
-                             uint32_t esz, uint32_t grid, hipStream_t stream);
+                             uint32_t esz, uint32_t grid, uint32_t tiles_per_block, hipStream_t stream);
 
 }  // namespace hcclx

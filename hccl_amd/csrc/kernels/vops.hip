@@ -126,9 +126,9 @@ __device__ __forceinline__ void copy_tile(const char *src, uint64_t dst0, uint64
     }
 }
 
+template <typename Ptrs, typename Tabs>
 __global__ void __launch_bounds__(kThreads)
-k_alltoallv(VRankPtrs ptrs, const uint64_t *__restrict__ send_counts, const uint64_t *__restrict__ sdispls,
-            const uint64_t *__restrict__ rdispls, uint32_t n, uint32_t esz)
+k_alltoallv(Ptrs ptrs, Tabs tabs, uint32_t n, uint32_t esz, uint32_t tiles_per_block)
 {
     extern __shared__ uint64_t s_end[];  // n*n entries, then 4 wave totals
     const uint32_t m = n * n;
@@ -136,44 +136,50 @@ k_alltoallv(VRankPtrs ptrs, const uint64_t *__restrict__ send_counts, const uint
     for (uint32_t p = threadIdx.x; p < m; p += kThreads) {
         const uint32_t i = p / n;
         const uint32_t j = p - i * n;
-        const uint64_t dst = reinterpret_cast<uint64_t>(ptrs.recv[j]) + rdispls[j * n + i] * esz;
-        s_end[p] = tiles_of(send_counts[p] * esz, dst);
+        const uint64_t dst = reinterpret_cast<uint64_t>(ptrs.recv[j]) + tabs.rdispl(j * n + i) * esz;
+        s_end[p] = tiles_of(tabs.count(p) * esz, dst);
     }
     __syncthreads();
     block_inclusive_scan(s_end, m, s_wave);
     const uint64_t total = s_end[m - 1];
 
-    for (uint64_t t = blockIdx.x; t < total; t += gridDim.x) {
+    // A workgroup takes runs of tiles_per_block consecutive tiles, so that the table set-up above is
+    // paid once per run.
+    const uint64_t stride = static_cast<uint64_t>(gridDim.x) * tiles_per_block;
+    for (uint64_t run = static_cast<uint64_t>(blockIdx.x) * tiles_per_block; run < total; run += stride)
+    for (uint64_t t = run; t < run + tiles_per_block && t < total; ++t) {
         const uint32_t p = find_block(s_end, m, t);
         const uint64_t tl = uniform64(t - (p ? s_end[p - 1] : 0));
         const uint32_t i = p / n;
         const uint32_t j = p - i * n;
-        const uint64_t bytes = send_counts[p] * esz;
-        const char *src = ptrs.send[i] + sdispls[p] * esz;
-        char *dst = ptrs.recv[j] + rdispls[j * n + i] * esz;
+        const uint64_t bytes = tabs.count(p) * esz;
+        const char *src = ptrs.send[i] + tabs.sdispl(p) * esz;
+        char *dst = ptrs.recv[j] + tabs.rdispl(j * n + i) * esz;
         copy_tile(src, reinterpret_cast<uint64_t>(dst), bytes, tl, 1, [=](uint32_t) { return dst; });
     }
 }
 
+template <typename Tabs>
 __global__ void __launch_bounds__(kThreads)
-k_allgatherv(VRankPtrs ptrs, const uint64_t *__restrict__ counts, const uint64_t *__restrict__ displs, uint32_t n,
-             uint32_t esz)
+k_allgatherv(VRankPtrs ptrs, Tabs tabs, uint32_t n, uint32_t esz, uint32_t tiles_per_block)
 {
     extern __shared__ uint64_t s_end[];  // n entries, then 4 wave totals
     uint64_t *s_wave = s_end + n;
     for (uint32_t i = threadIdx.x; i < n; i += kThreads) {
-        const uint64_t dst = reinterpret_cast<uint64_t>(ptrs.recv[0]) + displs[i] * esz;
-        s_end[i] = tiles_of(counts[i] * esz, dst);
+        const uint64_t dst = reinterpret_cast<uint64_t>(ptrs.recv[0]) + tabs.displ(i) * esz;
+        s_end[i] = tiles_of(tabs.count(i) * esz, dst);
     }
     __syncthreads();
     block_inclusive_scan(s_end, n, s_wave);
     const uint64_t total = s_end[n - 1];
 
-    for (uint64_t t = blockIdx.x; t < total; t += gridDim.x) {
+    const uint64_t stride = static_cast<uint64_t>(gridDim.x) * tiles_per_block;
+    for (uint64_t run = static_cast<uint64_t>(blockIdx.x) * tiles_per_block; run < total; run += stride)
+    for (uint64_t t = run; t < run + tiles_per_block && t < total; ++t) {
         const uint32_t i = find_block(s_end, n, t);
         const uint64_t tl = uniform64(t - (i ? s_end[i - 1] : 0));
-        const uint64_t bytes = counts[i] * esz;
-        const uint64_t off = displs[i] * esz;
+        const uint64_t bytes = tabs.count(i) * esz;
+        const uint64_t off = tabs.displ(i) * esz;
         const char *src = ptrs.send[i];
         copy_tile(src, reinterpret_cast<uint64_t>(ptrs.recv[0]) + off, bytes, tl, n,
                   [&](uint32_t d) { return ptrs.recv[d] + off; });
@@ -183,19 +189,41 @@ k_allgatherv(VRankPtrs ptrs, const uint64_t *__restrict__ counts, const uint64_t
 }  // namespace
 
 hipError_t launch_alltoallv(const VRankPtrs &ptrs, const uint64_t *send_counts, const uint64_t *sdispls,
-                            const uint64_t *rdispls, uint32_t n, uint32_t esz, uint32_t grid, hipStream_t stream)
+                            const uint64_t *rdispls, uint32_t n, uint32_t esz, uint32_t grid, uint32_t tiles_per_block,
+                            hipStream_t stream)
 {
     const size_t lds = (static_cast<size_t>(n) * n + 4) * sizeof(uint64_t);
-    hipLaunchKernelGGL(k_alltoallv, dim3(grid), dim3(kThreads), lds, stream, ptrs, send_counts, sdispls, rdispls, n,
-                       esz);
+    const A2avTablesPtr tabs{send_counts, sdispls, rdispls};
+    hipLaunchKernelGGL((k_alltoallv<VRankPtrs, A2avTablesPtr>), dim3(grid), dim3(kThreads), lds, stream, ptrs, tabs, n,
+                       esz, tiles_per_block);
+    return hipGetLastError();
+}
+
+hipError_t launch_alltoallv_inline(const VRankPtrs16 &ptrs, const A2avTablesInline &tabs, uint32_t n, uint32_t esz,
+                                   uint32_t grid, uint32_t tiles_per_block, hipStream_t stream)
+{
+    const size_t lds = (static_cast<size_t>(n) * n + 4) * sizeof(uint64_t);
+    hipLaunchKernelGGL((k_alltoallv<VRankPtrs16, A2avTablesInline>), dim3(grid), dim3(kThreads), lds, stream, ptrs, tabs,
+                       n, esz, tiles_per_block);
     return hipGetLastError();
 }
 
 hipError_t launch_allgatherv(const VRankPtrs &ptrs, const uint64_t *counts, const uint64_t *displs, uint32_t n,
-                             uint32_t esz, uint32_t grid, hipStream_t stream)
+                             uint32_t esz, uint32_t grid, uint32_t tiles_per_block, hipStream_t stream)
 {
     const size_t lds = (static_cast<size_t>(n) + 4) * sizeof(uint64_t);
-    hipLaunchKernelGGL(k_allgatherv, dim3(grid), dim3(kThreads), lds, stream, ptrs, counts, displs, n, esz);
+    const AgvTablesPtr tabs{counts, displs};
+    hipLaunchKernelGGL((k_allgatherv<AgvTablesPtr>), dim3(grid), dim3(kThreads), lds, stream, ptrs, tabs, n, esz,
+                       tiles_per_block);
+    return hipGetLastError();
+}
+
+hipError_t launch_allgatherv_inline(const VRankPtrs &ptrs, const AgvTablesInline &tabs, uint32_t n, uint32_t esz,
+                                    uint32_t grid, uint32_t tiles_per_block, hipStream_t stream)
+{
+    const size_t lds = (static_cast<size_t>(n) + 4) * sizeof(uint64_t);
+    hipLaunchKernelGGL((k_allgatherv<AgvTablesInline>), dim3(grid), dim3(kThreads), lds, stream, ptrs, tabs, n, esz,
+                       tiles_per_block);
     return hipGetLastError();
 }
 
