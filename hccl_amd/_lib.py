@@ -17,6 +17,7 @@ class Seg(ctypes.Structure):
         ("ndst", ctypes.c_uint32),
         ("src", ctypes.c_void_p * MAX_FAN),
         ("dst", ctypes.c_void_p * MAX_FAN),
+        ("prog", ctypes.c_uint8 * (2 * MAX_FAN)),
     ]
 
 

@@ -210,14 +210,70 @@ struct Built {
     uint64_t algo_bytes = 0;
 };
 
+// Embeds the (dst, src) step program of a tree segment into a complete binary tree with `slots` leaf
+// slots: fills the slot order of the sources, the per-node codes and the leaf mask.  Returns false when
+// the tree is deeper than log2(slots).
+bool embed_tree(const hcclx_seg_t &s, uint32_t slots, SegDev *sd)
+{
+    struct N {
+        int dst = -1, src = -1, leaf = -1;
+    };
+    std::vector<N> nodes(s.nsrc);
+    std::vector<int> holder(s.nsrc);  // node currently held by each register
+    for (uint32_t k = 0; k < s.nsrc; ++k) {
+        nodes[k].leaf = static_cast<int>(k);
+        holder[k] = static_cast<int>(k);
+    }
+    for (uint32_t t = 0; t + 1 < s.nsrc; ++t) {
+        N n;
+        n.dst = holder[s.prog[2 * t]];
+        n.src = holder[s.prog[2 * t + 1]];
+        nodes.push_back(n);
+        holder[s.prog[2 * t]] = static_cast<int>(nodes.size()) - 1;
+    }
+    sd->tree_codes = 0;
+    sd->leaf_mask = 0;
+    for (uint32_t k = 0; k < kMaxFan; ++k) sd->src[k] = nullptr;
+    bool ok = true;
+    // place(node, heap index): inner nodes combine their two children; a leaf above the bottom level is
+    // passed up from the left-most slot below it
+    std::vector<std::pair<int, uint32_t>> stack{{holder[0], 1u}};
+    while (!stack.empty() && ok) {
+        const int id = stack.back().first;
+        uint32_t at = stack.back().second;
+        stack.pop_back();
+        const N &n = nodes[id];
+        if (n.leaf >= 0) {
+            while (at < slots) {
+                sd->tree_codes |= 1u << (2 * at);
+                at *= 2;
+            }
+            sd->src[at - slots] = static_cast<const char *>(s.src[n.leaf]);
+            sd->leaf_mask |= 1u << (at - slots);
+        } else {
+            if (at >= slots) {
+                ok = false;
+                break;
+            }
+            sd->tree_codes |= 2u << (2 * at);
+            stack.push_back({n.dst, 2 * at});
+            stack.push_back({n.src, 2 * at + 1});
+        }
+    }
+    return ok;
+}
+
 int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, Built *out)
 {
     if (nseg != 0 && segs == nullptr) return fail(HCCL_E_PTR, "segs is null");
     const int esz = dtype_size(dtype);
     if (esz == 0) return fail(HCCL_E_NOT_SUPPORT, "unknown data type " + std::to_string(dtype));
-    if (mode != HCCLX_FOLD_CHAIN && mode != HCCLX_FOLD_SELF_FIRST) return fail(HCCL_E_PARA, "unknown fold mode");
+    if (mode != HCCLX_FOLD_CHAIN && mode != HCCLX_FOLD_SELF_FIRST && mode != HCCLX_FOLD_TREE) {
+        return fail(HCCL_E_PARA, "unknown fold mode");
+    }
 
     uint32_t max_src = 0;
+    uint32_t max_depth = 0;  // tree mode: levels of the deepest tree
     for (uint32_t i = 0; i < nseg; ++i) {
         const hcclx_seg_t &s = segs[i];
         if (s.nsrc == 0 || s.nsrc > HCCLX_MAX_FAN || s.ndst == 0 || s.ndst > HCCLX_MAX_FAN) {
@@ -235,6 +291,25 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
                 if (s.dst[k] == nullptr) return fail(HCCL_E_PTR, "segment " + std::to_string(i) + ": null destination");
             }
         }
+        if (mode == HCCLX_FOLD_TREE) {
+            // every register but 0 is consumed exactly once, register 0 never; a consumed register is dead
+            bool dead[HCCLX_MAX_FAN] = {false};
+            uint32_t depth[HCCLX_MAX_FAN] = {0};
+            for (uint32_t t = 0; t + 1 < s.nsrc; ++t) {
+                const uint32_t rd = s.prog[2 * t];
+                const uint32_t rs = s.prog[2 * t + 1];
+                if (rd >= s.nsrc || rs >= s.nsrc || rd == rs || rs == 0 || dead[rd] || dead[rs]) {
+                    return fail(HCCL_E_PARA, "segment " + std::to_string(i) + ": malformed tree program");
+                }
+                dead[rs] = true;
+                depth[rd] = (depth[rd] > depth[rs] ? depth[rd] : depth[rs]) + 1;
+            }
+            if (is_float_dtype(dtype) && (1u << depth[0]) > HCCLX_MAX_FAN) {
+                return fail(HCCL_E_NOT_SUPPORT, "segment " + std::to_string(i) + ": tree has " + std::to_string(depth[0]) +
+                                                    " levels, the kernel holds 4");
+            }
+            if (depth[0] > max_depth) max_depth = depth[0];
+        }
         if (s.nsrc > max_src) max_src = s.nsrc;
     }
 
@@ -247,6 +322,8 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
         if (!is_reduce_dtype(dtype)) return fail(HCCL_E_NOT_SUPPORT, "data type cannot be reduced");
         if (op < HCCL_REDUCE_SUM || op > HCCL_REDUCE_MIN) return fail(HCCL_E_NOT_SUPPORT, "unknown reduce op");
         proto.maxn = max_src <= 2 ? 2 : max_src <= 4 ? 4 : max_src <= 8 ? 8 : 16;
+        // a tree needs one leaf slot per position of the complete tree of its depth
+        if (mode == HCCLX_FOLD_TREE && is_float_dtype(dtype) && (1 << max_depth) > proto.maxn) proto.maxn = 1 << max_depth;
         // Integer folds are association-free: the self-first order gives the bits of the plain chain.
         // The kernel for it exists only for floating types, so integers take the chain kernel with the
         // self-first segment rewritten below.
@@ -254,7 +331,8 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
         proto.maxn = 1;
         proto.mode = HCCLX_FOLD_CHAIN;
     }
-    const bool rewrite_self = (!proto.copy && mode == HCCLX_FOLD_SELF_FIRST && !is_float_dtype(dtype));
+    // likewise a tree over integers equals the chain of its leaves
+    const bool rewrite_self = (!proto.copy && mode != HCCLX_FOLD_CHAIN && !is_float_dtype(dtype));
     if (rewrite_self) proto.mode = HCCLX_FOLD_CHAIN;
 
     const int ne = proto.copy ? 16 : 16 / esz;
@@ -269,6 +347,10 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
         sd.ndst = s.ndst;
         for (uint32_t k = 0; k < s.nsrc; ++k) sd.src[k] = static_cast<const char *>(s.src[k]);
         for (uint32_t k = 0; k < s.ndst; ++k) sd.dst[k] = static_cast<char *>(s.dst[k]);
+        if (proto.mode == HCCLX_FOLD_TREE && !embed_tree(s, static_cast<uint32_t>(proto.maxn), &sd)) {
+            return fail(HCCL_E_NOT_SUPPORT, "segment " + std::to_string(i) + ": tree deeper than log2(" +
+                                                std::to_string(proto.maxn) + ") levels");
+        }
         const uint64_t tiles = fold_tiles_of(sd.count, ne, proto.maxn);
         if (static_cast<int>(cur.segs.size()) == kMaxSegsPerLaunch) {
             out->batches.push_back(std::move(cur));

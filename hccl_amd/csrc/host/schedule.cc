@@ -293,7 +293,9 @@ struct Fold {
     std::vector<u64> src;
     u64 dst = 0;
     u64 bytes = 0;
-    bool chain = true;  // false: a tree that no chain reproduces
+    bool chain = true;        // false: a tree that no chain reproduces
+    bool fits = true;         // false: a tree too large for the tree kernel
+    std::vector<u8> prog;     // tree: (dst register, src register) per step over src[] as registers
 };
 
 bool IsFloatType(int dt)
@@ -331,6 +333,27 @@ std::string ExprText(const Tracer &tr, int e, u64 shift, const std::vector<OpPar
            ")";
 }
 
+// Post-order walk of a tree expression: leaves are numbered dst side first, so the value of every node
+// ends up in the register of its left-most leaf and the root in register 0.  Returns that register and
+// the number of levels below the node through *levels.
+u32 EmitTree(const Tracer &tr, int e, u64 shift, Fold &f, u32 *levels)
+{
+    if (e == 0) {
+        f.src.push_back(shift);
+        *levels = 0;
+        return static_cast<u32>(f.src.size()) - 1;
+    }
+    const Expr &x = tr.At(e);
+    u32 ld = 0;
+    u32 ls = 0;
+    const u32 rd = EmitTree(tr, x.dst, shift + x.dstShift, f, &ld);
+    const u32 rs = EmitTree(tr, x.src, shift + x.srcShift, f, &ls);
+    f.prog.push_back(static_cast<u8>(rd));
+    f.prog.push_back(static_cast<u8>(rs));
+    *levels = std::max(ld, ls) + 1;
+    return rd;
+}
+
 // Turns the expression of a piece into a fold.  A left-deep spine "leaf (+) acc" is a chain as it
 // stands.  Integer arithmetic (wrap-around sum and product, max, min) is associative and commutative, so
 // any tree equals the chain of its leaves.  For floating types IEEE addition and multiplication are
@@ -359,7 +382,12 @@ Fold Flatten(const Tracer &tr, int e, u64 shift, int dtype, int op)
             sh += x.srcShift;
             cur = x.src;
         } else {
+            // not a spine: keep the tree as it is, for the kernel that evaluates trees of up to
+            // log2(HCCLX_MAX_FAN) levels in registers
             f.chain = false;
+            u32 levels = 0;
+            (void)EmitTree(tr, e, shift, f, &levels);
+            f.fits = (f.src.size() <= HCCLX_MAX_FAN && (1u << levels) <= HCCLX_MAX_FAN);
             return f;
         }
     }
@@ -372,18 +400,19 @@ struct FusedPlan {
     std::vector<hcclx_seg_t> chainSegs;
     std::vector<hcclx_seg_t> selfSegs;
     std::vector<hcclx_seg_t> copySegs;
+    std::vector<hcclx_seg_t> treeSegs;
 };
 
 bool Overlaps(u64 a, u64 alen, u64 b, u64 blen) { return a < b + blen && b < a + alen; }
 
 // Builds the fused launch plan from the traced outputs.  Returns false when the schedule cannot be fused
-// (a floating-point tree, a source that is not an input, or an output that overlaps another fold's
+// (a floating-point tree with more than four levels, a source that is not an input, or an output that overlaps another fold's
 // source); the caller then runs the steps one by one.
 bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &params, int dtype, int op, u32 esz,
                     FusedPlan &plan, std::string *text)
 {
     std::vector<Fold> folds;
-    bool allChains = true;
+    bool allFit = true;
     for (size_t r = 0; r < params.size(); ++r) {
         const u64 out = reinterpret_cast<u64>(params[r].outputPtr);
         if (params[r].outputSize == 0) continue;
@@ -398,11 +427,11 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
                    << ExprText(tr, s.expr, s.shift, params) << "\n";
                 *text += os.str();
             }
-            if (!f.chain) allChains = false;
+            if (!f.fits) allFit = false;
             folds.push_back(std::move(f));
         }
     }
-    if (!allChains) return false;
+    if (!allFit) return false;
     // every source must be input data (or an output that the same fold overwrites in place)
     for (const Fold &f : folds) {
         for (u64 a : f.src) {
@@ -421,6 +450,7 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
     for (size_t i = 0; i < folds.size(); ++i) {
         std::vector<u64> key = folds[i].src;
         key.push_back(folds[i].bytes);
+        for (u8 b : folds[i].prog) key.push_back(b);  // same sources, different tree: different value
         bySrc[key].push_back(i);
     }
     // and find groups of N folds over the same N sources where fold j starts from source j and then takes
@@ -429,7 +459,7 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
     for (auto &kv : bySrc) {
         if (kv.second.size() != 1) continue;
         const Fold &f = folds[kv.second[0]];
-        if (f.src.size() < 2 || f.src.size() > HCCLX_MAX_FAN) continue;
+        if (!f.chain || f.src.size() < 2 || f.src.size() > HCCLX_MAX_FAN) continue;
         std::vector<u64> key = f.src;
         std::sort(key.begin(), key.end());
         key.push_back(f.bytes);
@@ -509,6 +539,10 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
             if (f.src.size() == 1) {
                 seg.count = f.bytes;  // a copy: counted in bytes
                 plan.copySegs.push_back(seg);
+            } else if (!f.chain) {
+                seg.count = f.bytes / esz;
+                std::memcpy(seg.prog, f.prog.data(), f.prog.size());
+                plan.treeSegs.push_back(seg);
             } else {
                 seg.count = f.bytes / esz;
                 plan.chainSegs.push_back(seg);
@@ -738,7 +772,7 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
         const bool ok = BuildFusedPlan(w, tr, params, foldType, op, esz, plan,
                                        (w->traceText || w->dryRun) ? &w->lastTrace : nullptr);
         w->lastFusedSegments =
-            static_cast<u32>(plan.chainSegs.size() + plan.selfSegs.size() + plan.copySegs.size());
+            static_cast<u32>(plan.chainSegs.size() + plan.selfSegs.size() + plan.copySegs.size() + plan.treeSegs.size());
         if (w->dryRun) {
             w->lastWasFused = ok;
             return HCCL_SUCCESS;
@@ -746,10 +780,10 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
         if (ok && fused) {
             CachedPlan c;
             c.key = key;
-            const std::pair<std::vector<hcclx_seg_t> *, int> parts[3] = {
+            const std::pair<std::vector<hcclx_seg_t> *, int> parts[4] = {
                 {&plan.selfSegs, HCCLX_FOLD_SELF_FIRST}, {&plan.chainSegs, HCCLX_FOLD_CHAIN},
-                {&plan.copySegs, HCCLX_FOLD_CHAIN}};
-            for (int i = 0; i < 3; ++i) {
+                {&plan.copySegs, HCCLX_FOLD_CHAIN}, {&plan.treeSegs, HCCLX_FOLD_TREE}};
+            for (int i = 0; i < 4; ++i) {
                 if (parts[i].first->empty()) continue;
                 hcclx_plan *hp = nullptr;
                 const int dt = (i == 2) ? HCCL_DATA_TYPE_INT8 : foldType;

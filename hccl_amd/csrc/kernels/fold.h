@@ -41,6 +41,29 @@ __device__ __forceinline__ uint64_t uniform64(uint64_t x)
     return (static_cast<uint64_t>(hi) << 32) | lo;
 }
 
+// Evaluates the embedded tree bottom-up.  leaf[k] are the MAXN leaf slots; every index below is a compile
+// time constant and every condition is wave-uniform, so the values stay in named registers.
+template <int DT, int OP, int MAXN, typename C, int NE>
+__device__ __forceinline__ void tree_eval(C (&leaf)[MAXN][NE], uint32_t codes)
+{
+    // level by level in place: after the pass for width w, leaf[0 .. w) hold the nodes w .. 2w-1
+#pragma unroll
+    for (int w = MAXN / 2; w >= 1; w /= 2) {
+#pragma unroll
+        for (int i = 0; i < w; ++i) {
+            const uint32_t code = (codes >> (2 * (w + i))) & 3u;
+            if (code == 2u) {
+#pragma unroll
+                for (int e = 0; e < NE; ++e) leaf[i][e] = Combine<DT, OP>::run(leaf[2 * i + 1][e], leaf[2 * i][e]);
+            } else if (code == 1u && i != 0) {
+                // pass the dst child up (for i == 0 it already sits in place)
+#pragma unroll
+                for (int e = 0; e < NE; ++e) leaf[i][e] = leaf[2 * i][e];
+            }
+        }
+    }
+}
+
 template <int DT, int OP, int MAXN, int MODE, bool CHECK>
 __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint32_t ndst, uint64_t v0, uint64_t nvec)
 {
@@ -51,9 +74,10 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
     using Op = Combine<DT, OP>;
 
     u32x4 raw[UNROLL][MAXN];
+    const uint32_t present = (MODE == kFoldTree) ? sd.leaf_mask : ((nsrc >= 32u) ? ~0u : ((1u << nsrc) - 1u));
 #pragma unroll
     for (int k = 0; k < MAXN; ++k) {
-        if (k < static_cast<int>(nsrc)) {
+        if ((present >> k) & 1u) {
             const char *p = sd.src[k] + v0 * 16;
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
@@ -86,6 +110,17 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
             for (uint32_t d = 0; d < ndst; ++d) {
                 st16(sd.dst[d] + vi * 16, out);
             }
+        } else if constexpr (MODE == kFoldTree) {
+            C val[MAXN][NE];
+#pragma unroll
+            for (int k = 0; k < MAXN; ++k) {
+                if ((present >> k) & 1u) V::unpack(raw[u][k], val[k]);
+            }
+            tree_eval<DT, OP, MAXN, C, NE>(val, sd.tree_codes);
+            const u32x4 out = V::pack(val[0]);
+            for (uint32_t d = 0; d < ndst; ++d) {
+                st16(sd.dst[d] + vi * 16, out);
+            }
         } else {
             C val[MAXN][NE];
 #pragma unroll
@@ -113,7 +148,7 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
 }
 
 // The last (count % NE) elements of a segment, one per thread.
-template <int DT, int OP, int MODE>
+template <int DT, int OP, int MAXN, int MODE>
 __device__ __forceinline__ void fold_tail(const SegDev &sd, uint32_t nsrc, uint32_t ndst, uint64_t idx)
 {
     using D = DTypeOf<DT>;
@@ -126,6 +161,15 @@ __device__ __forceinline__ void fold_tail(const SegDev &sd, uint32_t nsrc, uint3
             acc = Op::run(D::widen(reinterpret_cast<const S *>(sd.src[k])[idx]), acc);
         }
         const S out = D::narrow(acc);
+        for (uint32_t d = 0; d < ndst; ++d) reinterpret_cast<S *>(sd.dst[d])[idx] = out;
+    } else if constexpr (MODE == kFoldTree) {
+        C val[MAXN][1];
+#pragma unroll
+        for (int k = 0; k < MAXN; ++k) {
+            if ((sd.leaf_mask >> k) & 1u) val[k][0] = D::widen(reinterpret_cast<const S *>(sd.src[k])[idx]);
+        }
+        tree_eval<DT, OP, MAXN, C, 1>(val, sd.tree_codes);
+        const S out = D::narrow(val[0][0]);
         for (uint32_t d = 0; d < ndst; ++d) reinterpret_cast<S *>(sd.dst[d])[idx] = out;
     } else {
         // Every source is read before the first destination is written: a destination may alias a source.
@@ -179,7 +223,7 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
         } else {
             fold_tile<DT, OP, MAXN, MODE, true>(sd, nsrc, ndst, v0, nvec);
             if (rem != 0 && tl == nvec / TV && threadIdx.x < rem) {
-                fold_tail<DT, OP, MODE>(sd, nsrc, ndst, nvec * NE + threadIdx.x);
+                fold_tail<DT, OP, MAXN, MODE>(sd, nsrc, ndst, nvec * NE + threadIdx.x);
             }
         }
     }

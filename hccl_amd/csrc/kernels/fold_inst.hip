@@ -1,7 +1,7 @@
 // One data type's instantiations of the fold kernel.  Built once per type with
 //   -DHCCLX_DT=<HcclDataType enumerator> -DHCCLX_NAME=<suffix> -DHCCLX_ORDERED=<0|1>
-// HCCLX_ORDERED=1 (floating types) also builds the self-first mode; for integers every fold order gives
-// the same bits, so the launcher maps that mode onto the chain kernel.
+// HCCLX_ORDERED=1 (floating types) also builds the self-first and tree modes; for integers every fold
+// order gives the same bits, so the launcher maps those modes onto the chain kernel.
 // With -DHCCLX_COPY the unit holds the byte copy kernel instead (one source, many destinations).
 #include "fold.h"
 
@@ -59,6 +59,9 @@ hipError_t HCCLX_CAT(fold_dispatch_, HCCLX_NAME)(int op, int maxn, int mode, con
 #if HCCLX_ORDERED
     if (mode == kFoldSelfFirst) {
         return by_op<kFoldSelfFirst>(op, maxn, l);
+    }
+    if (mode == kFoldTree) {
+        return by_op<kFoldTree>(op, maxn, l);
     }
 #endif
     return hipErrorInvalidValue;

@@ -19,6 +19,12 @@ struct SegDev {
     uint32_t ndst;
     const char *src[kMaxFan];  // in fold order
     char *dst[kMaxFan];
+    // Tree mode: the tree is embedded in a complete binary tree with MAXN leaf slots (heap numbering: root
+    // 1, children of i are 2i = the step's dst side and 2i+1 = its src side, leaf slots MAXN .. 2*MAXN-1
+    // hold src[slot - MAXN]).  Two bits per inner node i at bit 2*i: 0 = nothing below, 1 = take the dst
+    // child unchanged, 2 = child(2i+1) (+) child(2i).  leaf_mask has bit k set when src[k] is present.
+    uint32_t tree_codes;
+    uint32_t leaf_mask;
 };
 
 // How the sources of a segment are folded.
@@ -27,6 +33,9 @@ enum FoldMode : int {
     kFoldChain = 0,
     // nsrc == ndst; dst[j] = fold starting from src[j], then src[k] for k ascending, k != j.
     kFoldSelfFirst = 1,
+    // A binary tree of at most log2(MAXN) levels over the sources (see SegDev::tree_codes); the value of
+    // the root goes to every dst.
+    kFoldTree = 2,
 };
 
 }  // namespace hcclx

@@ -6,13 +6,18 @@ from ._lib import Seg, check
 
 FOLD_CHAIN = 0
 FOLD_SELF_FIRST = 1
+FOLD_TREE = 2
 
 
 def make_segs(segs):
-    """segs: iterable of (count, [src addresses], [dst addresses]) -> ctypes array of hcclx_seg_t."""
+    """segs: iterable of (count, [src addresses], [dst addresses][, tree program]) -> ctypes array of
+    hcclx_seg_t.  The tree program is a flat list dst0, src0, dst1, src1, ... (FOLD_TREE only)."""
     segs = list(segs)
     arr = (Seg * max(1, len(segs)))()
-    for i, (count, srcs, dsts) in enumerate(segs):
+    for i, seg in enumerate(segs):
+        count, srcs, dsts = seg[0], seg[1], seg[2]
+        for k, b in enumerate((seg[3] if len(seg) > 3 else [])[:2 * _lib.MAX_FAN]):
+            arr[i].prog[k] = b
         arr[i].count = count
         arr[i].nsrc = len(srcs)
         arr[i].ndst = len(dsts)

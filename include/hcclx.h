@@ -41,7 +41,13 @@ typedef enum {
     /* nsrc == ndst; dst[j] = fold that starts from src[j] and then takes src[k], k ascending, k != j:
      * the per-rank order of the one-shot AllReduce and of the CPU-reduce NHR AllReduce
      * (ins_temp_all_reduce_mesh_1D_one_shot.cc:182-197, ins_temp_all_reduce_aicpu_reduce_nhr.cc:226-233). */
-    HCCLX_FOLD_SELF_FIRST = 1
+    HCCLX_FOLD_SELF_FIRST = 1,
+    /* A binary tree over the sources, for schedules that no chain reproduces (the NHR and recursive
+     * halving-doubling reduce-scatter phases, ins_temp_all_reduce_nhr.cc:183-243).  Registers 0 .. nsrc-1
+     * start as src[0 .. nsrc-1]; step t does  reg[prog[2t]] = reg[prog[2t+1]] (+) reg[prog[2t]];  there are
+     * nsrc-1 steps, every register but 0 is consumed exactly once as a source, and register 0 holds the
+     * result, which goes to dst[0 .. ndst-1]. */
+    HCCLX_FOLD_TREE = 2
 } hcclx_fold_mode_t;
 
 /* One contiguous run of `count` elements: nsrc sources (fold order), ndst destinations.
@@ -53,6 +59,7 @@ typedef struct {
     uint32_t ndst;
     const void *src[HCCLX_MAX_FAN];
     void *dst[HCCLX_MAX_FAN];
+    uint8_t prog[2 * HCCLX_MAX_FAN]; /* HCCLX_FOLD_TREE only: (dst register, src register) per step */
 } hcclx_seg_t;
 
 /* Library set-up for the current device: creates the descriptor arena.  Idempotent.  Called lazily by the

@@ -85,6 +85,96 @@ def test_self_first_in_place_allreduce():
         assert_same_bits(bufs[r].get(np.float32), fold_oracle(xs, T.FP32, T.SUM, order, False), T.FP32)
 
 
+def random_tree(rng, nsrc, max_levels=4):
+    """A random (dst register, src register) program over nsrc registers whose tree has at most
+    max_levels levels, register 0 holding the root."""
+    while True:
+        depth = {k: 0 for k in range(nsrc)}
+        prog = []
+        for _ in range(nsrc - 1):
+            live = list(depth)
+            pairs = [(d, s) for d in live for s in live
+                     if d != s and s != 0 and max(depth[d], depth[s]) + 1 <= max_levels]
+            if not pairs:
+                break
+            d, s = pairs[rng.integers(len(pairs))]
+            depth[d] = max(depth[d], depth[s]) + 1
+            del depth[s]
+            prog += [d, s]
+        if len(prog) == 2 * (nsrc - 1):
+            return prog
+
+
+def tree_oracle(xs, dtype, op, prog, wide):
+    if wide:
+        regs = [T.widen16(x, dtype) for x in xs]
+        e = T.NumericElems(T.FP32, op)
+    else:
+        regs = [np.ascontiguousarray(x).copy() for x in xs]
+        e = T.NumericElems(dtype, op)
+    for t in range(len(prog) // 2):
+        d, s = prog[2 * t], prog[2 * t + 1]
+        e.reduce(regs[d], 0, regs[s], 0, regs[d].size)
+    return T.narrow16(regs[0], dtype) if wide else regs[0]
+
+
+@pytest.mark.parametrize("nsrc", [2, 3, 4, 5, 7, 8, 11, 12, 16])
+@pytest.mark.parametrize("dtype,op", [(T.FP32, T.SUM), (T.FP32, T.MAX), (T.BFP16, T.SUM), (T.FP16, T.PROD),
+                                      (T.FP64, T.SUM), (T.INT32, T.SUM), (T.FP16, T.MIN)])
+def test_tree_fold_keeps_the_association_of_the_program(nsrc, dtype, op):
+    """Log-step schedules (NHR, halving-doubling) pair partial results with partial results; the tree
+    mode evaluates exactly that pairing, operand order included."""
+    rng = np.random.default_rng(nsrc * 31 + dtype * 5 + op)
+    kind = "prod" if op == T.PROD else "uniform" if dtype in (T.FP32, T.FP64) else "normal"
+    segs, cases = [], []
+    for count in (4096 * 3 + 7, 1, 1000):
+        xs = [payload(rng, dtype, count, kind) for _ in range(nsrc)]
+        prog = random_tree(rng, nsrc)
+        bufs = [DevBuf(x) for x in xs]
+        outs = [DevBuf(nbytes=xs[0].nbytes) for _ in range(2)]
+        segs.append((count, [b.ptr for b in bufs], [o.ptr for o in outs], prog))
+        cases.append((xs, prog, bufs, outs))
+    hcclx.fold(segs, dtype, op, hcclx.FOLD_TREE)
+    sync()
+    for xs, prog, bufs, outs in cases:
+        want = tree_oracle(xs, dtype, op, prog, fused_is_wide(dtype, op))
+        for o in outs:
+            assert_same_bits(o.get(T.NP_STORAGE[dtype]), want, dtype, f"program {prog}")
+            assert o.guard_intact()
+
+
+def test_tree_fold_in_place_and_chain_shaped_program():
+    """The result may overwrite register 0's source; a left-deep program of up to four steps equals the
+    chain fold of the same order."""
+    rng = np.random.default_rng(77)
+    n = 30011
+    xs = [payload(rng, T.FP32, n, "uniform") for _ in range(5)]
+    bufs = [DevBuf(x) for x in xs]
+    prog = [0, 1, 0, 2, 0, 3, 0, 4]
+    hcclx.fold([(n, [b.ptr for b in bufs], [bufs[0].ptr], prog)], T.FP32, T.SUM, hcclx.FOLD_TREE)
+    sync()
+    assert_same_bits(bufs[0].get(np.float32), fold_oracle(xs, T.FP32, T.SUM, [0, 1, 2, 3, 4], False), T.FP32)
+
+
+def test_tree_fold_rejects_what_the_kernel_cannot_hold():
+    b = DevBuf(nbytes=64)
+    deep = [0, 1, 0, 2, 0, 3, 0, 4, 0, 5]     # five levels
+    with pytest.raises(HcclError) as e:
+        hcclx.fold([(4, [b.ptr] * 6, [b.ptr], deep)], T.FP32, T.SUM, hcclx.FOLD_TREE)
+    assert e.value.code == 5
+    for bad in ([1, 0, 1, 2], [0, 1, 0, 1], [0, 3, 0, 1], [0, 1, 1, 2]):   # consumes 0 / twice / out of range / dead dst
+        with pytest.raises(HcclError) as e:
+            hcclx.fold([(4, [b.ptr] * 3, [b.ptr], bad)], T.FP32, T.SUM, hcclx.FOLD_TREE)
+        assert e.value.code == 1, bad
+    # integers are association-free: any well-formed program is taken, however deep
+    x = np.arange(16, dtype=np.int32)
+    bufs = [DevBuf(x + k) for k in range(6)]
+    out = DevBuf(nbytes=64)
+    hcclx.fold([(16, [q.ptr for q in bufs], [out.ptr], deep)], T.INT32, T.SUM, hcclx.FOLD_TREE)
+    sync()
+    assert np.array_equal(out.get(np.int32), 6 * x + 15)
+
+
 def test_fp32_subnormals_and_signed_zeros_survive():
     a = np.array([1e-45, -1e-45, 1e-39, 0.0, -0.0, 3e-39, 1.17549435e-38] * 37, dtype=np.float32)
     b = np.array([1e-45, 1e-45, -2e-39, -0.0, -0.0, 3e-39, -1e-45] * 37, dtype=np.float32)

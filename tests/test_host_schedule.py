@@ -119,10 +119,10 @@ def test_reduce_scatter_values_with_executor_chunks(alg):
 
 
 def test_which_templates_fuse():
-    """Chains (and every integer schedule) become fused passes; floating-point trees do not."""
+    """Chains, every integer schedule and floating-point trees of up to four levels become fused passes."""
     for alg, dtype, fused in [("InsAllReduceMesh1DOneShot", T.FP32, 1), ("InsAllReduceMesh1DTwoShot", T.FP32, 1),
                               ("InsAllReduceAicpuReduceNHR", T.FP32, 1), ("InsAllReduceRing", T.FP32, 1),
-                              ("InsAllReduceNHR", T.FP32, 0), ("InsAllReduceRHD", T.FP32, 0),
+                              ("InsAllReduceNHR", T.FP32, 1), ("InsAllReduceRHD", T.FP32, 1),
                               ("InsAllReduceNHR", T.INT32, 1), ("InsAllReduceRHD", T.INT32, 1)]:
         _, info = dry_allreduce(12, 1200, dtype, T.SUM, alg)
         assert info.fused == fused, alg
@@ -130,8 +130,11 @@ def test_which_templates_fuse():
     # the one-shot order of all 12 ranks is one segment: 12 sources read once, 12 outputs
     _, info = dry_allreduce(12, 1200, T.FP32, T.SUM, "InsAllReduceMesh1DOneShot")
     assert info.fusedSegments == 1
-    # float max keeps operand order: the ring's "acc (+) leaf" steps are not swapped into a chain
+    # float max keeps operand order: the ring's "acc (+) leaf" steps are not swapped into a chain.  With 4
+    # ranks the 3-level tree still fits the tree kernel; with 12 ranks (11 levels) the steps run one by one
     _, info = dry_allreduce(4, 64, T.FP32, T.MAX, "InsAllReduceRing")
+    assert info.fused == 1
+    _, info = dry_allreduce(12, 1200, T.FP32, T.MAX, "InsAllReduceRing")
     assert info.fused == 0
 
 
