@@ -4,7 +4,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libhccl_amd.so")
+# HCCL_AMD_LIBRARY names another build of the same library (e.g. one with different tile parameters)
+LIB_PATH = os.environ.get("HCCL_AMD_LIBRARY") or os.path.join(_HERE, "lib", "libhccl_amd.so")
 
 MAX_FAN = 16
 

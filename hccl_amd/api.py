@@ -9,6 +9,7 @@ from ._lib import HcclError
 EXEC_FUSED, EXEC_STEP = 0, 1
 CMD_ALLREDUCE, CMD_ALLGATHER, CMD_REDUCE_SCATTER, CMD_ALLTOALLV, CMD_ALLTOALLVC, CMD_ALLTOALL, CMD_ALLGATHER_V = \
     2, 6, 7, 8, 9, 10, 16
+CMD_REDUCE_SCATTER_V = 17
 SHAPE_CLOS, SHAPE_MESH_1D = 0, 1
 
 
@@ -39,6 +40,7 @@ def lib():
             "hcclxCommSetTrace": [vp, ci],
             "HcclAllReduce": [vp, vp, u64, ci, ci, vp, vp],
             "HcclReduceScatter": [vp, vp, u64, ci, ci, vp, vp],
+            "HcclReduceScatterV": [vp, vp, vp, vp, u64, ci, ci, vp, vp],
             "HcclAllGather": [vp, vp, u64, ci, vp, vp],
             "HcclAllGatherV": [vp, u64, vp, vp, vp, ci, vp, vp],
             "HcclAlltoAllV": [vp, vp, vp, ci, vp, vp, vp, ci, vp, vp],
@@ -117,6 +119,11 @@ class World:
 
     def reduce_scatter(self, rank, send, recv, recv_count, dtype, op, stream):
         return lib().HcclReduceScatter(send, recv, recv_count, int(dtype), int(op), self.comms[rank], stream)
+
+    def reduce_scatter_v(self, rank, send, counts, displs, recv, recv_count, dtype, op, stream):
+        c, d = _u64(counts), _u64(displs)
+        return lib().HcclReduceScatterV(send, ctypes.cast(c, ctypes.c_void_p), ctypes.cast(d, ctypes.c_void_p), recv,
+                                        recv_count, int(dtype), int(op), self.comms[rank], stream)
 
     def all_gather(self, rank, send, recv, send_count, dtype, stream):
         return lib().HcclAllGather(send, recv, send_count, int(dtype), self.comms[rank], stream)

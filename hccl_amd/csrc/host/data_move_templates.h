@@ -1,4 +1,4 @@
-// ReduceScatter, AllGather, AllGatherV and AlltoAllV templates: see the .cc files for what each restates.
+// ReduceScatter, ReduceScatterV, AllGather, AllGatherV and AlltoAllV templates: see the .cc files for what each restates.
 #pragma once
 #include "all_reduce_templates.h"
 
@@ -9,6 +9,9 @@ namespace ops_hccl {
 HCCL_DECLARE_TEMPLATE(InsTempReduceScatterMesh1D, "ReduceScatter mesh 1D",
                       (templateRankSize_ > 1 ? templateRankSize_ : 1), templateRankSize_);
 HCCL_DECLARE_TEMPLATE(InsTempReduceScatterNHR, "ReduceScatter NHR", 1, templateRankSize_);
+// reduce_scatter_v mesh_1D.cc:26-48: N-1 threads (the main thread sends too), N scratch slots
+HCCL_DECLARE_TEMPLATE(InsTempReduceScatterVMesh1D, "ReduceScatterV mesh 1D",
+                      (templateRankSize_ > 1 ? templateRankSize_ - 1 : 1), templateRankSize_);
 HCCL_DECLARE_TEMPLATE(InsTempAllGatherMesh1D, "AllGather mesh 1D",
                       (templateRankSize_ > 1 ? templateRankSize_ - 1 : 1), templateRankSize_);
 HCCL_DECLARE_TEMPLATE(InsTempAllGatherNHR, "AllGather NHR", 1, templateRankSize_);

@@ -263,6 +263,63 @@ public:
 };
 
 // ---------------------------------------------------------------------------------------------------
+// ReduceScatterV (src/ops/reduce_scatter_v/executor/ins_v2_reduce_scatter_v_sole_executor.cc:75-170)
+// ---------------------------------------------------------------------------------------------------
+template <typename AlgTopoMatch, typename InsAlgTemplate>
+class InsV2ReduceScatterVSoleExecutor : public InsCollAlgBase {
+public:
+    std::string Describe() const override { return "ReduceScatterV sole executor"; }
+    u64 CalcThreadNum(const OpParam &param, u32 rank, u32 rankSize) override
+    {
+        InsAlgTemplate t(param, rank, AlgTopoMatch::Match(rankSize));
+        return t.GetThreadNum();
+    }
+    HcclResult Orchestrate(const OpParam &param, const AlgResourceCtxSerializable &resCtx) override
+    {
+        myRank_ = resCtx.topoInfo.userRank;
+        rankSize_ = resCtx.topoInfo.userRankSize;
+        dataType_ = param.vDataDes.dataType;
+        dataTypeSize_ = DATATYPE_SIZE_TABLE[dataType_];
+        TemplateResource res;
+        TemplateDataParams t;
+        FillBuffInfo(param, resCtx, t, res);
+        t.repeatNum = 1;
+        t.inputRepeatStride = 0;
+        t.outputRepeatStride = 0;
+        const std::vector<u64> &counts = param.vDataDes.counts;
+        t.allRankDispls = param.vDataDes.displs;
+        for (u64 &d : t.allRankDispls) d *= dataTypeSize_;
+        InsAlgTemplate alg(param, myRank_, resCtx.subCommRanks);
+        const u64 mult = alg.CalcScratchMultiple(t.buffInfo.inBuffType, t.buffInfo.outBuffType);
+        maxTmpMemSize_ = t.buffInfo.hcclBuff.size;
+        const u64 maxCount = MaxDataSizePerLoop(maxTmpMemSize_, mult, UB_MAX_DATA_SIZE) / dataTypeSize_;
+        CHK_PRT_RET(maxCount == 0, HCCL_ERROR("[ReduceScatterV executor] maxDataCountPerLoop is 0"), HCCL_E_INTERNAL);
+        u64 maxRecv = 0;
+        for (u32 i = 0; i < rankSize_; ++i) maxRecv = std::max(maxRecv, counts[i]);
+        if (maxRecv == 0) return HCCL_SUCCESS;   // the op entry returns before it gets here
+        const u64 loops = 1 + ((maxRecv - 1) / maxCount);
+        u64 processed = 0;
+        t.allRankSliceSize.assign(rankSize_, 0);
+        for (u64 loop = 0; loop < loops; ++loop) {
+            u64 largest = 0;
+            for (u32 i = 0; i < rankSize_; ++i) {
+                const u64 left = processed < counts[i] ? std::min(maxCount, counts[i] - processed) : 0;
+                t.allRankSliceSize[i] = left * dataTypeSize_;
+                largest = std::max(largest, left);
+            }
+            // every rank's part advances by the same element offset
+            t.buffInfo.inBuffBaseOff = processed * dataTypeSize_;
+            t.buffInfo.outBuffBaseOff = processed * dataTypeSize_;
+            t.buffInfo.hcclBuffBaseOff = 0;
+            t.outputSliceStride = maxCount * dataTypeSize_;
+            CHK_RET(alg.KernelRun(param, t, res));
+            processed += largest;
+        }
+        return HCCL_SUCCESS;
+    }
+};
+
+// ---------------------------------------------------------------------------------------------------
 // AlltoAll / AlltoAllV / AlltoAllVC (src/ops/all_to_all_v/executor/ins_v2_all_to_all_v_sole_executor.cc:183-368)
 // ---------------------------------------------------------------------------------------------------
 template <typename AlgTopoMatch, typename InsAlgTemplate> class InsV2AlltoAllVSoleExecutor : public InsCollAlgBase {
@@ -354,6 +411,8 @@ REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_ALLGATHER, InsAllGatherMesh1D, InsV2AllGa
                  InsTempAllGatherMesh1D);
 REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_ALLGATHER, InsAllGatherNHR, InsV2AllGatherSoleExecutor, TopoMatch1D,
                  InsTempAllGatherNHR);
+REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_REDUCE_SCATTER_V, InsReduceScatterVMesh1D, InsV2ReduceScatterVSoleExecutor,
+                 TopoMatch1D, InsTempReduceScatterVMesh1D);
 REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_ALLGATHER_V, InsAllGatherVMesh1D, InsV2AllGatherVSoleExecutor, TopoMatch1D,
                  InsTempAllGatherVMesh1D);
 REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_ALLTOALLV, InsAlltoAllVMesh1D, InsV2AlltoAllVSoleExecutor, TopoMatch1D,

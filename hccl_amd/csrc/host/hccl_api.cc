@@ -3,6 +3,7 @@
 // Check order and error codes follow the reference's op files:
 //   HcclAllReduce      src/ops/all_reduce/all_reduce_op.cc:23-56, :106-178
 //   HcclReduceScatter  src/ops/reduce_scatter/reduce_scatter_op.cc:23, :180
+//   HcclReduceScatterV src/ops/reduce_scatter_v/reduce_scatter_v_op.cc:24-72, :142-167, :169-222
 //   HcclAllGather      src/ops/all_gather/all_gather_op.cc:24, :167
 //   HcclAllGatherV     src/ops/all_gather_v/all_gather_v_op.cc:22-67, :140-262
 //   HcclAlltoAll[V|VC] src/ops/all_to_all_v/all_to_all_v_op.cc:84-142, :385-430, :470-500
@@ -289,6 +290,45 @@ HcclResult HcclReduceScatter(void *sendBuf, void *recvBuf, uint64_t recvCount, H
     p.DataDes.count = recvCount;
     p.DataDes.dataType = dataType;
     if (rc->world->rankSize == 1) return SingleRankProc(p, p.outputSize, rc->world);
+    return SubmitOp(rc, p);
+}
+
+HcclResult HcclReduceScatterV(void *sendBuf, const void *sendCounts, const void *sendDispls, void *recvBuf,
+                              uint64_t recvCount, HcclDataType dataType, HcclReduceOp op, HcclComm comm,
+                              aclrtStream stream)
+{
+    CHK_PTR_NULL(stream);
+    CHK_PTR_NULL(comm);
+    CHK_PTR_NULL(sendCounts);
+    CHK_PTR_NULL(sendDispls);
+    if (recvCount > 0) CHK_PTR_NULL(recvBuf);
+    RankComm *rc = AsRankComm(comm);
+    CHK_PTR_NULL(rc);
+    const u32 n = rc->world->rankSize;
+    const u64 *counts = static_cast<const u64 *>(sendCounts);
+    const u64 *displs = static_cast<const u64 *>(sendDispls);
+    if (std::all_of(counts, counts + n, [](u64 c) { return c == 0; })) return HCCL_SUCCESS;
+    CHK_RET(CheckCount(recvCount));
+    CHK_RET(CheckDataType(dataType, true));
+    CHK_RET(CheckReduceOp(dataType, op));
+    // The reference trusts these two; here a wrong value would make a kernel read or write out of bounds.
+    CHK_PTR_NULL(sendBuf);
+    CHK_PRT_RET(counts[rc->rank] != recvCount, HCCL_ERROR("[HcclReduceScatterV] recvCount != sendCounts[rank]"),
+                HCCL_E_PARA);
+    OpParam p;
+    FillCommon(p, rc, "ReduceScatterV", HcclCMDType::HCCL_CMD_REDUCE_SCATTER_V, stream, sendBuf, recvBuf);
+    const u64 esz = DATATYPE_SIZE_TABLE[dataType];
+    p.reduceType = op;
+    p.vDataDes.counts.assign(counts, counts + n);
+    p.vDataDes.displs.assign(displs, displs + n);
+    p.vDataDes.dataType = dataType;
+    p.DataDes.dataType = dataType;
+    p.DataDes.count = recvCount;
+    u64 inElems = 0;
+    for (u32 i = 0; i < n; ++i) inElems = std::max(inElems, displs[i] + counts[i]);
+    p.inputSize = inElems * esz;
+    p.outputSize = recvCount * esz;
+    if (n == 1) return SingleRankProc(p, counts[0] * esz, rc->world);
     return SubmitOp(rc, p);
 }
 

@@ -2,6 +2,8 @@
 // (src/ops/reduce_scatter/template/aicpu/):
 //   InsTempReduceScatterMesh1D   ins_temp_reduce_scatter_mesh_1D.cc:65-227
 //   InsTempReduceScatterNHR      ins_temp_reduce_scatter_nhr.cc:77-425
+// and src/ops/reduce_scatter_v/template/aicpu/:
+//   InsTempReduceScatterVMesh1D  ins_temp_reduce_scatter_v_mesh_1D.cc:50-179
 #include "data_move_templates.h"
 
 namespace ops_hccl {
@@ -140,6 +142,66 @@ HcclResult InsTempReduceScatterNHR::KernelRun(const OpParam &param, const Templa
     const u64 size = sizeOf(me);
     return LocalCopy(th, DataSlice(ccl, p.buffInfo.hcclBuffBaseOff + p.sliceSize * me, size),
                      DataSlice(p.buffInfo.outputPtr, p.buffInfo.outBuffBaseOff + me * p.outputSliceStride, size));
+}
+
+// Ragged mesh ReduceScatter: rank k owns allRankSliceSize[k] bytes at allRankDispls[k] of every input.
+// Every rank writes its part for rank k into slot <own rank> of rank k's scratch (slots are
+// outputSliceStride apart); rank k copies its own part to the output and folds the other slots in,
+// ranks ascending.  The main thread takes the first peer itself, so N - 1 threads are used.
+HcclResult InsTempReduceScatterVMesh1D::KernelRun(const OpParam &param, const TemplateDataParams &p,
+                                                  TemplateResource &res)
+{
+    threadNum_ = static_cast<u32>(GetThreadNum());
+    CHK_PRT_RET(res.threads.size() < threadNum_, HCCL_ERROR("[RSV mesh] thread num is invalid"), HCCL_E_INTERNAL);
+    dataType_ = param.vDataDes.dataType;
+    const u64 esz = DATATYPE_SIZE_TABLE[dataType_];
+    const u32 n = templateRankSize_;
+    CHK_PRT_RET(p.allRankSliceSize.size() != n || p.allRankDispls.size() != n,
+                HCCL_ERROR("[RSV mesh] slice tables do not match the rank size"), HCCL_E_INTERNAL);
+    u32 me = 0;
+    CHK_RET(GetAlgRank(myRank_, subCommRanks_[0], me));
+    std::vector<ThreadHandle> threads(res.threads.begin(), res.threads.begin() + threadNum_);
+
+    CHK_RET(PreSync(threads));
+    for (u32 que = 0; que < threadNum_ && n > 1; ++que) {
+        const u32 next = (me + 1 + que) % n;
+        const ChannelInfo &link = res.channels.at(subCommRanks_[0][next])[0];
+        const u64 size = p.allRankSliceSize[next];
+        std::vector<DataSlice> txSrc, txDst, rxSrc, rxDst;
+        for (u64 rpt = 0; rpt < p.repeatNum; ++rpt) {
+            txSrc.emplace_back(p.buffInfo.inputPtr,
+                               p.buffInfo.inBuffBaseOff + rpt * p.inputRepeatStride + p.allRankDispls[next], size,
+                               size / esz);
+            txDst.emplace_back(link.remoteCclMem.addr,
+                               p.buffInfo.hcclBuffBaseOff + rpt * p.outputRepeatStride + me * p.outputSliceStride, size,
+                               size / esz);
+        }
+        SendRecvInfo info{{link, link}, {{txSrc, txDst}, {rxSrc, rxDst}}, dataType_};
+        CHK_RET(SendRecvWrite(info, threads[que]));
+    }
+    CHK_RET(PostSync(threads));
+
+    const u64 size = p.allRankSliceSize[me];
+    const u64 count = size / esz;
+    for (u64 rpt = 0; rpt < p.repeatNum; ++rpt) {
+        DataSlice dst(p.buffInfo.outputPtr, p.buffInfo.outBuffBaseOff + rpt * p.outputRepeatStride, size, count);
+        DataSlice own(p.buffInfo.inputPtr,
+                      p.buffInfo.inBuffBaseOff + rpt * p.inputRepeatStride + p.allRankDispls[me], size, count);
+        CHK_RET(LocalCopy(threads[0], own, dst));
+        // the CPU reduce loop runs on the host: flush what was queued so far (mesh_1D.cc:103-108)
+        if (dataType_ == HCCL_DATA_TYPE_INT64 || reduceOp_ == HCCL_REDUCE_PROD) {
+            CHK_RET(HcommBatchModeEnd(param.algTag.c_str()));
+            CHK_RET(HcommBatchModeStart(param.algTag.c_str()));
+            for (ThreadHandle t : threads) CHK_RET(HcommThreadJoin(t, CUSTOM_TIMEOUT));
+        }
+        for (u32 k = 0; k < n; ++k) {
+            if (k == me) continue;
+            DataSlice src(p.buffInfo.hcclBuff.addr,
+                          p.buffInfo.hcclBuffBaseOff + rpt * p.outputRepeatStride + k * p.outputSliceStride, size, count);
+            CHK_RET(LocalReduce(threads[0], src, dst, dataType_, reduceOp_));
+        }
+    }
+    return HCCL_SUCCESS;
 }
 
 }  // namespace ops_hccl

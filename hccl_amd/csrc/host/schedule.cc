@@ -559,6 +559,8 @@ std::string PlanKey(const std::vector<OpParam> &params, const std::string &alg, 
     const OpParam &p0 = params[0];
     os << static_cast<int>(p0.opType) << "|" << alg << "|" << p0.DataDes.dataType << "|" << p0.reduceType << "|"
        << p0.DataDes.count << "|" << cclBytes;
+    for (u64 c : p0.vDataDes.counts) os << "|c" << c;
+    for (u64 d : p0.vDataDes.displs) os << "|d" << d;
     for (const OpParam &p : params) os << "|" << p.inputPtr << "," << p.outputPtr << "," << p.inputSize;
     return os.str();
 }
@@ -587,6 +589,9 @@ bool SameOperands(const OpParam &a, const OpParam &b)
         case HcclCMDType::HCCL_CMD_ALLGATHER_V:
             return a.vDataDes.dataType == b.vDataDes.dataType && a.vDataDes.counts == b.vDataDes.counts &&
                    a.vDataDes.displs == b.vDataDes.displs;
+        case HcclCMDType::HCCL_CMD_REDUCE_SCATTER_V:
+            return a.vDataDes.dataType == b.vDataDes.dataType && a.vDataDes.counts == b.vDataDes.counts &&
+                   a.vDataDes.displs == b.vDataDes.displs && a.reduceType == b.reduceType;
         default:
             return a.all2AllVDataDes.sendType == b.all2AllVDataDes.sendType;
     }

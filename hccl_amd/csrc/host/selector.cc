@@ -131,6 +131,21 @@ protected:
     }
 };
 
+// ---- ReduceScatterV (src/ops/reduce_scatter_v/selector/reduce_scatter_v_auto_selector.cc:204-220): the mesh
+//      template for one to three topology levels; uint64 and fp64 have no AICPU algorithm
+class ReduceScatterVAutoSelector : public AutoSelectorBase {
+protected:
+    SelectorStatus SelectAicpuAlgo(const TopoInfoWithNetLayerDetails *topo, const OpParam &p,
+                                   std::string &name) const override
+    {
+        const HcclDataType dt = p.vDataDes.dataType;
+        if (dt == HCCL_DATA_TYPE_UINT64 || dt == HCCL_DATA_TYPE_FP64) return SelectorStatus::NOT_MATCH;
+        if (topo->topoLevelNums < 1 || topo->topoLevelNums > 3) return SelectorStatus::NOT_MATCH;
+        name = "InsReduceScatterVMesh1D";
+        return SelectorStatus::MATCH;
+    }
+};
+
 // ---- AlltoAll family (src/ops/all_to_all_v/selector/alltoallv_auto_selector.cc:94-128,
 //      alltoall_auto_selector.cc:111-154, alltoallvc_auto_selector.cc:53-62) -------------------------------
 template <int KIND> class AlltoAllFamilySelector : public AutoSelectorBase {
@@ -152,6 +167,7 @@ using AlltoAllVCAutoSelector = AlltoAllFamilySelector<2>;
 
 REGISTER_SELECTOR_BY_OPTYPE(HcclCMDType::HCCL_CMD_ALLREDUCE, SELECTOR_PRIORITY_BUILTIN, AllReduceAutoSelector);
 REGISTER_SELECTOR_BY_OPTYPE(HcclCMDType::HCCL_CMD_REDUCE_SCATTER, SELECTOR_PRIORITY_BUILTIN, ReduceScatterAutoSelector);
+REGISTER_SELECTOR_BY_OPTYPE(HcclCMDType::HCCL_CMD_REDUCE_SCATTER_V, SELECTOR_PRIORITY_BUILTIN, ReduceScatterVAutoSelector);
 REGISTER_SELECTOR_BY_OPTYPE(HcclCMDType::HCCL_CMD_ALLGATHER, SELECTOR_PRIORITY_BUILTIN, AllGatherAutoSelector);
 REGISTER_SELECTOR_BY_OPTYPE(HcclCMDType::HCCL_CMD_ALLGATHER_V, SELECTOR_PRIORITY_BUILTIN, AllGatherVAutoSelector);
 REGISTER_SELECTOR_BY_OPTYPE(HcclCMDType::HCCL_CMD_ALLTOALL, SELECTOR_PRIORITY_BUILTIN, AlltoAllAutoSelector);

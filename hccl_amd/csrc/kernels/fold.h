@@ -17,13 +17,21 @@ namespace hcclx {
 
 // 16-byte vectors each thread keeps in flight per source.  More sources -> fewer vectors per source, so
 // the loads outstanding per thread stay near 16 and the register file still holds several wavefronts.
+#ifndef HCCLX_FOLD_UNROLLS
+#define HCCLX_FOLD_UNROLLS 8, 4, 4, 2, 1   // for up to 1, 2, 4, 8, 16 sources
+#endif
+#ifndef HCCLX_FOLD_THREADS
+#define HCCLX_FOLD_THREADS 256
+#endif
+constexpr int kFoldThreads = HCCLX_FOLD_THREADS;
 __host__ __device__ constexpr int fold_unroll(int maxn)
 {
-    return maxn <= 1 ? 8 : maxn <= 4 ? 4 : maxn <= 8 ? 2 : 1;
+    constexpr int u[5] = {HCCLX_FOLD_UNROLLS};
+    return maxn <= 1 ? u[0] : maxn <= 2 ? u[1] : maxn <= 4 ? u[2] : maxn <= 8 ? u[3] : u[4];
 }
 __host__ __device__ constexpr uint64_t fold_tile_vecs(int maxn)
 {
-    return static_cast<uint64_t>(kThreads) * fold_unroll(maxn);
+    return static_cast<uint64_t>(kFoldThreads) * fold_unroll(maxn);
 }
 
 __device__ __forceinline__ u32x4 ld16(const char *p)
@@ -81,8 +89,8 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
             const char *p = sd.src[k] + v0 * 16;
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
-                if (!CHECK || v0 + static_cast<uint64_t>(u) * kThreads < nvec) {
-                    raw[u][k] = ld16(p + static_cast<uint64_t>(u) * kThreads * 16);
+                if (!CHECK || v0 + static_cast<uint64_t>(u) * kFoldThreads < nvec) {
+                    raw[u][k] = ld16(p + static_cast<uint64_t>(u) * kFoldThreads * 16);
                 }
             }
         }
@@ -90,7 +98,7 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
 
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-        const uint64_t vi = v0 + static_cast<uint64_t>(u) * kThreads;
+        const uint64_t vi = v0 + static_cast<uint64_t>(u) * kFoldThreads;
         if (CHECK && vi >= nvec) {
             continue;
         }
@@ -186,13 +194,13 @@ __device__ __forceinline__ void fold_tail(const SegDev &sd, uint32_t nsrc, uint3
 }
 
 template <int DT, int OP, int MAXN, int MODE>
-__global__ void __launch_bounds__(kThreads)
+__global__ void __launch_bounds__(kFoldThreads)
 k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, uint32_t nseg, uint64_t total_tiles)
 {
     constexpr int NE = Vec16<DT>::NE;
     constexpr uint64_t TV = fold_tile_vecs(MAXN);
     extern __shared__ uint64_t s_end[];  // nseg entries, sized by the launcher
-    for (uint32_t i = threadIdx.x; i < nseg; i += kThreads) {
+    for (uint32_t i = threadIdx.x; i < nseg; i += kFoldThreads) {
         s_end[i] = tile_end[i];
     }
     __syncthreads();

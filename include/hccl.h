@@ -32,6 +32,12 @@ extern HcclResult HcclAllReduce(void *sendBuf, void *recvBuf, uint64_t count, Hc
 extern HcclResult HcclReduceScatter(void *sendBuf, void *recvBuf, uint64_t recvCount, HcclDataType dataType,
     HcclReduceOp op, HcclComm comm, aclrtStream stream);
 
+/* reference include/hccl.h:85-86.  Ragged ReduceScatter: rank r receives the reduction of every rank's
+ * sendBuf[sendDispls[r] .. +sendCounts[r]); recvCount == sendCounts[own rank].  sendCounts / sendDispls are
+ * host uint64_t[rankSize] in elements, the same on every rank. */
+extern HcclResult HcclReduceScatterV(void *sendBuf, const void *sendCounts, const void *sendDispls,
+    void *recvBuf, uint64_t recvCount, HcclDataType dataType, HcclReduceOp op, HcclComm comm, aclrtStream stream);
+
 /* reference include/hccl.h:116-117.  recvBuf holds rankSize * sendCount elements. */
 extern HcclResult HcclAllGather(void *sendBuf, void *recvBuf, uint64_t sendCount, HcclDataType dataType,
     HcclComm comm, aclrtStream stream);

@@ -20,6 +20,8 @@ Reference followed (paths relative to the reference tree, src/ops/...):
   allreduce_aicpu_reduce_nhr   all_reduce/template/aicpu/ins_temp_all_reduce_aicpu_reduce_nhr.cc:65-271
   reduce_scatter_mesh          reduce_scatter/template/aicpu/ins_temp_reduce_scatter_mesh_1D.cc:65-227
   reduce_scatter_nhr           reduce_scatter/template/aicpu/ins_temp_reduce_scatter_nhr.cc:77-425
+  reduce_scatter_v_mesh        reduce_scatter_v/template/aicpu/ins_temp_reduce_scatter_v_mesh_1D.cc:50-179,
+                               chunk loop reduce_scatter_v/executor/ins_v2_reduce_scatter_v_sole_executor.cc:75-170
   executor chunk loops         all_reduce/executor/ins_v2_all_reduce_sole_executor.cc:92-185,
                                reduce_scatter/executor/ins_v2_reduce_scatter_sole_executor.cc:123-170
   allreduce_ring, allreduce_rhd  no executable reference exists; defined from the prose of
@@ -472,6 +474,45 @@ def run_reduce_scatter(elems, inputs, recv_count, esz, alg, ccl_bytes=CCL_BYTES_
     usable = ccl_bytes - 1024 * 1024          # ins_v2_reduce_scatter_sole_executor.cc:126-128
     for base, cur in chunk_counts(recv_count, usable, mult(w.n), esz, usable):
         fn(w, base, cur, recv_count)          # inputSliceStride = recvCount * esz (:160)
+    return w.out
+
+
+def reduce_scatter_v_mesh(w, done, sizes, displs, slot):
+    """One chunk of the ragged mesh ReduceScatter: rank k's part is inp[*][displs[k] + done .. +sizes[k]);
+    rank r writes its part for k into slot r of ccl[k] (slots `slot` elements apart); rank k copies its own
+    part to out[k][done ..) and folds the other slots in, ranks ascending."""
+    n, e = w.n, w.e
+    slot = min(slot, max(sizes))      # where a slot sits in the scratch changes no value: keep the buffers small
+    w.need_ccl(slot * n)
+    for r in range(n):                                   # RunReduceScatterV :131-179
+        for q in range(n - 1):
+            k = (r + 1 + q) % n
+            e.copy(w.ccl[k], r * slot, w.inp[r], displs[k] + done, sizes[k])
+    for r in range(n):                                   # PostCopy :79-129
+        e.copy(w.out[r], done, w.inp[r], displs[r] + done, sizes[r])
+        for k in range(n):
+            if k != r:
+                e.reduce(w.out[r], done, w.ccl[r], k * slot, sizes[r])
+
+
+def run_reduce_scatter_v(elems, inputs, counts, displs, esz, ccl_bytes=CCL_BYTES_DEFAULT):
+    """HcclReduceScatterV through its sole executor: every loop takes up to maxDataCountPerLoop elements of
+    every rank's part, all parts advancing by the same offset (sole_executor.cc:133-166)."""
+    n = len(inputs)
+    w = World(elems, inputs, 0, esz, ccl_bytes)
+    w.out = [elems.empty(counts[r]) for r in range(n)]
+    max_bytes = min(UB_MAX_DATA_SIZE, ccl_bytes // n // HCCL_MIN_SLICE_ALIGN * HCCL_MIN_SLICE_ALIGN)
+    max_count = max_bytes // esz
+    if max_count == 0:
+        raise ValueError("maxDataCountPerLoop is 0")
+    biggest = max(counts)
+    if biggest == 0:
+        return w.out
+    done = 0
+    for _ in range(1 + (biggest - 1) // max_count):
+        sizes = [min(max_count, c - done) if done < c else 0 for c in counts]
+        reduce_scatter_v_mesh(w, done, sizes, displs, max_count)
+        done += max(sizes)
     return w.out
 
 

@@ -72,6 +72,8 @@ def is_nan_bits(a, dtype):
 def assert_same_bits(got, want, dtype, what=""):
     """Bit-exact, except that NaNs only have to be NaNs (their payload is host-FPU specific)."""
     assert got.shape == want.shape, what
+    if got.size == 0:
+        return
     gn, wn = is_nan_bits(got, dtype), is_nan_bits(want, dtype)
     assert np.array_equal(gn, wn), f"{what}: NaN positions differ"
     g = got.view(np.uint8).reshape(got.size, -1)[~gn]

@@ -155,6 +155,52 @@ def test_reduce_scatter_both_templates_both_modes(stream, mode, alg, dtype, op, 
         w.close()
 
 
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("dtype,op,counts", [
+    (T.FP32, T.SUM, [100, 100, 100, 100, 100, 100, 100, 100, 500, 500]),       # reduce_scatter_v_testcase.cc:131-141
+    (T.INT8, T.SUM, [700, 700, 600, 600, 500, 500, 400, 400, 300, 300, 200, 200, 100, 100]),   # :120-129
+    (T.BFP16, T.SUM, [120001, 0, 7, 65536, 33333, 1, 250000, 4096]),
+    (T.INT64, T.MIN, [30000, 5, 0, 70001]),
+    (T.FP16, T.PROD, [50000, 20001, 3])])
+def test_reduce_scatter_v_ragged(stream, mode, dtype, op, counts):
+    """HcclReduceScatterV: ragged parts with gaps between them, zero-length parts, several executor loops."""
+    n = len(counts)
+    rng = np.random.default_rng(sum(counts))
+    displs, off = [], 3
+    for c in counts:
+        displs.append(off)
+        off += c + 5
+    xs = [payload(rng, dtype, off, "prod" if op == T.PROD else "normal") for _ in range(n)]
+    esz = T.DTYPE_SIZE[dtype]
+    w = api.World(n, ccl_bytes=SMALL_CCL)
+    try:
+        w.set_mode(mode)
+        send = [DevBuf(x) for x in xs]
+        recv = [DevBuf(nbytes=max(counts[r], 1) * esz) for r in range(n)]
+        torch.cuda.synchronize()
+        for r in range(n):
+            assert w.reduce_scatter_v(r, send[r].ptr, counts, displs, recv[r].ptr, counts[r], dtype, op,
+                                      stream.cuda_stream) == 0
+        stream.synchronize()
+        info = w.last_info()
+        assert info.algName.decode() == "InsReduceScatterVMesh1D"
+        assert info.fused == (1 if mode == api.EXEC_FUSED else 0)
+        if info.fused and dtype in (T.FP16, T.BFP16) and op == T.SUM:
+            wide = [T.widen16(x, dtype) for x in xs]
+            want = [T.narrow16(o, dtype) for o in
+                    T.run_reduce_scatter_v(T.NumericElems(T.FP32, T.SUM), wide, counts, displs, esz, ccl_bytes=SMALL_CCL)]
+        else:
+            want = T.run_reduce_scatter_v(T.NumericElems(dtype, op), xs, counts, displs, esz, ccl_bytes=SMALL_CCL)
+        for r in range(n):
+            got = recv[r].get(T.NP_STORAGE[dtype])[:counts[r]]
+            assert_same_bits(got, want[r], dtype, f"rank {r} fused={info.fused}")
+            if counts[r]:
+                assert recv[r].guard_intact()
+            assert send[r].guard_intact()
+    finally:
+        w.close()
+
+
 def test_reduce_scatter_bf16_within_one_ulp_of_fp32_accumulation(stream):
     """The tolerance the baseline states for 16-bit floats: every output within 1 bf16 ULP of the sum
     accumulated in fp32 (here: in float64, then compared on the bf16 grid)."""

@@ -1,13 +1,18 @@
 """The host runtime without a GPU: op entry -> selector -> executor -> template -> recorded steps ->
 dependency order -> symbolic trace.  The trace of every output is evaluated with the oracle's element
 arithmetic and compared, bit for bit, with the oracle's own restatement of the same template."""
+import json
+import os
+
 import numpy as np
 import pytest
 
 from oracle import templates as T
 from hccl_amd import api
 
-from host_util import (FAKE_STREAM, eval_trace, expr_to_oracle_string, fake_ptrs, parse_expr, parse_trace)
+from host_util import (FAKE_STREAM, eval_expr, eval_trace, expr_to_oracle_string, fake_ptrs, parse_expr, parse_trace)
+
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "st_cases.json")))
 
 SMALL_CCL = 1024 * 1024 + 64 * 1024     # forces several executor chunks at a few thousand elements
 AR_ALGS = list(T.ALLREDUCE_TEMPLATES)
@@ -116,6 +121,74 @@ def test_reduce_scatter_values_with_executor_chunks(alg):
     assert len(T.chunk_counts(rc, SMALL_CCL - (1 << 20), n, 4, SMALL_CCL - (1 << 20))) == 5
     for r in range(n):
         assert np.array_equal(got[r].view(np.uint32), want[r].view(np.uint32))
+
+
+def dry_reduce_scatter_v(counts, displs, dtype, op, ccl=SMALL_CCL):
+    n = len(counts)
+    w = api.World(n, ccl_bytes=ccl, dry=True)
+    try:
+        ins, outs = fake_ptrs(n)
+        for r in range(n):
+            assert w.reduce_scatter_v(r, ins[r], counts, displs, outs[r], counts[r], dtype, op, FAKE_STREAM) == 0
+        return w.last_trace(), w.last_info()
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("case", GOLD["reducescatterv"], ids=lambda c: c["name"])
+def test_reduce_scatter_v_reference_lists_trace_equals_oracle(case):
+    """The reference's own ReduceScatterV shapes (reduce_scatter_v_testcase.cc:64-141): the traced
+    expression of every output element is the oracle's, own rank first then ranks ascending."""
+    counts, displs = case["counts"], case["displs"]
+    dtype = {"int8": T.INT8, "int16": T.INT16, "int32": T.INT32, "fp16": T.FP16, "fp32": T.FP32}[case["dtype"]]
+    esz = T.DTYPE_SIZE[dtype]
+    n = len(counts)
+    text, info = dry_reduce_scatter_v(counts, displs, dtype, T.SUM)
+    assert info.algName.decode() == "InsReduceScatterVMesh1D" and info.fused == 1
+    total = max(d + c for d, c in zip(displs, counts))
+    want = T.run_reduce_scatter_v(T.SymbolicElems(), sym_inputs(n, total), counts, displs, esz, ccl_bytes=SMALL_CCL)
+    seen = [0] * n
+    for rank, off, nbytes, expr in parse_trace(text):
+        tree = parse_expr(expr)
+        for elem in (0, nbytes // esz - 1):
+            assert expr_to_oracle_string(tree, elem, esz, off) == want[rank][off // esz + elem]
+        seen[rank] += nbytes
+    assert seen == [c * esz for c in counts]
+
+
+def test_reduce_scatter_v_values_with_ragged_chunks_and_checks():
+    rng = np.random.default_rng(23)
+    counts = [120000, 0, 1, 60001, 333]       # scratch / 5 slots = 55,705 fp32 per loop: 3 loops
+    displs, off = [], 1
+    for c in counts:
+        displs.append(off)
+        off += c + 3
+    n = len(counts)
+    xs = [(rng.random(off) * 2 - 1).astype(np.float32) for _ in range(n)]
+    text, _ = dry_reduce_scatter_v(counts, displs, T.FP32, T.SUM, ccl=SMALL_CCL)
+    want = T.run_reduce_scatter_v(T.NumericElems(T.FP32, T.SUM), xs, counts, displs, 4, ccl_bytes=SMALL_CCL)
+    got = [np.zeros(c, dtype=np.float32) for c in counts]
+    for rank, o, nbytes, expr in parse_trace(text):
+        got[rank][o // 4:(o + nbytes) // 4] = eval_expr(parse_expr(expr), xs, nbytes, T.FP32, T.SUM)
+    for r in range(n):
+        assert np.array_equal(got[r].view(np.uint32), want[r].view(np.uint32)), r
+    # parameter checks (reduce_scatter_v_op.cc:142-167 and :49-66)
+    w = api.World(3, ccl_bytes=SMALL_CCL, dry=True)
+    try:
+        ins, outs = fake_ptrs(3)
+        c, d = [4, 4, 4], [0, 4, 8]
+        assert w.reduce_scatter_v(0, ins[0], c, d, outs[0], 4, T.FP32, T.SUM, 0) == 2             # null stream
+        assert w.reduce_scatter_v(0, ins[0], c, d, 0, 4, T.FP32, T.SUM, FAKE_STREAM) == 2         # null recvBuf
+        assert w.reduce_scatter_v(0, ins[0], [0, 0, 0], d, 0, 0, T.FP32, T.SUM, FAKE_STREAM) == 0  # nothing to do
+        assert w.reduce_scatter_v(0, ins[0], c, d, outs[0], 4, T.UINT8, T.SUM, FAKE_STREAM) == 5   # not a reduce type
+        assert w.reduce_scatter_v(0, ins[0], c, d, outs[0], 4, T.BFP16, T.PROD, FAKE_STREAM) == 5  # PROD on bf16
+        assert w.reduce_scatter_v(0, ins[0], c, d, outs[0], 5, T.FP32, T.SUM, FAKE_STREAM) == 1    # recvCount != counts[rank]
+        # uint64 / fp64 have no algorithm in the AICPU branch: the selector finds no match
+        for r in range(3):
+            rc = w.reduce_scatter_v(r, ins[r], c, d, outs[r], 4, T.FP64, T.SUM, FAKE_STREAM)
+        assert rc == 5
+    finally:
+        w.close()
 
 
 def test_which_templates_fuse():

@@ -6,6 +6,8 @@ import json
 import math
 import os
 
+import re
+
 import numpy as np
 import pytest
 
@@ -229,3 +231,67 @@ def test_allgatherv_contract_on_reference_lists(case):
     outs = T.run_allgatherv(ins, counts, displs, displs[-1] + counts[-1], 0)
     for o in outs:
         assert np.array_equal(o, np.concatenate(ins))
+
+
+DT_BY_NAME = {"int8": T.INT8, "int16": T.INT16, "int32": T.INT32, "fp16": T.FP16, "fp32": T.FP32}
+
+
+def symbolic_inputs(n, length):
+    out = []
+    for r in range(n):
+        a = np.empty(length, dtype=object)
+        a[:] = [f"x{r}[{i}]" for i in range(length)]
+        out.append(a)
+    return out
+
+
+@pytest.mark.parametrize("case", GOLD["reducescatterv"], ids=lambda c: c["name"])
+@pytest.mark.parametrize("ccl", [T.CCL_BYTES_DEFAULT, 16 * 1024])
+def test_reduce_scatter_v_on_reference_lists_satisfies_the_checker(case, ccl):
+    """The predicates of reduce_scatter_v_semantics_checker.cc:17-95 on the symbolic run: output r is
+    gap-free, every element reduces all N ranks exactly once, each taken at displs[r] + position; and the
+    order is own rank first, then ranks ascending."""
+    counts, displs = case["counts"], case["displs"]
+    n = len(counts)
+    esz = T.DTYPE_SIZE[DT_BY_NAME[case["dtype"]]]
+    total = max(d + c for d, c in zip(displs, counts))
+    outs = T.run_reduce_scatter_v(T.SymbolicElems(), symbolic_inputs(n, total), counts, displs, esz, ccl_bytes=ccl)
+    for r in range(n):
+        assert len(outs[r]) == counts[r]
+        for t in (0, counts[r] // 2, counts[r] - 1):
+            leaves = re.findall(r"x(\d+)\[(\d+)\]", outs[r][t])
+            assert sorted(int(k) for k, _ in leaves) == list(range(n))
+            assert all(int(i) == displs[r] + t for _, i in leaves)
+            order = [r] + [k for k in range(n) if k != r]
+            want = f"x{order[0]}[{displs[r] + t}]"
+            for k in order[1:]:
+                want = f"(x{k}[{displs[r] + t}]+{want})"
+            assert outs[r][t] == want
+
+
+def test_reduce_scatter_v_integers_equal_numpy_fold_with_ragged_chunks():
+    rng = np.random.default_rng(17)
+    counts = [5000, 0, 1, 4097, 333, 2048]
+    displs, off = [], 3
+    for c in counts:
+        displs.append(off)
+        off += c + 2
+    n = len(counts)
+    xs = [rng.integers(-2**31, 2**31 - 1, size=off, dtype=np.int32) for _ in range(n)]
+    ccl = 6 * 4 * 1024                  # 1024 int32 per slot: the longest part takes 5 loops
+    for op, fold in ((T.SUM, lambda a: a.sum(axis=0, dtype=np.int64).astype(np.int32)),
+                     (T.MAX, lambda a: a.max(axis=0)), (T.MIN, lambda a: a.min(axis=0))):
+        outs = T.run_reduce_scatter_v(T.NumericElems(T.INT32, op), xs, counts, displs, 4, ccl_bytes=ccl)
+        for r in range(n):
+            part = np.stack([x[displs[r]:displs[r] + counts[r]] for x in xs])
+            assert np.array_equal(outs[r], fold(part)), (op, r)
+
+
+def test_reduce_scatter_v_with_equal_counts_is_reduce_scatter():
+    rng = np.random.default_rng(4)
+    n, rc = 5, 777
+    xs = [(rng.random(n * rc) * 2 - 1).astype(np.float32) for _ in range(n)]
+    a = T.run_reduce_scatter_v(T.NumericElems(T.FP32, T.SUM), xs, [rc] * n, [r * rc for r in range(n)], 4)
+    b = T.run_reduce_scatter(T.NumericElems(T.FP32, T.SUM), xs, rc, 4, "InsReduceScatterMesh1D")
+    for r in range(n):
+        assert np.array_equal(a[r].view(np.uint32), b[r].view(np.uint32))
