@@ -130,7 +130,8 @@ template <int DT> struct Vec16 {
     using D = DTypeOf<DT>;
     using S = typename D::S;
     using C = typename D::C;
-    static constexpr int NE = 16 / static_cast<int>(sizeof(S));
+    static constexpr int NE = 16 / static_cast<int>(sizeof(S));   // compute registers per 16 bytes
+    static constexpr int kElems = NE;                             // elements per 16 bytes
 
     static __device__ __forceinline__ void unpack(u32x4 raw, C (&out)[NE])
     {
@@ -148,6 +149,71 @@ template <int DT> struct Vec16 {
         u32x4 raw;
         __builtin_memcpy(&raw, tmp, 16);
         return raw;
+    }
+
+    template <int OP> static __device__ __forceinline__ C combine(C s, C d) { return Combine<DT, OP>::run(s, d); }
+};
+
+// int8 stays packed, four elements to a 32-bit register: byte-wise arithmetic element by element costs
+// several instructions per byte and makes the fold compute-bound.
+typedef short i16x2 __attribute__((ext_vector_type(2)));
+template <> struct Vec16<HCCL_DATA_TYPE_INT8> {
+    using D = DTypeOf<HCCL_DATA_TYPE_INT8>;
+    using S = int8_t;
+    using C = uint32_t;   // four int8
+    static constexpr int NE = 4;
+    static constexpr int kElems = 16;
+
+    static __device__ __forceinline__ void unpack(u32x4 raw, C (&out)[NE])
+    {
+        out[0] = raw.x;
+        out[1] = raw.y;
+        out[2] = raw.z;
+        out[3] = raw.w;
+    }
+    static __device__ __forceinline__ u32x4 pack(const C (&in)[NE])
+    {
+        u32x4 raw = {in[0], in[1], in[2], in[3]};
+        return raw;
+    }
+
+    template <int OP> static __device__ __forceinline__ C combine(C s, C d)
+    {
+        if constexpr (OP == HCCL_REDUCE_SUM) {
+            // add the low 7 bits of every byte, then put the top bits back without carrying across bytes
+            return ((s & 0x7f7f7f7fu) + (d & 0x7f7f7f7fu)) ^ ((s ^ d) & 0x80808080u);
+        } else if constexpr (OP == HCCL_REDUCE_PROD) {
+            C r = 0;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                r |= (((s >> (8 * b)) & 0xffu) * ((d >> (8 * b)) & 0xffu) & 0xffu) << (8 * b);
+            }
+            return r;
+        } else {
+            // A byte in the high half of a 16-bit lane orders like the signed byte itself: even bytes are
+            // shifted up, odd bytes are already there; two packed 16-bit max/min cover all four.
+            const C se = (s << 8) & 0xff00ff00u;
+            const C de = (d << 8) & 0xff00ff00u;
+            const C so = s & 0xff00ff00u;
+            const C dp = d & 0xff00ff00u;
+            i16x2 a, b, c, e;
+            __builtin_memcpy(&a, &se, 4);
+            __builtin_memcpy(&b, &de, 4);
+            __builtin_memcpy(&c, &so, 4);
+            __builtin_memcpy(&e, &dp, 4);
+            i16x2 me, mo;
+            if constexpr (OP == HCCL_REDUCE_MAX) {
+                me = __builtin_elementwise_max(a, b);
+                mo = __builtin_elementwise_max(c, e);
+            } else {
+                me = __builtin_elementwise_min(a, b);
+                mo = __builtin_elementwise_min(c, e);
+            }
+            C ue, uo;
+            __builtin_memcpy(&ue, &me, 4);
+            __builtin_memcpy(&uo, &mo, 4);
+            return (ue >> 8) | uo;
+        }
     }
 };
 

@@ -62,7 +62,7 @@ __device__ __forceinline__ void tree_eval(C (&leaf)[MAXN][NE], uint32_t codes)
             const uint32_t code = (codes >> (2 * (w + i))) & 3u;
             if (code == 2u) {
 #pragma unroll
-                for (int e = 0; e < NE; ++e) leaf[i][e] = Combine<DT, OP>::run(leaf[2 * i + 1][e], leaf[2 * i][e]);
+                for (int e = 0; e < NE; ++e) leaf[i][e] = Vec16<DT>::template combine<OP>(leaf[2 * i + 1][e], leaf[2 * i][e]);
             } else if (code == 1u && i != 0) {
                 // pass the dst child up (for i == 0 it already sits in place)
 #pragma unroll
@@ -79,8 +79,6 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
     using V = Vec16<DT>;
     using C = typename V::C;
     constexpr int NE = V::NE;
-    using Op = Combine<DT, OP>;
-
     u32x4 raw[UNROLL][MAXN];
     const uint32_t present = (MODE == kFoldTree) ? sd.leaf_mask : ((nsrc >= 32u) ? ~0u : ((1u << nsrc) - 1u));
 #pragma unroll
@@ -111,7 +109,7 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
                     C x[NE];
                     V::unpack(raw[u][k], x);
 #pragma unroll
-                    for (int e = 0; e < NE; ++e) acc[e] = Op::run(x[e], acc[e]);
+                    for (int e = 0; e < NE; ++e) acc[e] = V::template combine<OP>(x[e], acc[e]);
                 }
             }
             const u32x4 out = V::pack(acc);
@@ -145,7 +143,7 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
                     for (int k = 0; k < MAXN; ++k) {
                         if (k != j && k < static_cast<int>(nsrc)) {
 #pragma unroll
-                            for (int e = 0; e < NE; ++e) acc[e] = Op::run(val[k][e], acc[e]);
+                            for (int e = 0; e < NE; ++e) acc[e] = V::template combine<OP>(val[k][e], acc[e]);
                         }
                     }
                     st16(sd.dst[j] + vi * 16, V::pack(acc));
@@ -197,7 +195,7 @@ template <int DT, int OP, int MAXN, int MODE>
 __global__ void __launch_bounds__(kFoldThreads)
 k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, uint32_t nseg, uint64_t total_tiles)
 {
-    constexpr int NE = Vec16<DT>::NE;
+    constexpr int NE = Vec16<DT>::kElems;   // elements per 16-byte vector
     constexpr uint64_t TV = fold_tile_vecs(MAXN);
     extern __shared__ uint64_t s_end[];  // nseg entries, sized by the launcher
     for (uint32_t i = threadIdx.x; i < nseg; i += kFoldThreads) {

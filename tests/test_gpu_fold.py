@@ -38,7 +38,8 @@ def test_pairwise_step_in_place_matches_reference_loop(dtype, op):
 
 @pytest.mark.parametrize("nsrc", [3, 4, 5, 8, 9, 12, 16])
 @pytest.mark.parametrize("dtype,op", [(T.FP32, T.SUM), (T.FP32, T.PROD), (T.BFP16, T.SUM), (T.FP16, T.SUM),
-                                      (T.FP16, T.PROD), (T.FP64, T.SUM), (T.INT32, T.MAX), (T.FP32, T.MAX)])
+                                      (T.FP16, T.PROD), (T.FP64, T.SUM), (T.INT32, T.MAX), (T.FP32, T.MAX),
+                                      (T.INT8, T.SUM), (T.INT8, T.PROD), (T.INT8, T.MAX), (T.INT8, T.MIN)])
 def test_chain_fold_reproduces_the_fold_order(nsrc, dtype, op):
     rng = np.random.default_rng(nsrc * 100 + dtype)
     n = 2 * 4096 + 13
