@@ -42,6 +42,10 @@ class Workload:
     name = ""
     dtype = ""
     kernel = ""          # name of the dominant kernel as rocprofv3 prints it (prefix)
+    # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters
+    # read on a plain 1 GiB copy (x2.0 and x1.0); measured once per workload, see profiles/<file>.txt
+    traffic = None
+    profile = None
 
     def __init__(self, torch, api, T, n):
         self.torch, self.api, self.T, self.n = torch, api, T, n
@@ -73,6 +77,8 @@ class ReduceScatterMesh(Workload):
     r's own data, then ranks ascending (ins_temp_reduce_scatter_mesh_1D.cc:132-154), as one fused pass."""
     dtype = "bf16"
     kernel = "hcclx::k_fold<11, 0, 8, 0>"
+    traffic = 604072042
+    profile = "profiles/k_fold_reduce_scatter_bf16_8x64MiB.txt"
 
     def __init__(self, torch, api, T, n=8, recv=4 * 1024 * 1024):
         super().__init__(torch, api, T, n)
@@ -114,6 +120,8 @@ class AllReduce(Workload):
     ranks, so each input is read once and the result is written to the eight outputs."""
     dtype = "f32"
     kernel = "hcclx::k_fold<4, 0, 8, 0>"
+    traffic = 1073830848
+    profile = "profiles/k_fold_all_reduce_fp32_8x64MiB.txt"
 
     def __init__(self, torch, api, T, n=8, count=16 * 1024 * 1024):
         super().__init__(torch, api, T, n)
@@ -141,6 +149,8 @@ class AllGather(Workload):
     output; each source byte is read once and written eight times."""
     dtype = "u8"
     kernel = "hcclx::(anonymous namespace)::k_allgatherv"
+    traffic = 4835821763
+    profile = "profiles/k_allgatherv_fp16_8x64MiB.txt"
 
     def __init__(self, torch, api, T, n=8, count=32 * 1024 * 1024):
         super().__init__(torch, api, T, n)
@@ -166,6 +176,8 @@ class AllToAllV(Workload):
     destination rank per token Zipf(s=1.2), tokens grouped by destination."""
     dtype = "u8"
     kernel = "hcclx::(anonymous namespace)::k_alltoallv"
+    traffic = 939543635
+    profile = "profiles/k_alltoallv_bf16_moe_8x4096x7168.txt"
 
     def __init__(self, torch, api, T, n=8, tokens=4096, hidden=7168, seed=0):
         import numpy as np
@@ -201,6 +213,8 @@ class CopyCalibration(Workload):
     used to scale the HBM traffic counters of a profiler run.  Not part of the per-op table."""
     dtype = "u8"
     kernel = "hcclx::k_fold<0, 0, 1, 0>"
+    traffic = 2147483648
+    profile = "profiles/k_fold_copy_1GiB_counter_calibration.txt"
 
     def __init__(self, torch, api, T, nbytes=1 << 30):
         from hccl_amd import hcclx
@@ -295,7 +309,8 @@ def main():
                         "pct_of_hbm_peak": round(gbs / HBM_PEAK_GBS * 100, 1), "entry": "HcclReduceScatter"
                         if "reduce_scatter" in wl.name else "Hccl* entry points"}, **wl.info()),
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": wl.kernel,
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": wl.traffic, "traffic_source": wl.profile,
+                     "algorithmic_bytes": wl.algo_bytes(), "kernel": wl.kernel,
                      "kernel_us": round(ev_ms * 1e3, 2)},
     }
 
@@ -321,7 +336,8 @@ def main():
         vp, _ = wl.cpu_baseline(parallel=True)
         line["cpu_baseline"] = {"value": round(v1, 3), "unit": "GB/s", "cores": 1, "kind": "port",
                                 "sample": sample,
-                                "all_cores": {"value": round(vp, 3), "cores": os.cpu_count()}}
+                                "all_cores": {"value": round(vp, 3),
+                                              "cores": int(os.environ.get("OMP_NUM_THREADS") or os.cpu_count())}}
     print(json.dumps(line))
 
 
