@@ -8,7 +8,8 @@ Every function below walks the same copy / reduce steps, in the same order and t
 inter-rank handshakes of the reference only order those steps; here the order is the program order of
 each function (all transfers of a phase, then the phase that consumes them).
 
-Two element back-ends run the same schedules:
+Three element back-ends run the same schedules (SampledElems: the numeric one on a sample of the element
+columns, for sizes where a dense run is too slow):
   * NumericElems  -- numpy buffers, reductions through oracle/elem_oracle.c (dst = src (+) dst);
   * SymbolicElems -- buffers of strings; a reduce builds "(src+dst)", a copy moves the string.  It shows
                      the association order of a template as text, e.g. "(x2+(x1+x0))".
@@ -139,6 +140,66 @@ class SymbolicElems:
             if dst[doff + i] == "?" or src[soff + i] == "?":
                 raise AssertionError("reduce reads an undefined element")
             dst[doff + i] = "(" + src[soff + i] + "+" + dst[doff + i] + ")"
+
+
+class SampledBuf:
+    """A buffer of which only some positions are known: sorted positions and their values."""
+
+    def __init__(self, length, np_dtype, pos=None, val=None):
+        self.n = length
+        self.pos = np.empty(0, dtype=np.int64) if pos is None else np.asarray(pos, dtype=np.int64)
+        self.val = np.empty(0, dtype=np_dtype) if val is None else np.ascontiguousarray(val, dtype=np_dtype)
+
+    def __len__(self):
+        return self.n
+
+    def window(self, off, n):
+        a, b = np.searchsorted(self.pos, [off, off + n])
+        return a, b
+
+
+class SampledElems:
+    """Runs a schedule on a sample of the element columns only, so that a template can be followed at
+    sizes (GiB per rank) where a dense CPU run would take minutes.  Every rank's input must be sampled at
+    the same positions; copies move the samples that fall inside the copied range, reduces combine the
+    samples of two ranges, which then sit at the same relative positions (both ranges derive from the same
+    input range of different ranks).  Arithmetic is the same C loop as NumericElems."""
+
+    def __init__(self, dtype, op):
+        self.dtype, self.op = dtype, op
+        self.np_dtype = NP_STORAGE[dtype]
+
+    def empty(self, n):
+        return SampledBuf(n, self.np_dtype)
+
+    def sample(self, length, positions, values):
+        return SampledBuf(length, self.np_dtype, positions, values)
+
+    def copy(self, dst, doff, src, soff, n):
+        if not n:
+            return
+        assert soff + n <= len(src) and doff + n <= len(dst), "copy outside a buffer"
+        a, b = src.window(soff, n)
+        c, d = dst.window(doff, n)
+        dst.val = np.concatenate([dst.val[:c], src.val[a:b], dst.val[d:]])
+        dst.pos = np.concatenate([dst.pos[:c], src.pos[a:b] - soff + doff, dst.pos[d:]])
+
+    def reduce(self, dst, doff, src, soff, n):
+        if not n:
+            return
+        assert soff + n <= len(src) and doff + n <= len(dst), "reduce outside a buffer"
+        a, b = src.window(soff, n)
+        c, d = dst.window(doff, n)
+        if b - a != d - c or not np.array_equal(src.pos[a:b] - soff, dst.pos[c:d] - doff):
+            raise AssertionError("reduce combines ranges with different samples")
+        if b == a:
+            return
+        tmp = np.ascontiguousarray(dst.val[c:d])
+        s = np.ascontiguousarray(src.val[a:b])
+        rc = lib().orc_reduce(tmp.ctypes.data, s.ctypes.data, b - a, self.dtype, self.op)
+        if rc != 0:
+            raise ValueError(f"reduce unsupported: dtype {self.dtype} op {self.op}")
+        dst.val[c:d] = tmp
 
 
 class World:

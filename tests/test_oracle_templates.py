@@ -295,3 +295,34 @@ def test_reduce_scatter_v_with_equal_counts_is_reduce_scatter():
     b = T.run_reduce_scatter(T.NumericElems(T.FP32, T.SUM), xs, rc, 4, "InsReduceScatterMesh1D")
     for r in range(n):
         assert np.array_equal(a[r].view(np.uint32), b[r].view(np.uint32))
+
+
+@pytest.mark.parametrize("alg", AR_ALGS)
+def test_sampled_run_equals_dense_run_allreduce(alg):
+    """SampledElems follows a template on a subset of the columns: it must give the dense run's values there,
+    with executor chunks and ragged slices in play."""
+    rng = np.random.default_rng(31)
+    n, count, ccl = 12, 50021, 64 * 1024
+    xs = [(0.9 + 0.2 * rng.random(count)).astype(np.float32) for _ in range(n)]
+    dense = T.run_allreduce(T.NumericElems(T.FP32, T.PROD), xs, count, 4, alg, ccl_bytes=ccl)
+    pos = np.unique(np.concatenate([rng.integers(0, count, 3000), np.arange(40), np.arange(count - 40, count)]))
+    e = T.SampledElems(T.FP32, T.PROD)
+    outs = T.run_allreduce(e, [e.sample(count, pos, x[pos]) for x in xs], count, 4, alg, ccl_bytes=ccl)
+    for r in range(n):
+        assert np.array_equal(outs[r].pos, pos)
+        assert np.array_equal(outs[r].val.view(np.uint32), dense[r][pos].view(np.uint32)), (alg, r)
+
+
+@pytest.mark.parametrize("alg", RS_ALGS)
+def test_sampled_run_equals_dense_run_reduce_scatter(alg):
+    rng = np.random.default_rng(32)
+    n, rc, ccl = 5, 30011, 1024 * 1024 + 40 * 1024
+    xs = [rng.standard_normal(n * rc).astype(np.float32) for _ in range(n)]
+    dense = T.run_reduce_scatter(T.NumericElems(T.FP32, T.SUM), xs, rc, 4, alg, ccl_bytes=ccl)
+    pos = np.unique(rng.integers(0, n * rc, 5000))
+    e = T.SampledElems(T.FP32, T.SUM)
+    outs = T.run_reduce_scatter(e, [e.sample(n * rc, pos, x[pos]) for x in xs], rc, 4, alg, ccl_bytes=ccl)
+    for r in range(n):
+        mine = pos[(pos >= r * rc) & (pos < (r + 1) * rc)] - r * rc
+        assert np.array_equal(outs[r].pos, mine)
+        assert np.array_equal(outs[r].val.view(np.uint32), dense[r][mine].view(np.uint32)), (alg, r)
