@@ -30,6 +30,7 @@ def parse():
     ap.add_argument("--workload", default="reduce_scatter_sum_bf16_mesh_8x64MiB")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-ops", action="store_true", help="skip the per-op table")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the 12-rank AllReduce size sweep")
     return ap.parse_args()
 
 
@@ -247,6 +248,49 @@ WORKLOADS = {
 EXTRA_WORKLOADS = {"copy_calibration_1024MiB": lambda *a: CopyCalibration(*a)}
 
 
+def sweep_allreduce_12_ranks(torch, api, T, steps):
+    """BASELINE config 5: AllReduce on 12 ranks, 4 KiB ... 1 GiB per rank in powers of 4; int32 MAX through the
+    NHR and halving-doubling templates, fp32 PROD through the CPU-reduce NHR template (what the selector
+    takes for PROD) and halving-doubling.  Small sizes are bound by the launch, so microseconds are reported
+    beside GB/s (algorithmic bytes = 2 * 12 * size)."""
+    n = 12
+    cases = [("int32_max_nhr", T.INT32, T.MAX, "InsAllReduceNHR"), ("int32_max_rhd", T.INT32, T.MAX, "InsAllReduceRHD"),
+             ("fp32_prod_aicpu_nhr", T.FP32, T.PROD, "InsAllReduceAicpuReduceNHR"),
+             ("fp32_prod_rhd", T.FP32, T.PROD, "InsAllReduceRHD")]
+    stream_obj = torch.cuda.Stream()
+    out = {}
+    big = 1 << 30
+    ins = [torch.rand(big // 4, device="cuda:0") * 0.2 + 0.9 for _ in range(n)]     # reused at every size
+    outs = [torch.empty(big // 4, device="cuda:0") for _ in range(n)]
+    for k in range(10):
+        nbytes = 4096 * 4 ** k
+        count = nbytes // 4
+        row = {}
+        for name, dt, op, alg in cases:
+            w = api.World(n)
+            w.set_algorithm(api.CMD_ALLREDUCE, alg)
+
+            class Step:
+                stream_obj_ = stream_obj
+
+                def step(self_inner):
+                    for r in range(n):
+                        rc = w.all_reduce(r, ins[r].data_ptr(), outs[r].data_ptr(), count, dt, op, stream_obj.cuda_stream)
+                        assert rc == 0, rc
+            st = Step()
+            st.stream_obj = stream_obj
+            reps = max(3, min(steps, (1 << 32) // max(nbytes * n, 1)))
+            _, ms = time_steps(torch, st, reps, 2)
+            info = w.last_info()
+            row[name] = {"us": round(ms * 1e3, 1), "GB/s": round(2 * n * nbytes / (ms * 1e-3) / 1e9, 1),
+                         "fused": bool(info.fused), "launches": info.launches}
+            w.close()
+        out["%d" % nbytes] = row
+    del ins, outs
+    torch.cuda.empty_cache()
+    return out
+
+
 def time_steps(torch, wl, steps, warmup):
     """W untimed steps, then K steps bracketed by synchronisation; events sit on the launch stream."""
     import gc
@@ -330,6 +374,8 @@ def main():
                 del w2
                 torch.cuda.empty_cache()
         line["ops"] = ops
+    if not args.no_ops and not args.no_sweep:
+        line["allreduce_12_ranks_sweep"] = sweep_allreduce_12_ranks(torch, api, T, args.steps)
 
     if not args.no_cpu and hasattr(wl, "cpu_baseline"):
         v1, sample = wl.cpu_baseline(parallel=False)

@@ -351,7 +351,9 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
             return fail(HCCL_E_NOT_SUPPORT, "segment " + std::to_string(i) + ": tree deeper than log2(" +
                                                 std::to_string(proto.maxn) + ") levels");
         }
-        const uint64_t tiles = fold_tiles_of(sd.count, ne, proto.maxn);
+        sd.head = fold_head_of(sd.count, proto.copy ? 1 : esz, sd.dst[0]);
+        sd.shift = fold_shift_of(sd.head, proto.copy ? 1 : esz, proto.maxn, sd.dst[0]);
+        const uint64_t tiles = fold_tiles_of(sd.count, ne, proto.maxn, sd.head, sd.shift);
         if (static_cast<int>(cur.segs.size()) == kMaxSegsPerLaunch) {
             out->batches.push_back(std::move(cur));
             cur = proto;

@@ -73,7 +73,8 @@ __device__ __forceinline__ void tree_eval(C (&leaf)[MAXN][NE], uint32_t codes)
 }
 
 template <int DT, int OP, int MAXN, int MODE, bool CHECK>
-__device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint32_t ndst, uint64_t v0, uint64_t nvec)
+__device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint32_t ndst, uint64_t v0, uint64_t nvec,
+                                          uint32_t head_bytes)
 {
     constexpr int UNROLL = fold_unroll(MAXN);
     using V = Vec16<DT>;
@@ -84,7 +85,7 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
 #pragma unroll
     for (int k = 0; k < MAXN; ++k) {
         if ((present >> k) & 1u) {
-            const char *p = sd.src[k] + v0 * 16;
+            const char *p = sd.src[k] + head_bytes + v0 * 16;
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 if (!CHECK || v0 + static_cast<uint64_t>(u) * kFoldThreads < nvec) {
@@ -114,7 +115,7 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
             }
             const u32x4 out = V::pack(acc);
             for (uint32_t d = 0; d < ndst; ++d) {
-                st16(sd.dst[d] + vi * 16, out);
+                st16(sd.dst[d] + head_bytes + vi * 16, out);
             }
         } else if constexpr (MODE == kFoldTree) {
             C val[MAXN][NE];
@@ -125,7 +126,7 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
             tree_eval<DT, OP, MAXN, C, NE>(val, sd.tree_codes);
             const u32x4 out = V::pack(val[0]);
             for (uint32_t d = 0; d < ndst; ++d) {
-                st16(sd.dst[d] + vi * 16, out);
+                st16(sd.dst[d] + head_bytes + vi * 16, out);
             }
         } else {
             C val[MAXN][NE];
@@ -146,7 +147,7 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
                             for (int e = 0; e < NE; ++e) acc[e] = V::template combine<OP>(val[k][e], acc[e]);
                         }
                     }
-                    st16(sd.dst[j] + vi * 16, V::pack(acc));
+                    st16(sd.dst[j] + head_bytes + vi * 16, V::pack(acc));
                 }
             }
         }
@@ -221,28 +222,58 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
         const uint32_t nsrc = sd.nsrc;
         const uint32_t ndst = sd.ndst;
         const uint64_t count = sd.count;
-        const uint64_t nvec = count / NE;
-        const uint32_t rem = static_cast<uint32_t>(count % NE);
-        const uint64_t v0 = tl * TV + threadIdx.x;
-        if ((tl + 1) * TV <= nvec) {
-            fold_tile<DT, OP, MAXN, MODE, false>(sd, nsrc, ndst, v0, nvec);
+        const uint32_t head = sd.head;                      // elements before the aligned body
+        const uint64_t body = count - head;
+        const uint64_t nvec = body / NE;
+        const uint32_t rem = static_cast<uint32_t>(body % NE);
+        const uint32_t head_bytes = head * (16 / NE);
+        const uint32_t shift = sd.shift;
+        // In the first tile of a shifted grid v0 wraps below zero for the vectors in front of the segment;
+        // they fail the bound check of the checked path like the ones behind its end.
+        const uint64_t v0 = tl * TV + threadIdx.x - shift;
+        if (tl * TV >= shift && (tl + 1) * TV - shift <= nvec) {
+            fold_tile<DT, OP, MAXN, MODE, false>(sd, nsrc, ndst, v0, nvec, head_bytes);
         } else {
-            fold_tile<DT, OP, MAXN, MODE, true>(sd, nsrc, ndst, v0, nvec);
-            if (rem != 0 && tl == nvec / TV && threadIdx.x < rem) {
-                fold_tail<DT, OP, MAXN, MODE>(sd, nsrc, ndst, nvec * NE + threadIdx.x);
+            fold_tile<DT, OP, MAXN, MODE, true>(sd, nsrc, ndst, v0, nvec, head_bytes);
+            // the last tile also takes the elements in front of and behind the vector body, one per thread
+            if (tl == (nvec + shift) / TV && threadIdx.x < head + rem) {
+                const uint64_t idx = threadIdx.x < head ? threadIdx.x : head + nvec * NE + (threadIdx.x - head);
+                fold_tail<DT, OP, MAXN, MODE>(sd, nsrc, ndst, idx);
             }
         }
     }
 }
 
 // Host-side geometry, used by the launcher to build tile_end[].
-inline uint64_t fold_tiles_of(uint64_t count, int ne, int maxn)
+// Elements of a segment in front of the first 16-byte boundary of its first destination.
+inline uint32_t fold_head_of(uint64_t count, int esz, const void *dst0)
+{
+    const uint64_t bytes = (16 - (reinterpret_cast<uint64_t>(dst0) & 15)) & 15;
+    if (bytes % esz != 0) {
+        return 0;   // the pointer is not element-aligned: no element boundary falls on a 16-byte boundary
+    }
+    const uint64_t head = bytes / esz;
+    return static_cast<uint32_t>(head < count ? head : count);
+}
+
+// Vectors by which the tile grid is shifted so that tiles are aligned in the address space of dst0.
+inline uint32_t fold_shift_of(uint32_t head, int esz, int maxn, const void *dst0)
+{
+    const uint64_t body_addr = reinterpret_cast<uint64_t>(dst0) + static_cast<uint64_t>(head) * esz;
+    if (body_addr % 16 != 0) {
+        return 0;   // no aligned body (see fold_head_of)
+    }
+    return static_cast<uint32_t>((body_addr % (fold_tile_vecs(maxn) * 16)) / 16);
+}
+
+inline uint64_t fold_tiles_of(uint64_t count, int ne, int maxn, uint32_t head, uint32_t shift)
 {
     if (count == 0) {
         return 0;
     }
-    const uint64_t nvec = count / ne;
-    const uint64_t units = nvec + ((count % ne) ? 1 : 0);
+    const uint64_t body = count - head;
+    const uint64_t nvec = body / ne;
+    const uint64_t units = shift + nvec + ((head + body % ne) ? 1 : 0);
     const uint64_t tv = fold_tile_vecs(maxn);
     return (units + tv - 1) / tv;
 }

@@ -25,6 +25,13 @@ struct SegDev {
     // child unchanged, 2 = child(2i+1) (+) child(2i).  leaf_mask has bit k set when src[k] is present.
     uint32_t tree_codes;
     uint32_t leaf_mask;
+    // Elements in front of the first 16-byte boundary of dst[0]; they are handled one by one so that the
+    // vector stores to dst[0] (and every pointer that shares its alignment) are aligned.
+    uint32_t head;
+    // The tile grid is shifted by this many 16-byte vectors so that tile boundaries fall on multiples of
+    // the tile size in dst[0]'s address space: every wavefront then stores whole, aligned cache lines.
+    // The first tile is partial when shift != 0.
+    uint32_t shift;
 };
 
 // How the sources of a segment are folded.

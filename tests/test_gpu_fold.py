@@ -46,8 +46,9 @@ def test_chain_fold_reproduces_the_fold_order(nsrc, dtype, op):
     kind = "prod" if op == T.PROD else "uniform" if dtype in (T.FP32, T.FP64) else "normal"
     xs = [payload(rng, dtype, n, kind) for _ in range(nsrc)]
     order = list(rng.permutation(nsrc))
-    bufs = [DevBuf(x) for x in xs]
-    outs = [DevBuf(nbytes=xs[0].nbytes) for _ in range(3)]
+    esz = T.DTYPE_SIZE[dtype]
+    bufs = [DevBuf(x, offset=(k % 3) * esz) for k, x in enumerate(xs)]       # element-aligned, not 16-byte aligned
+    outs = [DevBuf(nbytes=xs[0].nbytes, offset=(1 + 2 * k) * esz) for k in range(3)]
     hcclx.fold([(n, [bufs[k].ptr for k in order], [o.ptr for o in outs])], dtype, op)
     sync()
     want = fold_oracle(xs, dtype, op, order, wide=fused_is_wide(dtype, op))
