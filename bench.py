@@ -172,6 +172,36 @@ class AllGather(Workload):
         return 2 * self.n * self.n * self.count * 2
 
 
+class AllGatherV(Workload):
+    """BASELINE config 3: HcclAllGatherV fp16, 16 ranks, per-rank counts uniform in [0, 8,388,608] from a
+    seed, displacements their prefix sum (so most blocks start at addresses that are only 2-byte aligned)."""
+    dtype = "u8"
+    kernel = "hcclx::(anonymous namespace)::k_allgatherv"
+
+    def __init__(self, torch, api, T, n=16, seed=3):
+        import numpy as np
+        super().__init__(torch, api, T, n)
+        self.name = "all_gather_v_fp16_16_ranks_ragged"
+        rng = np.random.default_rng(seed)
+        self.counts = [int(c) for c in rng.integers(0, 8388608, size=n, endpoint=True)]
+        self.displs = [int(d) for d in np.concatenate([[0], np.cumsum(self.counts)[:-1]])]
+        total = sum(self.counts)
+        self.x = [torch.randint(-32768, 32767, (max(c, 1),), device="cuda:0", dtype=torch.int16) for c in self.counts]
+        self.out = [torch.empty(total, device="cuda:0", dtype=torch.int16) for _ in range(n)]
+        self.sp = [t.data_ptr() for t in self.x]
+        self.rp = [t.data_ptr() for t in self.out]
+        self.ct, self.dt = api.u64_table(self.counts), api.u64_table(self.displs)
+
+    def step(self):
+        w, T = self.world, self.T
+        for r in range(self.n):
+            rc = w.all_gather_v(r, self.sp[r], self.counts[r], self.rp[r], self.ct, self.dt, T.FP16, self.stream)
+            assert rc == 0, rc
+
+    def algo_bytes(self):
+        return 2 * self.n * sum(self.counts) * 2
+
+
 class AllToAllV(Workload):
     """BASELINE config 4: HcclAlltoAllV bf16, MoE dispatch: 8 ranks x 4096 tokens x hidden 7168,
     destination rank per token Zipf(s=1.2), tokens grouped by destination."""
@@ -244,6 +274,7 @@ WORKLOADS = {
     "all_reduce_sum_fp32_8x64MiB": lambda *a: AllReduce(*a),
     "all_gather_fp16_8x64MiB": lambda *a: AllGather(*a),
     "all_to_all_v_bf16_moe_8x4096x7168": lambda *a: AllToAllV(*a),
+    "all_gather_v_fp16_16_ranks_ragged": lambda *a: AllGatherV(*a),
 }
 EXTRA_WORKLOADS = {"copy_calibration_1024MiB": lambda *a: CopyCalibration(*a)}
 
@@ -349,7 +380,7 @@ def main():
         "vs_baseline": None,
         "dtype": wl.dtype,
         "data": "synthetic",
-        "config": dict({"workload": wl.name, "virtual_ranks": 8, "algorithmic_bytes": wl.algo_bytes(),
+        "config": dict({"workload": wl.name, "virtual_ranks": wl.n, "algorithmic_bytes": wl.algo_bytes(),
                         "pct_of_hbm_peak": round(gbs / HBM_PEAK_GBS * 100, 1), "entry": "HcclReduceScatter"
                         if "reduce_scatter" in wl.name else "Hccl* entry points"}, **wl.info()),
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -15,12 +15,22 @@ constexpr uint32_t kTileVecs = 256 * kCopyUnroll;
 // aligned: the bytes before the first 16-byte boundary of dst (head) and after the last whole vector
 // (tail) are moved one byte per thread by the block's last tile.  Used by the kernels and, when the
 // tables are on the host, by the launcher to size the grid exactly.
+// The tile grid of a block is shifted by v_shift_of() vectors so that every wavefront's 64 x 16 bytes start
+// on a 1 KiB boundary of dst: whole cache lines are stored.  The first tile is then partial.
+__host__ __device__ inline uint64_t v_head_of(uint64_t bytes, uint64_t dst)
+{
+    const uint64_t head = (16 - (dst & 15)) & 15;
+    return head > bytes ? bytes : head;
+}
+__host__ __device__ inline uint32_t v_shift_of(uint64_t head, uint64_t dst)
+{
+    return static_cast<uint32_t>(((dst + head) & 1023) / 16);
+}
 __host__ __device__ inline uint64_t v_tiles_of(uint64_t bytes, uint64_t dst)
 {
     if (bytes == 0) return 0;
-    uint64_t head = (16 - (dst & 15)) & 15;
-    if (head > bytes) head = bytes;
-    return (bytes - head) / 16 / kTileVecs + 1;
+    const uint64_t head = v_head_of(bytes, dst);
+    return ((bytes - head) / 16 + v_shift_of(head, dst)) / kTileVecs + 1;
 }
 
 // Base pointers of every virtual rank's send and receive buffer, passed by value as a kernel argument.

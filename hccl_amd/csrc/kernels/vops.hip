@@ -83,13 +83,15 @@ template <typename DstFn>
 __device__ __forceinline__ void copy_tile(const char *src, uint64_t dst0, uint64_t bytes, uint64_t tl, uint32_t ndst,
                                           DstFn dst_of)
 {
-    uint64_t head = (16 - (dst0 & 15)) & 15;
-    if (head > bytes) head = bytes;
+    const uint64_t head = v_head_of(bytes, dst0);
     const uint64_t body = bytes - head;
     const uint64_t nvec = body / 16;
-    const uint64_t v0 = tl * kTileVecs + threadIdx.x;
+    const uint32_t shift = v_shift_of(head, dst0);
+    // in the first tile of a shifted grid v0 wraps below zero for the vectors in front of the block and
+    // fails the bound check below
+    const uint64_t v0 = tl * kTileVecs + threadIdx.x - shift;
     const char *sb = src + head;
-    if ((tl + 1) * kTileVecs <= nvec) {
+    if (tl * kTileVecs >= shift && (tl + 1) * kTileVecs - shift <= nvec) {
         u32x4 r[kCopyUnroll];
 #pragma unroll
         for (int u = 0; u < kCopyUnroll; ++u) r[u] = ld16(sb + (v0 + static_cast<uint64_t>(u) * kThreads) * 16);
@@ -100,7 +102,7 @@ __device__ __forceinline__ void copy_tile(const char *src, uint64_t dst0, uint64
         }
         return;
     }
-    // last tile of the block: remaining vectors, then head and tail bytes
+    // first or last tile of the block: the vectors inside it; the last one also moves head and tail bytes
     u32x4 r[kCopyUnroll];
 #pragma unroll
     for (int u = 0; u < kCopyUnroll; ++u) {
@@ -110,7 +112,7 @@ __device__ __forceinline__ void copy_tile(const char *src, uint64_t dst0, uint64
     const uint64_t tail = body - nvec * 16;
     char edge = 0;
     uint64_t edge_off = 0;
-    const bool has_edge = threadIdx.x < head + tail;
+    const bool has_edge = tl == (nvec + shift) / kTileVecs && threadIdx.x < head + tail;
     if (has_edge) {
         edge_off = (threadIdx.x < head) ? threadIdx.x : head + nvec * 16 + (threadIdx.x - head);
         edge = src[edge_off];
