@@ -68,7 +68,7 @@ int hcclx_alltoallv(const void *const *send, void *const *recv, const uint64_t *
         for (uint32_t i = 0; i < n; ++i) {
             for (uint32_t j = 0; j < n; ++j) {
                 const uint64_t dst = reinterpret_cast<uint64_t>(ptrs.recv[j]) + rdispls[j * n + i] * esz;
-                total += v_tiles_of(send_counts[i * n + j] * esz, dst);
+                total += v_tiles_of(send_counts[i * n + j] * esz, dst, kA2avUnroll);
             }
         }
         if (total == 0) return HCCL_SUCCESS;
@@ -123,7 +123,7 @@ int hcclx_allgatherv(const void *const *send, void *const *recv, const uint64_t 
     if (!tables_on_device) {
         uint64_t total = 0;
         for (uint32_t i = 0; i < n; ++i) {
-            total += v_tiles_of(counts[i] * esz, reinterpret_cast<uint64_t>(ptrs.recv[0]) + displs[i] * esz);
+            total += v_tiles_of(counts[i] * esz, reinterpret_cast<uint64_t>(ptrs.recv[0]) + displs[i] * esz, kAgvUnroll);
         }
         if (total == 0) return HCCL_SUCCESS;
         grid = (total + ctx->v_tiles_per_block - 1) / ctx->v_tiles_per_block;

@@ -34,13 +34,27 @@ __host__ __device__ constexpr uint64_t fold_tile_vecs(int maxn)
     return static_cast<uint64_t>(kFoldThreads) * fold_unroll(maxn);
 }
 
+#ifndef HCCLX_NT_LOAD
+#define HCCLX_NT_LOAD 1
+#endif
+#ifndef HCCLX_NT_STORE
+#define HCCLX_NT_STORE 1
+#endif
 __device__ __forceinline__ u32x4 ld16(const char *p)
 {
+#if HCCLX_NT_LOAD
     return __builtin_nontemporal_load(reinterpret_cast<const u32x4_u *>(p));
+#else
+    return *reinterpret_cast<const u32x4_u *>(p);
+#endif
 }
 __device__ __forceinline__ void st16(char *p, u32x4 v)
 {
+#if HCCLX_NT_STORE
     __builtin_nontemporal_store(v, reinterpret_cast<u32x4_u *>(p));
+#else
+    *reinterpret_cast<u32x4_u *>(p) = v;
+#endif
 }
 __device__ __forceinline__ uint64_t uniform64(uint64_t x)
 {
@@ -284,6 +298,7 @@ struct FoldLaunch {
     uint32_t nseg;
     uint64_t total_tiles;
     uint32_t grid;
+    uint32_t lds_pad;          // extra dynamic LDS per workgroup: bounds the workgroups resident per CU
     hipStream_t stream;
 };
 

@@ -7,9 +7,18 @@ namespace hcclx {
 
 constexpr uint32_t kMaxVRanks = 64;
 
-// Tile geometry of the V kernels: 256 threads x 8 vectors of 16 bytes = 32 KiB per tile.
-constexpr int kCopyUnroll = 8;
-constexpr uint32_t kTileVecs = 256 * kCopyUnroll;
+// Tile geometry of the V kernels: 256 threads x `unroll` vectors of 16 bytes per tile.
+// 16-byte vectors each thread moves per tile.  AlltoAllV stages and scans an n x n table per workgroup, so its
+// tiles are large (32 KiB); AllGatherV's set-up is n entries, and small tiles (4 KiB: every workgroup sweeps
+// a compact range and retires quickly) measured faster for its write-heavy traffic.
+#ifndef HCCLX_A2AV_UNROLL
+#define HCCLX_A2AV_UNROLL 8
+#endif
+#ifndef HCCLX_AGV_UNROLL
+#define HCCLX_AGV_UNROLL 1
+#endif
+constexpr int kA2avUnroll = HCCLX_A2AV_UNROLL;
+constexpr int kAgvUnroll = HCCLX_AGV_UNROLL;
 
 // Tiles of a block of `bytes` bytes whose first destination byte sits at address `dst`.  Stores are
 // aligned: the bytes before the first 16-byte boundary of dst (head) and after the last whole vector
@@ -26,8 +35,9 @@ __host__ __device__ inline uint32_t v_shift_of(uint64_t head, uint64_t dst)
 {
     return static_cast<uint32_t>(((dst + head) & 1023) / 16);
 }
-__host__ __device__ inline uint64_t v_tiles_of(uint64_t bytes, uint64_t dst)
+__host__ __device__ inline uint64_t v_tiles_of(uint64_t bytes, uint64_t dst, int unroll)
 {
+    const uint64_t kTileVecs = 256ull * unroll;
     if (bytes == 0) return 0;
     const uint64_t head = v_head_of(bytes, dst);
     return ((bytes - head) / 16 + v_shift_of(head, dst)) / kTileVecs + 1;

@@ -23,10 +23,6 @@ namespace hcclx {
 
 namespace {
 
-constexpr uint32_t kTileBytes = kTileVecs * 16;  // 32 KiB
-
-__device__ __forceinline__ uint64_t tiles_of(uint64_t bytes, uint64_t dst) { return v_tiles_of(bytes, dst); }
-
 __device__ __forceinline__ uint64_t wave_inclusive_scan(uint64_t v)
 {
     const int lane = threadIdx.x & 63;
@@ -79,10 +75,11 @@ __device__ __forceinline__ uint32_t find_block(const uint64_t *s_end, uint32_t m
 
 // One tile of a block copy: tile `tl` of a block of `bytes` bytes from src to dst[0..ndst) (all
 // destinations share dst[0]'s alignment modulo 16, or lose only speed if they do not).
-template <typename DstFn>
+template <int kCopyUnroll, typename DstFn>
 __device__ __forceinline__ void copy_tile(const char *src, uint64_t dst0, uint64_t bytes, uint64_t tl, uint32_t ndst,
                                           DstFn dst_of)
 {
+    constexpr uint64_t kTileVecs = 256ull * kCopyUnroll;
     const uint64_t head = v_head_of(bytes, dst0);
     const uint64_t body = bytes - head;
     const uint64_t nvec = body / 16;
@@ -139,7 +136,7 @@ k_alltoallv(Ptrs ptrs, Tabs tabs, uint32_t n, uint32_t esz, uint32_t tiles_per_b
         const uint32_t i = p / n;
         const uint32_t j = p - i * n;
         const uint64_t dst = reinterpret_cast<uint64_t>(ptrs.recv[j]) + tabs.rdispl(j * n + i) * esz;
-        s_end[p] = tiles_of(tabs.count(p) * esz, dst);
+        s_end[p] = v_tiles_of(tabs.count(p) * esz, dst, kA2avUnroll);
     }
     __syncthreads();
     block_inclusive_scan(s_end, m, s_wave);
@@ -157,7 +154,7 @@ k_alltoallv(Ptrs ptrs, Tabs tabs, uint32_t n, uint32_t esz, uint32_t tiles_per_b
         const uint64_t bytes = tabs.count(p) * esz;
         const char *src = ptrs.send[i] + tabs.sdispl(p) * esz;
         char *dst = ptrs.recv[j] + tabs.rdispl(j * n + i) * esz;
-        copy_tile(src, reinterpret_cast<uint64_t>(dst), bytes, tl, 1, [=](uint32_t) { return dst; });
+        copy_tile<kA2avUnroll>(src, reinterpret_cast<uint64_t>(dst), bytes, tl, 1, [=](uint32_t) { return dst; });
     }
 }
 
@@ -169,7 +166,7 @@ k_allgatherv(VRankPtrs ptrs, Tabs tabs, uint32_t n, uint32_t esz, uint32_t tiles
     uint64_t *s_wave = s_end + n;
     for (uint32_t i = threadIdx.x; i < n; i += kThreads) {
         const uint64_t dst = reinterpret_cast<uint64_t>(ptrs.recv[0]) + tabs.displ(i) * esz;
-        s_end[i] = tiles_of(tabs.count(i) * esz, dst);
+        s_end[i] = v_tiles_of(tabs.count(i) * esz, dst, kAgvUnroll);
     }
     __syncthreads();
     block_inclusive_scan(s_end, n, s_wave);
@@ -183,7 +180,7 @@ k_allgatherv(VRankPtrs ptrs, Tabs tabs, uint32_t n, uint32_t esz, uint32_t tiles
         const uint64_t bytes = tabs.count(i) * esz;
         const uint64_t off = tabs.displ(i) * esz;
         const char *src = ptrs.send[i];
-        copy_tile(src, reinterpret_cast<uint64_t>(ptrs.recv[0]) + off, bytes, tl, n,
+        copy_tile<kAgvUnroll>(src, reinterpret_cast<uint64_t>(ptrs.recv[0]) + off, bytes, tl, n,
                   [&](uint32_t d) { return ptrs.recv[d] + off; });
     }
 }
