@@ -68,6 +68,7 @@ void init_slot(DeviceSlot *s, int dev)
     if (const char *v = std::getenv("HCCLX_BLOCKS_PER_CU")) {
         c.blocks_per_cu = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
     }
+    if (const char *v = std::getenv("HCCLX_A2AV_DIRECT")) c.a2av_direct_unroll = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
     if (const char *v = std::getenv("HCCLX_LDS_PAD")) c.lds_pad = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
     if (const char *v = std::getenv("HCCLX_V_BLOCKS_PER_CU")) {
         const uint32_t b = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));

@@ -78,6 +78,36 @@ int hcclx_alltoallv(const void *const *send, void *const *recv, const uint64_t *
             inline_ok = send_counts[k] <= 0xffffffffull && sdispls[k] <= 0xffffffffull && rdispls[k] <= 0xffffffffull;
         }
     }
+    if (inline_ok && n <= kA2avDirectRanks && ctx->a2av_direct_unroll != 0) {
+        // small host tables and their tile prefix ride in the kernel arguments: one small tile per workgroup
+        const int unroll = ctx->a2av_direct_unroll == 1 ? 1 : ctx->a2av_direct_unroll == 2 ? 2 : 4;
+        VRankPtrs16 p16;
+        A2avTablesDirect tabs;
+        std::memset(&p16, 0, sizeof(p16));
+        std::memset(&tabs, 0, sizeof(tabs));
+        for (uint32_t i = 0; i < n; ++i) {
+            p16.send[i] = ptrs.send[i];
+            p16.recv[i] = ptrs.recv[i];
+        }
+        uint64_t tiles = 0;
+        for (uint32_t i = 0; i < n; ++i) {
+            for (uint32_t j = 0; j < n; ++j) {
+                const uint32_t k = i * n + j;
+                const uint64_t dst = reinterpret_cast<uint64_t>(ptrs.recv[j]) + rdispls[j * n + i] * esz;
+                tiles += v_tiles_of(send_counts[k] * esz, dst, unroll);
+                tabs.send_counts[k] = static_cast<uint32_t>(send_counts[k]);
+                tabs.sdispls[k] = static_cast<uint32_t>(sdispls[k]);
+                tabs.rdispls[k] = static_cast<uint32_t>(rdispls[j * n + i]);
+                tabs.tile_end[k] = static_cast<uint32_t>(tiles);
+            }
+        }
+        if (tiles <= 0x7fffffffull) {
+            hipError_t e = launch_alltoallv_direct(p16, tabs, n, static_cast<uint32_t>(esz), static_cast<uint32_t>(tiles),
+                                                   unroll, st);
+            if (e != hipSuccess) return fail_hip(e, "alltoallv kernel launch");
+            return HCCL_SUCCESS;
+        }
+    }
     if (inline_ok) {
         // small host tables ride in the kernel arguments: nothing is copied in front of the kernel
         VRankPtrs16 p16;

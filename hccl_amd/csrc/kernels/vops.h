@@ -69,6 +69,16 @@ struct A2avTablesInline {
     __device__ uint64_t sdispl(uint32_t p) const { return sdispls[p]; }
     __device__ uint64_t rdispl(uint32_t p) const { return rdispls[p]; }
 };
+// Host tables of up to 15 ranks with the tile prefix worked out by the host: a workgroup finds its block
+// with a binary search over kernel arguments (scalar loads), with no LDS table and no barrier, which is
+// what makes 4 KiB tiles affordable.  15 x 15 x 4 tables of uint32 = 3600 bytes of kernel arguments.
+constexpr uint32_t kA2avDirectRanks = 15;
+struct A2avTablesDirect {
+    uint32_t send_counts[kA2avDirectRanks * kA2avDirectRanks];
+    uint32_t sdispls[kA2avDirectRanks * kA2avDirectRanks];
+    uint32_t rdispls[kA2avDirectRanks * kA2avDirectRanks];   // indexed like send_counts: block (i, j) at i * n + j
+    uint32_t tile_end[kA2avDirectRanks * kA2avDirectRanks];  // inclusive prefix of tiles per block
+};
 // Base pointers for up to kA2avInlineRanks ranks, for the inline-table launch.
 struct VRankPtrs16 {
     const char *send[kA2avInlineRanks];
@@ -89,6 +99,9 @@ struct AgvTablesInline {
 
 hipError_t launch_alltoallv_inline(const VRankPtrs16 &ptrs, const A2avTablesInline &tabs, uint32_t n, uint32_t esz,
                                    uint32_t grid, uint32_t tiles_per_block, hipStream_t stream);
+// unroll: 1, 2 or 4 vectors per thread and tile; grid = total number of tiles
+hipError_t launch_alltoallv_direct(const VRankPtrs16 &ptrs, const A2avTablesDirect &tabs, uint32_t n, uint32_t esz,
+                                   uint32_t grid, int unroll, hipStream_t stream);
 hipError_t launch_allgatherv_inline(const VRankPtrs &ptrs, const AgvTablesInline &tabs, uint32_t n, uint32_t esz,
                                     uint32_t grid, uint32_t tiles_per_block, hipStream_t stream);
 

@@ -158,6 +158,33 @@ k_alltoallv(Ptrs ptrs, Tabs tabs, uint32_t n, uint32_t esz, uint32_t tiles_per_b
     }
 }
 
+// One tile per workgroup; the block of a tile is found in the host-made prefix that rides in the kernel
+// arguments.  Every index below is wave-uniform, so the table reads are scalar loads.
+template <int UNROLL>
+__global__ void __launch_bounds__(kThreads)
+k_alltoallv_direct(VRankPtrs16 ptrs, A2avTablesDirect tabs, uint32_t n, uint32_t esz)
+{
+    const uint32_t t = blockIdx.x;
+    uint32_t lo = 0;
+    uint32_t hi = n * n - 1;
+    while (lo < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (tabs.tile_end[mid] > t) {
+            hi = mid;
+        } else {
+            lo = mid + 1;
+        }
+    }
+    const uint32_t p = lo;
+    const uint64_t tl = t - (p ? tabs.tile_end[p - 1] : 0);
+    const uint32_t i = p / n;
+    const uint32_t j = p - i * n;
+    const uint64_t bytes = static_cast<uint64_t>(tabs.send_counts[p]) * esz;
+    const char *src = ptrs.send[i] + static_cast<uint64_t>(tabs.sdispls[p]) * esz;
+    char *dst = ptrs.recv[j] + static_cast<uint64_t>(tabs.rdispls[p]) * esz;
+    copy_tile<UNROLL>(src, reinterpret_cast<uint64_t>(dst), bytes, tl, 1, [=](uint32_t) { return dst; });
+}
+
 template <typename Tabs>
 __global__ void __launch_bounds__(kThreads)
 k_allgatherv(VRankPtrs ptrs, Tabs tabs, uint32_t n, uint32_t esz, uint32_t tiles_per_block)
@@ -204,6 +231,19 @@ hipError_t launch_alltoallv_inline(const VRankPtrs16 &ptrs, const A2avTablesInli
     const size_t lds = (static_cast<size_t>(n) * n + 4) * sizeof(uint64_t);
     hipLaunchKernelGGL((k_alltoallv<VRankPtrs16, A2avTablesInline>), dim3(grid), dim3(kThreads), lds, stream, ptrs, tabs,
                        n, esz, tiles_per_block);
+    return hipGetLastError();
+}
+
+hipError_t launch_alltoallv_direct(const VRankPtrs16 &ptrs, const A2avTablesDirect &tabs, uint32_t n, uint32_t esz,
+                                   uint32_t grid, int unroll, hipStream_t stream)
+{
+    if (unroll == 1) {
+        hipLaunchKernelGGL((k_alltoallv_direct<1>), dim3(grid), dim3(kThreads), 0, stream, ptrs, tabs, n, esz);
+    } else if (unroll == 2) {
+        hipLaunchKernelGGL((k_alltoallv_direct<2>), dim3(grid), dim3(kThreads), 0, stream, ptrs, tabs, n, esz);
+    } else {
+        hipLaunchKernelGGL((k_alltoallv_direct<4>), dim3(grid), dim3(kThreads), 0, stream, ptrs, tabs, n, esz);
+    }
     return hipGetLastError();
 }
 
