@@ -239,6 +239,65 @@ class AllToAllV(Workload):
         return 2 * self.payload
 
 
+class _NoWorld:
+    def close(self):
+        pass
+
+
+class MoeDispatchPack(Workload):
+    """The caller side of BASELINE config 4, timed on its own: per-token destinations (Zipf 1.2) -> AlltoAllV
+    tables and the stable row permutation (hcclx_moe_route), then the row gather that packs the send buffers
+    (hcclx_moe_pack); 8 ranks x 4096 tokens x hidden 7168 bf16.  Algorithmic bytes: every token row read once
+    and written once."""
+    dtype = "u8"
+    kernel = "k_moe_rows<true>"
+
+    def __init__(self, torch, api, T, n=8, tokens=4096, hidden=7168, seed=0, combine=False):
+        import numpy as np
+        from hccl_amd import hcclx
+        self.torch, self.T, self.n, self.hx = torch, T, n, hcclx
+        self.stream_obj = torch.cuda.Stream()
+        self.stream = self.stream_obj.cuda_stream
+        self.world = _NoWorld()
+        self.combine = combine
+        self.name = ("moe_combine_bf16_%dx%dx%d" if combine else "moe_dispatch_pack_bf16_%dx%dx%d") % (n, tokens, hidden)
+        self.tokens, self.hidden = tokens, hidden
+        rng = np.random.default_rng(seed)
+        w = 1.0 / np.arange(1, n + 1) ** 1.2
+        w /= w.sum()
+        self.dest = [torch.from_numpy(rng.choice(n, size=tokens, p=w).astype(np.int32)).to("cuda:0") for _ in range(n)]
+        self.tok = [torch.randint(-32768, 32767, (tokens * hidden,), device="cuda:0", dtype=torch.int16) for _ in range(n)]
+        self.packed = [torch.empty(tokens * hidden, device="cuda:0", dtype=torch.int16) for _ in range(n)]
+        self.out = [torch.empty(tokens * hidden, device="cuda:0", dtype=torch.int16) for _ in range(n)]
+        self.tabs = [torch.zeros(n * n, dtype=torch.int64, device="cuda:0") for _ in range(4)]
+        self.perm = [torch.empty(tokens, dtype=torch.int32, device="cuda:0") for _ in range(n)]
+        self.ws = torch.empty(hcclx.moe_workspace_bytes(n, tokens), dtype=torch.uint8, device="cuda:0")
+        self.p = lambda ts: [t.data_ptr() for t in ts]
+        self._route()
+        self.hx.moe_pack(self.p(self.tok), self.p(self.perm), tokens, 1, hidden * 2, self.p(self.packed), stream=self.stream)
+
+    def _route(self):
+        t = self.tabs
+        self.hx.moe_route(self.p(self.dest), self.tokens, self.hidden, t[0].data_ptr(), t[1].data_ptr(), t[2].data_ptr(),
+                          t[3].data_ptr(), self.p(self.perm), self.ws.data_ptr(), stream=self.stream)
+
+    def step(self):
+        if self.combine:
+            self.hx.moe_combine(self.p(self.packed), self.p(self.perm), self.tokens, 1, self.hidden, self.T.BFP16,
+                                self.p(self.out), stream=self.stream)
+        else:
+            self._route()
+            self.hx.moe_pack(self.p(self.tok), self.p(self.perm), self.tokens, 1, self.hidden * 2, self.p(self.packed),
+                             stream=self.stream)
+
+    def algo_bytes(self):
+        return 2 * self.n * self.tokens * self.hidden * 2
+
+    def info(self):
+        return {"algorithm": "moe combine (top-1)" if self.combine else "moe route + pack", "fused": True,
+                "launches": 1 if self.combine else 5, "plan_cache_hit": False}
+
+
 class CopyCalibration(Workload):
     """A plain device copy of 1 GiB through the fold kernel's copy instantiation: a kernel of known size,
     used to scale the HBM traffic counters of a profiler run.  Not part of the per-op table."""
@@ -275,6 +334,8 @@ WORKLOADS = {
     "all_gather_fp16_8x64MiB": lambda *a: AllGather(*a),
     "all_to_all_v_bf16_moe_8x4096x7168": lambda *a: AllToAllV(*a),
     "all_gather_v_fp16_16_ranks_ragged": lambda *a: AllGatherV(*a),
+    "moe_dispatch_pack_bf16_8x4096x7168": lambda *a: MoeDispatchPack(*a),
+    "moe_combine_bf16_8x4096x7168": lambda *a: MoeDispatchPack(*a, combine=True),
 }
 EXTRA_WORKLOADS = {"copy_calibration_1024MiB": lambda *a: CopyCalibration(*a)}
 

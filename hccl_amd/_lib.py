@@ -56,6 +56,18 @@ def load():
     lib.hcclx_alltoallv.restype = ctypes.c_int
     lib.hcclx_alltoallv.argtypes = [vpp, vpp, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32,
                                     ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    lib.hcclx_moe_workspace_bytes.restype = ctypes.c_uint64
+    lib.hcclx_moe_workspace_bytes.argtypes = [ctypes.c_uint32, ctypes.c_uint32]
+    lib.hcclx_moe_route.restype = ctypes.c_int
+    lib.hcclx_moe_route.argtypes = [vpp, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p,
+                                    ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, vpp, ctypes.c_void_p,
+                                    ctypes.c_void_p]
+    lib.hcclx_moe_pack.restype = ctypes.c_int
+    lib.hcclx_moe_pack.argtypes = [vpp, vpp, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64, vpp,
+                                   ctypes.c_void_p]
+    lib.hcclx_moe_combine.restype = ctypes.c_int
+    lib.hcclx_moe_combine.argtypes = [vpp, vpp, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint64,
+                                      ctypes.c_int, vpp, ctypes.c_void_p]
     lib.hcclx_allgatherv.restype = ctypes.c_int
     lib.hcclx_allgatherv.argtypes = [vpp, vpp, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_int,
                                      ctypes.c_int, ctypes.c_void_p]

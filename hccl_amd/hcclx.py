@@ -92,3 +92,24 @@ def allgatherv(send, recv, counts, displs, dtype, on_device=False, stream=0):
     b, kb = _table(displs)
     check(_lib.load().hcclx_allgatherv(_ptr_array(send), _ptr_array(recv), a, b, n, int(dtype),
                                        1 if on_device else 0, ctypes.c_void_p(stream)))
+
+
+def moe_workspace_bytes(n, entries):
+    return _lib.load().hcclx_moe_workspace_bytes(n, entries)
+
+
+def moe_route(dest, entries, row_elems, send_counts, sdispls, recv_counts, rdispls, perm, workspace, stream=0):
+    """dest / perm: lists of n device addresses; the tables and the workspace are device addresses."""
+    check(_lib.load().hcclx_moe_route(_ptr_array(dest), len(dest), entries, row_elems, ctypes.c_void_p(send_counts),
+                                      ctypes.c_void_p(sdispls), ctypes.c_void_p(recv_counts), ctypes.c_void_p(rdispls),
+                                      _ptr_array(perm), ctypes.c_void_p(workspace), ctypes.c_void_p(stream)))
+
+
+def moe_pack(tokens, perm, entries, topk, row_bytes, packed, stream=0):
+    check(_lib.load().hcclx_moe_pack(_ptr_array(tokens), _ptr_array(perm), len(tokens), entries, topk, row_bytes,
+                                     _ptr_array(packed), ctypes.c_void_p(stream)))
+
+
+def moe_combine(packed, perm, tokens, topk, row_elems, dtype, out, stream=0):
+    check(_lib.load().hcclx_moe_combine(_ptr_array(packed), _ptr_array(perm), len(packed), tokens, topk, row_elems,
+                                        int(dtype), _ptr_array(out), ctypes.c_void_p(stream)))

@@ -103,6 +103,43 @@ int hcclx_alltoallv(const void *const *send, void *const *recv, const uint64_t *
 int hcclx_allgatherv(const void *const *send, void *const *recv, const uint64_t *counts,
                      const uint64_t *displs, uint32_t n, int dtype, int tables_on_device, void *stream);
 
+/* ---- The caller side of an MoE AlltoAllV, for n virtual ranks at once -------------------------------------
+ * No counterpart in the reference, whose AlltoAllV takes finished send buffers and tables; the nearest code is
+ * the staging either side of the transfer (PreCopy / PostCopy,
+ * src/ops/all_to_all_v/template/aicpu/ins_temp_all_to_all_v_mesh_1D.cc:412-440).
+ *
+ * Every rank i holds `tokens` rows and `entries = tokens * topk` routing entries; entry e belongs to token
+ * e / topk and goes to rank dest[i][e].  Rows are grouped by destination rank, and inside a group they keep
+ * their entry order (a stable grouping).  An entry whose destination is outside 0 .. n-1 is dropped: it is
+ * not sent, perm marks it 0xFFFFFFFF, and it adds nothing when results are combined.
+ * All pointer arrays are host arrays of n device pointers; all tables are device arrays. */
+
+/* Bytes of device workspace hcclx_moe_route needs. */
+uint64_t hcclx_moe_workspace_bytes(uint32_t n, uint32_t entries);
+
+/* From dest[i] (device int32[entries]) to the tables of the AlltoAllV that follows, all n x n row-major
+ * uint64 in elements (row_elems per row), laid out as hcclx_alltoallv reads them with tables_on_device = 1:
+ *   send_counts[i*n + j], sdispls[i*n + j]   what rank i sends to rank j and where it starts in i's packed buffer
+ *   rdispls[j*n + i]                         where that block lands in rank j's receive buffer (blocks in rank order)
+ *   recv_counts[j*n + i] = send_counts[i*n + j]   (the send counts of the way back)
+ * and perm[i] (device uint32[entries]): the row of rank i's packed buffer that entry e goes to.
+ * The AlltoAllV of the way back uses (recv_counts, rdispls, sdispls) in the places of
+ * (send_counts, sdispls, rdispls). */
+int hcclx_moe_route(const int32_t *const *dest, uint32_t n, uint32_t entries, uint64_t row_elems, uint64_t *send_counts,
+                    uint64_t *sdispls, uint64_t *recv_counts, uint64_t *rdispls, uint32_t *const *perm, void *workspace,
+                    void *stream);
+
+/* packed[i][perm[i][e]] = tokens[i][e / topk]: rows of row_bytes bytes (a multiple of 16; buffers 16-byte
+ * aligned). */
+int hcclx_moe_pack(const void *const *tokens, const uint32_t *const *perm, uint32_t n, uint32_t entries, uint32_t topk,
+                   uint64_t row_bytes, void *const *packed, void *stream);
+
+/* out[i][t] = sum over j < topk of packed[i][perm[i][t*topk + j]], j ascending, dropped entries skipped (all
+ * dropped: zeros).  topk == 1 is a pure row permute for any dtype.  topk > 1 takes fp32, fp16 or bf16; 16-bit
+ * floats are accumulated in fp32 and narrowed once (round to nearest even). */
+int hcclx_moe_combine(const void *const *packed, const uint32_t *const *perm, uint32_t n, uint32_t tokens, uint32_t topk,
+                      uint64_t row_elems, int dtype, void *const *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -32,6 +32,9 @@ Reference followed (paths relative to the reference tree, src/ops/...):
                                (test/st/algorithm/utils/src/hccl_verifier/semantics_check/
                                allgather_v_semantics_checker.cc:17-100, all2allv_semantics_checker.cc:19-95)
 
+  moe_route / moe_pack / moe_combine  no reference code; the contract of include/hcclx.h (stable grouping by
+                               destination rank, its inverse, fp32-accumulated combine)
+
 PARITY UNPINNED: allreduce_ring and allreduce_rhd restate documentation prose only; no reference code,
 test or fixture fixes their step order.
 """
@@ -610,6 +613,68 @@ def run_alltoallv(inputs, send_counts, sdispls, recv_counts, rdispls, out_lens, 
             o[rdispls[j][i]:rdispls[j][i] + c] = inputs[i][sdispls[i][j]:sdispls[i][j] + c]
         outs.append(o)
     return outs
+
+
+# ------------------------------------------------------------------------------------------------
+# The caller side of an MoE AlltoAllV (no reference code: defined by its contract)
+# ------------------------------------------------------------------------------------------------
+MOE_DROPPED = 0xFFFFFFFF
+
+
+def moe_route(dests, n, row_elems):
+    """dests[i]: destination rank per routing entry of rank i.  Entries are grouped by destination, entry
+    order kept inside a group; destinations outside 0..n-1 are dropped.  Returns send_counts, sdispls,
+    recv_counts, rdispls (n x n lists, in elements) and perm[i] (row of the packed buffer per entry)."""
+    counts = [[0] * n for _ in range(n)]
+    perms = []
+    for i in range(n):
+        d = np.asarray(dests[i], dtype=np.int64)
+        ok = (d >= 0) & (d < n)
+        for j in range(n):
+            counts[i][j] = int(np.count_nonzero(d == j))
+        starts = np.concatenate([[0], np.cumsum(counts[i])[:-1]])
+        perm = np.full(d.size, MOE_DROPPED, dtype=np.uint32)
+        kept = np.nonzero(ok)[0]
+        order = kept[np.argsort(d[kept], kind="stable")]      # kept entries, grouped by destination, stable
+        perm[order] = np.arange(order.size, dtype=np.uint32)
+        perms.append(perm)
+        del starts
+    send_counts = [[c * row_elems for c in row] for row in counts]
+    sdispls = [[sum(row[:j]) for j in range(n)] for row in send_counts]
+    recv_counts = [[send_counts[i][j] for i in range(n)] for j in range(n)]
+    rdispls = [[sum(recv_counts[j][:i]) for i in range(n)] for j in range(n)]
+    return send_counts, sdispls, recv_counts, rdispls, perms
+
+
+def moe_pack(tokens, perm, topk, out_rows):
+    """tokens: (rows, width) array; packed[perm[e]] = tokens[e // topk]."""
+    packed = np.zeros((out_rows, tokens.shape[1]), dtype=tokens.dtype)
+    for e, p in enumerate(perm):
+        if p != MOE_DROPPED:
+            packed[p] = tokens[e // topk]
+    return packed
+
+
+def moe_combine(packed, perm, topk, dtype):
+    """out[t] = sum_j packed[perm[t*topk + j]], j ascending from the first kept entry; 16-bit floats in fp32 with
+    one narrowing; topk == 1 moves rows as they are."""
+    tokens = len(perm) // topk
+    out = np.zeros((tokens, packed.shape[1]), dtype=packed.dtype)
+    for t in range(tokens):
+        rows = [packed[p] for p in perm[t * topk:(t + 1) * topk] if p != MOE_DROPPED]
+        if not rows:
+            continue
+        if topk == 1:
+            out[t] = rows[0]
+            continue
+        wide = dtype in (FP16, BFP16)
+        acc = widen16(rows[0], dtype) if wide else rows[0].astype(np.float32).copy()
+        e = NumericElems(FP32, SUM)
+        for r in rows[1:]:
+            x = widen16(r, dtype) if wide else np.ascontiguousarray(r, dtype=np.float32)
+            e.reduce(acc, 0, x, 0, acc.size)
+        out[t] = narrow16(acc, dtype) if wide else acc
+    return out
 
 
 def alltoallvc_to_v(matrix, rank):

@@ -326,3 +326,54 @@ def test_sampled_run_equals_dense_run_reduce_scatter(alg):
         mine = pos[(pos >= r * rc) & (pos < (r + 1) * rc)] - r * rc
         assert np.array_equal(outs[r].pos, mine)
         assert np.array_equal(outs[r].val.view(np.uint32), dense[r][mine].view(np.uint32)), (alg, r)
+
+
+def test_moe_route_is_a_stable_grouping_brute_force():
+    """Row of entry e = number of kept entries with a smaller destination + number of earlier kept entries with
+    the same destination; tables follow from the counts (checked with plain loops on small inputs)."""
+    rng = np.random.default_rng(41)
+    for n, entries in ((1, 7), (3, 50), (8, 301), (5, 1)):
+        dests = [rng.integers(-1, n + 1, size=entries) for _ in range(n)]       # -1 and n are dropped
+        sc, sd, rc, rd, perms = T.moe_route(dests, n, 6)
+        for i in range(n):
+            d = dests[i]
+            for e in range(entries):
+                if d[e] < 0 or d[e] >= n:
+                    assert perms[i][e] == T.MOE_DROPPED
+                    continue
+                smaller = sum(1 for x in d if 0 <= x < d[e])
+                earlier = sum(1 for x in d[:e] if x == d[e])
+                assert perms[i][e] == smaller + earlier
+            for j in range(n):
+                assert sc[i][j] == 6 * sum(1 for x in d if x == j)
+                assert sd[i][j] == sum(sc[i][:j])
+                assert rc[j][i] == sc[i][j]
+                assert rd[j][i] == sum(sc[k][j] for k in range(i))
+
+
+def test_moe_dispatch_alltoallv_and_back_is_the_identity():
+    """pack -> AlltoAllV -> AlltoAllV with the tables of the way back -> combine(topk = 1) returns the tokens
+    (dropped ones come back as zeros): ties the routing tables to run_alltoallv."""
+    rng = np.random.default_rng(42)
+    n, tokens, width = 4, 37, 8
+    dests = [rng.integers(0, n + 1, size=tokens) for _ in range(n)]               # n = dropped
+    toks = [rng.integers(0, 60000, size=(tokens, width)).astype(np.uint16) for _ in range(n)]
+    sc, sd, rc, rd, perms = T.moe_route(dests, n, width)
+    packed = [T.moe_pack(toks[i], perms[i], 1, max(1, sum(sc[i]) // width)).reshape(-1) for i in range(n)]
+    recv = T.run_alltoallv(packed, sc, sd, rc, rd, [sum(rc[j]) for j in range(n)])
+    back = T.run_alltoallv(recv, rc, rd, sc, sd, [sum(sc[i]) for i in range(n)])
+    for i in range(n):
+        rows = back[i].reshape(-1, width) if back[i].size else np.zeros((0, width), np.uint16)
+        pad = np.zeros((max(1, rows.shape[0]), width), np.uint16)
+        pad[:rows.shape[0]] = rows
+        out = T.moe_combine(pad, perms[i], 1, T.BFP16)
+        want = toks[i].copy()
+        want[(dests[i] < 0) | (dests[i] >= n)] = 0
+        assert np.array_equal(out, want)
+    # what rank j receives from rank i are i's tokens for j, in token order
+    for j in range(n):
+        pos = 0
+        for i in range(n):
+            mine = toks[i][dests[i] == j].reshape(-1)
+            assert np.array_equal(recv[j][pos:pos + mine.size], mine)
+            pos += mine.size
