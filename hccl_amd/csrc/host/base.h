@@ -29,6 +29,7 @@ constexpr u32 INVALID_VALUE_RANKID = 0xFFFFFFFFu;
 constexpr u64 SYS_MAX_COUNT = 0x7FFFFFFFFull;
 constexpr u64 HCCL_MIN_SLICE_ALIGN = 128;
 constexpr u64 UB_MAX_DATA_SIZE = 256ull * 1024 * 1024;
+constexpr u64 AICPU_ALIGN_SIZE = 4096;   // src/ops/op_common/inc/alg_param.h:75
 constexpr u64 HCCL_CCL_BUFFER_DEFAULT = 200ull * 1024 * 1024;  // HCCL_BUFFSIZE default, 200 MiB in the ST harness
 constexpr u32 NOTIFY_IDX_ACK = 0;
 constexpr u32 NOTIFY_IDX_DATA_SIGNAL = 1;

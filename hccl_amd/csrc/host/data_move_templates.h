@@ -12,6 +12,12 @@ HCCL_DECLARE_TEMPLATE(InsTempReduceScatterNHR, "ReduceScatter NHR", 1, templateR
 // reduce_scatter_v mesh_1D.cc:26-48: N-1 threads (the main thread sends too), N scratch slots
 HCCL_DECLARE_TEMPLATE(InsTempReduceScatterVMesh1D, "ReduceScatterV mesh 1D",
                       (templateRankSize_ > 1 ? templateRankSize_ - 1 : 1), templateRankSize_);
+// mesh-chunk templates (mesh_chunk_templates.cc): reduce_scatter meshchunk.cc:25-52 (N-1 threads, N-1 scratch
+// multiple); all_reduce two_shot_mesh_chunk.cc:17-38 (N threads, scratch multiple 2)
+HCCL_DECLARE_TEMPLATE(InsTempReduceScatterMesh1DMeshChunk, "ReduceScatter mesh 1D, chunked",
+                      (templateRankSize_ > 1 ? templateRankSize_ - 1 : 1), (templateRankSize_ > 0 ? templateRankSize_ - 1 : 0));
+HCCL_DECLARE_TEMPLATE(InsTempAllReduceMesh1DTwoShotMeshChunk, "AllReduce mesh 1D two-shot, chunked",
+                      (templateRankSize_ > 1 ? templateRankSize_ : 1), 2);
 HCCL_DECLARE_TEMPLATE(InsTempAllGatherMesh1D, "AllGather mesh 1D",
                       (templateRankSize_ > 1 ? templateRankSize_ - 1 : 1), templateRankSize_);
 HCCL_DECLARE_TEMPLATE(InsTempAllGatherNHR, "AllGather NHR", 1, templateRankSize_);

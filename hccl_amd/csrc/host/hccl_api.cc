@@ -127,9 +127,23 @@ HcclResult AlltoAllCommon(RankComm *rc, OpParam &p, const void *sendBuf, const v
 extern "C" {
 
 // ---- communicators -------------------------------------------------------------------------------
+namespace {
+// HCCL_BUFFSIZE (MiB) or 200 MiB (test/st/algorithm/utils/inc/sim_common.h:36)
+u64 DefaultCclBytes()
+{
+    u64 ccl = HCCL_CCL_BUFFER_DEFAULT;
+    if (const char *mb = std::getenv("HCCL_BUFFSIZE")) {
+        const u64 v = std::strtoull(mb, nullptr, 10);
+        if (v >= 2) ccl = v * 1024 * 1024;
+    }
+    return ccl;
+}
+}  // namespace
+
 HcclResult hcclxCommInitAll(uint32_t nranks, uint64_t cclBytes, int dry, HcclComm *comms)
 {
     CHK_PTR_NULL(comms);
+    if (cclBytes == 0) cclBytes = DefaultCclBytes();
     if (!dry && hcclx_init() != HCCL_SUCCESS) return HCCL_E_RUNTIME;
     std::vector<HcclComm> v;
     CHK_RET(WorldCreate(nranks, cclBytes, dry != 0, v));
@@ -140,12 +154,7 @@ HcclResult hcclxCommInitAll(uint32_t nranks, uint64_t cclBytes, int dry, HcclCom
 HcclResult HcclCommInitAll(uint32_t ndev, int32_t *devices, HcclComm *comms)
 {
     (void)devices;
-    u64 ccl = HCCL_CCL_BUFFER_DEFAULT;
-    if (const char *mb = std::getenv("HCCL_BUFFSIZE")) {
-        const u64 v = std::strtoull(mb, nullptr, 10);
-        if (v >= 2) ccl = v * 1024 * 1024;
-    }
-    return hcclxCommInitAll(ndev, ccl, 0, comms);
+    return hcclxCommInitAll(ndev, 0, 0, comms);
 }
 
 HcclResult HcclCommDestroy(HcclComm comm) { return WorldDestroyRank(comm); }

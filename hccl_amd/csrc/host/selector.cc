@@ -44,6 +44,8 @@ bool IsSpecial(HcclDataType dt, HcclReduceOp op)
 constexpr u64 AR_AICPU_1D_SMALL_DATA_SIZE = 8ull * 1024 * 1024;
 constexpr u64 AR_AICPU_1D_MAX_DATA_SIZE = 32ull * 1024 * 1024;
 constexpr u64 AR_AICPU_1D_64DATATYPE_DATA_SIZE = 8ull * 1024 * 1024;
+constexpr u64 RS_AICPU_1D_MAX_DATA_SIZE = 16ull * 1024 * 1024;   // reduce_scatter_auto_selector.cc:20
+constexpr double DEFAULT_RANK_SIZE = 8.0;                        // op_common/selector/auto_selector_base.h:27
 
 class AllReduceAutoSelector : public AutoSelectorBase {
 protected:
@@ -52,6 +54,7 @@ protected:
     {
         const u64 dataSize = p.DataDes.count * DATATYPE_SIZE_TABLE[p.DataDes.dataType];
         const bool special = IsSpecial(p.DataDes.dataType, p.reduceType);
+        const double n = topo->userRankSize ? static_cast<double>(topo->userRankSize) : 1.0;
         if (topo->topoLevelNums > 1) {
             // several levels: the flat log-step algorithm; the reference's hierarchical mesh+NHR
             // combinations (:396-409) need real link tiers and are not built
@@ -64,9 +67,11 @@ protected:
                                                                     : "InsAllReduceMesh1DTwoShot";
             } else if (dataSize <= AR_AICPU_1D_SMALL_DATA_SIZE) {
                 name = "InsAllReduceMesh1DOneShot";
+            } else if (static_cast<double>(dataSize) * (DEFAULT_RANK_SIZE / n / n) > AR_AICPU_1D_MAX_DATA_SIZE) {
+                // large messages reduce in place, chunk by chunk (:485-487; the Z-axis detour variant of
+                // two-level machines is not modelled)
+                name = "InsAllReduceMesh1DTwoShotMeshChunk";
             } else {
-                // Above size * 8 / N^2 > 32 MiB the reference moves on to its mesh-chunk template
-                // (:485-487), which is not built; the two-shot template takes those sizes too.
                 name = "InsAllReduceMesh1DTwoShot";
             }
             return SelectorStatus::MATCH;
@@ -93,9 +98,16 @@ protected:
             return SelectorStatus::MATCH;
         }
         if (topo->level0Topo == Level0Shape::MESH_1D) {
-            // dataSize * (8/N)^2 > 16 MiB selects the mesh-chunk template in the reference (:404-408);
-            // it is not built, the mesh template takes those sizes too.
-            name = "InsReduceScatterMesh1D";
+            // 64-bit types and PROD stay with the slot-per-rank template; otherwise a shard of more than
+            // 16 MiB * (N/8)^2 is reduced in place, chunk by chunk (:383-408)
+            const u64 dataSize = p.DataDes.count * DATATYPE_SIZE_TABLE[p.DataDes.dataType];
+            const double n = topo->userRankSize ? static_cast<double>(topo->userRankSize) : 1.0;
+            const double ratio = topo->userRankSize ? (DEFAULT_RANK_SIZE / n) * (DEFAULT_RANK_SIZE / n) : 1.0;
+            if (!IsSpecial(p.DataDes.dataType, p.reduceType) && static_cast<double>(dataSize) * ratio > RS_AICPU_1D_MAX_DATA_SIZE) {
+                name = "InsReduceScatterMesh1DMeshChunk";
+            } else {
+                name = "InsReduceScatterMesh1D";
+            }
             return SelectorStatus::MATCH;
         }
         return SelectorStatus::NOT_MATCH;

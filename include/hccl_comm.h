@@ -28,7 +28,7 @@ HcclResult HcclCommDestroy(HcclComm comm);
 HcclResult HcclGetRankSize(HcclComm comm, uint32_t *rankSize);
 HcclResult HcclGetRankId(HcclComm comm, uint32_t *rank);
 
-/* The same with an explicit scratch-buffer size per rank (bytes, > 1 MiB + 8 KiB; the default is 200 MiB, or
+/* The same with an explicit scratch-buffer size per rank (bytes, > 1 MiB + 8 KiB; 0 = the default: 200 MiB, or
  * HCCL_BUFFSIZE megabytes).  dry != 0 creates a world without a GPU behind it: collectives record, order
  * and trace their schedule and launch nothing. */
 HcclResult hcclxCommInitAll(uint32_t nranks, uint64_t cclBytes, int dry, HcclComm *comms);

@@ -21,6 +21,8 @@ Reference followed (paths relative to the reference tree, src/ops/...):
   allreduce_aicpu_reduce_nhr   all_reduce/template/aicpu/ins_temp_all_reduce_aicpu_reduce_nhr.cc:65-271
   reduce_scatter_mesh          reduce_scatter/template/aicpu/ins_temp_reduce_scatter_mesh_1D.cc:65-227
   reduce_scatter_nhr           reduce_scatter/template/aicpu/ins_temp_reduce_scatter_nhr.cc:77-425
+  reduce_scatter_mesh_chunk    reduce_scatter/template/aicpu/ins_temp_reduce_scatter_mesh_1D_meshchunk.cc:69-263
+  allreduce_mesh_two_shot_mesh_chunk  all_reduce/template/aicpu/ins_temp_all_reduce_mesh_1D_two_shot_mesh_chunk.cc:49-336
   reduce_scatter_v_mesh        reduce_scatter_v/template/aicpu/ins_temp_reduce_scatter_v_mesh_1D.cc:50-179,
                                chunk loop reduce_scatter_v/executor/ins_v2_reduce_scatter_v_sole_executor.cc:75-170
   executor chunk loops         all_reduce/executor/ins_v2_all_reduce_sole_executor.cc:92-185,
@@ -446,12 +448,55 @@ def allreduce_rhd(w, base, count):
         e.copy(w.out[r], base, w.ccl[r], 0, count)
 
 
+def chunk_distance(step, chunk, n):
+    """Mesh-chunk rotation: in step `step`, chunk `chunk` of a shard is written by the rank this many places
+    above the owner: step + chunk + 1, skipping the multiples of n
+    (ins_temp_reduce_scatter_mesh_1D_meshchunk.cc:187-191, ins_temp_all_reduce_mesh_1D_two_shot_mesh_chunk.cc:176-181)."""
+    d = step + chunk + 1
+    if d >= n:
+        d += 1
+    return d % n
+
+
+def split_even(count, parts):
+    """count elements in `parts` chunks, the first count % parts one longer (two_shot_mesh_chunk.cc:131-142)."""
+    return [count // parts + (1 if i < count % parts else 0) for i in range(parts)]
+
+
+def allreduce_mesh_two_shot_mesh_chunk(w, base, count):
+    """Two-shot mesh for large messages: the owner's slice sits in its scratch buffer at the slice's own offset
+    and every peer reduce-writes its chunks straight onto it, chunk c in step s coming from the rank
+    chunk_distance(s, c) above the owner; then every rank reads every owner's slice."""
+    n, e = w.n, w.e
+    if count == 0:
+        return
+    sl = split_data(count, n)
+    w.need_ccl(count)
+    for r in range(n):                                   # PreCopy :313-336
+        off, c = sl[r]
+        e.copy(w.ccl[r], off, w.inp[r], base + off, c)
+    for step in range(n - 1):                            # RunReduceScatter :122-238
+        for owner in range(n):
+            off, c = sl[owner]
+            sizes = split_even(c, n - 1)
+            pos = 0
+            for ch in range(n - 1):
+                src = (owner + chunk_distance(step, ch, n)) % n
+                e.reduce(w.ccl[owner], off + pos, w.inp[src], base + off + pos, sizes[ch])
+                pos += sizes[ch]
+    for r in range(n):                                   # RunAllgather :240-311
+        for k in range(n):
+            off, c = sl[k]
+            e.copy(w.out[r], base + off, w.ccl[k], off, c)
+
+
 ALLREDUCE_TEMPLATES = {
     # name -> (function, scratch multiple as CalcScratchMultiple returns it)
     "InsAllReduceMesh1DOneShot": (allreduce_mesh_one_shot, lambda n: n),      # one_shot.cc:42-48
     "InsAllReduceMesh1DTwoShot": (allreduce_mesh_two_shot, lambda n: 2),      # two_shot.cc:20-27
     "InsAllReduceNHR": (allreduce_nhr, lambda n: 1),                           # nhr.cc:20-26
     "InsAllReduceAicpuReduceNHR": (allreduce_aicpu_reduce_nhr, lambda n: n),  # aicpu_reduce_nhr.cc:22-28
+    "InsAllReduceMesh1DTwoShotMeshChunk": (allreduce_mesh_two_shot_mesh_chunk, lambda n: 2),   # mesh_chunk.cc:17-24
     "InsAllReduceRing": (allreduce_ring, lambda n: 1),
     "InsAllReduceRHD": (allreduce_rhd, lambda n: 1),
 }
@@ -526,9 +571,36 @@ def reduce_scatter_nhr(w, base, count, stride):
         e.copy(w.out[r], base, w.ccl[r], r * count, count)
 
 
+def reduce_scatter_mesh_chunk(w, base, count, stride):
+    """Mesh ReduceScatter for large shards: the own shard is copied to the scratch buffer and the peers reduce-
+    write their chunks onto it in the chunk_distance rotation; N-1 chunks, all but the last rounded down to
+    4 KiB, shards too small for that cut evenly (meshchunk.cc:139-162)."""
+    n, e = w.n, w.e
+    w.need_ccl(max(count, 1))
+    for r in range(n):                                   # PreCopy :110-123
+        e.copy(w.ccl[r], 0, w.inp[r], r * stride + base, count)
+    if n > 1:
+        parts = n - 1
+        aligned = (count * w.esz // parts) // 4096 * 4096
+        if parts >= 2 and aligned > 0:
+            sizes = [aligned // w.esz] * (parts - 1) + [count - (aligned // w.esz) * (parts - 1)]
+        else:
+            sizes = split_even(count, parts)
+        for step in range(n - 1):                        # DoMeshChunk :171-243
+            for owner in range(n):
+                pos = 0
+                for ch in range(n - 1):
+                    src = (owner + chunk_distance(step, ch, n)) % n
+                    e.reduce(w.ccl[owner], pos, w.inp[src], owner * stride + base + pos, sizes[ch])
+                    pos += sizes[ch]
+    for r in range(n):                                   # PostCopy :245-263
+        e.copy(w.out[r], base, w.ccl[r], 0, count)
+
+
 REDUCE_SCATTER_TEMPLATES = {
     "InsReduceScatterMesh1D": (reduce_scatter_mesh, lambda n: n),   # mesh_1D.cc:59-63
     "InsReduceScatterNHR": (reduce_scatter_nhr, lambda n: n),       # nhr.cc:369-377
+    "InsReduceScatterMesh1DMeshChunk": (reduce_scatter_mesh_chunk, lambda n: n - 1),   # meshchunk.cc:46-52
 }
 
 

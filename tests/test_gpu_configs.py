@@ -251,3 +251,66 @@ def test_config5_allreduce_12_ranks_fp32_prod(stream, nbytes):
     pos, want = oracle_on_samples(xs, count, T.FP32, T.PROD, "InsAllReduceRHD", rng, 20000)
     for r in range(n):
         assert np.array_equal(take(outs[r], pos).view(np.uint32), want[r].val.view(np.uint32)), r
+
+
+# ---------------------------------------------------------------------------------------------------
+# beyond the baseline's sizes: what the selector moves to for large messages (mesh-chunk templates)
+# ---------------------------------------------------------------------------------------------------
+def test_large_reduce_scatter_takes_the_chunked_mesh_template(stream):
+    """bf16 shards of 32 MiB on 8 ranks (256 MiB per rank): above 16 MiB the selector picks the template that
+    reduces in place chunk by chunk; every chunk of a shard has its own rotation of the ranks."""
+    n, rc = 8, 16 * 1024 * 1024
+    g = torch.Generator(device=DEV)
+    xs = []
+    for k in range(n):
+        g.manual_seed(700 + k)
+        xs.append(torch.randn(n * rc, device=DEV, generator=g).to(torch.bfloat16))
+    outs = [torch.zeros(rc, device=DEV, dtype=torch.bfloat16) for _ in range(n)]
+    torch.cuda.synchronize()
+    w = api.World(n)
+    try:
+        for r in range(n):
+            assert w.reduce_scatter(r, xs[r].data_ptr(), outs[r].data_ptr(), rc, T.BFP16, T.SUM, stream.cuda_stream) == 0
+        stream.synchronize()
+        info = w.last_info()
+        assert info.algName.decode() == "InsReduceScatterMesh1DMeshChunk" and info.fused == 1
+        rng = np.random.default_rng(7)
+        pos = sample_positions(rng, n * rc, 100000, marks=[k * rc for k in range(1, n)])
+        e = T.SampledElems(T.FP32, T.SUM)
+        ins = [e.sample(n * rc, pos, take(x.float(), pos)) for x in xs]
+        want = T.run_reduce_scatter(e, ins, rc, 2, "InsReduceScatterMesh1DMeshChunk")
+        for r in range(n):
+            got = take(outs[r].view(torch.int16), want[r].pos).view(np.uint16)
+            assert np.array_equal(got, T.narrow16(want[r].val, T.BFP16)), r
+        # any order gives the same value up to rounding: within 1 bf16 ULP of the float64 sum on rank 0's shard
+        exact = sum(x[:rc].double() for x in xs)
+        err = (outs[0].double() - exact).abs()
+        ulp = torch.clamp(exact.abs(), min=2.0 ** -126) * 2.0 ** -7
+        assert bool((err <= ulp).all())
+    finally:
+        w.close()
+
+
+def test_large_allreduce_takes_the_chunked_two_shot_template(stream):
+    n, count = 8, 64 * 1024 * 1024 + 5            # 256 MiB + 20 bytes of fp32 per rank
+    xs = [uniform(count, 800 + k, -1.0, 1.0) for k in range(n)]
+    outs = [torch.empty(count, device=DEV) for _ in range(n)]
+    torch.cuda.synchronize()
+    w = api.World(n)
+    try:
+        for r in range(n):
+            assert w.all_reduce(r, xs[r].data_ptr(), outs[r].data_ptr(), count, T.FP32, T.SUM, stream.cuda_stream) == 0
+        stream.synchronize()
+        info = w.last_info()
+        assert info.algName.decode() == "InsAllReduceMesh1DTwoShotMeshChunk" and info.fused == 1
+        for r in range(1, n):
+            assert torch.equal(outs[r].view(torch.int32), outs[0].view(torch.int32)), r
+        rng = np.random.default_rng(8)
+        pos = sample_positions(rng, count, 100000)
+        e = T.SampledElems(T.FP32, T.SUM)
+        want = T.run_allreduce(e, [e.sample(count, pos, take(x, pos)) for x in xs], count, 4,
+                               "InsAllReduceMesh1DTwoShotMeshChunk")
+        for r in range(n):
+            assert np.array_equal(take(outs[r], pos).view(np.uint32), want[r].val.view(np.uint32)), r
+    finally:
+        w.close()

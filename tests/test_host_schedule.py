@@ -191,6 +191,35 @@ def test_reduce_scatter_v_values_with_ragged_chunks_and_checks():
         w.close()
 
 
+def test_mesh_chunk_rotation_and_4k_chunks():
+    """Chunk i of rank f's shard takes f's own data, then the ranks f+i+1, f+i+2, ... (wrapping, skipping f);
+    with a shard of 20,000 bytes on 4 ranks the chunks are 4096, 4096 and 11,808 bytes."""
+    n, rc = 4, 5000
+    text, info = dry_reduce_scatter(n, rc, T.FP32, T.SUM, "InsReduceScatterMesh1DMeshChunk")
+    assert info.fused == 1
+    pieces = {}
+    for rank, off, nbytes, expr in parse_trace(text):
+        pieces.setdefault(rank, []).append((off, nbytes, expr))
+    for f in range(n):
+        got = sorted(pieces[f])
+        assert [(o, b) for o, b, _ in got] == [(0, 4096), (4096, 4096), (8192, 11808)]
+        for i, (off, _, expr) in enumerate(got):
+            order = [f] + [(f + i + 1 + s + (1 if i + 1 + s >= n else 0)) % n for s in range(n - 1)]
+            want = f"x{order[0]}@{f * rc * 4 + off}"
+            for k in order[1:]:
+                want = f"(x{k}@{f * rc * 4 + off}+{want})"
+            assert expr == want
+    # AllReduce: first level ceil(count / N), second level N-1 even chunks, same rotation
+    text, info = dry_allreduce(5, 1003, T.FP32, T.SUM, "InsAllReduceMesh1DTwoShotMeshChunk")
+    assert info.fused == 1
+    want = T.run_allreduce(T.SymbolicElems(), sym_inputs(5, 1003), 1003, 4, "InsAllReduceMesh1DTwoShotMeshChunk",
+                           ccl_bytes=SMALL_CCL)
+    for rank, off, nbytes, expr in parse_trace(text):
+        tree = parse_expr(expr)
+        for elem in (0, nbytes // 4 - 1):
+            assert expr_to_oracle_string(tree, elem, 4, off) == want[rank][off // 4 + elem]
+
+
 def test_which_templates_fuse():
     """Chains, every integer schedule and floating-point trees of up to four levels become fused passes."""
     for alg, dtype, fused in [("InsAllReduceMesh1DOneShot", T.FP32, 1), ("InsAllReduceMesh1DTwoShot", T.FP32, 1),
@@ -213,7 +242,8 @@ def test_which_templates_fuse():
 
 def test_selector_choices_follow_the_reference_thresholds():
     def pick(n, count, dtype, op, topo=None, cmd="ar"):
-        w = api.World(n, ccl_bytes=SMALL_CCL, dry=True)
+        # the default 200 MiB scratch for large counts: a small one would mean thousands of executor loops
+        w = api.World(n, ccl_bytes=SMALL_CCL if count < (1 << 22) else 0, dry=True)
         try:
             if topo:
                 w.set_topo(*topo)
@@ -231,6 +261,16 @@ def test_selector_choices_follow_the_reference_thresholds():
 
     mib = 1 << 20
     assert pick(8, 8 * mib // 4, T.FP32, T.SUM) == "InsAllReduceMesh1DOneShot"          # <= 8 MiB
+    # size * 8 / N^2 > 32 MiB: the chunked two-shot (all_reduce_auto_selector.cc:485-487)
+    assert pick(8, 256 * mib // 4, T.FP32, T.SUM) == "InsAllReduceMesh1DTwoShot"
+    assert pick(8, 256 * mib // 4 + 1, T.FP32, T.SUM) == "InsAllReduceMesh1DTwoShotMeshChunk"
+    assert pick(4, 64 * mib // 4 + 1, T.FP32, T.SUM) == "InsAllReduceMesh1DTwoShotMeshChunk"
+    assert pick(8, 512 * mib // 8, T.FP64, T.SUM) == "InsAllReduceMesh1DTwoShot"        # 64-bit types never
+    # shard * (8/N)^2 > 16 MiB: the chunked mesh ReduceScatter (reduce_scatter_auto_selector.cc:383-408)
+    assert pick(8, 16 * mib // 2, T.BFP16, T.SUM, cmd="rs") == "InsReduceScatterMesh1D"
+    assert pick(8, 16 * mib // 2 + 1, T.BFP16, T.SUM, cmd="rs") == "InsReduceScatterMesh1DMeshChunk"
+    assert pick(16, 16 * mib // 2 + 1, T.BFP16, T.SUM, cmd="rs") == "InsReduceScatterMesh1D"
+    assert pick(8, 64 * mib // 4, T.FP32, T.PROD, cmd="rs") == "InsReduceScatterMesh1D"
     assert pick(8, 8 * mib // 4 + 1, T.FP32, T.SUM) == "InsAllReduceMesh1DTwoShot"
     assert pick(8, 1024, T.FP32, T.PROD) == "InsAllReduceMesh1DOneShot"
     assert pick(8, 8 * mib // 8 + 1, T.FP64, T.SUM) == "InsAllReduceMesh1DTwoShot"
