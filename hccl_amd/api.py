@@ -18,6 +18,12 @@ class LastOpInfo(ctypes.Structure):
                 ("fusedSegments", ctypes.c_uint32), ("fused", ctypes.c_int), ("planCacheHit", ctypes.c_int)]
 
 
+class CheckReport(ctypes.Structure):
+    _fields_ = [("steps", ctypes.c_uint32), ("levels", ctypes.c_uint32), ("copies", ctypes.c_uint32),
+                ("reduces", ctypes.c_uint32), ("races", ctypes.c_uint32), ("semanticErrors", ctypes.c_uint32),
+                ("exhaustive", ctypes.c_int), ("firstProblem", ctypes.c_char * 256)]
+
+
 _bound = False
 
 
@@ -38,6 +44,8 @@ def lib():
             "hcclxCommSetTopo": [vp, u32, ci, u32],
             "hcclxCommGetLastOpInfo": [vp, ctypes.POINTER(LastOpInfo)],
             "hcclxCommSetTrace": [vp, ci],
+            "hcclxCommSetCheck": [vp, ci],
+            "hcclxCommGetLastCheck": [vp, ctypes.POINTER(CheckReport)],
             "HcclAllReduce": [vp, vp, u64, ci, ci, vp, vp],
             "HcclReduceScatter": [vp, vp, u64, ci, ci, vp, vp],
             "HcclReduceScatterV": [vp, vp, vp, vp, u64, ci, ci, vp, vp],
@@ -101,6 +109,14 @@ class World:
 
     def set_trace(self, on):
         check(lib().hcclxCommSetTrace(self.comms[0], 1 if on else 0))
+
+    def set_check(self, on):
+        check(lib().hcclxCommSetCheck(self.comms[0], 1 if on else 0))
+
+    def last_check(self):
+        rep = CheckReport()
+        check(lib().hcclxCommGetLastCheck(self.comms[0], ctypes.byref(rep)))
+        return rep
 
     def last_info(self):
         info = LastOpInfo()

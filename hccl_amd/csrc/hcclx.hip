@@ -69,7 +69,6 @@ void init_slot(DeviceSlot *s, int dev)
         c.blocks_per_cu = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
     }
     if (const char *v = std::getenv("HCCLX_A2AV_DIRECT")) c.a2av_direct_unroll = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
-    if (const char *v = std::getenv("HCCLX_LDS_PAD")) c.lds_pad = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
     if (const char *v = std::getenv("HCCLX_V_BLOCKS_PER_CU")) {
         const uint32_t b = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
         if (b != 0) c.v_blocks_per_cu = b;
@@ -383,7 +382,6 @@ int launch_batch(const DeviceCtx *ctx, const Batch &b, const char *d_table, hipS
     l.nseg = static_cast<uint32_t>(b.segs.size());
     l.total_tiles = b.total_tiles;
     l.grid = grid_for(ctx, b.total_tiles);
-    l.lds_pad = ctx->lds_pad;
     l.stream = stream;
     hipError_t e;
     if (b.copy) {

@@ -27,7 +27,6 @@ struct DeviceCtx {
     // the grid at blocks_per_cu x CUs instead.
     uint32_t blocks_per_cu = 0;
     uint32_t a2av_direct_unroll = 2;   // HCCLX_A2AV_DIRECT: 0 = off, 1 / 2 / 4 = vectors per thread and tile
-    uint32_t lds_pad = 0;   // HCCLX_LDS_PAD: extra LDS bytes per fold workgroup (occupancy experiments)
     // V kernels whose tables live on the device cannot know their tile count on the host and run as a
     // persistent grid of this many workgroups per CU.
     uint32_t v_blocks_per_cu = 2;

@@ -1,0 +1,49 @@
+// HCCL_ALGO: the environment override of the algorithm choice.
+//
+// Grammar and checks follow the reference's parser (src/common/alg_env_config.cc:330-349, :370-590):
+//   one common setting           level0:<algo>;level1:<algo>[;level2:..;level3:..]
+//   or one setting per op type   <op>=level0:..;level1:.. / <op>=..   (op: allreduce allgather reducescatter
+//                                alltoall broadcast reduce send receive gather scatter sendrecv others)
+// Blanks are ignored; the two forms cannot be mixed; a level may appear once; algo is one of
+//   null ring pipeline fullmesh H-D_R pairwise NHR NHR_V1 AHC AHC_BROKE NB NA.
+// A per-op setting must not put null at level 0; alltoall settings also cover alltoallv / alltoallvc.
+//
+// The reference's AICPU selectors receive this map and ignore it (all_reduce_auto_selector.cc:354).  Here
+// the ranks form one flat level, and the setting picks the template of that level: level1 when it names an
+// algorithm, otherwise level0.
+#pragma once
+#include <map>
+#include <string>
+#include <vector>
+
+#include "base.h"
+
+namespace ops_hccl {
+
+enum class HcclAlgoType {
+    HCCL_ALGO_TYPE_DEFAULT = 0,
+    HCCL_ALGO_TYPE_RING,
+    HCCL_ALGO_TYPE_PIPELINE,
+    HCCL_ALGO_TYPE_FULLMESH,
+    HCCL_ALGO_TYPE_HDR,
+    HCCL_ALGO_TYPE_PAIRWISE,
+    HCCL_ALGO_TYPE_NHR,
+    HCCL_ALGO_TYPE_NHR_V1,
+    HCCL_ALGO_TYPE_AHC,
+    HCCL_ALGO_TYPE_AHC_BROKE,
+    HCCL_ALGO_TYPE_NB,
+    HCCL_ALGO_TYPE_NULL,
+    HCCL_ALGO_TYPE_NA,
+};
+constexpr u32 HCCL_ALGO_LEVEL_NUM = 4;
+
+using HcclAlgoConfig = std::map<HcclCMDType, std::vector<HcclAlgoType>>;
+
+// Parses a HCCL_ALGO value into per-op level settings (ops that are not mentioned stay absent).
+HcclResult SetHcclAlgoConfig(const std::string &hcclAlgo, HcclAlgoConfig &config);
+
+// The executor name the setting asks for on a flat world, "" when it leaves the choice to the selector.
+// cpuReduce: 64-bit types and PROD, which take the CPU-reduce variants.
+std::string AlgNameFromConfig(const HcclAlgoConfig &config, HcclCMDType type, bool cpuReduce);
+
+}  // namespace ops_hccl

@@ -239,6 +239,35 @@ HcclResult hcclxCommSetTrace(HcclComm comm, int on)
     return HCCL_SUCCESS;
 }
 
+HcclResult hcclxCommSetCheck(HcclComm comm, int on)
+{
+    RankComm *rc = AsRankComm(comm);
+    CHK_PTR_NULL(rc);
+    std::lock_guard<std::mutex> lock(rc->world->mu);
+    rc->world->check = (on != 0);
+    return HCCL_SUCCESS;
+}
+
+HcclResult hcclxCommGetLastCheck(HcclComm comm, hcclxCheckReport *report)
+{
+    RankComm *rc = AsRankComm(comm);
+    CHK_PTR_NULL(rc);
+    CHK_PTR_NULL(report);
+    World *w = rc->world;
+    std::lock_guard<std::mutex> lock(w->mu);
+    const CheckReport &c = w->lastCheck;
+    std::memset(report, 0, sizeof(*report));
+    report->steps = c.steps;
+    report->levels = c.levels;
+    report->copies = c.copies;
+    report->reduces = c.reduces;
+    report->races = c.races;
+    report->semanticErrors = c.semanticErrors;
+    report->exhaustive = c.exhaustive ? 1 : 0;
+    std::strncpy(report->firstProblem, c.firstProblem.c_str(), sizeof(report->firstProblem) - 1);
+    return HCCL_SUCCESS;
+}
+
 uint64_t hcclxCommGetLastTrace(HcclComm comm, char *buf, uint64_t size)
 {
     RankComm *rc = AsRankComm(comm);

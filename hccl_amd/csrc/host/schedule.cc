@@ -47,7 +47,12 @@ struct Node {
 // Flattens every thread's items into `order` (a topological order) and gives each data step a level:
 // steps of one level do not depend on each other.  Fails when a wait has no matching record (the
 // schedule would hang) or the dependencies form a cycle.
-HcclResult BuildOrder(World *w, std::vector<Node> &order, u32 &numLevels)
+// With `report`, also looks for data races: two steps that the handshakes leave unordered and that touch
+// the same bytes, at least one of them writing.  Up to kExhaustiveSteps steps every such pair is tested
+// for a dependency path; beyond that only steps of the same level (which are unordered by construction).
+constexpr size_t kExhaustiveSteps = 4096;
+
+HcclResult BuildOrder(World *w, std::vector<Node> &order, u32 &numLevels, CheckReport *report = nullptr)
 {
     struct Flat {
         const TaskItem *item;
@@ -106,6 +111,75 @@ HcclResult BuildOrder(World *w, std::vector<Node> &order, u32 &numLevels)
         }
     }
     CHK_PRT_RET(head != flat.size(), HCCL_ERROR("[schedule] the recorded handshakes deadlock"), HCCL_E_INTERNAL);
+    if (report != nullptr) {
+        // data steps, numbered in topological order
+        std::vector<int> dataId(flat.size(), -1);
+        std::vector<int> dataFlat;
+        for (int id : ready) {
+            if (IsDataOp(*flat[id].item)) {
+                dataId[id] = static_cast<int>(dataFlat.size());
+                dataFlat.push_back(id);
+            }
+        }
+        const size_t nd = dataFlat.size();
+        report->steps = static_cast<u32>(nd);
+        report->levels = numLevels;
+        for (int id : dataFlat) (flat[id].item->kind == ItemKind::COPY ? report->copies : report->reduces)++;
+        report->exhaustive = nd <= kExhaustiveSteps;
+        // reach[id]: the data steps that come after flat node id (bit set), built backwards over the order
+        const size_t words = (nd + 63) / 64;
+        std::vector<std::vector<uint64_t>> reach;
+        if (report->exhaustive) {
+            reach.assign(flat.size(), std::vector<uint64_t>(words, 0));
+            for (size_t k = ready.size(); k-- > 0;) {
+                const int id = ready[k];
+                for (int sx : succ[id]) {
+                    for (size_t wd = 0; wd < words; ++wd) reach[id][wd] |= reach[sx][wd];
+                    if (dataId[sx] >= 0) reach[id][dataId[sx] / 64] |= 1ull << (dataId[sx] % 64);
+                }
+            }
+        }
+        auto ordered = [&](int a, int b) {   // flat ids of two data steps
+            if (!report->exhaustive) return flat[a].level != flat[b].level;
+            const int da = dataId[a];
+            const int db = dataId[b];
+            return ((reach[a][db / 64] >> (db % 64)) & 1ull) != 0 || ((reach[b][da / 64] >> (da % 64)) & 1ull) != 0;
+        };
+        struct Access {
+            u64 lo, hi;
+            int id;
+            bool write;
+        };
+        std::vector<Access> acc;
+        for (int id : dataFlat) {
+            const TaskItem &it = *flat[id].item;
+            if (it.bytes == 0) continue;
+            const u64 d = reinterpret_cast<u64>(it.dst);
+            const u64 sA = reinterpret_cast<u64>(it.src);
+            acc.push_back({d, d + it.bytes, id, true});
+            acc.push_back({sA, sA + it.bytes, id, false});
+        }
+        std::sort(acc.begin(), acc.end(), [](const Access &a, const Access &b) { return a.lo < b.lo; });
+        std::vector<size_t> active;
+        for (size_t k = 0; k < acc.size(); ++k) {
+            size_t keep = 0;
+            for (size_t a : active) {
+                if (acc[a].hi > acc[k].lo) active[keep++] = a;
+            }
+            active.resize(keep);
+            for (size_t a : active) {
+                if (acc[a].id == acc[k].id || (!acc[a].write && !acc[k].write)) continue;
+                if (ordered(acc[a].id, acc[k].id)) continue;
+                if (report->races++ == 0) {
+                    std::ostringstream os;
+                    os << "race: steps " << dataId[acc[a].id] << " and " << dataId[acc[k].id]
+                       << " are not ordered and overlap at address 0x" << std::hex << std::max(acc[a].lo, acc[k].lo);
+                    report->firstProblem = os.str();
+                }
+            }
+            active.push_back(k);
+        }
+    }
     std::stable_sort(order.begin(), order.end(), [](const Node &a, const Node &b) { return a.level < b.level; });
     return HCCL_SUCCESS;
 }
@@ -553,6 +627,128 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
     return true;
 }
 
+// Every output piece against the contract of the collective (what the reference's semantics checkers
+// demand of a recorded task list: test/st/algorithm/utils/src/hccl_verifier/semantics_check/).
+void CheckSemantics(const Tracer &tr, const std::vector<OpParam> &params, CheckReport &rep)
+{
+    const u32 n = static_cast<u32>(params.size());
+    const HcclCMDType type = params[0].opType;
+    auto problem = [&](u32 rank, u64 off, const std::string &what) {
+        if (rep.semanticErrors++ == 0 && rep.firstProblem.empty()) {
+            std::ostringstream os;
+            os << "rank " << rank << " output byte " << off << ": " << what;
+            rep.firstProblem = os.str();
+        }
+    };
+    auto inputOf = [&](u64 addr, u32 &rank, u64 &off) {
+        for (u32 k = 0; k < n; ++k) {
+            const u64 base = reinterpret_cast<u64>(params[k].inputPtr);
+            if (addr >= base && addr < base + std::max<u64>(params[k].inputSize, 1)) {
+                rank = k;
+                off = addr - base;
+                return true;
+            }
+        }
+        return false;
+    };
+    const bool reduceOp = type == HcclCMDType::HCCL_CMD_ALLREDUCE || type == HcclCMDType::HCCL_CMD_REDUCE_SCATTER ||
+                          type == HcclCMDType::HCCL_CMD_REDUCE_SCATTER_V;
+    for (u32 r = 0; r < n; ++r) {
+        const OpParam &p = params[r];
+        const u64 out = reinterpret_cast<u64>(p.outputPtr);
+        const u64 esz = reduceOp ? DATATYPE_SIZE_TABLE[p.DataDes.dataType] : 1;
+        // expected source of output byte `off`: rank (or every rank for a reduction) and input offset;
+        // false = this byte is not part of the result and must stay untouched
+        auto expect = [&](u64 off, u32 &srcRank, u64 &srcOff) {
+            switch (type) {
+                case HcclCMDType::HCCL_CMD_ALLREDUCE:
+                    srcOff = off;
+                    return off < p.DataDes.count * esz;
+                case HcclCMDType::HCCL_CMD_REDUCE_SCATTER:
+                    srcOff = r * p.outputSize + off;
+                    return true;
+                case HcclCMDType::HCCL_CMD_REDUCE_SCATTER_V:
+                    srcOff = p.vDataDes.displs[r] * esz + off;
+                    return off < p.vDataDes.counts[r] * esz;
+                case HcclCMDType::HCCL_CMD_ALLGATHER:
+                    srcRank = static_cast<u32>(off / p.inputSize);
+                    srcOff = off % p.inputSize;
+                    return true;
+                case HcclCMDType::HCCL_CMD_ALLGATHER_V: {
+                    const u64 ez = DATATYPE_SIZE_TABLE[p.vDataDes.dataType];
+                    for (u32 k = 0; k < n; ++k) {
+                        const u64 lo = p.vDataDes.displs[k] * ez;
+                        if (off >= lo && off < lo + p.vDataDes.counts[k] * ez) {
+                            srcRank = k;
+                            srcOff = off - lo;
+                            return true;
+                        }
+                    }
+                    return false;
+                }
+                default: {   // the AlltoAll family
+                    const u64 ez = DATATYPE_SIZE_TABLE[p.all2AllVDataDes.recvType];
+                    for (u32 k = 0; k < n; ++k) {
+                        const u64 lo = p.all2AllVDataDes.rdispls[k] * ez;
+                        if (off >= lo && off < lo + p.all2AllVDataDes.recvCounts[k] * ez) {
+                            srcRank = k;
+                            srcOff = params[k].all2AllVDataDes.sdispls[r] * ez + (off - lo);
+                            return true;
+                        }
+                    }
+                    return false;
+                }
+            }
+        };
+        for (const Sub &s : tr.Lookup(out, std::max<u64>(p.outputSize, 0))) {
+            const u64 off = s.start - out;
+            const bool untouched = (s.expr == 0 && s.shift == s.start);
+            // a piece is uniform only if the expectation does not change inside it: test both ends
+            for (u64 probe : {off, off + s.len - 1}) {
+                u32 wantRank = 0;
+                u64 wantOff = 0;
+                const bool part = expect(probe, wantRank, wantOff);
+                const u64 delta = probe - off;
+                if (!part) {
+                    if (!untouched) problem(r, probe, "written, but not part of the result");
+                    continue;
+                }
+                if (untouched) {
+                    // in place: the byte already holds the right input only for a copy from the same address
+                    u32 k = 0;
+                    u64 o = 0;
+                    if (!reduceOp && inputOf(s.start + delta, k, o) && k == wantRank && o == wantOff) continue;
+                    problem(r, probe, "never written");
+                    continue;
+                }
+                std::vector<u64> leaves;
+                CollectLeaves(tr, s.expr, s.shift + delta, leaves);
+                if (!reduceOp) {
+                    u32 k = 0;
+                    u64 o = 0;
+                    if (leaves.size() != 1 || !inputOf(leaves[0], k, o) || k != wantRank || o != wantOff) {
+                        problem(r, probe, "copied from the wrong place");
+                    }
+                    continue;
+                }
+                std::vector<u32> seen(n, 0);
+                bool ok = leaves.size() == n;
+                for (u64 a : leaves) {
+                    u32 k = 0;
+                    u64 o = 0;
+                    if (!inputOf(a, k, o) || o != wantOff) {
+                        ok = false;
+                        break;
+                    }
+                    seen[k]++;
+                }
+                for (u32 k = 0; k < n && ok; ++k) ok = seen[k] == 1;
+                if (!ok) problem(r, probe, "not the reduction of every rank's element at the matching offset");
+            }
+        }
+    }
+}
+
 std::string PlanKey(const std::vector<OpParam> &params, const std::string &alg, u64 cclBytes)
 {
     std::ostringstream os;
@@ -705,8 +901,14 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
         }
     }
 
-    // algorithm: forced for this world, or the selector's choice
+    // algorithm: forced for this world, asked for by HCCL_ALGO, or the selector's choice
     std::string algName = GetForcedAlgorithm(w, type);
+    if (algName.empty()) {
+        const HcclDataType dt = params[0].DataDes.dataType;
+        const bool cpuReduce = dt == HCCL_DATA_TYPE_INT64 || dt == HCCL_DATA_TYPE_UINT64 || dt == HCCL_DATA_TYPE_FP64 ||
+                               params[0].reduceType == HCCL_REDUCE_PROD;
+        algName = AlgNameFromConfig(w->algoConfig, type, cpuReduce);
+    }
     if (algName.empty()) {
         TopoInfoWithNetLayerDetails topo;
         topo.userRankSize = n;
@@ -725,12 +927,12 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
     const int dtype = params[0].DataDes.dataType;
     const int op = params[0].reduceType;
     const bool fused = (w->mode == ExecMode::FUSED);
-    if (fused && !w->dryRun && !w->traceText && IsDataMove(type)) {
+    if (fused && !w->dryRun && !w->traceText && !w->check && IsDataMove(type)) {
         w->lastWasFused = true;
         return LaunchDataMove(w, params, stream);
     }
     std::string key;
-    if (fused && !w->dryRun && !w->traceText) {
+    if (fused && !w->dryRun && !w->traceText && !w->check) {
         key = PlanKey(params, algName, w->cclBytes);
         for (CachedPlan &c : w->planCache) {
             if (c.key == key) {
@@ -757,12 +959,13 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
     }
     std::vector<Node> order;
     u32 numLevels = 0;
-    CHK_RET(BuildOrder(w, order, numLevels));
+    w->lastCheck = CheckReport();
+    CHK_RET(BuildOrder(w, order, numLevels, w->check ? &w->lastCheck : nullptr));
     w->lastLevels = numLevels;
 
     const u32 esz = IsDataMove(type) ? 1 : DATATYPE_SIZE_TABLE[dtype];
     const int foldType = IsDataMove(type) ? HCCL_DATA_TYPE_INT8 : dtype;
-    if (fused || w->dryRun || w->traceText) {
+    if (fused || w->dryRun || w->traceText || w->check) {
         Tracer tr;
         for (const Node &nd : order) {
             const TaskItem &it = *nd.item;
@@ -771,6 +974,11 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
             } else {
                 tr.Reduce(reinterpret_cast<u64>(it.dst), reinterpret_cast<u64>(it.src), it.bytes);
             }
+        }
+        if (w->check) {
+            CheckSemantics(tr, params, w->lastCheck);
+            CHK_PRT_RET(w->lastCheck.races != 0 || w->lastCheck.semanticErrors != 0,
+                        HCCL_ERROR("[schedule check] %s", w->lastCheck.firstProblem.c_str()), HCCL_E_INTERNAL);
         }
         FusedPlan plan;
         w->lastTrace.clear();

@@ -117,6 +117,14 @@ HcclResult WorldCreate(u32 rankSize, u64 cclBytes, bool dryRun, std::vector<Hccl
         if (std::strcmp(m, "step") == 0) w->mode = ExecMode::STEP;
     }
     if (const char *b = std::getenv("HCCL_VRANK_BLOCKING")) w->blocking = (std::atoi(b) != 0);
+    if (const char *c = std::getenv("HCCL_VRANK_CHECK")) w->check = (std::atoi(c) != 0);
+    if (const char *a = std::getenv("HCCL_ALGO")) {
+        const HcclResult rc = SetHcclAlgoConfig(a, w->algoConfig);
+        if (rc != HCCL_SUCCESS) {
+            delete w;
+            return rc;
+        }
+    }
     w->cclBuf.assign(rankSize, nullptr);
     w->queue.resize(rankSize);
     w->launched.assign(rankSize, 0);

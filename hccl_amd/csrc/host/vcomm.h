@@ -15,6 +15,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include "alg_env_config.h"
 #include "alg_param.h"
 
 struct hcclx_plan;
@@ -72,6 +73,18 @@ struct CachedPlan {
     u64 lastUse = 0;
 };
 
+// What the schedule check found in the last collective (see hcclxCommSetCheck).
+struct CheckReport {
+    u32 steps = 0;           // copy + reduce steps recorded
+    u32 levels = 0;
+    u32 copies = 0;
+    u32 reduces = 0;
+    u32 races = 0;           // pairs of unordered steps that touch the same bytes, at least one writing
+    u32 semanticErrors = 0;  // output pieces that are not what the collective's contract says
+    bool exhaustive = false; // true: every pair of steps was tested for order; false: only steps of one level
+    std::string firstProblem;
+};
+
 struct World {
     u32 rankSize = 0;
     int device = 0;
@@ -102,12 +115,15 @@ struct World {
     bool lastPlanCacheHit = false;
     std::string lastTrace;  // expression of every output piece, filled when traceText is set
     bool traceText = false;
+    bool check = false;     // verify every schedule before it is launched
+    CheckReport lastCheck;
 
     std::vector<CachedPlan> planCache;
     u64 useCounter = 0;
 
     // configuration
     std::map<int, std::string> forcedAlg;  // per HcclCMDType; empty = selector decides
+    HcclAlgoConfig algoConfig;             // HCCL_ALGO as it was when the world was made
     u32 topoLevels = 1;
     Level0Shape topoShape = Level0Shape::MESH_1D;
     u32 devicesPerServer = 0;

@@ -298,7 +298,6 @@ struct FoldLaunch {
     uint32_t nseg;
     uint64_t total_tiles;
     uint32_t grid;
-    uint32_t lds_pad;          // extra dynamic LDS per workgroup: bounds the workgroups resident per CU
     hipStream_t stream;
 };
 

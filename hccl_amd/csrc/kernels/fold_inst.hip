@@ -10,7 +10,7 @@ namespace hcclx {
 template <int DT, int OP, int MAXN, int MODE>
 static hipError_t launch_one(const FoldLaunch &l)
 {
-    hipLaunchKernelGGL((k_fold<DT, OP, MAXN, MODE>), dim3(l.grid), dim3(kFoldThreads), l.nseg * sizeof(uint64_t) + l.lds_pad, l.stream,
+    hipLaunchKernelGGL((k_fold<DT, OP, MAXN, MODE>), dim3(l.grid), dim3(kFoldThreads), l.nseg * sizeof(uint64_t), l.stream,
                        l.tile_end, l.segs, l.nseg, l.total_tiles);
     return hipGetLastError();
 }

@@ -42,7 +42,7 @@ HcclResult hcclxCommSetBlocking(HcclComm comm, int blocking);
 /* HcclCMDType values used by hcclxCommSetAlgorithm. */
 typedef enum {
     HCCLX_CMD_ALLREDUCE = 2, HCCLX_CMD_ALLGATHER = 6, HCCLX_CMD_REDUCE_SCATTER = 7, HCCLX_CMD_ALLTOALLV = 8,
-    HCCLX_CMD_ALLTOALLVC = 9, HCCLX_CMD_ALLTOALL = 10, HCCLX_CMD_ALLGATHER_V = 16
+    HCCLX_CMD_ALLTOALLVC = 9, HCCLX_CMD_ALLTOALL = 10, HCCLX_CMD_ALLGATHER_V = 16, HCCLX_CMD_REDUCE_SCATTER_V = 17
 } hcclxCmdType;
 /* Forces the algorithm (executor name, e.g. "InsAllReduceRing") of an op type; NULL or "" = selector. */
 HcclResult hcclxCommSetAlgorithm(HcclComm comm, int cmdType, const char *algName);
@@ -66,6 +66,25 @@ HcclResult hcclxCommGetLastOpInfo(HcclComm comm, hcclxLastOpInfo *info);
  * the full length. */
 HcclResult hcclxCommSetTrace(HcclComm comm, int on);
 uint64_t hcclxCommGetLastTrace(HcclComm comm, char *buf, uint64_t size);
+
+/* Schedule check.  When on (also: HCCL_VRANK_CHECK=1), every collective's recorded steps are verified before
+ * anything is launched, the way the reference's system-test harness verifies a recorded task list
+ * (test/st/algorithm/utils/src/hccl_verifier/): (1) every wait has a record and the handshakes do not deadlock,
+ * (2) no two steps that the handshakes leave unordered touch the same bytes with at least one of them writing
+ * (check_rank_mem / the task-graph race rules), (3) every output piece is what the collective's contract says:
+ * reduced from each rank exactly once at the matching offset, or copied from the right rank and offset
+ * (semantics_check/*_semantics_checker.cc).  A collective that fails returns HCCL_E_INTERNAL and launches
+ * nothing.  Checked collectives bypass the plan cache. */
+typedef struct {
+    uint32_t steps, levels, copies, reduces;
+    uint32_t races;
+    uint32_t semanticErrors;
+    int exhaustive;           /* 1: all pairs of steps were tested for order; 0 (schedules of more than 4096
+                                 steps): only steps of the same dependency level */
+    char firstProblem[256];
+} hcclxCheckReport;
+HcclResult hcclxCommSetCheck(HcclComm comm, int on);
+HcclResult hcclxCommGetLastCheck(HcclComm comm, hcclxCheckReport *report);
 
 #ifdef __cplusplus
 }
