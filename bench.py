@@ -124,9 +124,15 @@ class AllReduce(Workload):
     traffic = 1073830848
     profile = "profiles/k_fold_all_reduce_fp32_8x64MiB.txt"
 
-    def __init__(self, torch, api, T, n=8, count=16 * 1024 * 1024):
+    def __init__(self, torch, api, T, n=8, count=16 * 1024 * 1024, alg=None, step_mode=False):
         super().__init__(torch, api, T, n)
         self.name = "all_reduce_sum_fp32_%dx%dMiB" % (n, count * 4 >> 20)
+        if alg:
+            self.world.set_algorithm(api.CMD_ALLREDUCE, alg)
+            self.name += "_" + alg
+        if step_mode:
+            self.world.set_mode(api.EXEC_STEP)
+            self.name += "_step_by_step"
         self.count = count
         g = torch.Generator(device="cuda:0")
         g.manual_seed(7)
@@ -334,6 +340,12 @@ WORKLOADS = {
     "all_gather_fp16_8x64MiB": lambda *a: AllGather(*a),
     "all_to_all_v_bf16_moe_8x4096x7168": lambda *a: AllToAllV(*a),
     "all_gather_v_fp16_16_ranks_ragged": lambda *a: AllGatherV(*a),
+    # BASELINE config 1 (ring template, 8 x 1,048,576 fp32): one fused pass, and every step of the ring
+    # launched through the scratch buffers (the step-faithful variant, with the ring's own larger traffic)
+    "all_reduce_sum_fp32_8x4MiB_ring": lambda *a: AllReduce(*a, count=1048576, alg="InsAllReduceRing"),
+    "all_reduce_sum_fp32_8x4MiB_ring_step_by_step": lambda *a: AllReduce(*a, count=1048576, alg="InsAllReduceRing",
+                                                                         step_mode=True),
+    "all_reduce_sum_fp32_8x64MiB_two_shot_step_by_step": lambda *a: AllReduce(*a, step_mode=True),
     "moe_dispatch_pack_bf16_8x4096x7168": lambda *a: MoeDispatchPack(*a),
     "moe_combine_bf16_8x4096x7168": lambda *a: MoeDispatchPack(*a, combine=True),
 }

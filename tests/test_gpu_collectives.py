@@ -90,6 +90,26 @@ def test_allreduce_in_place(stream, mode):
         w.close()
 
 
+def test_checked_world_verifies_then_launches(stream):
+    """With the schedule check on, a collective is verified (no race, right semantics) and then runs as usual."""
+    rng = np.random.default_rng(21)
+    n, count = 8, 50001
+    xs = [payload(rng, T.FP32, count, "uniform") for _ in range(n)]
+    w = api.World(n, ccl_bytes=SMALL_CCL)
+    try:
+        w.set_check(True)
+        for alg in ("InsAllReduceNHR", "InsAllReduceMesh1DTwoShotMeshChunk"):
+            w.set_algorithm(api.CMD_ALLREDUCE, alg)
+            got, _ = run_allreduce(w, stream, xs, count, T.FP32, T.SUM)
+            rep = w.last_check()
+            assert rep.races == 0 and rep.semanticErrors == 0 and rep.steps > 0 and w.last_info().fused == 1
+            want = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs, count, 4, alg, ccl_bytes=SMALL_CCL)
+            for r in range(n):
+                assert_same_bits(got[r], want[r], T.FP32, f"{alg} rank {r}")
+    finally:
+        w.close()
+
+
 def test_allreduce_default_selector_and_plan_cache(stream):
     """Config 1 of the baseline: AllReduce SUM fp32, 8 ranks x 1,048,576 elements, uniform[-1,1): the
     selector takes the one-shot mesh template at this size; the ring template is forced next."""
