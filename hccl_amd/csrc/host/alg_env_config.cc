@@ -1,6 +1,7 @@
 #include "alg_env_config.h"
 
 #include <algorithm>
+#include <cctype>
 
 namespace ops_hccl {
 
@@ -155,6 +156,38 @@ std::string AlgNameFromConfig(const HcclAlgoConfig &config, HcclCMDType type, bo
         default:
             return "";   // one template each: nothing to choose
     }
+}
+
+HcclResult ParseDeterministic(const std::string &text, u8 &level)
+{
+    std::string t = text;
+    std::transform(t.begin(), t.end(), t.begin(), [](unsigned char c) { return static_cast<char>(std::toupper(c)); });
+    if (t == "FALSE") {
+        level = static_cast<u8>(DeterministicEnableLevel::DETERMINISTIC_DISABLE);
+    } else if (t == "TRUE") {
+        level = static_cast<u8>(DeterministicEnableLevel::DETERMINISTIC_ENABLE);
+    } else if (t == "STRICT") {
+        level = static_cast<u8>(DeterministicEnableLevel::DETERMINISTIC_STRICT);
+    } else {
+        HCCL_ERROR("HCCL_DETERMINISTIC is set to [%s]: should be true, false or strict", text.c_str());
+        return HCCL_E_PARA;
+    }
+    return HCCL_SUCCESS;
+}
+
+namespace {
+u8 g_deterministic = static_cast<u8>(DeterministicEnableLevel::DETERMINISTIC_DISABLE);
+}
+u8 GetExternalInputHcclDeterministic() { return g_deterministic; }
+void SetExternalInputHcclDeterministic(u8 level) { g_deterministic = level; }
+
+bool IsNeedStrictModeForOrderPreserved(HcclDataType dataType, HcclReduceOp reduceType, u32 rankSize)
+{
+    return GetExternalInputHcclDeterministic() == static_cast<u8>(DeterministicEnableLevel::DETERMINISTIC_STRICT) &&
+           (dataType == HCCL_DATA_TYPE_FP16 || dataType == HCCL_DATA_TYPE_FP32 || dataType == HCCL_DATA_TYPE_BFP16 ||
+            dataType == HCCL_DATA_TYPE_FP64) &&
+           (reduceType == HCCL_REDUCE_SUM || reduceType == HCCL_REDUCE_PROD) &&
+           rankSize > MIN_STRICT_RANK_NUM_ORDER_PRESERVED;
 }
 
 }  // namespace ops_hccl

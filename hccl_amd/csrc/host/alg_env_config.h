@@ -46,4 +46,17 @@ HcclResult SetHcclAlgoConfig(const std::string &hcclAlgo, HcclAlgoConfig &config
 // cpuReduce: 64-bit types and PROD, which take the CPU-reduce variants.
 std::string AlgNameFromConfig(const HcclAlgoConfig &config, HcclCMDType type, bool cpuReduce);
 
+// HCCL_DETERMINISTIC: false / true / strict, any case (src/common/alg_env_config.cc:948-990).  strict asks for
+// a reduction order that does not depend on which rank computes: the order-preserved ReduceScatter.
+enum class DeterministicEnableLevel : u8 { DETERMINISTIC_DISABLE = 0, DETERMINISTIC_ENABLE, DETERMINISTIC_STRICT };
+HcclResult ParseDeterministic(const std::string &text, u8 &level);
+// Process-wide value, as the selectors read it; set from the environment whenever a world is made.
+u8 GetExternalInputHcclDeterministic();
+void SetExternalInputHcclDeterministic(u8 level);
+
+// Strict mode applies to floating-point SUM / PROD among more than two ranks (src/common/order_preserved_common.h:63-76).
+constexpr u32 MIN_STRICT_RANK_NUM_ORDER_PRESERVED = 2;
+constexpr u32 MAX_RANK_NUM_FOR_ORDER_PRESERVED = 32;
+bool IsNeedStrictModeForOrderPreserved(HcclDataType dataType, HcclReduceOp reduceType, u32 rankSize);
+
 }  // namespace ops_hccl

@@ -18,6 +18,32 @@ HCCL_DECLARE_TEMPLATE(InsTempReduceScatterMesh1DMeshChunk, "ReduceScatter mesh 1
                       (templateRankSize_ > 1 ? templateRankSize_ - 1 : 1), (templateRankSize_ > 0 ? templateRankSize_ - 1 : 0));
 HCCL_DECLARE_TEMPLATE(InsTempAllReduceMesh1DTwoShotMeshChunk, "AllReduce mesh 1D two-shot, chunked",
                       (templateRankSize_ > 1 ? templateRankSize_ : 1), 2);
+// Where each rank's block sits in the scratch buffer during one loop of the order-preserved ReduceScatter
+// (ins_v2_reduce_scatter_order_preserved_executor.h:37-42).
+struct MemBlockInfo {
+    std::vector<u64> size;
+    std::vector<u64> userInputOffsets;
+    std::vector<u64> inputOffsets;
+    std::vector<u64> outputOffsets;
+};
+
+// order_preserved_level1.cc:35-50, :128-131: N threads, N scratch slots
+class InsTempReduceScatterOrderPreservedLevel1 : public InsAlgTemplateBase {
+public:
+    using InsAlgTemplateBase::InsAlgTemplateBase;
+    std::string Describe() const override { return "ReduceScatter, order preserved"; }
+    u64 GetThreadNum() const override { return templateRankSize_ > 1 ? templateRankSize_ : 1; }
+    u64 CalcScratchMultiple(BufferType, BufferType) override { return templateRankSize_; }
+    HcclResult KernelRun(const OpParam &param, const TemplateDataParams &tempAlgParams,
+                         TemplateResource &templateResource) override;
+    void SetMemBlockInfo(const MemBlockInfo &info) { memBlockInfo_ = info; }
+
+private:
+    // slot of the block that rank `peer` sent to rank `localRank` (:153-158)
+    u32 CalcOutputIndex(u32 peer, u32 localRank) const { return (peer + localRank) % templateRankSize_; }
+    MemBlockInfo memBlockInfo_;
+};
+
 HCCL_DECLARE_TEMPLATE(InsTempAllGatherMesh1D, "AllGather mesh 1D",
                       (templateRankSize_ > 1 ? templateRankSize_ - 1 : 1), templateRankSize_);
 HCCL_DECLARE_TEMPLATE(InsTempAllGatherNHR, "AllGather NHR", 1, templateRankSize_);

@@ -71,6 +71,8 @@ REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_ALLREDUCE, InsAllReduceMesh1DTwoShotMeshC
                  TopoMatch1D, InsTempAllReduceMesh1DTwoShotMeshChunk);
 REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_REDUCE_SCATTER, InsReduceScatterMesh1DMeshChunk, InsV2ReduceScatterSoleExecutor,
                  TopoMatch1D, InsTempReduceScatterMesh1DMeshChunk);
+REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_REDUCE_SCATTER, ReduceScatterOrderPreserved, InsV2ReduceScatterOrderPreservedExecutor,
+                 TopoMatch1D, InsTempReduceScatterOrderPreservedLevel1);
 REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_REDUCE_SCATTER_V, InsReduceScatterVMesh1D, InsV2ReduceScatterVSoleExecutor,
                  TopoMatch1D, InsTempReduceScatterVMesh1D);
 REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_ALLGATHER_V, InsAllGatherVMesh1D, InsV2AllGatherVSoleExecutor, TopoMatch1D,

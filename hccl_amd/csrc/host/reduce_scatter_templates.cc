@@ -2,6 +2,7 @@
 // (src/ops/reduce_scatter/template/aicpu/):
 //   InsTempReduceScatterMesh1D   ins_temp_reduce_scatter_mesh_1D.cc:65-227
 //   InsTempReduceScatterNHR      ins_temp_reduce_scatter_nhr.cc:77-425
+//   InsTempReduceScatterOrderPreservedLevel1   ins_temp_reduce_scatter_order_preserved_level1.cc:52-330
 // and src/ops/reduce_scatter_v/template/aicpu/:
 //   InsTempReduceScatterVMesh1D  ins_temp_reduce_scatter_v_mesh_1D.cc:50-179
 #include "data_move_templates.h"
@@ -200,6 +201,74 @@ HcclResult InsTempReduceScatterVMesh1D::KernelRun(const OpParam &param, const Te
                           p.buffInfo.hcclBuffBaseOff + rpt * p.outputRepeatStride + k * p.outputSliceStride, size, count);
             CHK_RET(LocalReduce(threads[0], src, dst, dataType_, reduceOp_));
         }
+    }
+    return HCCL_SUCCESS;
+}
+
+// Strictly deterministic ReduceScatter: every rank sends shard k of its input to rank k (an all-to-all into
+// scratch slots), and rank k folds the N blocks in a tree that is the same on every rank: while more than one
+// block remains, with M the largest power of two below the number of blocks, block v >= M is folded into block
+// v % M, then M blocks remain.  Blocks are numbered by the rank they came from, so the
+// association does not depend on which rank owns the shard.
+HcclResult InsTempReduceScatterOrderPreservedLevel1::KernelRun(const OpParam &param, const TemplateDataParams &p,
+                                                               TemplateResource &res)
+{
+    if (p.sliceSize == 0 && p.tailSize == 0) return HCCL_SUCCESS;
+    const u32 n = templateRankSize_;
+    threadNum_ = static_cast<u32>(res.threads.size());
+    CHK_PRT_RET(threadNum_ == 0, HCCL_ERROR("[RS order preserved] no thread"), HCCL_E_INTERNAL);
+    dataType_ = param.DataDes.dataType;
+    reduceOp_ = param.reduceType;
+    const u64 esz = DATATYPE_SIZE_TABLE[dataType_];
+    const MemBlockInfo &mb = memBlockInfo_;
+    CHK_PRT_RET(mb.size.size() != n || mb.userInputOffsets.size() != n || mb.outputOffsets.size() != n,
+                HCCL_ERROR("[RS order preserved] block table does not match the rank size"), HCCL_E_INTERNAL);
+    u32 me = 0;
+    CHK_RET(GetAlgRank(myRank_, subCommRanks_[0], me));
+    void *in = p.buffInfo.inputPtr;
+    void *ccl = p.buffInfo.hcclBuff.addr;
+    const u64 size = mb.size[me];
+
+    if (size != 0) {   // own shard into its slot
+        CHK_RET(LocalCopy(res.threads[0], DataSlice(in, mb.userInputOffsets[me], size),
+                          DataSlice(ccl, mb.outputOffsets[CalcOutputIndex(me, me)], size)));
+    }
+    CHK_RET(PreSync(res.threads));
+    u32 que = 1;
+    for (u32 i = 1; i < n; ++i) {   // all-to-all: shard `next` goes to rank `next`, into the slot of this rank
+        const u32 next = (me + i) % n;
+        const auto ch = res.channels.find(subCommRanks_[0][next]);
+        CHK_PRT_RET(ch == res.channels.end() || ch->second.empty(), HCCL_ERROR("[RS order preserved] channel not found"),
+                    HCCL_E_INTERNAL);
+        const ChannelInfo &link = ch->second[0];
+        DataSlice txSrc(in, mb.userInputOffsets[next], mb.size[next]);
+        DataSlice txDst(link.remoteCclMem.addr, mb.outputOffsets[CalcOutputIndex(next, me)], mb.size[next]);
+        SendRecvInfo info{{link, link}, {{{txSrc}, {txDst}}, {{}, {}}}, dataType_};
+        CHK_RET(SendRecvWrite(info, res.threads[threadNum_ > 1 ? que : 0]));
+        if (++que >= threadNum_) que = 1;
+    }
+    CHK_RET(PostSync(res.threads));
+    if (dataType_ == HCCL_DATA_TYPE_FP64 || reduceOp_ == HCCL_REDUCE_PROD) {
+        CHK_RET(HcommBatchModeEnd(param.algTag.c_str()));
+        CHK_RET(HcommBatchModeStart(param.algTag.c_str()));
+        for (ThreadHandle t : res.threads) CHK_RET(HcommThreadJoin(t, CUSTOM_TIMEOUT));
+    }
+
+    // the tree: block v of this rank sits in slot (v + me) % n
+    u32 remaining = n;
+    while (remaining > 1 && size != 0) {
+        u32 m = 1;
+        while (m * 2 < remaining) m *= 2;   // largest power of two below `remaining`
+        for (u32 v = m; v < remaining; ++v) {
+            DataSlice src(ccl, mb.outputOffsets[CalcOutputIndex(v, me)], size, size / esz);
+            DataSlice dst(ccl, mb.outputOffsets[CalcOutputIndex(v % m, me)], size, size / esz);
+            CHK_RET(LocalReduce(res.threads[0], src, dst, dataType_, reduceOp_));
+        }
+        remaining = m;
+    }
+    if (size != 0) {
+        CHK_RET(LocalCopy(res.threads[0], DataSlice(ccl, mb.outputOffsets[CalcOutputIndex(0, me)], size),
+                          DataSlice(p.buffInfo.outputPtr, p.buffInfo.outBuffBaseOff, size)));
     }
     return HCCL_SUCCESS;
 }

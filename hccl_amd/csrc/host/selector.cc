@@ -1,5 +1,7 @@
 #include "selector.h"
 
+#include "alg_env_config.h"
+
 namespace ops_hccl {
 
 SelectorRegistry *SelectorRegistry::Global()
@@ -90,6 +92,13 @@ protected:
     SelectorStatus SelectAicpuAlgo(const TopoInfoWithNetLayerDetails *topo, const OpParam &p,
                                    std::string &name) const override
     {
+        if (IsNeedStrictModeForOrderPreserved(p.DataDes.dataType, p.reduceType, topo->userRankSize)) {
+            // strict determinism (:337-347): an all-to-all of the shards, then a fixed tree over the ranks.
+            // The grouped variant for more than 32 ranks is not built.
+            if (topo->userRankSize > MAX_RANK_NUM_FOR_ORDER_PRESERVED) return SelectorStatus::NOT_MATCH;
+            name = "ReduceScatterOrderPreserved";
+            return SelectorStatus::MATCH;
+        }
         if (topo->topoLevelNums > 1 || topo->level0Topo == Level0Shape::CLOS) {
             // The reference picks InsReduceScatterAicpuReduceNHR for PROD / 64-bit here (:350, :430);
             // its fold order is the NHR gather followed by the own-data-first fold, which is what

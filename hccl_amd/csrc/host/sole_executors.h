@@ -6,6 +6,7 @@
 #pragma once
 #include <algorithm>
 
+#include "data_move_templates.h"
 #include "executor.h"
 
 namespace ops_hccl {
@@ -355,5 +356,65 @@ public:
 
 // Names as the reference registers them (e.g. ins_v2_reduce_scatter_sole_executor.cc:256-265); the two
 // documentation-derived AllReduce templates are added under their own names.
+
+// ---------------------------------------------------------------------------------------------------
+// Order-preserved ReduceScatter
+// (src/ops/reduce_scatter/executor/ins_v2_reduce_scatter_order_preserved_executor.cc:77-186): the chunk loop of
+// the sole executor with the whole scratch buffer, the 256 MiB transport bound and a table of where each
+// rank's block sits in this loop.
+// ---------------------------------------------------------------------------------------------------
+template <typename AlgTopoMatch, typename InsAlgTemplate>
+class InsV2ReduceScatterOrderPreservedExecutor : public InsCollAlgBase {
+public:
+    std::string Describe() const override { return "ReduceScatter order-preserved executor"; }
+    u64 CalcThreadNum(const OpParam &param, u32 rank, u32 rankSize) override
+    {
+        InsAlgTemplate t(param, rank, AlgTopoMatch::Match(rankSize));
+        return t.GetThreadNum();
+    }
+    HcclResult Orchestrate(const OpParam &param, const AlgResourceCtxSerializable &resCtx) override
+    {
+        myRank_ = resCtx.topoInfo.userRank;
+        rankSize_ = resCtx.topoInfo.userRankSize;
+        dataType_ = param.DataDes.dataType;
+        dataTypeSize_ = DATATYPE_SIZE_TABLE[dataType_];
+        dataCount_ = param.DataDes.count;
+        dataSize_ = dataCount_ * dataTypeSize_;
+        TemplateResource res;
+        TemplateDataParams t;
+        detail::FillBuffInfo(param, resCtx, t, res);
+        InsAlgTemplate alg(param, myRank_, resCtx.subCommRanks);
+        const u64 mult = alg.CalcScratchMultiple(t.buffInfo.inBuffType, t.buffInfo.outBuffType);
+        maxTmpMemSize_ = t.buffInfo.hcclBuff.size;
+        const u64 maxCount = MaxDataSizePerLoop(maxTmpMemSize_, mult, UB_MAX_DATA_SIZE) / dataTypeSize_;
+        CHK_PRT_RET(maxCount == 0, HCCL_ERROR("[ReduceScatter order-preserved executor] maxDataCountPerLoop is 0"),
+                    HCCL_E_INTERNAL);
+        const u64 loops = dataCount_ / maxCount + (dataCount_ % maxCount != 0);
+        u64 done = 0;
+        for (u64 loop = 0; loop < loops; ++loop) {
+            const u64 cur = (loop == loops - 1) ? dataCount_ - done : maxCount;
+            const u64 blockSize = cur * dataTypeSize_;
+            t.count = cur;
+            t.buffInfo.inBuffBaseOff = done * dataTypeSize_;
+            t.buffInfo.outBuffBaseOff = done * dataTypeSize_;
+            t.buffInfo.hcclBuffBaseOff = 0;
+            MemBlockInfo blocks;
+            for (u32 k = 0; k < rankSize_; ++k) {
+                blocks.size.push_back(blockSize);
+                blocks.userInputOffsets.push_back(done * dataTypeSize_ + k * dataSize_);
+                blocks.inputOffsets.push_back(k * blockSize);
+                blocks.outputOffsets.push_back(k * blockSize);
+            }
+            t.sliceSize = blockSize;
+            t.tailSize = blockSize;
+            t.inputSliceStride = dataSize_;
+            t.outputSliceStride = 0;
+            alg.SetMemBlockInfo(blocks);
+            CHK_RET(alg.KernelRun(param, t, res));
+            done += cur;
+        }
+        return HCCL_SUCCESS;
+    }
+};
 
 }  // namespace ops_hccl

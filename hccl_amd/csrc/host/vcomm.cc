@@ -118,6 +118,16 @@ HcclResult WorldCreate(u32 rankSize, u64 cclBytes, bool dryRun, std::vector<Hccl
     }
     if (const char *b = std::getenv("HCCL_VRANK_BLOCKING")) w->blocking = (std::atoi(b) != 0);
     if (const char *c = std::getenv("HCCL_VRANK_CHECK")) w->check = (std::atoi(c) != 0);
+    {
+        u8 level = static_cast<u8>(DeterministicEnableLevel::DETERMINISTIC_DISABLE);
+        if (const char *d = std::getenv("HCCL_DETERMINISTIC")) {
+            if (ParseDeterministic(d, level) != HCCL_SUCCESS) {
+                delete w;
+                return HCCL_E_PARA;
+            }
+        }
+        SetExternalInputHcclDeterministic(level);
+    }
     if (const char *a = std::getenv("HCCL_ALGO")) {
         const HcclResult rc = SetHcclAlgoConfig(a, w->algoConfig);
         if (rc != HCCL_SUCCESS) {

@@ -21,6 +21,8 @@ Reference followed (paths relative to the reference tree, src/ops/...):
   allreduce_aicpu_reduce_nhr   all_reduce/template/aicpu/ins_temp_all_reduce_aicpu_reduce_nhr.cc:65-271
   reduce_scatter_mesh          reduce_scatter/template/aicpu/ins_temp_reduce_scatter_mesh_1D.cc:65-227
   reduce_scatter_nhr           reduce_scatter/template/aicpu/ins_temp_reduce_scatter_nhr.cc:77-425
+  reduce_scatter_order_preserved  reduce_scatter/template/aicpu/ins_temp_reduce_scatter_order_preserved_level1.cc:52-330,
+                               executor reduce_scatter/executor/ins_v2_reduce_scatter_order_preserved_executor.cc:77-186
   reduce_scatter_mesh_chunk    reduce_scatter/template/aicpu/ins_temp_reduce_scatter_mesh_1D_meshchunk.cc:69-263
   allreduce_mesh_two_shot_mesh_chunk  all_reduce/template/aicpu/ins_temp_all_reduce_mesh_1D_two_shot_mesh_chunk.cc:49-336
   reduce_scatter_v_mesh        reduce_scatter_v/template/aicpu/ins_temp_reduce_scatter_v_mesh_1D.cc:50-179,
@@ -597,10 +599,33 @@ def reduce_scatter_mesh_chunk(w, base, count, stride):
         e.copy(w.out[r], base, w.ccl[r], 0, count)
 
 
+def reduce_scatter_order_preserved(w, base, count, stride):
+    """Strict determinism: all-to-all of the shards into scratch slots (the block from rank k sits in slot
+    (k + r) % n of rank r), then a tree that is the same on every rank: with m the largest power of two below
+    the number of remaining blocks, block v >= m is folded into block v % m
+    (ins_temp_reduce_scatter_order_preserved_level1.cc:170-330)."""
+    n, e = w.n, w.e
+    w.need_ccl(max(count, 1) * n)
+    for r in range(n):                                   # PreLocalCopy + RunAllToAll
+        for k in range(n):
+            e.copy(w.ccl[k], ((r + k) % n) * count, w.inp[r], k * stride + base, count)
+    for r in range(n):                                   # RunLocalReduce
+        remaining = n
+        while remaining > 1:
+            m = 1
+            while m * 2 < remaining:
+                m *= 2
+            for v in range(m, remaining):
+                e.reduce(w.ccl[r], ((v % m + r) % n) * count, w.ccl[r], ((v + r) % n) * count, count)
+            remaining = m
+        e.copy(w.out[r], base, w.ccl[r], (r % n) * count, count)    # PostCopy: block 0
+
+
 REDUCE_SCATTER_TEMPLATES = {
     "InsReduceScatterMesh1D": (reduce_scatter_mesh, lambda n: n),   # mesh_1D.cc:59-63
     "InsReduceScatterNHR": (reduce_scatter_nhr, lambda n: n),       # nhr.cc:369-377
     "InsReduceScatterMesh1DMeshChunk": (reduce_scatter_mesh_chunk, lambda n: n - 1),   # meshchunk.cc:46-52
+    "ReduceScatterOrderPreserved": (reduce_scatter_order_preserved, lambda n: n),      # level1.cc:46-50
 }
 
 
@@ -608,7 +633,10 @@ def run_reduce_scatter(elems, inputs, recv_count, esz, alg, ccl_bytes=CCL_BYTES_
     fn, mult = REDUCE_SCATTER_TEMPLATES[alg]
     w = World(elems, inputs, recv_count, esz, ccl_bytes)
     usable = ccl_bytes - 1024 * 1024          # ins_v2_reduce_scatter_sole_executor.cc:126-128
-    for base, cur in chunk_counts(recv_count, usable, mult(w.n), esz, usable):
+    bound = usable
+    if alg == "ReduceScatterOrderPreserved":  # its own executor: whole buffer, 256 MiB transport bound
+        usable, bound = ccl_bytes, UB_MAX_DATA_SIZE   # ins_v2_reduce_scatter_order_preserved_executor.cc:108-119
+    for base, cur in chunk_counts(recv_count, usable, mult(w.n), esz, bound):
         fn(w, base, cur, recv_count)          # inputSliceStride = recvCount * esz (:160)
     return w.out
 

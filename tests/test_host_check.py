@@ -213,3 +213,32 @@ def test_hccl_algo_environment_override(monkeypatch):
         assert e.value.code == 1, bad
     monkeypatch.setenv("HCCL_ALGO", "  ")
     assert run_ar(8, 1000, T.FP32, T.SUM) == "InsAllReduceMesh1DOneShot"
+
+
+def test_strict_determinism_selects_the_order_preserved_reduce_scatter(monkeypatch):
+    """HCCL_DETERMINISTIC=strict (alg_env_config.cc:948-990): floating-point SUM / PROD among more than two ranks
+    take the order-preserved template (reduce_scatter_auto_selector.cc:337-347, order_preserved_common.h:63-76)."""
+    def pick_rs(n, dtype, op):
+        w = api.World(n, ccl_bytes=SMALL_CCL, dry=True)
+        try:
+            ins, outs = fake_ptrs(n)
+            rc = 0
+            for r in range(n):
+                rc = w.reduce_scatter(r, ins[r], outs[r], 1000, dtype, op, FAKE_STREAM)
+            return rc, w.last_info().algName.decode()
+        finally:
+            w.close()
+
+    monkeypatch.setenv("HCCL_DETERMINISTIC", "Strict")
+    assert pick_rs(8, T.BFP16, T.SUM) == (0, "ReduceScatterOrderPreserved")
+    assert pick_rs(5, T.FP64, T.PROD) == (0, "ReduceScatterOrderPreserved")
+    assert pick_rs(8, T.FP32, T.MAX) == (0, "InsReduceScatterMesh1D")          # max / min need no order
+    assert pick_rs(8, T.INT32, T.SUM) == (0, "InsReduceScatterMesh1D")         # integers neither
+    assert pick_rs(2, T.FP32, T.SUM) == (0, "InsReduceScatterMesh1D")          # two ranks: one pairwise op
+    assert pick_rs(33, T.FP32, T.SUM)[0] == 5                                  # the grouped variant is not built
+    monkeypatch.setenv("HCCL_DETERMINISTIC", "true")
+    assert pick_rs(8, T.BFP16, T.SUM) == (0, "InsReduceScatterMesh1D")
+    monkeypatch.setenv("HCCL_DETERMINISTIC", "sometimes")
+    with pytest.raises(_lib.HcclError) as e:
+        api.World(2, ccl_bytes=SMALL_CCL, dry=True)
+    assert e.value.code == 1

@@ -377,3 +377,28 @@ def test_moe_dispatch_alltoallv_and_back_is_the_identity():
             mine = toks[i][dests[i] == j].reshape(-1)
             assert np.array_equal(recv[j][pos:pos + mine.size], mine)
             pos += mine.size
+
+
+def test_order_preserved_tree_is_the_same_on_every_rank():
+    """Strict determinism: the association over the ranks' blocks does not depend on the rank that owns the
+    shard.  Hand-worked from the fold rule (upper blocks onto block v % m): 8 ranks and 12 ranks."""
+    want = {
+        3: "(x1+(x2+x0))",
+        8: "(((x7+x3)+(x5+x1))+((x6+x2)+(x4+x0)))",
+    }
+    for n in (3, 8):
+        outs = T.run_reduce_scatter(T.SymbolicElems(), sym_inputs(n, n * 2), 2, 4, "ReduceScatterOrderPreserved")
+        for r in range(n):
+            assert outs[r][0] == want[n], (n, r, outs[r][0])
+    # 12 ranks: blocks 8..11 fold onto 0..3 first, then 4..7 onto 0..3, then 2,3 onto 0,1, then 1 onto 0
+    outs = T.run_reduce_scatter(T.SymbolicElems(), sym_inputs(12, 12), 1, 4, "ReduceScatterOrderPreserved")
+    b = [f"x{k}" for k in range(12)]
+    for v in range(8, 12):
+        b[v - 8] = f"({b[v]}+{b[v - 8]})"
+    for v in range(4, 8):
+        b[v - 4] = f"({b[v]}+{b[v - 4]})"
+    for v in range(2, 4):
+        b[v - 2] = f"({b[v]}+{b[v - 2]})"
+    b[0] = f"({b[1]}+{b[0]})"
+    for r in range(12):
+        assert outs[r][0] == b[0]
