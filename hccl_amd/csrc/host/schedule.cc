@@ -2,6 +2,7 @@
 
 #include <algorithm>
 #include <cstring>
+#include <functional>
 #include <map>
 #include <sstream>
 #include <unordered_map>
@@ -749,16 +750,27 @@ void CheckSemantics(const Tracer &tr, const std::vector<OpParam> &params, CheckR
     }
 }
 
-std::string PlanKey(const std::vector<OpParam> &params, const std::string &alg, u64 cclBytes)
+// What a cached plan depends on, as plain numbers (a string would cost more to build than the launch).
+std::vector<u64> PlanKey(const std::vector<OpParam> &params, const std::string &alg, u64 cclBytes)
 {
-    std::ostringstream os;
     const OpParam &p0 = params[0];
-    os << static_cast<int>(p0.opType) << "|" << alg << "|" << p0.DataDes.dataType << "|" << p0.reduceType << "|"
-       << p0.DataDes.count << "|" << cclBytes;
-    for (u64 c : p0.vDataDes.counts) os << "|c" << c;
-    for (u64 d : p0.vDataDes.displs) os << "|d" << d;
-    for (const OpParam &p : params) os << "|" << p.inputPtr << "," << p.outputPtr << "," << p.inputSize;
-    return os.str();
+    std::vector<u64> key;
+    key.reserve(8 + 2 * p0.vDataDes.counts.size() + 3 * params.size());
+    key.push_back(static_cast<u64>(p0.opType));
+    key.push_back(std::hash<std::string>()(alg));
+    key.push_back(static_cast<u64>(p0.DataDes.dataType));
+    key.push_back(static_cast<u64>(p0.reduceType));
+    key.push_back(p0.DataDes.count);
+    key.push_back(cclBytes);
+    key.push_back(p0.vDataDes.counts.size());
+    key.insert(key.end(), p0.vDataDes.counts.begin(), p0.vDataDes.counts.end());
+    key.insert(key.end(), p0.vDataDes.displs.begin(), p0.vDataDes.displs.end());
+    for (const OpParam &p : params) {
+        key.push_back(reinterpret_cast<u64>(p.inputPtr));
+        key.push_back(reinterpret_cast<u64>(p.outputPtr));
+        key.push_back(p.inputSize);
+    }
+    return key;
 }
 
 HcclResult LaunchPlans(World *w, const std::vector<hcclx_plan *> &plans, void *stream)
@@ -931,7 +943,7 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
         w->lastWasFused = true;
         return LaunchDataMove(w, params, stream);
     }
-    std::string key;
+    std::vector<u64> key;
     if (fused && !w->dryRun && !w->traceText && !w->check) {
         key = PlanKey(params, algName, w->cclBytes);
         for (CachedPlan &c : w->planCache) {

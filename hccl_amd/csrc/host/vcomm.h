@@ -68,7 +68,7 @@ struct QueuedOp {
 };
 
 struct CachedPlan {
-    std::string key;
+    std::vector<u64> key;
     std::vector<hcclx_plan *> plans;
     u64 lastUse = 0;
 };
