@@ -24,6 +24,7 @@ namespace hcclx {
 #define HCCLX_FOLD_THREADS 256
 #endif
 constexpr int kFoldThreads = HCCLX_FOLD_THREADS;
+constexpr uint32_t kFoldDirectSegs = 64;   // up to this many segments the tile prefix is searched in place
 __host__ __device__ constexpr int fold_unroll(int maxn)
 {
     constexpr int u[5] = {HCCLX_FOLD_UNROLLS};
@@ -128,8 +129,11 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
                 }
             }
             const u32x4 out = V::pack(acc);
-            for (uint32_t d = 0; d < ndst; ++d) {
-                st16(sd.dst[d] + head_bytes + vi * 16, out);
+            // a constant trip count with a uniform guard: the destination pointers are then fetched in one
+            // batch of scalar loads instead of one dependent load per iteration
+#pragma unroll
+            for (int d = 0; d < kMaxFan; ++d) {
+                if (d < static_cast<int>(ndst)) st16(sd.dst[d] + head_bytes + vi * 16, out);
             }
         } else if constexpr (MODE == kFoldTree) {
             C val[MAXN][NE];
@@ -139,8 +143,11 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
             }
             tree_eval<DT, OP, MAXN, C, NE>(val, sd.tree_codes);
             const u32x4 out = V::pack(val[0]);
-            for (uint32_t d = 0; d < ndst; ++d) {
-                st16(sd.dst[d] + head_bytes + vi * 16, out);
+            // a constant trip count with a uniform guard: the destination pointers are then fetched in one
+            // batch of scalar loads instead of one dependent load per iteration
+#pragma unroll
+            for (int d = 0; d < kMaxFan; ++d) {
+                if (d < static_cast<int>(ndst)) st16(sd.dst[d] + head_bytes + vi * 16, out);
             }
         } else {
             C val[MAXN][NE];
@@ -213,25 +220,45 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
     constexpr int NE = Vec16<DT>::kElems;   // elements per 16-byte vector
     constexpr uint64_t TV = fold_tile_vecs(MAXN);
     extern __shared__ uint64_t s_end[];  // nseg entries, sized by the launcher
-    for (uint32_t i = threadIdx.x; i < nseg; i += kFoldThreads) {
-        s_end[i] = tile_end[i];
+    // Few segments: the prefix is searched where it lies (every index is wave-uniform, so these are scalar
+    // loads that hit the constant cache after the first workgroup); staging it in LDS would cost a barrier
+    // before the first data load.  Many segments: staged once per workgroup.
+    const bool direct = nseg <= kFoldDirectSegs;
+    if (!direct) {
+        for (uint32_t i = threadIdx.x; i < nseg; i += kFoldThreads) {
+            s_end[i] = tile_end[i];
+        }
+        __syncthreads();
     }
-    __syncthreads();
 
     for (uint64_t t = blockIdx.x; t < total_tiles; t += gridDim.x) {
         // first segment whose inclusive tile prefix exceeds t
         uint32_t lo = 0;
         uint32_t hi = nseg - 1;
-        while (lo < hi) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if (s_end[mid] > t) {
-                hi = mid;
-            } else {
-                lo = mid + 1;
+        uint64_t before = 0;   // tiles of the segments in front of the one found
+        if (direct) {
+            while (lo < hi) {
+                const uint32_t mid = (lo + hi) >> 1;
+                if (tile_end[mid] > t) {
+                    hi = mid;
+                } else {
+                    lo = mid + 1;
+                }
             }
+            before = lo ? tile_end[lo - 1] : 0;
+        } else {
+            while (lo < hi) {
+                const uint32_t mid = (lo + hi) >> 1;
+                if (s_end[mid] > t) {
+                    hi = mid;
+                } else {
+                    lo = mid + 1;
+                }
+            }
+            before = lo ? s_end[lo - 1] : 0;
         }
         const uint32_t s = __builtin_amdgcn_readfirstlane(lo);
-        const uint64_t tl = uniform64(t - (s ? s_end[s - 1] : 0));
+        const uint64_t tl = uniform64(t - before);
         const SegDev &sd = segs[s];
         const uint32_t nsrc = sd.nsrc;
         const uint32_t ndst = sd.ndst;
