@@ -73,7 +73,7 @@ def _randn_bits16(torch, n, seed, dt):
 
 
 class ReduceScatterMesh(Workload):
-    """BASELINE config 2: HcclReduceScatter SUM bf16, 8 ranks x 33,554,432 elements in (64 MiB per rank).
+    """benchmark configuration 2: HcclReduceScatter SUM bf16, 8 ranks x 33,554,432 elements in (64 MiB per rank).
     The selector picks the mesh template; output shard r folds slice r of every rank starting from rank
     r's own data, then ranks ascending (ins_temp_reduce_scatter_mesh_1D.cc:132-154), as one fused pass."""
     dtype = "bf16"
@@ -179,7 +179,7 @@ class AllGather(Workload):
 
 
 class AllGatherV(Workload):
-    """BASELINE config 3: HcclAllGatherV fp16, 16 ranks, per-rank counts uniform in [0, 8,388,608] from a
+    """benchmark configuration 3: HcclAllGatherV fp16, 16 ranks, per-rank counts uniform in [0, 8,388,608] from a
     seed, displacements their prefix sum (so most blocks start at addresses that are only 2-byte aligned)."""
     dtype = "u8"
     kernel = "hcclx::(anonymous namespace)::k_allgatherv"
@@ -209,7 +209,7 @@ class AllGatherV(Workload):
 
 
 class AllToAllV(Workload):
-    """BASELINE config 4: HcclAlltoAllV bf16, MoE dispatch: 8 ranks x 4096 tokens x hidden 7168,
+    """benchmark configuration 4: HcclAlltoAllV bf16, MoE dispatch: 8 ranks x 4096 tokens x hidden 7168,
     destination rank per token Zipf(s=1.2), tokens grouped by destination."""
     dtype = "u8"
     kernel = "hcclx::(anonymous namespace)::k_alltoallv_direct<2>"
@@ -251,7 +251,7 @@ class _NoWorld:
 
 
 class MoeDispatchPack(Workload):
-    """The caller side of BASELINE config 4, timed on its own: per-token destinations (Zipf 1.2) -> AlltoAllV
+    """The caller side of benchmark configuration 4, timed on its own: per-token destinations (Zipf 1.2) -> AlltoAllV
     tables and the stable row permutation (hcclx_moe_route), then the row gather that packs the send buffers
     (hcclx_moe_pack); 8 ranks x 4096 tokens x hidden 7168 bf16.  Algorithmic bytes: every token row read once
     and written once."""
@@ -340,7 +340,7 @@ WORKLOADS = {
     "all_gather_fp16_8x64MiB": lambda *a: AllGather(*a),
     "all_to_all_v_bf16_moe_8x4096x7168": lambda *a: AllToAllV(*a),
     "all_gather_v_fp16_16_ranks_ragged": lambda *a: AllGatherV(*a),
-    # BASELINE config 1 (ring template, 8 x 1,048,576 fp32): one fused pass, and every step of the ring
+    # benchmark configuration 1 (ring template, 8 x 1,048,576 fp32): one fused pass, and every step of the ring
     # launched through the scratch buffers (the step-faithful variant, with the ring's own larger traffic)
     "all_reduce_sum_fp32_8x4MiB_ring": lambda *a: AllReduce(*a, count=1048576, alg="InsAllReduceRing"),
     "all_reduce_sum_fp32_8x4MiB_ring_step_by_step": lambda *a: AllReduce(*a, count=1048576, alg="InsAllReduceRing",
@@ -353,7 +353,7 @@ EXTRA_WORKLOADS = {"copy_calibration_1024MiB": lambda *a: CopyCalibration(*a)}
 
 
 def sweep_allreduce_12_ranks(torch, api, T, steps):
-    """BASELINE config 5: AllReduce on 12 ranks, 4 KiB ... 1 GiB per rank in powers of 4; int32 MAX through the
+    """benchmark configuration 5: AllReduce on 12 ranks, 4 KiB ... 1 GiB per rank in powers of 4; int32 MAX through the
     NHR and halving-doubling templates, fp32 PROD through the CPU-reduce NHR template (what the selector
     takes for PROD) and halving-doubling.  Small sizes are bound by the launch, so microseconds are reported
     beside GB/s (algorithmic bytes = 2 * 12 * size)."""
