@@ -73,7 +73,7 @@ uint64_t hcclxCommGetLastTrace(HcclComm comm, char *buf, uint64_t size);
  * (2) no two steps that the handshakes leave unordered touch the same bytes with at least one of them writing
  * (check_rank_mem / the task-graph race rules), (3) every output piece is what the collective's contract says:
  * reduced from each rank exactly once at the matching offset, or copied from the right rank and offset
- * (semantics_check/*_semantics_checker.cc).  A collective that fails returns HCCL_E_INTERNAL and launches
+ * (semantics_check/<op>_semantics_checker.cc).  A collective that fails returns HCCL_E_INTERNAL and launches
  * nothing.  Checked collectives bypass the plan cache. */
 typedef struct {
     uint32_t steps, levels, copies, reduces;

@@ -40,6 +40,57 @@ def test_every_declared_function_is_exported():
     assert len(names) >= 45
 
 
+C_PROGRAM = r'''
+#include <stdio.h>
+#include <stdint.h>
+#include "hccl.h"
+#include "hccl_comm.h"
+#include "hcclx.h"
+#include "hcomm_primitives.h"
+int main(void)
+{
+    HcclComm comm[4];
+    uint32_t n = 0, id = 9;
+    char trace[4096];
+    hcclxLastOpInfo info;
+    hcclxCheckReport rep;
+    if (hcclxCommInitAll(4, 0, 1, comm) != HCCL_SUCCESS) return 1;
+    if (HcclGetRankSize(comm[2], &n) != HCCL_SUCCESS || n != 4) return 2;
+    if (HcclGetRankId(comm[2], &id) != HCCL_SUCCESS || id != 2) return 3;
+    hcclxCommSetCheck(comm[0], 1);
+    hcclxCommSetTrace(comm[0], 1);
+    for (int r = 0; r < 4; ++r) {
+        void *in = (void *)(uintptr_t)(0x100000000000ull + (uint64_t)r * 0x1000000000ull);
+        void *out = (void *)(uintptr_t)(0x200000000000ull + (uint64_t)r * 0x1000000000ull);
+        if (HcclAllReduce(in, out, 1000, HCCL_DATA_TYPE_FP32, HCCL_REDUCE_SUM, comm[r], (aclrtStream)1) != HCCL_SUCCESS) return 4;
+    }
+    hcclxCommGetLastOpInfo(comm[0], &info);
+    hcclxCommGetLastCheck(comm[0], &rep);
+    hcclxCommGetLastTrace(comm[0], trace, sizeof(trace));
+    printf("%s fused=%d steps=%u races=%u semantic=%u\n%.60s\n", info.algName, info.fused, rep.steps, rep.races, rep.semanticErrors, trace);
+    if (HcclAllReduce(0, 0, 1000, HCCL_DATA_TYPE_FP32, HCCL_REDUCE_SUM, comm[0], (aclrtStream)1) != HCCL_E_PTR) return 5;
+    for (int r = 0; r < 4; ++r) HcclCommDestroy(comm[r]);
+    return (rep.races == 0 && rep.semanticErrors == 0) ? 0 : 6;
+}
+'''
+
+
+def test_headers_are_plain_c_and_a_c_program_drives_a_dry_world(tmp_path):
+    """gcc -std=c99 -pedantic -Werror on all four headers; the program makes a dry world of four ranks, runs a
+    checked and traced HcclAllReduce, and reads the reports back."""
+    import subprocess
+    c = tmp_path / "c_abi.c"
+    c.write_text(C_PROGRAM)
+    exe = tmp_path / "c_abi"
+    lib_dir = os.path.dirname(_lib.LIB_PATH)
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
+                           str(c), "-o", str(exe), "-L", lib_dir, "-lhccl_amd", "-Wl,-rpath," + lib_dir])
+    out = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "InsAllReduceMesh1DOneShot fused=1" in out.stdout and "races=0 semantic=0" in out.stdout
+    assert "rank 0 out[0,4000) = (x3@0+(x2@0+(x1@0+x0@0)))" in out.stdout
+
+
 def test_no_compute_entry_point_runs_without_a_gpu_silently():
     """Without a GPU the kernel layer reports an error instead of falling back to anything."""
     import torch
