@@ -146,7 +146,7 @@ std::string AlgNameFromConfig(const HcclAlgoConfig &config, HcclCMDType type, bo
             return "";   // fullmesh: the selector's one-shot / two-shot / chunked choice by size
         case HcclCMDType::HCCL_CMD_REDUCE_SCATTER:
             if (algo == HcclAlgoType::HCCL_ALGO_TYPE_NHR || algo == HcclAlgoType::HCCL_ALGO_TYPE_NHR_V1) {
-                return cpuReduce ? "" : "InsReduceScatterNHR";
+                return cpuReduce ? "InsReduceScatterAicpuReduceNHR" : "InsReduceScatterNHR";
             }
             return "";
         case HcclCMDType::HCCL_CMD_ALLGATHER:

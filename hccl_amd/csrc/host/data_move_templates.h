@@ -9,6 +9,8 @@ namespace ops_hccl {
 HCCL_DECLARE_TEMPLATE(InsTempReduceScatterMesh1D, "ReduceScatter mesh 1D",
                       (templateRankSize_ > 1 ? templateRankSize_ : 1), templateRankSize_);
 HCCL_DECLARE_TEMPLATE(InsTempReduceScatterNHR, "ReduceScatter NHR", 1, templateRankSize_);
+// reduce_scatter aicpu_reduce_nhr.cc:46-50, :242-249: one thread, N scratch slots
+HCCL_DECLARE_TEMPLATE(InsTempReduceScatterAicpuReduceNHR, "ReduceScatter NHR gather + local reduce", 1, templateRankSize_);
 // reduce_scatter_v mesh_1D.cc:26-48: N-1 threads (the main thread sends too), N scratch slots
 HCCL_DECLARE_TEMPLATE(InsTempReduceScatterVMesh1D, "ReduceScatterV mesh 1D",
                       (templateRankSize_ > 1 ? templateRankSize_ - 1 : 1), templateRankSize_);

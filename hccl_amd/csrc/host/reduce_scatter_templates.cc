@@ -2,6 +2,7 @@
 // (src/ops/reduce_scatter/template/aicpu/):
 //   InsTempReduceScatterMesh1D   ins_temp_reduce_scatter_mesh_1D.cc:65-227
 //   InsTempReduceScatterNHR      ins_temp_reduce_scatter_nhr.cc:77-425
+//   InsTempReduceScatterAicpuReduceNHR   ins_temp_reduce_scatter_aicpu_reduce_nhr.cc:52-300
 //   InsTempReduceScatterOrderPreservedLevel1   ins_temp_reduce_scatter_order_preserved_level1.cc:52-330
 // and src/ops/reduce_scatter_v/template/aicpu/:
 //   InsTempReduceScatterVMesh1D  ins_temp_reduce_scatter_v_mesh_1D.cc:50-179
@@ -83,6 +84,75 @@ HcclResult InsTempReduceScatterMesh1D::KernelRun(const OpParam &param, const Tem
             DataSlice src(p.buffInfo.hcclBuff.addr, p.buffInfo.hcclBuffBaseOff + rpt * p.outputRepeatStride + k * size,
                           size, count);
             CHK_RET(LocalReduce(threads[0], src, dst, dataType_, reduceOp_));
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
+// One round per shard: every rank puts its copy of shard k into slot <own rank> of its scratch, the NHR
+// all-gather steps spread the slots until every rank holds all N copies, and rank k alone folds them: own
+// input first, then the slots of the other ranks ascending.  N all-gathers move N times the data a
+// reduce-scatter needs; the reference accepts that for PROD and 64-bit types, which its CPU has to reduce.
+HcclResult InsTempReduceScatterAicpuReduceNHR::KernelRun(const OpParam &param, const TemplateDataParams &p,
+                                                         TemplateResource &res)
+{
+    CHK_PRT_RET(res.threads.empty(), HCCL_ERROR("[RS AicpuReduceNHR] no thread"), HCCL_E_INTERNAL);
+    if (p.sliceSize == 0) return HCCL_SUCCESS;
+    dataType_ = param.DataDes.dataType;
+    const u32 n = templateRankSize_;
+    u32 me = 0;
+    CHK_RET(GetAlgRank(myRank_, subCommRanks_[0], me));
+    const ThreadHandle th = res.threads[0];
+    void *ccl = p.buffInfo.hcclBuff.addr;
+    const u64 size = p.sliceSize;
+    const u64 count = p.count;
+    const u64 rpts = p.repeatNum > 1 ? p.repeatNum : 1;
+    auto slot = [&](void *buf, u64 rpt, u32 k) {  // :250-262: scratch repeats are N slots apart
+        return DataSlice(buf, p.buffInfo.hcclBuffBaseOff + rpt * size * n + k * size, size, count);
+    };
+    std::vector<NHRStepInfo> steps;
+    if (n > 1) GetNHRAllGatherSteps(n, me, steps);  // GetStepInfo :268-300
+
+    for (u32 shard = 0; shard < n; ++shard) {
+        for (u64 rpt = 0; rpt < rpts; ++rpt) {  // LocalDataCopy :82-113
+            const u64 inOff = p.buffInfo.inBuffBaseOff + rpt * p.inputRepeatStride + shard * p.inputSliceStride;
+            const u64 scOff = p.buffInfo.hcclBuffBaseOff + rpt * p.outputRepeatStride + me * size;
+            if (p.buffInfo.inBuffType != p.buffInfo.hcclBuffType || inOff != scOff) {
+                CHK_RET(LocalCopy(th, DataSlice(p.buffInfo.inputPtr, inOff, size, count), DataSlice(ccl, scOff, size, count)));
+            }
+            if (shard != me) continue;  // LocalCopyToOutput :115-138
+            const u64 outOff = p.buffInfo.outBuffBaseOff + rpt * p.outputRepeatStride;
+            if (p.buffInfo.inBuffType != p.buffInfo.outBuffType || inOff != outOff) {
+                CHK_RET(LocalCopy(th, DataSlice(p.buffInfo.inputPtr, inOff, size, count),
+                                  DataSlice(p.buffInfo.outputPtr, outOff, size, count)));
+            }
+        }
+        for (const NHRStepInfo &st : steps) {  // RunAllGather :180-240
+            const ChannelInfo &recv = res.channels.at(subCommRanks_[0][st.fromRank]).at(0);
+            const ChannelInfo &send = res.channels.at(subCommRanks_[0][st.toRank]).at(0);
+            std::vector<DataSlice> txSrc, txDst, rxSrc, rxDst;
+            for (u64 rpt = 0; rpt < rpts; ++rpt) {
+                for (u32 i = 0; i < st.nSlices; ++i) {
+                    txSrc.push_back(slot(ccl, rpt, st.txSliceIdxs[i]));
+                    txDst.push_back(slot(send.remoteCclMem.addr, rpt, st.txSliceIdxs[i]));
+                    rxSrc.push_back(slot(recv.remoteCclMem.addr, rpt, st.rxSliceIdxs[i]));
+                    rxDst.push_back(slot(ccl, rpt, st.rxSliceIdxs[i]));
+                }
+            }
+            SendRecvInfo info{{send, recv}, {{txSrc, txDst}, {rxSrc, rxDst}}};
+            CHK_RET(SendRecvWrite(info, th));
+        }
+        CHK_RET(HcommBatchModeEnd(param.algTag.c_str()));  // :66-70: the CPU fold needs the data to have landed
+        CHK_RET(HcommBatchModeStart(param.algTag.c_str()));
+        for (ThreadHandle t : res.threads) CHK_RET(HcommThreadJoin(t, CUSTOM_TIMEOUT));
+        if (shard != me) continue;
+        for (u64 rpt = 0; rpt < rpts; ++rpt) {  // PostLocalReduce :140-178
+            DataSlice dst(p.buffInfo.outputPtr, p.buffInfo.outBuffBaseOff + rpt * p.outputRepeatStride, size, count);
+            for (u32 k = 0; k < n; ++k) {
+                if (k == me) continue;
+                DataSlice src(ccl, p.buffInfo.hcclBuffBaseOff + rpt * p.outputRepeatStride + k * size, size, count);
+                CHK_RET(LocalReduce(th, src, dst, dataType_, reduceOp_));
+            }
         }
     }
     return HCCL_SUCCESS;

@@ -100,10 +100,8 @@ protected:
             return SelectorStatus::MATCH;
         }
         if (topo->topoLevelNums > 1 || topo->level0Topo == Level0Shape::CLOS) {
-            // The reference picks InsReduceScatterAicpuReduceNHR for PROD / 64-bit here (:350, :430);
-            // its fold order is the NHR gather followed by the own-data-first fold, which is what
-            // InsReduceScatterMesh1D computes, so that template serves those types.
-            name = IsSpecial(p.DataDes.dataType, p.reduceType) ? "InsReduceScatterMesh1D" : "InsReduceScatterNHR";
+            // PROD and 64-bit types gather and fold locally (:350, :430)
+            name = IsSpecial(p.DataDes.dataType, p.reduceType) ? "InsReduceScatterAicpuReduceNHR" : "InsReduceScatterNHR";
             return SelectorStatus::MATCH;
         }
         if (topo->level0Topo == Level0Shape::MESH_1D) {
@@ -169,14 +167,23 @@ protected:
 
 // ---- AlltoAll family (src/ops/all_to_all_v/selector/alltoallv_auto_selector.cc:94-128,
 //      alltoall_auto_selector.cc:111-154, alltoallvc_auto_selector.cc:53-62) -------------------------------
+constexpr u64 ALLTOALL_ENABLE_MULTI_CHANNEL_DATA_SIZE_LIMIT = 150ull * 1024 * 1024;
 template <int KIND> class AlltoAllFamilySelector : public AutoSelectorBase {
 protected:
-    SelectorStatus SelectAicpuAlgo(const TopoInfoWithNetLayerDetails *topo, const OpParam &, std::string &name) const override
+    SelectorStatus SelectAicpuAlgo(const TopoInfoWithNetLayerDetails *topo, const OpParam &p, std::string &name) const override
     {
         if (topo->level0Topo != Level0Shape::MESH_1D && topo->level0Topo != Level0Shape::CLOS) {
             return SelectorStatus::NOT_MATCH;
         }
         name = KIND == 0 ? "InsAlltoAllMesh1D" : KIND == 1 ? "InsAlltoAllVMesh1D" : "InsAlltoAllVCMesh1D";
+        if (KIND == 0 && !p.all2AllVDataDes.sendCounts.empty()) {
+            // up to 150 MiB per rank one link per pair is used (alltoall_auto_selector.cc:127-135); the
+            // steps the template records are the same, only the number of links it would spread them over differs
+            const u64 bytes = p.all2AllVDataDes.sendCounts[0] * DATATYPE_SIZE_TABLE[p.all2AllVDataDes.sendType];
+            if (bytes * topo->userRankSize <= ALLTOALL_ENABLE_MULTI_CHANNEL_DATA_SIZE_LIMIT) {
+                name = "InsAlltoAllMesh1DSingleChannel";
+            }
+        }
         return SelectorStatus::MATCH;
     }
 };

@@ -573,6 +573,26 @@ def reduce_scatter_nhr(w, base, count, stride):
         e.copy(w.out[r], base, w.ccl[r], r * count, count)
 
 
+def reduce_scatter_aicpu_reduce_nhr(w, base, count, stride):
+    """ins_temp_reduce_scatter_aicpu_reduce_nhr.cc:52-80: one round per shard k: every rank copies its shard k
+    into slot <own rank> of its scratch (:82-113), the NHR all-gather steps spread the slots (:180-240), and rank
+    k folds: own input to the output (:115-138), then the other ranks' slots ascending (:140-178)."""
+    n, e = w.n, w.e
+    w.need_ccl(count * n)
+    for k in range(n):
+        for r in range(n):
+            e.copy(w.ccl[r], r * count, w.inp[r], k * stride + base, count)
+        e.copy(w.out[k], base, w.inp[k], k * stride + base, count)
+        for s in range(nhr_step_num(n)):
+            for r in range(n):
+                to, _, txs, _ = nhr_ag_steps(n, r)[s]
+                for idx in txs:
+                    e.copy(w.ccl[to], idx * count, w.ccl[r], idx * count, count)
+        for q in range(n):
+            if q != k:
+                e.reduce(w.out[k], base, w.ccl[k], q * count, count)
+
+
 def reduce_scatter_mesh_chunk(w, base, count, stride):
     """Mesh ReduceScatter for large shards: the own shard is copied to the scratch buffer and the peers reduce-
     write their chunks onto it in the chunk_distance rotation; N-1 chunks, all but the last rounded down to
@@ -624,6 +644,7 @@ def reduce_scatter_order_preserved(w, base, count, stride):
 REDUCE_SCATTER_TEMPLATES = {
     "InsReduceScatterMesh1D": (reduce_scatter_mesh, lambda n: n),   # mesh_1D.cc:59-63
     "InsReduceScatterNHR": (reduce_scatter_nhr, lambda n: n),       # nhr.cc:369-377
+    "InsReduceScatterAicpuReduceNHR": (reduce_scatter_aicpu_reduce_nhr, lambda n: n),  # aicpu_reduce_nhr.cc:242-249
     "InsReduceScatterMesh1DMeshChunk": (reduce_scatter_mesh_chunk, lambda n: n - 1),   # meshchunk.cc:46-52
     "ReduceScatterOrderPreserved": (reduce_scatter_order_preserved, lambda n: n),      # level1.cc:46-50
 }

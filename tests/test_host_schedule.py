@@ -253,6 +253,8 @@ def test_selector_choices_follow_the_reference_thresholds():
                     assert w.all_reduce(r, ins[r], outs[r], count, dtype, op, FAKE_STREAM) == 0
                 elif cmd == "rs":
                     assert w.reduce_scatter(r, ins[r], outs[r], count, dtype, op, FAKE_STREAM) == 0
+                elif cmd == "a2a":
+                    assert w.all_to_all(r, ins[r], count, outs[r], dtype, FAKE_STREAM) == 0
                 else:
                     assert w.all_gather(r, ins[r], outs[r], count, dtype, FAKE_STREAM) == 0
             return w.last_info().algName.decode()
@@ -280,7 +282,13 @@ def test_selector_choices_follow_the_reference_thresholds():
     assert pick(12, 4096, T.FP32, T.SUM, topo=(1, api.SHAPE_CLOS, 0)) == "InsAllReduceNHR"
     assert pick(8, 4096, T.BFP16, T.SUM, cmd="rs") == "InsReduceScatterMesh1D"
     assert pick(8, 4096, T.BFP16, T.SUM, topo=(2, api.SHAPE_MESH_1D, 1), cmd="rs") == "InsReduceScatterNHR"
+    # reduce_scatter_auto_selector.cc:350-352, :429-431
+    assert pick(8, 4096, T.FP32, T.PROD, topo=(2, api.SHAPE_MESH_1D, 1), cmd="rs") == "InsReduceScatterAicpuReduceNHR"
+    assert pick(6, 4096, T.INT64, T.SUM, topo=(1, api.SHAPE_CLOS, 0), cmd="rs") == "InsReduceScatterAicpuReduceNHR"
     assert pick(8, 4096, T.FP16, None, cmd="ag") == "InsAllGatherMesh1D"
+    # one link per pair up to 150 MiB per rank (alltoall_auto_selector.cc:127-135)
+    assert pick(8, 150 * mib // 8 // 2, T.FP16, None, cmd="a2a") == "InsAlltoAllMesh1DSingleChannel"
+    assert pick(8, 150 * mib // 8 // 2 + 1, T.FP16, None, cmd="a2a") == "InsAlltoAllMesh1D"
     assert pick(8, 4096, T.FP16, None, topo=(1, api.SHAPE_CLOS, 0), cmd="ag") == "InsAllGatherNHR"
 
 
@@ -434,7 +442,7 @@ def test_alltoall_and_alltoallvc_reduce_to_alltoallv():
         ins, outs = fake_ptrs(n)
         for r in range(n):
             assert w.all_to_all(r, ins[r], c, outs[r], T.UINT8, FAKE_STREAM) == 0
-        assert w.last_info().algName.decode() == "InsAlltoAllMesh1D"
+        assert w.last_info().algName.decode() == "InsAlltoAllMesh1DSingleChannel"   # <= 150 MiB per rank
         got = copy_trace_outputs(w.last_trace(), xs, [n * c] * n, 1)
         for j in range(n):
             assert np.array_equal(got[j], np.concatenate([xs[i][j * c:(j + 1) * c] for i in range(n)]))
