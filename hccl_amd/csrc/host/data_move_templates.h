@@ -40,10 +40,30 @@ public:
                          TemplateResource &templateResource) override;
     void SetMemBlockInfo(const MemBlockInfo &info) { memBlockInfo_ = info; }
 
-private:
+protected:
+    // the peers in the order their shards are sent: ranks me+1, me+2, ... (:200-240)
+    virtual std::vector<u32> SendOrder(u32 me) const;
     // slot of the block that rank `peer` sent to rank `localRank` (:153-158)
     u32 CalcOutputIndex(u32 peer, u32 localRank) const { return (peer + localRank) % templateRankSize_; }
     MemBlockInfo memBlockInfo_;
+};
+
+// The variant for more than 32 ranks (order_preserved_group.cc:35-61, :132-141, :236-262): at most
+// ORDER_PRESERVED_MAX_THREADS threads, and the shards go out by growing distance, right neighbour then left.
+// Slots and the tree are the ones of the level-1 template, so the results are the same bits.
+constexpr u32 ORDER_PRESERVED_MAX_THREADS = 32;  // src/common/order_preserved_common.h:24-33
+class InsTempReduceScatterOrderPreservedGroup : public InsTempReduceScatterOrderPreservedLevel1 {
+public:
+    using InsTempReduceScatterOrderPreservedLevel1::InsTempReduceScatterOrderPreservedLevel1;
+    std::string Describe() const override { return "ReduceScatter, order preserved, grouped all-to-all"; }
+    u64 GetThreadNum() const override
+    {
+        const u32 n = templateRankSize_ > 1 ? templateRankSize_ : 1;
+        return n < ORDER_PRESERVED_MAX_THREADS ? n : ORDER_PRESERVED_MAX_THREADS;
+    }
+
+protected:
+    std::vector<u32> SendOrder(u32 me) const override;
 };
 
 HCCL_DECLARE_TEMPLATE(InsTempAllGatherMesh1D, "AllGather mesh 1D",

@@ -75,6 +75,8 @@ REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_REDUCE_SCATTER, InsReduceScatterMesh1DMes
                  TopoMatch1D, InsTempReduceScatterMesh1DMeshChunk);
 REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_REDUCE_SCATTER, ReduceScatterOrderPreserved, InsV2ReduceScatterOrderPreservedExecutor,
                  TopoMatch1D, InsTempReduceScatterOrderPreservedLevel1);
+REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_REDUCE_SCATTER, ReduceScatterOrderPreservedGroup, InsV2ReduceScatterOrderPreservedExecutor,
+                 TopoMatch1D, InsTempReduceScatterOrderPreservedGroup);
 REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_REDUCE_SCATTER_V, InsReduceScatterVMesh1D, InsV2ReduceScatterVSoleExecutor,
                  TopoMatch1D, InsTempReduceScatterVMesh1D);
 REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_ALLGATHER_V, InsAllGatherVMesh1D, InsV2AllGatherVSoleExecutor, TopoMatch1D,

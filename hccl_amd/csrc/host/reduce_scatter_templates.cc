@@ -4,6 +4,7 @@
 //   InsTempReduceScatterNHR      ins_temp_reduce_scatter_nhr.cc:77-425
 //   InsTempReduceScatterAicpuReduceNHR   ins_temp_reduce_scatter_aicpu_reduce_nhr.cc:52-300
 //   InsTempReduceScatterOrderPreservedLevel1   ins_temp_reduce_scatter_order_preserved_level1.cc:52-330
+//   InsTempReduceScatterOrderPreservedGroup    ins_temp_reduce_scatter_order_preserved_group.cc:63-413
 // and src/ops/reduce_scatter_v/template/aicpu/:
 //   InsTempReduceScatterVMesh1D  ins_temp_reduce_scatter_v_mesh_1D.cc:50-179
 #include "data_move_templates.h"
@@ -280,6 +281,26 @@ HcclResult InsTempReduceScatterVMesh1D::KernelRun(const OpParam &param, const Te
 // block remains, with M the largest power of two below the number of blocks, block v >= M is folded into block
 // v % M, then M blocks remain.  Blocks are numbered by the rank they came from, so the
 // association does not depend on which rank owns the shard.
+std::vector<u32> InsTempReduceScatterOrderPreservedLevel1::SendOrder(u32 me) const
+{
+    std::vector<u32> order;
+    for (u32 i = 1; i < templateRankSize_; ++i) order.push_back((me + i) % templateRankSize_);
+    return order;
+}
+
+std::vector<u32> InsTempReduceScatterOrderPreservedGroup::SendOrder(u32 me) const
+{
+    std::vector<u32> order;
+    const u32 n = templateRankSize_;
+    for (u32 distance = 1; distance <= n / 2; ++distance) {
+        const u32 right = (me + distance) % n;
+        const u32 left = (me + n - distance) % n;
+        order.push_back(right);
+        if (left != right) order.push_back(left);
+    }
+    return order;
+}
+
 HcclResult InsTempReduceScatterOrderPreservedLevel1::KernelRun(const OpParam &param, const TemplateDataParams &p,
                                                                TemplateResource &res)
 {
@@ -305,8 +326,7 @@ HcclResult InsTempReduceScatterOrderPreservedLevel1::KernelRun(const OpParam &pa
     }
     CHK_RET(PreSync(res.threads));
     u32 que = 1;
-    for (u32 i = 1; i < n; ++i) {   // all-to-all: shard `next` goes to rank `next`, into the slot of this rank
-        const u32 next = (me + i) % n;
+    for (const u32 next : SendOrder(me)) {   // all-to-all: shard `next` goes to rank `next`, into the slot of this rank
         const auto ch = res.channels.find(subCommRanks_[0][next]);
         CHK_PRT_RET(ch == res.channels.end() || ch->second.empty(), HCCL_ERROR("[RS order preserved] channel not found"),
                     HCCL_E_INTERNAL);

@@ -93,10 +93,10 @@ protected:
                                    std::string &name) const override
     {
         if (IsNeedStrictModeForOrderPreserved(p.DataDes.dataType, p.reduceType, topo->userRankSize)) {
-            // strict determinism (:337-347): an all-to-all of the shards, then a fixed tree over the ranks.
-            // The grouped variant for more than 32 ranks is not built.
-            if (topo->userRankSize > MAX_RANK_NUM_FOR_ORDER_PRESERVED) return SelectorStatus::NOT_MATCH;
-            name = "ReduceScatterOrderPreserved";
+            // strict determinism (:337-347): an all-to-all of the shards, then a fixed tree over the ranks;
+            // above 32 ranks the all-to-all runs on a capped number of threads
+            name = topo->userRankSize > MAX_RANK_NUM_FOR_ORDER_PRESERVED ? "ReduceScatterOrderPreservedGroup"
+                                                                         : "ReduceScatterOrderPreserved";
             return SelectorStatus::MATCH;
         }
         if (topo->topoLevelNums > 1 || topo->level0Topo == Level0Shape::CLOS) {

@@ -647,6 +647,9 @@ REDUCE_SCATTER_TEMPLATES = {
     "InsReduceScatterAicpuReduceNHR": (reduce_scatter_aicpu_reduce_nhr, lambda n: n),  # aicpu_reduce_nhr.cc:242-249
     "InsReduceScatterMesh1DMeshChunk": (reduce_scatter_mesh_chunk, lambda n: n - 1),   # meshchunk.cc:46-52
     "ReduceScatterOrderPreserved": (reduce_scatter_order_preserved, lambda n: n),      # level1.cc:46-50
+    # ins_temp_reduce_scatter_order_preserved_group.cc: the same slots and tree; only the order in which the
+    # all-to-all sends go out (:236-262) and the thread count differ, which changes no value
+    "ReduceScatterOrderPreservedGroup": (reduce_scatter_order_preserved, lambda n: n),
 }
 
 
@@ -655,7 +658,7 @@ def run_reduce_scatter(elems, inputs, recv_count, esz, alg, ccl_bytes=CCL_BYTES_
     w = World(elems, inputs, recv_count, esz, ccl_bytes)
     usable = ccl_bytes - 1024 * 1024          # ins_v2_reduce_scatter_sole_executor.cc:126-128
     bound = usable
-    if alg == "ReduceScatterOrderPreserved":  # its own executor: whole buffer, 256 MiB transport bound
+    if alg.startswith("ReduceScatterOrderPreserved"):  # its own executor: whole buffer, 256 MiB transport bound
         usable, bound = ccl_bytes, UB_MAX_DATA_SIZE   # ins_v2_reduce_scatter_order_preserved_executor.cc:108-119
     for base, cur in chunk_counts(recv_count, usable, mult(w.n), esz, bound):
         fn(w, base, cur, recv_count)          # inputSliceStride = recvCount * esz (:160)

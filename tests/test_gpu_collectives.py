@@ -175,6 +175,31 @@ def test_reduce_scatter_both_templates_both_modes(stream, mode, alg, dtype, op, 
         w.close()
 
 
+def test_reduce_scatter_order_preserved_at_40_ranks(stream):
+    """The grouped variant for more than 32 ranks; its 40-leaf tree is deeper than the fold kernel's tree
+    mode takes, so the steps are launched one by one."""
+    n, rc, dtype = 40, 5003, T.FP32
+    rng = np.random.default_rng(40)
+    xs = [payload(rng, dtype, n * rc, "normal") for _ in range(n)]
+    w = api.World(n, ccl_bytes=SMALL_CCL)
+    try:
+        w.set_algorithm(api.CMD_REDUCE_SCATTER, "ReduceScatterOrderPreservedGroup")
+        send = [DevBuf(x) for x in xs]
+        recv = [DevBuf(nbytes=rc * 4) for _ in range(n)]
+        torch.cuda.synchronize()
+        for r in range(n):
+            assert w.reduce_scatter(r, send[r].ptr, recv[r].ptr, rc, dtype, T.SUM, stream.cuda_stream) == 0
+        stream.synchronize()
+        assert not w.last_info().fused
+        want = T.run_reduce_scatter(T.NumericElems(dtype, T.SUM), xs, rc, 4, "ReduceScatterOrderPreservedGroup",
+                                    ccl_bytes=SMALL_CCL)
+        for r in range(n):
+            assert_same_bits(recv[r].get(np.float32), want[r], dtype, f"rank {r}")
+            assert recv[r].guard_intact()
+    finally:
+        w.close()
+
+
 @pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("dtype,op,counts", [
     (T.FP32, T.SUM, [100, 100, 100, 100, 100, 100, 100, 100, 500, 500]),       # reduce_scatter_v_testcase.cc:131-141

@@ -235,7 +235,8 @@ def test_strict_determinism_selects_the_order_preserved_reduce_scatter(monkeypat
     assert pick_rs(8, T.FP32, T.MAX) == (0, "InsReduceScatterMesh1D")          # max / min need no order
     assert pick_rs(8, T.INT32, T.SUM) == (0, "InsReduceScatterMesh1D")         # integers neither
     assert pick_rs(2, T.FP32, T.SUM) == (0, "InsReduceScatterMesh1D")          # two ranks: one pairwise op
-    assert pick_rs(33, T.FP32, T.SUM)[0] == 5                                  # the grouped variant is not built
+    assert pick_rs(32, T.FP32, T.SUM) == (0, "ReduceScatterOrderPreserved")
+    assert pick_rs(33, T.FP32, T.SUM) == (0, "ReduceScatterOrderPreservedGroup")   # more than 32 ranks
     monkeypatch.setenv("HCCL_DETERMINISTIC", "true")
     assert pick_rs(8, T.BFP16, T.SUM) == (0, "InsReduceScatterMesh1D")
     monkeypatch.setenv("HCCL_DETERMINISTIC", "sometimes")

@@ -83,6 +83,22 @@ def test_reduce_scatter_association_order_equals_oracle(alg, n):
     assert all(s == set(range(rc)) for s in seen)
 
 
+def test_grouped_order_preserved_reduce_scatter_at_40_ranks():
+    """More than 32 ranks: the all-to-all runs on 32 threads, shards leave by growing distance
+    (ins_temp_reduce_scatter_order_preserved_group.cc:236-262); the tree is the one of the 32-rank template."""
+    n, rc = 40, 3
+    text, info = dry_reduce_scatter(n, rc, T.FP32, T.SUM, "ReduceScatterOrderPreservedGroup")
+    want = T.run_reduce_scatter(T.SymbolicElems(), sym_inputs(n, n * rc), rc, 4, "ReduceScatterOrderPreservedGroup")
+    plain = T.run_reduce_scatter(T.SymbolicElems(), sym_inputs(n, n * rc), rc, 4, "ReduceScatterOrderPreserved")
+    seen = [set() for _ in range(n)]
+    for rank, off, nbytes, expr in parse_trace(text):
+        tree = parse_expr(expr)
+        for e in range(nbytes // 4):
+            assert expr_to_oracle_string(tree, e, 4, off) == want[rank][off // 4 + e] == plain[rank][off // 4 + e]
+            seen[rank].add(off // 4 + e)
+    assert all(s == set(range(rc)) for s in seen)
+
+
 @pytest.mark.parametrize("alg", AR_ALGS)
 @pytest.mark.parametrize("dtype,op,n,count", [(T.FP32, T.SUM, 8, 70001), (T.FP32, T.PROD, 12, 30011),
                                              (T.FP64, T.SUM, 5, 40000), (T.INT32, T.MAX, 12, 50000),
