@@ -22,6 +22,20 @@ class Seg(ctypes.Structure):
     ]
 
 
+MAX_WIDE_FAN = 64
+
+
+class WideSeg(ctypes.Structure):
+    """hcclx_wide_seg_t of include/hcclx.h."""
+    _fields_ = [
+        ("count", ctypes.c_uint64),
+        ("nsrc", ctypes.c_uint32),
+        ("ndst", ctypes.c_uint32),
+        ("src", ctypes.c_void_p * MAX_WIDE_FAN),
+        ("dst", ctypes.c_void_p * MAX_WIDE_FAN),
+    ]
+
+
 _lib = None
 
 
@@ -47,6 +61,11 @@ def load():
     lib.hcclx_plan_create.restype = ctypes.c_int
     lib.hcclx_plan_create.argtypes = [ctypes.POINTER(Seg), ctypes.c_uint32, ctypes.c_int, ctypes.c_int,
                                       ctypes.c_int, ctypes.POINTER(ctypes.c_void_p)]
+    lib.hcclx_fold_wide.restype = ctypes.c_int
+    lib.hcclx_fold_wide.argtypes = [ctypes.POINTER(WideSeg), ctypes.c_uint32, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    lib.hcclx_plan_create_wide.restype = ctypes.c_int
+    lib.hcclx_plan_create_wide.argtypes = [ctypes.POINTER(WideSeg), ctypes.c_uint32, ctypes.c_int, ctypes.c_int,
+                                           ctypes.POINTER(ctypes.c_void_p)]
     lib.hcclx_plan_launch.restype = ctypes.c_int
     lib.hcclx_plan_launch.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
     lib.hcclx_plan_destroy.restype = ctypes.c_int

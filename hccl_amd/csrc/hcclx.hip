@@ -202,7 +202,12 @@ struct Batch {
     uint64_t total_tiles = 0;
     std::vector<uint64_t> tile_end;
     std::vector<SegDev> segs;
-    size_t bytes() const { return align256(tile_end.size() * 8) + segs.size() * sizeof(SegDev); }
+    std::vector<SegWide> wide;   // instead of segs when maxn == kMaxWideFan
+    size_t nseg() const { return segs.size() + wide.size(); }
+    size_t bytes() const
+    {
+        return align256(tile_end.size() * 8) + segs.size() * sizeof(SegDev) + wide.size() * sizeof(SegWide);
+    }
     static size_t align256(size_t x) { return (x + 255) & ~static_cast<size_t>(255); }
 };
 
@@ -368,18 +373,87 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
     return HCCL_SUCCESS;
 }
 
+// Wide segments: chain order, up to kMaxWideFan sources and destinations, one kernel for every fan-in.
+int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, Built *out)
+{
+    if (nseg != 0 && segs == nullptr) return fail(HCCL_E_PTR, "segs is null");
+    int esz = dtype_size(dtype);
+    if (esz == 0) return fail(HCCL_E_NOT_SUPPORT, "unknown data type " + std::to_string(dtype));
+    uint32_t max_src = 0;
+    for (uint32_t i = 0; i < nseg; ++i) {
+        const hcclx_wide_seg_t &s = segs[i];
+        if (s.nsrc == 0 || s.nsrc > HCCLX_MAX_WIDE_FAN || s.ndst == 0 || s.ndst > HCCLX_MAX_WIDE_FAN) {
+            return fail(HCCL_E_PARA, "segment " + std::to_string(i) + ": nsrc/ndst outside 1.." +
+                                         std::to_string(HCCLX_MAX_WIDE_FAN));
+        }
+        if (s.count != 0) {
+            for (uint32_t k = 0; k < s.nsrc; ++k) {
+                if (s.src[k] == nullptr) return fail(HCCL_E_PTR, "segment " + std::to_string(i) + ": null source");
+            }
+            for (uint32_t k = 0; k < s.ndst; ++k) {
+                if (s.dst[k] == nullptr) return fail(HCCL_E_PTR, "segment " + std::to_string(i) + ": null destination");
+            }
+        }
+        if (s.nsrc > max_src) max_src = s.nsrc;
+    }
+    Batch proto;
+    proto.dtype = dtype;
+    proto.op = op;
+    proto.mode = HCCLX_FOLD_CHAIN;
+    proto.maxn = kMaxWideFan;
+    uint64_t scale = 1;
+    if (max_src <= 1) {
+        // nothing is combined: any type is moved as bytes
+        proto.dtype = HCCL_DATA_TYPE_INT8;
+        proto.op = HCCL_REDUCE_SUM;
+        scale = static_cast<uint64_t>(esz);
+        esz = 1;
+    } else {
+        if (!is_reduce_dtype(dtype)) return fail(HCCL_E_NOT_SUPPORT, "data type cannot be reduced");
+        if (op < HCCL_REDUCE_SUM || op > HCCL_REDUCE_MIN) return fail(HCCL_E_NOT_SUPPORT, "unknown reduce op");
+    }
+    const int ne = 16 / esz;
+    Batch cur = proto;
+    for (uint32_t i = 0; i < nseg; ++i) {
+        const hcclx_wide_seg_t &s = segs[i];
+        if (s.count == 0) continue;
+        SegWide sd;
+        std::memset(&sd, 0, sizeof(sd));
+        sd.count = s.count * scale;
+        sd.nsrc = s.nsrc;
+        sd.ndst = s.ndst;
+        for (uint32_t k = 0; k < s.nsrc; ++k) sd.src[k] = static_cast<const char *>(s.src[k]);
+        for (uint32_t k = 0; k < s.ndst; ++k) sd.dst[k] = static_cast<char *>(s.dst[k]);
+        sd.head = fold_head_of(sd.count, esz, sd.dst[0]);
+        sd.shift = fold_shift_of(sd.head, esz, kMaxWideFan, sd.dst[0]);
+        const uint64_t tiles = fold_tiles_of(sd.count, ne, kMaxWideFan, sd.head, sd.shift);
+        if (static_cast<int>(cur.wide.size()) == kMaxWideSegsPerLaunch) {
+            out->batches.push_back(std::move(cur));
+            cur = proto;
+        }
+        cur.total_tiles += tiles;
+        cur.tile_end.push_back(cur.total_tiles);
+        cur.wide.push_back(sd);
+        out->algo_bytes += static_cast<uint64_t>(s.nsrc + s.ndst) * sd.count * esz;
+    }
+    if (!cur.wide.empty()) out->batches.push_back(std::move(cur));
+    return HCCL_SUCCESS;
+}
+
 void fill_table(const Batch &b, char *h)
 {
     std::memcpy(h, b.tile_end.data(), b.tile_end.size() * 8);
-    std::memcpy(h + Batch::align256(b.tile_end.size() * 8), b.segs.data(), b.segs.size() * sizeof(SegDev));
+    char *at = h + Batch::align256(b.tile_end.size() * 8);
+    if (!b.segs.empty()) std::memcpy(at, b.segs.data(), b.segs.size() * sizeof(SegDev));
+    if (!b.wide.empty()) std::memcpy(at, b.wide.data(), b.wide.size() * sizeof(SegWide));
 }
 
 int launch_batch(const DeviceCtx *ctx, const Batch &b, const char *d_table, hipStream_t stream)
 {
     FoldLaunch l;
     l.tile_end = reinterpret_cast<const uint64_t *>(d_table);
-    l.segs = reinterpret_cast<const SegDev *>(d_table + Batch::align256(b.tile_end.size() * 8));
-    l.nseg = static_cast<uint32_t>(b.segs.size());
+    l.segs = d_table + Batch::align256(b.tile_end.size() * 8);
+    l.nseg = static_cast<uint32_t>(b.nseg());
     l.total_tiles = b.total_tiles;
     l.grid = grid_for(ctx, b.total_tiles);
     l.stream = stream;
@@ -425,18 +499,12 @@ const char *hcclx_last_error(void) { return g_err.c_str(); }
 
 uint32_t hcclx_dtype_size(int dtype) { return static_cast<uint32_t>(dtype_size(dtype)); }
 
-int hcclx_fold(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, void *stream)
+static int launch_built(DeviceCtx *ctx, const Built &built, hipStream_t st)
 {
-    DeviceCtx *ctx = device_ctx();
-    if (!ctx) return HCCL_E_RUNTIME;
-    Built built;
-    int rc = build_batches(segs, nseg, dtype, op, mode, &built);
-    if (rc != HCCL_SUCCESS) return rc;
-    hipStream_t st = static_cast<hipStream_t>(stream);
     for (const Batch &b : built.batches) {
         char *h = nullptr;
         char *d = nullptr;
-        rc = ring_reserve(ctx, b.bytes(), st, &h, &d);
+        int rc = ring_reserve(ctx, b.bytes(), st, &h, &d);
         if (rc != HCCL_SUCCESS) return rc;
         fill_table(b, h);
         HCCLX_HIP(hipMemcpyAsync(d, h, b.bytes(), hipMemcpyHostToDevice, st));
@@ -446,15 +514,8 @@ int hcclx_fold(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mo
     return HCCL_SUCCESS;
 }
 
-int hcclx_plan_create(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, hcclx_plan_t **plan)
+static int plan_from(DeviceCtx *ctx, Built &built, hcclx_plan_t **plan)
 {
-    if (plan == nullptr) return fail(HCCL_E_PTR, "plan is null");
-    *plan = nullptr;
-    DeviceCtx *ctx = device_ctx();
-    if (!ctx) return HCCL_E_RUNTIME;
-    Built built;
-    int rc = build_batches(segs, nseg, dtype, op, mode, &built);
-    if (rc != HCCL_SUCCESS) return rc;
     hcclx_plan *p = new hcclx_plan;
     p->device = ctx->device;
     p->algo_bytes = built.algo_bytes;
@@ -477,6 +538,50 @@ int hcclx_plan_create(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op,
     }
     *plan = p;
     return HCCL_SUCCESS;
+}
+
+int hcclx_fold(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, void *stream)
+{
+    DeviceCtx *ctx = device_ctx();
+    if (!ctx) return HCCL_E_RUNTIME;
+    Built built;
+    int rc = build_batches(segs, nseg, dtype, op, mode, &built);
+    if (rc != HCCL_SUCCESS) return rc;
+    return launch_built(ctx, built, static_cast<hipStream_t>(stream));
+}
+
+int hcclx_fold_wide(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, void *stream)
+{
+    DeviceCtx *ctx = device_ctx();
+    if (!ctx) return HCCL_E_RUNTIME;
+    Built built;
+    int rc = build_wide_batches(segs, nseg, dtype, op, &built);
+    if (rc != HCCL_SUCCESS) return rc;
+    return launch_built(ctx, built, static_cast<hipStream_t>(stream));
+}
+
+int hcclx_plan_create(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, hcclx_plan_t **plan)
+{
+    if (plan == nullptr) return fail(HCCL_E_PTR, "plan is null");
+    *plan = nullptr;
+    DeviceCtx *ctx = device_ctx();
+    if (!ctx) return HCCL_E_RUNTIME;
+    Built built;
+    int rc = build_batches(segs, nseg, dtype, op, mode, &built);
+    if (rc != HCCL_SUCCESS) return rc;
+    return plan_from(ctx, built, plan);
+}
+
+int hcclx_plan_create_wide(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, hcclx_plan_t **plan)
+{
+    if (plan == nullptr) return fail(HCCL_E_PTR, "plan is null");
+    *plan = nullptr;
+    DeviceCtx *ctx = device_ctx();
+    if (!ctx) return HCCL_E_RUNTIME;
+    Built built;
+    int rc = build_wide_batches(segs, nseg, dtype, op, &built);
+    if (rc != HCCL_SUCCESS) return rc;
+    return plan_from(ctx, built, plan);
 }
 
 int hcclx_plan_launch(const hcclx_plan_t *plan, void *stream)

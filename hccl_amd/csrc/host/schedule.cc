@@ -476,6 +476,7 @@ struct FusedPlan {
     std::vector<hcclx_seg_t> selfSegs;
     std::vector<hcclx_seg_t> copySegs;
     std::vector<hcclx_seg_t> treeSegs;
+    std::vector<hcclx_wide_seg_t> wideSegs;   // chains over more than HCCLX_MAX_FAN sources
 };
 
 bool Overlaps(u64 a, u64 alen, u64 b, u64 blen) { return a < b + blen && b < a + alen; }
@@ -586,12 +587,29 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
     // self-first group (every thread reads all sources of an element before it writes any destination):
     // that is an in-place collective.  Any other overlap between what one fold writes and what another
     // reads would be a race inside a single pass.
-    for (size_t i = 0; i < folds.size(); ++i) {
+    {
+        struct Read {
+            u64 addr;
+            u64 bytes;
+            size_t fold;
+        };
+        std::vector<Read> reads;
+        u64 longest = 0;
         for (size_t j = 0; j < folds.size(); ++j) {
-            for (u64 a : folds[j].src) {
-                if (!Overlaps(folds[i].dst, folds[i].bytes, a, folds[j].bytes)) continue;
+            for (u64 a : folds[j].src) reads.push_back({a, folds[j].bytes, j});
+            longest = std::max(longest, folds[j].bytes);
+        }
+        std::sort(reads.begin(), reads.end(), [](const Read &x, const Read &y) { return x.addr < y.addr; });
+        for (size_t i = 0; i < folds.size(); ++i) {
+            // reads that can reach into [dst, dst + bytes) start after dst - longest
+            const u64 from = folds[i].dst > longest ? folds[i].dst - longest : 0;
+            auto it = std::lower_bound(reads.begin(), reads.end(), from,
+                                       [](const Read &x, u64 v) { return x.addr < v; });
+            for (; it != reads.end() && it->addr < folds[i].dst + folds[i].bytes; ++it) {
+                if (!Overlaps(folds[i].dst, folds[i].bytes, it->addr, it->bytes)) continue;
+                const size_t j = it->fold;
                 const bool sameUnit = (i == j) || (group[i] != -1 && group[i] == group[j]);
-                if (sameUnit && a == folds[i].dst) continue;
+                if (sameUnit && it->addr == folds[i].dst) continue;
                 return false;
             }
         }
@@ -601,9 +619,25 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
         for (size_t i : kv.second) {
             if (!taken[i]) rest.push_back(i);
         }
+        if (!rest.empty() && folds[rest[0]].src.size() > HCCLX_MAX_FAN) {
+            // more ranks than the register-resident kernels take: the wide chain kernel
+            const Fold &f = folds[rest[0]];
+            if (!f.chain || f.src.size() > HCCLX_MAX_WIDE_FAN) return false;
+            for (size_t at = 0; at < rest.size(); at += HCCLX_MAX_WIDE_FAN) {
+                hcclx_wide_seg_t seg;
+                std::memset(&seg, 0, sizeof(seg));
+                seg.count = f.bytes / esz;
+                seg.nsrc = static_cast<uint32_t>(f.src.size());
+                for (size_t k = 0; k < f.src.size(); ++k) seg.src[k] = reinterpret_cast<const void *>(f.src[k]);
+                for (size_t d = at; d < rest.size() && d < at + HCCLX_MAX_WIDE_FAN; ++d) {
+                    seg.dst[seg.ndst++] = reinterpret_cast<void *>(folds[rest[d]].dst);
+                }
+                plan.wideSegs.push_back(seg);
+            }
+            continue;
+        }
         for (size_t at = 0; at < rest.size(); at += HCCLX_MAX_FAN) {
             const Fold &f = folds[rest[at]];
-            if (f.src.size() > HCCLX_MAX_FAN) return false;
             hcclx_seg_t seg;
             std::memset(&seg, 0, sizeof(seg));
             seg.nsrc = static_cast<uint32_t>(f.src.size());
@@ -997,7 +1031,8 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
         const bool ok = BuildFusedPlan(w, tr, params, foldType, op, esz, plan,
                                        (w->traceText || w->dryRun) ? &w->lastTrace : nullptr);
         w->lastFusedSegments =
-            static_cast<u32>(plan.chainSegs.size() + plan.selfSegs.size() + plan.copySegs.size() + plan.treeSegs.size());
+            static_cast<u32>(plan.chainSegs.size() + plan.selfSegs.size() + plan.copySegs.size() + plan.treeSegs.size() +
+                             plan.wideSegs.size());
         if (w->dryRun) {
             w->lastWasFused = ok;
             return HCCL_SUCCESS;
@@ -1014,6 +1049,16 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
                 const int dt = (i == 2) ? HCCL_DATA_TYPE_INT8 : foldType;
                 const int rc = hcclx_plan_create(parts[i].first->data(), static_cast<uint32_t>(parts[i].first->size()),
                                                  dt, op, parts[i].second, &hp);
+                if (rc != HCCL_SUCCESS) {
+                    for (hcclx_plan *q : c.plans) (void)hcclx_plan_destroy(q);
+                    return static_cast<HcclResult>(rc);
+                }
+                c.plans.push_back(hp);
+            }
+            if (!plan.wideSegs.empty()) {
+                hcclx_plan *hp = nullptr;
+                const int rc = hcclx_plan_create_wide(plan.wideSegs.data(), static_cast<uint32_t>(plan.wideSegs.size()),
+                                                      foldType, op, &hp);
                 if (rc != HCCL_SUCCESS) {
                     for (hcclx_plan *q : c.plans) (void)hcclx_plan_destroy(q);
                     return static_cast<HcclResult>(rc);

@@ -28,7 +28,8 @@ constexpr uint32_t kFoldDirectSegs = 64;   // up to this many segments the tile 
 __host__ __device__ constexpr int fold_unroll(int maxn)
 {
     constexpr int u[5] = {HCCLX_FOLD_UNROLLS};
-    return maxn <= 1 ? u[0] : maxn <= 2 ? u[1] : maxn <= 4 ? u[2] : maxn <= 8 ? u[3] : u[4];
+    // more than kMaxFan sources: the wide kernel, which walks them in groups, one vector per thread
+    return maxn <= 1 ? u[0] : maxn <= 2 ? u[1] : maxn <= 4 ? u[2] : maxn <= 8 ? u[3] : maxn <= kMaxFan ? u[4] : 1;
 }
 __host__ __device__ constexpr uint64_t fold_tile_vecs(int maxn)
 {
@@ -176,8 +177,8 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
 }
 
 // The last (count % NE) elements of a segment, one per thread.
-template <int DT, int OP, int MAXN, int MODE>
-__device__ __forceinline__ void fold_tail(const SegDev &sd, uint32_t nsrc, uint32_t ndst, uint64_t idx)
+template <int DT, int OP, int MAXN, int MODE, typename SEG>
+__device__ __forceinline__ void fold_tail(const SEG &sd, uint32_t nsrc, uint32_t ndst, uint64_t idx)
 {
     using D = DTypeOf<DT>;
     using S = typename D::S;
@@ -213,6 +214,39 @@ __device__ __forceinline__ void fold_tail(const SegDev &sd, uint32_t nsrc, uint3
     }
 }
 
+// Maps tile number t of a launch to its segment (the first one whose inclusive tile prefix exceeds t) and
+// to the tile's number inside that segment.  Every value is wave-uniform.
+__device__ __forceinline__ void locate_tile(const uint64_t *__restrict__ tile_end, const uint64_t *s_end, uint32_t nseg,
+                                            bool direct, uint64_t t, uint32_t *seg, uint64_t *tile_in_seg)
+{
+    uint32_t lo = 0;
+    uint32_t hi = nseg - 1;
+    uint64_t before = 0;   // tiles of the segments in front of the one found
+    if (direct) {
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (tile_end[mid] > t) {
+                hi = mid;
+            } else {
+                lo = mid + 1;
+            }
+        }
+        before = lo ? tile_end[lo - 1] : 0;
+    } else {
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (s_end[mid] > t) {
+                hi = mid;
+            } else {
+                lo = mid + 1;
+            }
+        }
+        before = lo ? s_end[lo - 1] : 0;
+    }
+    *seg = __builtin_amdgcn_readfirstlane(lo);
+    *tile_in_seg = uniform64(t - before);
+}
+
 template <int DT, int OP, int MAXN, int MODE>
 __global__ void __launch_bounds__(kFoldThreads)
 k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, uint32_t nseg, uint64_t total_tiles)
@@ -232,33 +266,9 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
     }
 
     for (uint64_t t = blockIdx.x; t < total_tiles; t += gridDim.x) {
-        // first segment whose inclusive tile prefix exceeds t
-        uint32_t lo = 0;
-        uint32_t hi = nseg - 1;
-        uint64_t before = 0;   // tiles of the segments in front of the one found
-        if (direct) {
-            while (lo < hi) {
-                const uint32_t mid = (lo + hi) >> 1;
-                if (tile_end[mid] > t) {
-                    hi = mid;
-                } else {
-                    lo = mid + 1;
-                }
-            }
-            before = lo ? tile_end[lo - 1] : 0;
-        } else {
-            while (lo < hi) {
-                const uint32_t mid = (lo + hi) >> 1;
-                if (s_end[mid] > t) {
-                    hi = mid;
-                } else {
-                    lo = mid + 1;
-                }
-            }
-            before = lo ? s_end[lo - 1] : 0;
-        }
-        const uint32_t s = __builtin_amdgcn_readfirstlane(lo);
-        const uint64_t tl = uniform64(t - before);
+        uint32_t s;
+        uint64_t tl;
+        locate_tile(tile_end, s_end, nseg, direct, t, &s, &tl);
         const SegDev &sd = segs[s];
         const uint32_t nsrc = sd.nsrc;
         const uint32_t ndst = sd.ndst;
@@ -280,6 +290,88 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
             if (tl == (nvec + shift) / TV && threadIdx.x < head + rem) {
                 const uint64_t idx = threadIdx.x < head ? threadIdx.x : head + nvec * NE + (threadIdx.x - head);
                 fold_tail<DT, OP, MAXN, MODE>(sd, nsrc, ndst, idx);
+            }
+        }
+    }
+}
+
+// More than kMaxFan sources or destinations (chain order only): the sources are walked in groups of kMaxFan,
+// each group loaded before it is folded in, so the loads in flight per thread stay what the 16-source kernel
+// has.  One vector per thread and tile.
+template <int DT, int OP, bool CHECK>
+__device__ __forceinline__ void fold_tile_wide(const SegWide &sd, uint32_t nsrc, uint32_t ndst, uint64_t v, uint64_t nvec,
+                                               uint32_t head_bytes)
+{
+    using V = Vec16<DT>;
+    using C = typename V::C;
+    constexpr int NE = V::NE;
+    if (CHECK && v >= nvec) {
+        return;
+    }
+    const uint64_t off = head_bytes + v * 16;
+    C acc[NE];
+    V::unpack(ld16(sd.src[0] + off), acc);
+    for (uint32_t base = 1; base < nsrc; base += kMaxFan) {
+        u32x4 raw[kMaxFan];
+#pragma unroll
+        for (int k = 0; k < kMaxFan; ++k) {
+            if (base + k < nsrc) raw[k] = ld16(sd.src[base + k] + off);
+        }
+#pragma unroll
+        for (int k = 0; k < kMaxFan; ++k) {
+            if (base + k < nsrc) {
+                C x[NE];
+                V::unpack(raw[k], x);
+#pragma unroll
+                for (int e = 0; e < NE; ++e) acc[e] = V::template combine<OP>(x[e], acc[e]);
+            }
+        }
+    }
+    const u32x4 out = V::pack(acc);
+    for (uint32_t base = 0; base < ndst; base += kMaxFan) {
+#pragma unroll
+        for (int d = 0; d < kMaxFan; ++d) {
+            if (base + d < ndst) st16(sd.dst[base + d] + off, out);
+        }
+    }
+}
+
+template <int DT, int OP>
+__global__ void __launch_bounds__(kFoldThreads)
+k_fold_wide(const uint64_t *__restrict__ tile_end, const SegWide *__restrict__ segs, uint32_t nseg, uint64_t total_tiles)
+{
+    constexpr int NE = Vec16<DT>::kElems;
+    constexpr uint64_t TV = fold_tile_vecs(kMaxWideFan);
+    static_assert(TV == kFoldThreads, "the wide kernel moves one vector per thread and tile");
+    extern __shared__ uint64_t s_end[];
+    const bool direct = nseg <= kFoldDirectSegs;
+    if (!direct) {
+        for (uint32_t i = threadIdx.x; i < nseg; i += kFoldThreads) {
+            s_end[i] = tile_end[i];
+        }
+        __syncthreads();
+    }
+    for (uint64_t t = blockIdx.x; t < total_tiles; t += gridDim.x) {
+        uint32_t s;
+        uint64_t tl;
+        locate_tile(tile_end, s_end, nseg, direct, t, &s, &tl);
+        const SegWide &sd = segs[s];
+        const uint32_t nsrc = sd.nsrc;
+        const uint32_t ndst = sd.ndst;
+        const uint32_t head = sd.head;
+        const uint64_t body = sd.count - head;
+        const uint64_t nvec = body / NE;
+        const uint32_t rem = static_cast<uint32_t>(body % NE);
+        const uint32_t head_bytes = head * (16 / NE);
+        const uint32_t shift = sd.shift;
+        const uint64_t v = tl * TV + threadIdx.x - shift;   // wraps in front of a shifted segment: fails the check
+        if (tl * TV >= shift && (tl + 1) * TV - shift <= nvec) {
+            fold_tile_wide<DT, OP, false>(sd, nsrc, ndst, v, nvec, head_bytes);
+        } else {
+            fold_tile_wide<DT, OP, true>(sd, nsrc, ndst, v, nvec, head_bytes);
+            if (tl == (nvec + shift) / TV && threadIdx.x < head + rem) {
+                const uint64_t idx = threadIdx.x < head ? threadIdx.x : head + nvec * NE + (threadIdx.x - head);
+                fold_tail<DT, OP, kMaxWideFan, kFoldChain>(sd, nsrc, ndst, idx);
             }
         }
     }
@@ -321,7 +413,7 @@ inline uint64_t fold_tiles_of(uint64_t count, int ne, int maxn, uint32_t head, u
 
 struct FoldLaunch {
     const uint64_t *tile_end;  // device
-    const SegDev *segs;        // device
+    const void *segs;          // device: SegDev[], or SegWide[] for the wide kernel
     uint32_t nseg;
     uint64_t total_tiles;
     uint32_t grid;

@@ -10,8 +10,10 @@
 namespace hcclx {
 
 constexpr int kMaxFan = 16;        // sources fused in one pass / destinations written in one pass
+constexpr int kMaxWideFan = 64;    // the same for the wide chain kernel (communicators of more than 16 ranks)
 constexpr int kThreads = 256;      // workgroup size: 4 wavefronts of 64
 constexpr int kMaxSegsPerLaunch = 2048;  // tile_end[] must fit the LDS staging array (16 KiB)
+constexpr int kMaxWideSegsPerLaunch = 512;   // and a launch's table one slice of the descriptor ring
 
 struct SegDev {
     uint64_t count;            // elements (bytes for the copy kernel)
@@ -32,6 +34,18 @@ struct SegDev {
     // the tile size in dst[0]'s address space: every wavefront then stores whole, aligned cache lines.
     // The first tile is partial when shift != 0.
     uint32_t shift;
+};
+
+// A chain segment of the wide kernel: acc = src[0]; acc = src[k] (+) acc for k = 1 .. nsrc-1; the value goes
+// to every dst.  head and shift as in SegDev, for tiles of one vector per thread.
+struct SegWide {
+    uint64_t count;
+    uint32_t nsrc;
+    uint32_t ndst;
+    uint32_t head;
+    uint32_t shift;
+    const char *src[kMaxWideFan];
+    char *dst[kMaxWideFan];
 };
 
 // How the sources of a segment are folded.

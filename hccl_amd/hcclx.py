@@ -2,7 +2,7 @@
 import ctypes
 
 from . import _lib
-from ._lib import Seg, check
+from ._lib import Seg, WideSeg, check
 
 FOLD_CHAIN = 0
 FOLD_SELF_FIRST = 1
@@ -28,6 +28,21 @@ def make_segs(segs):
     return arr, len(segs)
 
 
+def make_wide_segs(segs):
+    """segs: iterable of (count, [src addresses], [dst addresses]) -> ctypes array of hcclx_wide_seg_t."""
+    segs = list(segs)
+    arr = (WideSeg * max(1, len(segs)))()
+    for i, (count, srcs, dsts) in enumerate(segs):
+        arr[i].count = count
+        arr[i].nsrc = len(srcs)
+        arr[i].ndst = len(dsts)
+        for k, p in enumerate(srcs[:_lib.MAX_WIDE_FAN]):   # the library rejects nsrc/ndst beyond MAX_WIDE_FAN
+            arr[i].src[k] = p
+        for k, p in enumerate(dsts[:_lib.MAX_WIDE_FAN]):
+            arr[i].dst[k] = p
+    return arr, len(segs)
+
+
 def init():
     check(_lib.load().hcclx_init())
 
@@ -37,13 +52,23 @@ def fold(segs, dtype, op=0, mode=FOLD_CHAIN, stream=0):
     check(_lib.load().hcclx_fold(arr, n, int(dtype), int(op), int(mode), ctypes.c_void_p(stream)))
 
 
+def fold_wide(segs, dtype, op=0, stream=0):
+    """Chain-order fold of segments with up to 64 sources and destinations."""
+    arr, n = make_wide_segs(segs)
+    check(_lib.load().hcclx_fold_wide(arr, n, int(dtype), int(op), ctypes.c_void_p(stream)))
+
+
 class Plan:
     """A fold whose table already sits in device memory: launch() is one kernel launch."""
 
-    def __init__(self, segs, dtype, op=0, mode=FOLD_CHAIN):
-        arr, n = make_segs(segs)
+    def __init__(self, segs, dtype, op=0, mode=FOLD_CHAIN, wide=False):
         h = ctypes.c_void_p()
-        check(_lib.load().hcclx_plan_create(arr, n, int(dtype), int(op), int(mode), ctypes.byref(h)))
+        if wide:
+            arr, n = make_wide_segs(segs)
+            check(_lib.load().hcclx_plan_create_wide(arr, n, int(dtype), int(op), ctypes.byref(h)))
+        else:
+            arr, n = make_segs(segs)
+            check(_lib.load().hcclx_plan_create(arr, n, int(dtype), int(op), int(mode), ctypes.byref(h)))
         self._h = h
 
     @property

@@ -175,6 +175,64 @@ def test_reduce_scatter_both_templates_both_modes(stream, mode, alg, dtype, op, 
         w.close()
 
 
+@pytest.mark.parametrize("alg,fusable", [("InsAllReduceMesh1DTwoShot", True), ("InsAllReduceMesh1DOneShot", True),
+                                         ("InsAllReduceRing", True), ("InsAllReduceAicpuReduceNHR", True),
+                                         ("InsAllReduceNHR", False), ("InsAllReduceRHD", False)])
+@pytest.mark.parametrize("dtype,op,n,count", [(T.FP32, T.SUM, 24, 50021), (T.BFP16, T.SUM, 32, 70001),
+                                             (T.INT32, T.MAX, 40, 30011), (T.FP64, T.PROD, 17, 20000)])
+def test_allreduce_among_more_than_16_ranks(stream, alg, fusable, dtype, op, n, count):
+    """Chains over more than 16 sources take the wide fold kernel and stay one pass; the trees of the log-step
+    templates are deeper than four levels for floating types and are launched step by step."""
+    rng = np.random.default_rng(n * 11 + count)
+    kind = "prod" if op == T.PROD else "uniform" if dtype == T.FP32 else "normal"
+    xs = [payload(rng, dtype, count, kind) for _ in range(n)]
+    w = api.World(n, ccl_bytes=SMALL_CCL)
+    try:
+        w.set_algorithm(api.CMD_ALLREDUCE, alg)
+        got, bufs = run_allreduce(w, stream, xs, count, dtype, op)
+        info = w.last_info()
+        assert bool(info.fused) == (fusable or dtype == T.INT32), alg
+        if info.fused and dtype in (T.FP16, T.BFP16) and op == T.SUM:
+            want = wide_oracle_allreduce(xs, count, dtype, alg, SMALL_CCL)
+        else:
+            want = T.run_allreduce(T.NumericElems(dtype, op), xs, count, T.DTYPE_SIZE[dtype], alg, ccl_bytes=SMALL_CCL)
+        for r in range(n):
+            assert_same_bits(got[r], want[r], dtype, f"{alg} rank {r} fused={info.fused}")
+            assert bufs[r].guard_intact()
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("alg", ["InsReduceScatterMesh1D", "InsReduceScatterNHR", "InsReduceScatterAicpuReduceNHR"])
+@pytest.mark.parametrize("dtype,op,n,rc", [(T.BFP16, T.SUM, 32, 9001), (T.FP32, T.SUM, 20, 12345), (T.INT8, T.MIN, 64, 5000)])
+def test_reduce_scatter_among_more_than_16_ranks(stream, alg, dtype, op, n, rc):
+    rng = np.random.default_rng(n + rc)
+    xs = [payload(rng, dtype, n * rc, "normal") for _ in range(n)]
+    w = api.World(n, ccl_bytes=SMALL_CCL)
+    try:
+        w.set_algorithm(api.CMD_REDUCE_SCATTER, alg)
+        send = [DevBuf(x) for x in xs]
+        recv = [DevBuf(nbytes=rc * T.DTYPE_SIZE[dtype]) for _ in range(n)]
+        torch.cuda.synchronize()
+        for r in range(n):
+            assert w.reduce_scatter(r, send[r].ptr, recv[r].ptr, rc, dtype, op, stream.cuda_stream) == 0
+        stream.synchronize()
+        info = w.last_info()
+        esz = T.DTYPE_SIZE[dtype]
+        assert bool(info.fused) == (alg != "InsReduceScatterNHR" or dtype == T.INT8), alg
+        if info.fused and dtype in (T.FP16, T.BFP16) and op == T.SUM:
+            wide = [T.widen16(x, dtype) for x in xs]
+            want = [T.narrow16(o, dtype) for o in
+                    T.run_reduce_scatter(T.NumericElems(T.FP32, T.SUM), wide, rc, esz, alg, ccl_bytes=SMALL_CCL)]
+        else:
+            want = T.run_reduce_scatter(T.NumericElems(dtype, op), xs, rc, esz, alg, ccl_bytes=SMALL_CCL)
+        for r in range(n):
+            assert_same_bits(recv[r].get(T.NP_STORAGE[dtype]), want[r], dtype, f"{alg} rank {r} fused={info.fused}")
+            assert recv[r].guard_intact()
+    finally:
+        w.close()
+
+
 def test_reduce_scatter_order_preserved_at_40_ranks(stream):
     """The grouped variant for more than 32 ranks; its 40-leaf tree is deeper than the fold kernel's tree
     mode takes, so the steps are launched one by one."""

@@ -87,6 +87,70 @@ def test_self_first_in_place_allreduce():
         assert_same_bits(bufs[r].get(np.float32), fold_oracle(xs, T.FP32, T.SUM, order, False), T.FP32)
 
 
+@pytest.mark.parametrize("nsrc,ndst", [(1, 40), (2, 1), (17, 3), (24, 24), (33, 17), (40, 1), (64, 64)])
+@pytest.mark.parametrize("dtype,op", [(T.FP32, T.SUM), (T.BFP16, T.SUM), (T.FP16, T.PROD), (T.FP64, T.PROD),
+                                      (T.INT8, T.MAX), (T.INT64, T.MIN), (T.INT16, T.SUM)])
+def test_wide_chain_fold_up_to_64_sources_and_destinations(nsrc, ndst, dtype, op):
+    """hcclx_fold_wide: the chain order over more sources than the register-resident kernel holds, operands at
+    element alignment, a count that leaves a head and a tail, two segments in one launch."""
+    rng = np.random.default_rng(nsrc * 1000 + ndst * 10 + dtype)
+    esz = T.DTYPE_SIZE[dtype]
+    counts = [3 * 4096 // esz + 13, 7]
+    kind = "prod" if op == T.PROD else "uniform" if dtype in (T.FP32, T.FP64) else "normal"
+    segs, checks = [], []
+    for si, n in enumerate(counts):
+        xs = [payload(rng, dtype, n, kind) for _ in range(nsrc)]
+        order = list(rng.permutation(nsrc))
+        bufs = [DevBuf(x, offset=(k % 5) * esz) for k, x in enumerate(xs)]
+        outs = [DevBuf(nbytes=xs[0].nbytes, offset=((si + k) % 7) * esz) for k in range(ndst)]
+        segs.append((n, [bufs[k].ptr for k in order], [o.ptr for o in outs]))
+        checks.append((xs, order, bufs, outs))
+    hcclx.fold_wide(segs, dtype, op)
+    sync()
+    for xs, order, bufs, outs in checks:
+        want = fold_oracle(xs, dtype, op, order, wide=fused_is_wide(dtype, op))
+        for o in outs:
+            assert_same_bits(o.get(T.NP_STORAGE[dtype]), want, dtype)
+            assert o.guard_intact()
+        assert all(b.guard_intact() for b in bufs)
+
+
+def test_wide_fold_in_place_copy_of_any_type_plan_and_errors():
+    rng = np.random.default_rng(77)
+    n, nsrc = 50001, 20
+    xs = [payload(rng, T.FP32, n, "uniform") for _ in range(nsrc)]
+    bufs = [DevBuf(x) for x in xs]
+    segs = [(n, [b.ptr for b in bufs], [bufs[0].ptr, bufs[7].ptr])]     # two destinations alias sources
+    plan = hcclx.Plan(segs, T.FP32, T.SUM, wide=True)
+    assert plan.bytes == (nsrc + 2) * n * 4
+    plan.launch()
+    sync()
+    want = fold_oracle(xs, T.FP32, T.SUM, list(range(nsrc)), False)
+    assert_same_bits(bufs[0].get(np.float32), want, T.FP32)
+    assert_same_bits(bufs[7].get(np.float32), want, T.FP32)
+    plan.close()
+    raw = rng.integers(0, 255, size=30011, dtype=np.uint8)              # a copy moves any type as bytes
+    src = DevBuf(raw, offset=3)
+    outs = [DevBuf(nbytes=raw.nbytes, offset=k % 16) for k in range(33)]
+    hcclx.fold_wide([(raw.size, [src.ptr], [o.ptr for o in outs])], T.UINT8)
+    sync()
+    for o in outs:
+        assert np.array_equal(o.get(np.uint8), raw) and o.guard_intact()
+    b = DevBuf(nbytes=64)
+    with pytest.raises(HcclError) as e:
+        hcclx.fold_wide([(4, [b.ptr] * 65, [b.ptr])], T.FP32, T.SUM)
+    assert e.value.code == 1
+    with pytest.raises(HcclError) as e:
+        hcclx.fold_wide([(4, [b.ptr] * 20, [b.ptr] * 19 + [0])], T.FP32, T.SUM)
+    assert e.value.code == 2
+    with pytest.raises(HcclError) as e:
+        hcclx.fold_wide([(4, [b.ptr] * 20, [b.ptr])], T.UINT8, T.SUM)
+    assert e.value.code == 5
+    hcclx.fold_wide([], T.FP32, T.SUM)
+    hcclx.fold_wide([(0, [0] * 20, [0])], T.FP32)
+    sync()
+
+
 def random_tree(rng, nsrc, max_levels=4):
     """A random (dst register, src register) program over nsrc registers whose tree has at most
     max_levels levels, register 0 holding the root."""
