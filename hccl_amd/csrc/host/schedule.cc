@@ -188,10 +188,12 @@ HcclResult BuildOrder(World *w, std::vector<Node> &order, u32 &numLevels, CheckR
 // ---------------------------------------------------------------------------------------------------
 // STEP mode: every recorded copy / reduce is launched, one fold launch per level and kind
 // ---------------------------------------------------------------------------------------------------
-HcclResult LaunchSteps(World *w, const std::vector<Node> &order, u32 numLevels, int dtype, int op, void *stream)
+// STEP mode: the recorded steps as they are, level by level; the copies of a level are one launch and its
+// reduce steps another.  The launches are built as plans so that a repeated collective only replays them.
+HcclResult BuildStepPlans(const std::vector<Node> &order, u32 numLevels, int dtype, int op,
+                          std::vector<hcclx_plan *> &plans)
 {
     size_t i = 0;
-    w->lastLaunches = 0;
     for (u32 level = 0; level < numLevels; ++level) {
         std::vector<hcclx_seg_t> copies;
         std::vector<hcclx_seg_t> reduces;
@@ -216,17 +218,14 @@ HcclResult LaunchSteps(World *w, const std::vector<Node> &order, u32 numLevels, 
                 reduces.push_back(s);
             }
         }
-        if (!copies.empty()) {
-            const int rc = hcclx_fold(copies.data(), static_cast<uint32_t>(copies.size()), HCCL_DATA_TYPE_INT8, 0,
-                                      HCCLX_FOLD_CHAIN, stream);
+        for (int part = 0; part < 2; ++part) {
+            const std::vector<hcclx_seg_t> &segs = part == 0 ? copies : reduces;
+            if (segs.empty()) continue;
+            hcclx_plan *hp = nullptr;
+            const int rc = hcclx_plan_create(segs.data(), static_cast<uint32_t>(segs.size()),
+                                             part == 0 ? HCCL_DATA_TYPE_INT8 : dtype, part == 0 ? 0 : op, HCCLX_FOLD_CHAIN, &hp);
             if (rc != HCCL_SUCCESS) return static_cast<HcclResult>(rc);
-            w->lastLaunches++;
-        }
-        if (!reduces.empty()) {
-            const int rc = hcclx_fold(reduces.data(), static_cast<uint32_t>(reduces.size()), dtype, op,
-                                      HCCLX_FOLD_CHAIN, stream);
-            if (rc != HCCL_SUCCESS) return static_cast<HcclResult>(rc);
-            w->lastLaunches++;
+            plans.push_back(hp);
         }
     }
     return HCCL_SUCCESS;
@@ -818,6 +817,37 @@ HcclResult LaunchPlans(World *w, const std::vector<hcclx_plan *> &plans, void *s
     return HCCL_SUCCESS;
 }
 
+void DropPlans(std::vector<hcclx_plan *> &plans)
+{
+    for (hcclx_plan *q : plans) (void)hcclx_plan_destroy(q);
+    plans.clear();
+}
+
+// Launches a freshly built plan and, when it has a key, keeps it for the next identical collective (the least
+// recently used of 32 makes room).  A plan that is not kept is destroyed once its kernels have finished.
+HcclResult LaunchAndKeep(World *w, CachedPlan &&c, void *stream)
+{
+    const HcclResult res = LaunchPlans(w, c.plans, stream);
+    if (!c.key.empty() && res == HCCL_SUCCESS) {
+        c.lastUse = ++w->useCounter;
+        if (w->planCache.size() >= 32) {
+            size_t victim = 0;
+            for (size_t i = 1; i < w->planCache.size(); ++i) {
+                if (w->planCache[i].lastUse < w->planCache[victim].lastUse) victim = i;
+            }
+            // its kernels may still be queued: wait for the device before the tables are freed
+            (void)hipDeviceSynchronize();
+            DropPlans(w->planCache[victim].plans);
+            w->planCache.erase(w->planCache.begin() + victim);
+        }
+        w->planCache.push_back(std::move(c));
+    } else {
+        (void)hipDeviceSynchronize();
+        DropPlans(c.plans);
+    }
+    return res;
+}
+
 bool SameOperands(const OpParam &a, const OpParam &b)
 {
     if (a.opType != b.opType) return false;
@@ -978,12 +1008,14 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
         return LaunchDataMove(w, params, stream);
     }
     std::vector<u64> key;
-    if (fused && !w->dryRun && !w->traceText && !w->check) {
+    if (!w->dryRun && !w->traceText && !w->check) {
         key = PlanKey(params, algName, w->cclBytes);
+        key.push_back(fused ? 1 : 0);
         for (CachedPlan &c : w->planCache) {
             if (c.key == key) {
                 c.lastUse = ++w->useCounter;
-                w->lastWasFused = true;
+                w->lastWasFused = c.fused;
+                w->lastLevels = c.levels;
                 w->lastPlanCacheHit = true;
                 return LaunchPlans(w, c.plans, stream);
             }
@@ -1040,6 +1072,7 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
         if (ok && fused) {
             CachedPlan c;
             c.key = key;
+            c.levels = numLevels;
             const std::pair<std::vector<hcclx_seg_t> *, int> parts[4] = {
                 {&plan.selfSegs, HCCLX_FOLD_SELF_FIRST}, {&plan.chainSegs, HCCLX_FOLD_CHAIN},
                 {&plan.copySegs, HCCLX_FOLD_CHAIN}, {&plan.treeSegs, HCCLX_FOLD_TREE}};
@@ -1050,7 +1083,7 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
                 const int rc = hcclx_plan_create(parts[i].first->data(), static_cast<uint32_t>(parts[i].first->size()),
                                                  dt, op, parts[i].second, &hp);
                 if (rc != HCCL_SUCCESS) {
-                    for (hcclx_plan *q : c.plans) (void)hcclx_plan_destroy(q);
+                    DropPlans(c.plans);
                     return static_cast<HcclResult>(rc);
                 }
                 c.plans.push_back(hp);
@@ -1060,34 +1093,25 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
                 const int rc = hcclx_plan_create_wide(plan.wideSegs.data(), static_cast<uint32_t>(plan.wideSegs.size()),
                                                       foldType, op, &hp);
                 if (rc != HCCL_SUCCESS) {
-                    for (hcclx_plan *q : c.plans) (void)hcclx_plan_destroy(q);
+                    DropPlans(c.plans);
                     return static_cast<HcclResult>(rc);
                 }
                 c.plans.push_back(hp);
             }
             w->lastWasFused = true;
-            const HcclResult res = LaunchPlans(w, c.plans, stream);
-            if (!key.empty() && res == HCCL_SUCCESS) {
-                c.lastUse = ++w->useCounter;
-                if (w->planCache.size() >= 32) {  // evict the least recently used plan
-                    size_t victim = 0;
-                    for (size_t i = 1; i < w->planCache.size(); ++i) {
-                        if (w->planCache[i].lastUse < w->planCache[victim].lastUse) victim = i;
-                    }
-                    // its kernels may still be queued: wait for the device before the tables are freed
-                    (void)hipDeviceSynchronize();
-                    for (hcclx_plan *q : w->planCache[victim].plans) (void)hcclx_plan_destroy(q);
-                    w->planCache.erase(w->planCache.begin() + victim);
-                }
-                w->planCache.push_back(std::move(c));
-            } else {
-                (void)hipDeviceSynchronize();
-                for (hcclx_plan *q : c.plans) (void)hcclx_plan_destroy(q);
-            }
-            return res;
+            return LaunchAndKeep(w, std::move(c), stream);
         }
     }
-    return LaunchSteps(w, order, numLevels, foldType, op, stream);
+    CachedPlan c;
+    c.key = key;
+    c.fused = false;
+    c.levels = numLevels;
+    const HcclResult built = BuildStepPlans(order, numLevels, foldType, op, c.plans);
+    if (built != HCCL_SUCCESS) {
+        DropPlans(c.plans);
+        return built;
+    }
+    return LaunchAndKeep(w, std::move(c), stream);
 }
 
 }  // namespace

@@ -69,8 +69,10 @@ struct QueuedOp {
 
 struct CachedPlan {
     std::vector<u64> key;
-    std::vector<hcclx_plan *> plans;
+    std::vector<hcclx_plan *> plans;   // launched in this order
     u64 lastUse = 0;
+    bool fused = true;                 // false: the recorded steps, one or two plans per level
+    u32 levels = 0;
 };
 
 // What the schedule check found in the last collective (see hcclxCommSetCheck).

@@ -110,6 +110,36 @@ def test_checked_world_verifies_then_launches(stream):
         w.close()
 
 
+def test_step_by_step_plans_are_replayed_with_new_data(stream):
+    """A schedule that cannot be fused (the NHR tree among 20 ranks is deeper than the tree kernel) and the
+    explicit step-by-step mode: the second identical call replays the per-level launches from the cache, on the
+    data the buffers hold then."""
+    n, count = 20, 40009
+    for mode, alg in [(api.EXEC_FUSED, "InsAllReduceNHR"), (api.EXEC_STEP, "InsAllReduceMesh1DTwoShot")]:
+        w = api.World(n, ccl_bytes=SMALL_CCL)
+        try:
+            w.set_mode(mode)
+            w.set_algorithm(api.CMD_ALLREDUCE, alg)
+            rng = np.random.default_rng(3)
+            send = [DevBuf(nbytes=count * 4) for _ in range(n)]
+            recv = [DevBuf(nbytes=count * 4) for _ in range(n)]
+            for rep in range(3):
+                xs = [payload(rng, T.FP32, count, "uniform") for _ in range(n)]
+                for r in range(n):
+                    send[r].t[:count * 4] = torch.from_numpy(xs[r].view(np.uint8).copy()).to("cuda:0")
+                torch.cuda.synchronize()
+                for r in range(n):
+                    assert w.all_reduce(r, send[r].ptr, recv[r].ptr, count, T.FP32, T.SUM, stream.cuda_stream) == 0
+                stream.synchronize()
+                info = w.last_info()
+                assert info.fused == 0 and info.planCacheHit == (rep > 0) and info.launches >= info.levels > 1
+                want = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs, count, 4, alg, ccl_bytes=SMALL_CCL)
+                for r in range(n):
+                    assert_same_bits(recv[r].get(np.float32), want[r], T.FP32, f"{alg} rep {rep} rank {r}")
+        finally:
+            w.close()
+
+
 def test_allreduce_default_selector_and_plan_cache(stream):
     """Config 1 of the baseline: AllReduce SUM fp32, 8 ranks x 1,048,576 elements, uniform[-1,1): the
     selector takes the one-shot mesh template at this size; the ring template is forced next."""
