@@ -33,6 +33,7 @@ class WideSeg(ctypes.Structure):
         ("ndst", ctypes.c_uint32),
         ("src", ctypes.c_void_p * MAX_WIDE_FAN),
         ("dst", ctypes.c_void_p * MAX_WIDE_FAN),
+        ("prog", ctypes.c_uint8 * (2 * MAX_WIDE_FAN)),
     ]
 
 
@@ -62,10 +63,11 @@ def load():
     lib.hcclx_plan_create.argtypes = [ctypes.POINTER(Seg), ctypes.c_uint32, ctypes.c_int, ctypes.c_int,
                                       ctypes.c_int, ctypes.POINTER(ctypes.c_void_p)]
     lib.hcclx_fold_wide.restype = ctypes.c_int
-    lib.hcclx_fold_wide.argtypes = [ctypes.POINTER(WideSeg), ctypes.c_uint32, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    lib.hcclx_fold_wide.argtypes = [ctypes.POINTER(WideSeg), ctypes.c_uint32, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                    ctypes.c_void_p]
     lib.hcclx_plan_create_wide.restype = ctypes.c_int
     lib.hcclx_plan_create_wide.argtypes = [ctypes.POINTER(WideSeg), ctypes.c_uint32, ctypes.c_int, ctypes.c_int,
-                                           ctypes.POINTER(ctypes.c_void_p)]
+                                           ctypes.c_int, ctypes.POINTER(ctypes.c_void_p)]
     lib.hcclx_plan_launch.restype = ctypes.c_int
     lib.hcclx_plan_launch.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
     lib.hcclx_plan_destroy.restype = ctypes.c_int

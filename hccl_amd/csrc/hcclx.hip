@@ -216,57 +216,85 @@ struct Built {
     uint64_t algo_bytes = 0;
 };
 
-// Embeds the (dst, src) step program of a tree segment into a complete binary tree with `slots` leaf
-// slots: fills the slot order of the sources, the per-node codes and the leaf mask.  Returns false when
-// the tree is deeper than log2(slots).
-bool embed_tree(const hcclx_seg_t &s, uint32_t slots, SegDev *sd)
+// Embeds the (dst, src) step program of a tree over nsrc registers into a complete binary tree with `slots`
+// leaf slots: code[i] of inner heap node i (0 = nothing below, 1 = take the dst child, 2 = combine) and, per
+// leaf slot, the register whose source sits there (-1 = empty).  Returns false when the tree is deeper than
+// log2(slots).
+bool embed_tree(uint32_t nsrc, const uint8_t *prog, uint32_t slots, std::vector<uint8_t> *code, std::vector<int> *slot_reg)
 {
     struct N {
         int dst = -1, src = -1, leaf = -1;
     };
-    std::vector<N> nodes(s.nsrc);
-    std::vector<int> holder(s.nsrc);  // node currently held by each register
-    for (uint32_t k = 0; k < s.nsrc; ++k) {
+    std::vector<N> nodes(nsrc);
+    std::vector<int> holder(nsrc);  // node currently held by each register
+    for (uint32_t k = 0; k < nsrc; ++k) {
         nodes[k].leaf = static_cast<int>(k);
         holder[k] = static_cast<int>(k);
     }
-    for (uint32_t t = 0; t + 1 < s.nsrc; ++t) {
+    for (uint32_t t = 0; t + 1 < nsrc; ++t) {
         N n;
-        n.dst = holder[s.prog[2 * t]];
-        n.src = holder[s.prog[2 * t + 1]];
+        n.dst = holder[prog[2 * t]];
+        n.src = holder[prog[2 * t + 1]];
         nodes.push_back(n);
-        holder[s.prog[2 * t]] = static_cast<int>(nodes.size()) - 1;
+        holder[prog[2 * t]] = static_cast<int>(nodes.size()) - 1;
     }
-    sd->tree_codes = 0;
-    sd->leaf_mask = 0;
-    for (uint32_t k = 0; k < kMaxFan; ++k) sd->src[k] = nullptr;
-    bool ok = true;
+    code->assign(slots, 0);
+    slot_reg->assign(slots, -1);
     // place(node, heap index): inner nodes combine their two children; a leaf above the bottom level is
     // passed up from the left-most slot below it
     std::vector<std::pair<int, uint32_t>> stack{{holder[0], 1u}};
-    while (!stack.empty() && ok) {
+    while (!stack.empty()) {
         const int id = stack.back().first;
         uint32_t at = stack.back().second;
         stack.pop_back();
         const N &n = nodes[id];
         if (n.leaf >= 0) {
             while (at < slots) {
-                sd->tree_codes |= 1u << (2 * at);
+                (*code)[at] = 1;
                 at *= 2;
             }
-            sd->src[at - slots] = static_cast<const char *>(s.src[n.leaf]);
-            sd->leaf_mask |= 1u << (at - slots);
+            (*slot_reg)[at - slots] = n.leaf;
         } else {
-            if (at >= slots) {
-                ok = false;
-                break;
-            }
-            sd->tree_codes |= 2u << (2 * at);
+            if (at >= slots) return false;
+            (*code)[at] = 2;
             stack.push_back({n.dst, 2 * at});
             stack.push_back({n.src, 2 * at + 1});
         }
     }
-    return ok;
+    return true;
+}
+
+bool embed_tree(const hcclx_seg_t &s, uint32_t slots, SegDev *sd)
+{
+    std::vector<uint8_t> code;
+    std::vector<int> slot_reg;
+    if (!embed_tree(s.nsrc, s.prog, slots, &code, &slot_reg)) return false;
+    sd->tree_codes = 0;
+    sd->leaf_mask = 0;
+    for (uint32_t k = 0; k < kMaxFan; ++k) sd->src[k] = nullptr;
+    for (uint32_t i = 1; i < slots; ++i) sd->tree_codes |= static_cast<uint32_t>(code[i]) << (2 * i);
+    for (uint32_t k = 0; k < slots; ++k) {
+        if (slot_reg[k] < 0) continue;
+        sd->src[k] = static_cast<const char *>(s.src[slot_reg[k]]);
+        sd->leaf_mask |= 1u << k;
+    }
+    return true;
+}
+
+// Checks a tree program: nsrc - 1 steps, every register but 0 consumed exactly once, register 0 never, no
+// step on a consumed register.  Returns the number of levels of the tree, or -1 when it is malformed.
+int tree_levels(uint32_t nsrc, const uint8_t *prog)
+{
+    std::vector<bool> dead(nsrc, false);
+    std::vector<uint32_t> depth(nsrc, 0);
+    for (uint32_t t = 0; t + 1 < nsrc; ++t) {
+        const uint32_t rd = prog[2 * t];
+        const uint32_t rs = prog[2 * t + 1];
+        if (rd >= nsrc || rs >= nsrc || rd == rs || rs == 0 || dead[rd] || dead[rs]) return -1;
+        dead[rs] = true;
+        depth[rd] = (depth[rd] > depth[rs] ? depth[rd] : depth[rs]) + 1;
+    }
+    return static_cast<int>(depth[0]);
 }
 
 int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, Built *out)
@@ -298,23 +326,13 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
             }
         }
         if (mode == HCCLX_FOLD_TREE) {
-            // every register but 0 is consumed exactly once, register 0 never; a consumed register is dead
-            bool dead[HCCLX_MAX_FAN] = {false};
-            uint32_t depth[HCCLX_MAX_FAN] = {0};
-            for (uint32_t t = 0; t + 1 < s.nsrc; ++t) {
-                const uint32_t rd = s.prog[2 * t];
-                const uint32_t rs = s.prog[2 * t + 1];
-                if (rd >= s.nsrc || rs >= s.nsrc || rd == rs || rs == 0 || dead[rd] || dead[rs]) {
-                    return fail(HCCL_E_PARA, "segment " + std::to_string(i) + ": malformed tree program");
-                }
-                dead[rs] = true;
-                depth[rd] = (depth[rd] > depth[rs] ? depth[rd] : depth[rs]) + 1;
-            }
-            if (is_float_dtype(dtype) && (1u << depth[0]) > HCCLX_MAX_FAN) {
-                return fail(HCCL_E_NOT_SUPPORT, "segment " + std::to_string(i) + ": tree has " + std::to_string(depth[0]) +
+            const int levels = tree_levels(s.nsrc, s.prog);
+            if (levels < 0) return fail(HCCL_E_PARA, "segment " + std::to_string(i) + ": malformed tree program");
+            if (is_float_dtype(dtype) && (1u << levels) > HCCLX_MAX_FAN) {
+                return fail(HCCL_E_NOT_SUPPORT, "segment " + std::to_string(i) + ": tree has " + std::to_string(levels) +
                                                     " levels, the kernel holds 4");
             }
-            if (depth[0] > max_depth) max_depth = depth[0];
+            if (static_cast<uint32_t>(levels) > max_depth) max_depth = static_cast<uint32_t>(levels);
         }
         if (s.nsrc > max_src) max_src = s.nsrc;
     }
@@ -374,9 +392,12 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
 }
 
 // Wide segments: chain order, up to kMaxWideFan sources and destinations, one kernel for every fan-in.
-int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, Built *out)
+int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, Built *out)
 {
     if (nseg != 0 && segs == nullptr) return fail(HCCL_E_PTR, "segs is null");
+    if (mode != HCCLX_FOLD_CHAIN && mode != HCCLX_FOLD_TREE) {
+        return fail(mode == HCCLX_FOLD_SELF_FIRST ? HCCL_E_NOT_SUPPORT : HCCL_E_PARA, "wide segments fold as a chain or as a tree");
+    }
     int esz = dtype_size(dtype);
     if (esz == 0) return fail(HCCL_E_NOT_SUPPORT, "unknown data type " + std::to_string(dtype));
     uint32_t max_src = 0;
@@ -394,12 +415,21 @@ int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, i
                 if (s.dst[k] == nullptr) return fail(HCCL_E_PTR, "segment " + std::to_string(i) + ": null destination");
             }
         }
+        if (mode == HCCLX_FOLD_TREE) {
+            const int levels = tree_levels(s.nsrc, s.prog);
+            if (levels < 0) return fail(HCCL_E_PARA, "segment " + std::to_string(i) + ": malformed tree program");
+            if (is_float_dtype(dtype) && (1u << levels) > HCCLX_MAX_WIDE_FAN) {
+                return fail(HCCL_E_NOT_SUPPORT, "segment " + std::to_string(i) + ": tree has " + std::to_string(levels) +
+                                                    " levels, the kernel holds 6");
+            }
+        }
         if (s.nsrc > max_src) max_src = s.nsrc;
     }
     Batch proto;
     proto.dtype = dtype;
     proto.op = op;
-    proto.mode = HCCLX_FOLD_CHAIN;
+    // a tree over integers equals the chain of its leaves
+    proto.mode = (mode == HCCLX_FOLD_TREE && is_float_dtype(dtype) && max_src > 1) ? HCCLX_FOLD_TREE : HCCLX_FOLD_CHAIN;
     proto.maxn = kMaxWideFan;
     uint64_t scale = 1;
     if (max_src <= 1) {
@@ -424,6 +454,20 @@ int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, i
         sd.ndst = s.ndst;
         for (uint32_t k = 0; k < s.nsrc; ++k) sd.src[k] = static_cast<const char *>(s.src[k]);
         for (uint32_t k = 0; k < s.ndst; ++k) sd.dst[k] = static_cast<char *>(s.dst[k]);
+        if (proto.mode == HCCLX_FOLD_TREE) {
+            std::vector<uint8_t> code;
+            std::vector<int> slot_reg;
+            if (!embed_tree(s.nsrc, s.prog, kMaxWideFan, &code, &slot_reg)) {
+                return fail(HCCL_E_NOT_SUPPORT, "segment " + std::to_string(i) + ": tree deeper than 6 levels");
+            }
+            for (uint32_t node = 1; node < static_cast<uint32_t>(kMaxWideFan); ++node) {
+                sd.tree_codes[node / 16] |= static_cast<uint32_t>(code[node]) << (2 * (node % 16));
+            }
+            for (uint32_t k = 0; k < static_cast<uint32_t>(kMaxWideFan); ++k) {
+                sd.src[k] = slot_reg[k] < 0 ? nullptr : static_cast<const char *>(s.src[slot_reg[k]]);
+                if (slot_reg[k] >= 0) sd.leaf_mask |= 1ull << k;
+            }
+        }
         sd.head = fold_head_of(sd.count, esz, sd.dst[0]);
         sd.shift = fold_shift_of(sd.head, esz, kMaxWideFan, sd.dst[0]);
         const uint64_t tiles = fold_tiles_of(sd.count, ne, kMaxWideFan, sd.head, sd.shift);
@@ -550,12 +594,12 @@ int hcclx_fold(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mo
     return launch_built(ctx, built, static_cast<hipStream_t>(stream));
 }
 
-int hcclx_fold_wide(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, void *stream)
+int hcclx_fold_wide(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, void *stream)
 {
     DeviceCtx *ctx = device_ctx();
     if (!ctx) return HCCL_E_RUNTIME;
     Built built;
-    int rc = build_wide_batches(segs, nseg, dtype, op, &built);
+    int rc = build_wide_batches(segs, nseg, dtype, op, mode, &built);
     if (rc != HCCL_SUCCESS) return rc;
     return launch_built(ctx, built, static_cast<hipStream_t>(stream));
 }
@@ -572,14 +616,15 @@ int hcclx_plan_create(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op,
     return plan_from(ctx, built, plan);
 }
 
-int hcclx_plan_create_wide(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, hcclx_plan_t **plan)
+int hcclx_plan_create_wide(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode,
+                           hcclx_plan_t **plan)
 {
     if (plan == nullptr) return fail(HCCL_E_PTR, "plan is null");
     *plan = nullptr;
     DeviceCtx *ctx = device_ctx();
     if (!ctx) return HCCL_E_RUNTIME;
     Built built;
-    int rc = build_wide_batches(segs, nseg, dtype, op, &built);
+    int rc = build_wide_batches(segs, nseg, dtype, op, mode, &built);
     if (rc != HCCL_SUCCESS) return rc;
     return plan_from(ctx, built, plan);
 }

@@ -368,7 +368,8 @@ struct Fold {
     u64 dst = 0;
     u64 bytes = 0;
     bool chain = true;        // false: a tree that no chain reproduces
-    bool fits = true;         // false: a tree too large for the tree kernel
+    bool fits = true;         // false: a tree too large for the tree kernels
+    u32 levels = 0;           // tree: levels below the root
     std::vector<u8> prog;     // tree: (dst register, src register) per step over src[] as registers
 };
 
@@ -456,12 +457,13 @@ Fold Flatten(const Tracer &tr, int e, u64 shift, int dtype, int op)
             sh += x.srcShift;
             cur = x.src;
         } else {
-            // not a spine: keep the tree as it is, for the kernel that evaluates trees of up to
-            // log2(HCCLX_MAX_FAN) levels in registers
+            // not a spine: keep the tree as it is, for the kernels that evaluate trees of up to four levels
+            // (six in the wide kernel) in registers
             f.chain = false;
             u32 levels = 0;
             (void)EmitTree(tr, e, shift, f, &levels);
-            f.fits = (f.src.size() <= HCCLX_MAX_FAN && (1u << levels) <= HCCLX_MAX_FAN);
+            f.levels = levels;
+            f.fits = (f.src.size() <= HCCLX_MAX_WIDE_FAN && levels <= 6);
             return f;
         }
     }
@@ -475,14 +477,15 @@ struct FusedPlan {
     std::vector<hcclx_seg_t> selfSegs;
     std::vector<hcclx_seg_t> copySegs;
     std::vector<hcclx_seg_t> treeSegs;
-    std::vector<hcclx_wide_seg_t> wideSegs;   // chains over more than HCCLX_MAX_FAN sources
+    std::vector<hcclx_wide_seg_t> wideSegs;       // chains over more than HCCLX_MAX_FAN sources
+    std::vector<hcclx_wide_seg_t> wideTreeSegs;   // trees with more leaves or levels than the 16-slot kernel holds
 };
 
 bool Overlaps(u64 a, u64 alen, u64 b, u64 blen) { return a < b + blen && b < a + alen; }
 
 // Builds the fused launch plan from the traced outputs.  Returns false when the schedule cannot be fused
-// (a floating-point tree with more than four levels, a source that is not an input, or an output that overlaps another fold's
-// source); the caller then runs the steps one by one.
+// (a floating-point tree with more than six levels or 64 leaves, a source that is not an input, or an output
+// that overlaps another fold's source); the caller then runs the steps one by one.
 bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &params, int dtype, int op, u32 esz,
                     FusedPlan &plan, std::string *text)
 {
@@ -618,10 +621,10 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
         for (size_t i : kv.second) {
             if (!taken[i]) rest.push_back(i);
         }
-        if (!rest.empty() && folds[rest[0]].src.size() > HCCLX_MAX_FAN) {
-            // more ranks than the register-resident kernels take: the wide chain kernel
+        if (!rest.empty() && (folds[rest[0]].src.size() > HCCLX_MAX_FAN || (1u << folds[rest[0]].levels) > HCCLX_MAX_FAN)) {
+            // more ranks than the register-resident kernels take: the wide kernels
             const Fold &f = folds[rest[0]];
-            if (!f.chain || f.src.size() > HCCLX_MAX_WIDE_FAN) return false;
+            if (f.src.size() > HCCLX_MAX_WIDE_FAN) return false;
             for (size_t at = 0; at < rest.size(); at += HCCLX_MAX_WIDE_FAN) {
                 hcclx_wide_seg_t seg;
                 std::memset(&seg, 0, sizeof(seg));
@@ -631,7 +634,12 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
                 for (size_t d = at; d < rest.size() && d < at + HCCLX_MAX_WIDE_FAN; ++d) {
                     seg.dst[seg.ndst++] = reinterpret_cast<void *>(folds[rest[d]].dst);
                 }
-                plan.wideSegs.push_back(seg);
+                if (f.chain) {
+                    plan.wideSegs.push_back(seg);
+                } else {
+                    std::memcpy(seg.prog, f.prog.data(), f.prog.size());
+                    plan.wideTreeSegs.push_back(seg);
+                }
             }
             continue;
         }
@@ -1064,7 +1072,7 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
                                        (w->traceText || w->dryRun) ? &w->lastTrace : nullptr);
         w->lastFusedSegments =
             static_cast<u32>(plan.chainSegs.size() + plan.selfSegs.size() + plan.copySegs.size() + plan.treeSegs.size() +
-                             plan.wideSegs.size());
+                             plan.wideSegs.size() + plan.wideTreeSegs.size());
         if (w->dryRun) {
             w->lastWasFused = ok;
             return HCCL_SUCCESS;
@@ -1088,10 +1096,12 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
                 }
                 c.plans.push_back(hp);
             }
-            if (!plan.wideSegs.empty()) {
+            for (int i = 0; i < 2; ++i) {
+                const std::vector<hcclx_wide_seg_t> &segs = i == 0 ? plan.wideSegs : plan.wideTreeSegs;
+                if (segs.empty()) continue;
                 hcclx_plan *hp = nullptr;
-                const int rc = hcclx_plan_create_wide(plan.wideSegs.data(), static_cast<uint32_t>(plan.wideSegs.size()),
-                                                      foldType, op, &hp);
+                const int rc = hcclx_plan_create_wide(segs.data(), static_cast<uint32_t>(segs.size()), foldType, op,
+                                                      i == 0 ? HCCLX_FOLD_CHAIN : HCCLX_FOLD_TREE, &hp);
                 if (rc != HCCL_SUCCESS) {
                     DropPlans(c.plans);
                     return static_cast<HcclResult>(rc);

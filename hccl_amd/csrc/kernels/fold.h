@@ -65,27 +65,35 @@ __device__ __forceinline__ uint64_t uniform64(uint64_t x)
     return (static_cast<uint64_t>(hi) << 32) | lo;
 }
 
-// Evaluates the embedded tree bottom-up.  leaf[k] are the MAXN leaf slots; every index below is a compile
-// time constant and every condition is wave-uniform, so the values stay in named registers.
-template <int DT, int OP, int MAXN, typename C, int NE>
-__device__ __forceinline__ void tree_eval(C (&leaf)[MAXN][NE], uint32_t codes)
+// Evaluates an embedded (sub)tree bottom-up.  leaf[k] are the SLOTS leaf slots below heap node ROOT; the node
+// at width w, position i of that subtree is heap node ROOT * w + i, and code(node) gives its 2-bit code.  Every
+// index below is a compile time constant and every condition is wave-uniform, so the values stay in named
+// registers.  The value of node ROOT ends up in leaf[0].
+template <int DT, int OP, int SLOTS, int ROOT, typename C, int NE, typename CODE>
+__device__ __forceinline__ void tree_eval_at(C (&leaf)[SLOTS][NE], CODE code)
 {
-    // level by level in place: after the pass for width w, leaf[0 .. w) hold the nodes w .. 2w-1
+    // level by level in place: after the pass for width w, leaf[0 .. w) hold the nodes ROOT*w .. ROOT*w + w-1
 #pragma unroll
-    for (int w = MAXN / 2; w >= 1; w /= 2) {
+    for (int w = SLOTS / 2; w >= 1; w /= 2) {
 #pragma unroll
         for (int i = 0; i < w; ++i) {
-            const uint32_t code = (codes >> (2 * (w + i))) & 3u;
-            if (code == 2u) {
+            const uint32_t c = code(ROOT * w + i);
+            if (c == 2u) {
 #pragma unroll
                 for (int e = 0; e < NE; ++e) leaf[i][e] = Vec16<DT>::template combine<OP>(leaf[2 * i + 1][e], leaf[2 * i][e]);
-            } else if (code == 1u && i != 0) {
+            } else if (c == 1u && i != 0) {
                 // pass the dst child up (for i == 0 it already sits in place)
 #pragma unroll
                 for (int e = 0; e < NE; ++e) leaf[i][e] = leaf[2 * i][e];
             }
         }
     }
+}
+
+template <int DT, int OP, int MAXN, typename C, int NE>
+__device__ __forceinline__ void tree_eval(C (&leaf)[MAXN][NE], uint32_t codes)
+{
+    tree_eval_at<DT, OP, MAXN, 1, C, NE>(leaf, [codes](int node) { return (codes >> (2 * node)) & 3u; });
 }
 
 template <int DT, int OP, int MAXN, int MODE, bool CHECK>
@@ -197,7 +205,11 @@ __device__ __forceinline__ void fold_tail(const SEG &sd, uint32_t nsrc, uint32_t
         for (int k = 0; k < MAXN; ++k) {
             if ((sd.leaf_mask >> k) & 1u) val[k][0] = D::widen(reinterpret_cast<const S *>(sd.src[k])[idx]);
         }
-        tree_eval<DT, OP, MAXN, C, 1>(val, sd.tree_codes);
+        if constexpr (MAXN > kMaxFan) {
+            tree_eval_at<DT, OP, MAXN, 1, C, 1>(val, [&sd](int node) { return (sd.tree_codes[node / 16] >> (2 * (node % 16))) & 3u; });
+        } else {
+            tree_eval<DT, OP, MAXN, C, 1>(val, sd.tree_codes);
+        }
         const S out = D::narrow(val[0][0]);
         for (uint32_t d = 0; d < ndst; ++d) reinterpret_cast<S *>(sd.dst[d])[idx] = out;
     } else {
@@ -295,7 +307,7 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
     }
 }
 
-// More than kMaxFan sources or destinations (chain order only): the sources are walked in groups of kMaxFan,
+// More than kMaxFan sources or destinations, chain order: the sources are walked in groups of kMaxFan,
 // each group loaded before it is folded in, so the loads in flight per thread stay what the 16-source kernel
 // has.  One vector per thread and tile.
 template <int DT, int OP, bool CHECK>
@@ -336,7 +348,69 @@ __device__ __forceinline__ void fold_tile_wide(const SegWide &sd, uint32_t nsrc,
     }
 }
 
-template <int DT, int OP>
+// The value of the subtree over leaf slots G * kMaxFan .. G * kMaxFan + kMaxFan - 1 (heap node
+// kMaxWideFan / kMaxFan + G); nothing is loaded and `out` is left alone when no leaf of it is present.
+template <int DT, int OP, int G>
+__device__ __forceinline__ void wide_subtree(const SegWide &sd, uint64_t off, uint64_t mask,
+                                             typename Vec16<DT>::C (&out)[Vec16<DT>::NE])
+{
+    using V = Vec16<DT>;
+    using C = typename V::C;
+    constexpr int NE = V::NE;
+    const uint32_t present = static_cast<uint32_t>(mask >> (G * kMaxFan)) & 0xffffu;
+    if (present == 0) {
+        return;
+    }
+    u32x4 raw[kMaxFan];
+#pragma unroll
+    for (int k = 0; k < kMaxFan; ++k) {
+        if ((present >> k) & 1u) raw[k] = ld16(sd.src[G * kMaxFan + k] + off);
+    }
+    C val[kMaxFan][NE];
+#pragma unroll
+    for (int k = 0; k < kMaxFan; ++k) {
+        if ((present >> k) & 1u) V::unpack(raw[k], val[k]);
+    }
+    tree_eval_at<DT, OP, kMaxFan, kMaxWideFan / kMaxFan + G, C, NE>(
+        val, [&sd](int node) { return (sd.tree_codes[node / 16] >> (2 * (node % 16))) & 3u; });
+#pragma unroll
+    for (int e = 0; e < NE; ++e) out[e] = val[0][e];
+}
+
+// A tree over up to kMaxWideFan leaf slots: the four subtrees of kMaxFan slots below heap nodes 4 .. 7 are
+// evaluated one after the other, each with its leaves loaded first as in the 16-slot kernel, and their values go
+// through the two top levels.
+template <int DT, int OP, bool CHECK>
+__device__ __forceinline__ void fold_tile_wide_tree(const SegWide &sd, uint32_t ndst, uint64_t v, uint64_t nvec,
+                                                    uint32_t head_bytes)
+{
+    using V = Vec16<DT>;
+    using C = typename V::C;
+    constexpr int NE = V::NE;
+    constexpr int kGroups = kMaxWideFan / kMaxFan;
+    if (CHECK && v >= nvec) {
+        return;
+    }
+    const uint64_t off = head_bytes + v * 16;
+    const uint64_t mask = sd.leaf_mask;
+    auto code = [&sd](int node) { return (sd.tree_codes[node / 16] >> (2 * (node % 16))) & 3u; };
+    C part[kGroups][NE];
+    wide_subtree<DT, OP, 0>(sd, off, mask, part[0]);
+    wide_subtree<DT, OP, 1>(sd, off, mask, part[1]);
+    wide_subtree<DT, OP, 2>(sd, off, mask, part[2]);
+    wide_subtree<DT, OP, 3>(sd, off, mask, part[3]);
+    static_assert(kGroups == 4, "the subtree roots above are heap nodes 4 .. 7");
+    tree_eval_at<DT, OP, kGroups, 1, C, NE>(part, code);
+    const u32x4 out = V::pack(part[0]);
+    for (uint32_t base = 0; base < ndst; base += kMaxFan) {
+#pragma unroll
+        for (int d = 0; d < kMaxFan; ++d) {
+            if (base + d < ndst) st16(sd.dst[base + d] + off, out);
+        }
+    }
+}
+
+template <int DT, int OP, int MODE>
 __global__ void __launch_bounds__(kFoldThreads)
 k_fold_wide(const uint64_t *__restrict__ tile_end, const SegWide *__restrict__ segs, uint32_t nseg, uint64_t total_tiles)
 {
@@ -366,12 +440,20 @@ k_fold_wide(const uint64_t *__restrict__ tile_end, const SegWide *__restrict__ s
         const uint32_t shift = sd.shift;
         const uint64_t v = tl * TV + threadIdx.x - shift;   // wraps in front of a shifted segment: fails the check
         if (tl * TV >= shift && (tl + 1) * TV - shift <= nvec) {
-            fold_tile_wide<DT, OP, false>(sd, nsrc, ndst, v, nvec, head_bytes);
+            if constexpr (MODE == kFoldTree) {
+                fold_tile_wide_tree<DT, OP, false>(sd, ndst, v, nvec, head_bytes);
+            } else {
+                fold_tile_wide<DT, OP, false>(sd, nsrc, ndst, v, nvec, head_bytes);
+            }
         } else {
-            fold_tile_wide<DT, OP, true>(sd, nsrc, ndst, v, nvec, head_bytes);
+            if constexpr (MODE == kFoldTree) {
+                fold_tile_wide_tree<DT, OP, true>(sd, ndst, v, nvec, head_bytes);
+            } else {
+                fold_tile_wide<DT, OP, true>(sd, nsrc, ndst, v, nvec, head_bytes);
+            }
             if (tl == (nvec + shift) / TV && threadIdx.x < head + rem) {
                 const uint64_t idx = threadIdx.x < head ? threadIdx.x : head + nvec * NE + (threadIdx.x - head);
-                fold_tail<DT, OP, kMaxWideFan, kFoldChain>(sd, nsrc, ndst, idx);
+                fold_tail<DT, OP, kMaxWideFan, MODE>(sd, nsrc, ndst, idx);
             }
         }
     }

@@ -15,10 +15,10 @@ static hipError_t launch_one(const FoldLaunch &l)
     return hipGetLastError();
 }
 
-template <int DT, int OP>
+template <int DT, int OP, int MODE>
 static hipError_t launch_wide(const FoldLaunch &l)
 {
-    hipLaunchKernelGGL((k_fold_wide<DT, OP>), dim3(l.grid), dim3(kFoldThreads), l.nseg * sizeof(uint64_t), l.stream,
+    hipLaunchKernelGGL((k_fold_wide<DT, OP, MODE>), dim3(l.grid), dim3(kFoldThreads), l.nseg * sizeof(uint64_t), l.stream,
                        l.tile_end, static_cast<const SegWide *>(l.segs), l.nseg, l.total_tiles);
     return hipGetLastError();
 }
@@ -40,7 +40,12 @@ static hipError_t by_fan(int maxn, const FoldLaunch &l)
         case 4: return launch_one<HCCLX_DT, OP, 4, MODE>(l);
         case 8: return launch_one<HCCLX_DT, OP, 8, MODE>(l);
         case 16: return launch_one<HCCLX_DT, OP, 16, MODE>(l);
-        case kMaxWideFan: return MODE == kFoldChain ? launch_wide<HCCLX_DT, OP>(l) : hipErrorInvalidValue;
+        case kMaxWideFan:
+            if constexpr (MODE == kFoldSelfFirst) {
+                return hipErrorInvalidValue;
+            } else {
+                return launch_wide<HCCLX_DT, OP, MODE>(l);
+            }
         default: return hipErrorInvalidValue;
     }
 }

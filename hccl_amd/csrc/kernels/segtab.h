@@ -36,14 +36,18 @@ struct SegDev {
     uint32_t shift;
 };
 
-// A chain segment of the wide kernel: acc = src[0]; acc = src[k] (+) acc for k = 1 .. nsrc-1; the value goes
-// to every dst.  head and shift as in SegDev, for tiles of one vector per thread.
+// A segment of the wide kernels.  Chain: acc = src[0]; acc = src[k] (+) acc for k = 1 .. nsrc-1.  Tree: as in
+// SegDev, embedded in a complete binary tree with kMaxWideFan leaf slots; the 2-bit code of inner node i sits at
+// bit 2 * (i % 16) of tree_codes[i / 16].  The value goes to every dst.  head and shift as in SegDev, for tiles
+// of one vector per thread.
 struct SegWide {
     uint64_t count;
     uint32_t nsrc;
     uint32_t ndst;
     uint32_t head;
     uint32_t shift;
+    uint64_t leaf_mask;
+    uint32_t tree_codes[4];
     const char *src[kMaxWideFan];
     char *dst[kMaxWideFan];
 };

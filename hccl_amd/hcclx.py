@@ -29,10 +29,14 @@ def make_segs(segs):
 
 
 def make_wide_segs(segs):
-    """segs: iterable of (count, [src addresses], [dst addresses]) -> ctypes array of hcclx_wide_seg_t."""
+    """segs: iterable of (count, [src addresses], [dst addresses][, tree program]) -> ctypes array of
+    hcclx_wide_seg_t."""
     segs = list(segs)
     arr = (WideSeg * max(1, len(segs)))()
-    for i, (count, srcs, dsts) in enumerate(segs):
+    for i, seg in enumerate(segs):
+        count, srcs, dsts = seg[0], seg[1], seg[2]
+        for k, b in enumerate((seg[3] if len(seg) > 3 else [])[:2 * _lib.MAX_WIDE_FAN]):
+            arr[i].prog[k] = b
         arr[i].count = count
         arr[i].nsrc = len(srcs)
         arr[i].ndst = len(dsts)
@@ -52,10 +56,10 @@ def fold(segs, dtype, op=0, mode=FOLD_CHAIN, stream=0):
     check(_lib.load().hcclx_fold(arr, n, int(dtype), int(op), int(mode), ctypes.c_void_p(stream)))
 
 
-def fold_wide(segs, dtype, op=0, stream=0):
-    """Chain-order fold of segments with up to 64 sources and destinations."""
+def fold_wide(segs, dtype, op=0, mode=FOLD_CHAIN, stream=0):
+    """Fold of segments with up to 64 sources and destinations (chain or tree order)."""
     arr, n = make_wide_segs(segs)
-    check(_lib.load().hcclx_fold_wide(arr, n, int(dtype), int(op), ctypes.c_void_p(stream)))
+    check(_lib.load().hcclx_fold_wide(arr, n, int(dtype), int(op), int(mode), ctypes.c_void_p(stream)))
 
 
 class Plan:
@@ -65,7 +69,7 @@ class Plan:
         h = ctypes.c_void_p()
         if wide:
             arr, n = make_wide_segs(segs)
-            check(_lib.load().hcclx_plan_create_wide(arr, n, int(dtype), int(op), ctypes.byref(h)))
+            check(_lib.load().hcclx_plan_create_wide(arr, n, int(dtype), int(op), int(mode), ctypes.byref(h)))
         else:
             arr, n = make_segs(segs)
             check(_lib.load().hcclx_plan_create(arr, n, int(dtype), int(op), int(mode), ctypes.byref(h)))

@@ -62,9 +62,9 @@ typedef struct {
     uint8_t prog[2 * HCCLX_MAX_FAN]; /* HCCLX_FOLD_TREE only: (dst register, src register) per step */
 } hcclx_seg_t;
 
-/* A chain-order segment with up to HCCLX_MAX_WIDE_FAN sources and destinations, for communicators of more than
- * HCCLX_MAX_FAN ranks:  acc = src[0]; acc = src[k] (+) acc for k = 1 .. nsrc-1; the result goes to
- * dst[0 .. ndst-1].  Aliasing rules as for hcclx_seg_t. */
+/* A segment with up to HCCLX_MAX_WIDE_FAN sources and destinations, for communicators of more than
+ * HCCLX_MAX_FAN ranks.  HCCLX_FOLD_CHAIN and HCCLX_FOLD_TREE as for hcclx_seg_t (a floating-point tree may have
+ * up to six levels); HCCLX_FOLD_SELF_FIRST is not taken.  Aliasing rules as for hcclx_seg_t. */
 #define HCCLX_MAX_WIDE_FAN 64
 typedef struct {
     uint64_t count;
@@ -72,6 +72,7 @@ typedef struct {
     uint32_t ndst;
     const void *src[HCCLX_MAX_WIDE_FAN];
     void *dst[HCCLX_MAX_WIDE_FAN];
+    uint8_t prog[2 * HCCLX_MAX_WIDE_FAN]; /* HCCLX_FOLD_TREE only */
 } hcclx_wide_seg_t;
 
 /* Library set-up for the current device: creates the descriptor arena.  Idempotent.  Called lazily by the
@@ -90,14 +91,15 @@ uint32_t hcclx_dtype_size(int dtype);
  * All segments of a call share nsrc's upper bound HCCLX_MAX_FAN.  segs is a host array, copied before
  * return. */
 int hcclx_fold(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, void *stream);
-/* The same for wide segments, chain order. */
-int hcclx_fold_wide(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, void *stream);
+/* The same for wide segments. */
+int hcclx_fold_wide(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, void *stream);
 
 /* The same, split in two so that a repeated collective uploads its table once. */
 typedef struct hcclx_plan hcclx_plan_t;
 int hcclx_plan_create(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, hcclx_plan_t **plan);
-/* A plan over wide segments (chain order); launched, measured and destroyed like any other plan. */
-int hcclx_plan_create_wide(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, hcclx_plan_t **plan);
+/* A plan over wide segments; launched, measured and destroyed like any other plan. */
+int hcclx_plan_create_wide(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode,
+                           hcclx_plan_t **plan);
 int hcclx_plan_launch(const hcclx_plan_t *plan, void *stream);
 int hcclx_plan_destroy(hcclx_plan_t *plan);
 /* Algorithmic bytes one launch of the plan moves: sum over segments of (nsrc + ndst) * count * size. */

@@ -111,11 +111,11 @@ def test_checked_world_verifies_then_launches(stream):
 
 
 def test_step_by_step_plans_are_replayed_with_new_data(stream):
-    """A schedule that cannot be fused (the NHR tree among 20 ranks is deeper than the tree kernel) and the
-    explicit step-by-step mode: the second identical call replays the per-level launches from the cache, on the
+    """A schedule that cannot be fused (among 9 ranks the ring's MAX fold is a spine of eight levels, and a
+    floating-point MAX cannot be reordered) and the explicit step-by-step mode: the second identical call replays the per-level launches from the cache, on the
     data the buffers hold then."""
-    n, count = 20, 40009
-    for mode, alg in [(api.EXEC_FUSED, "InsAllReduceNHR"), (api.EXEC_STEP, "InsAllReduceMesh1DTwoShot")]:
+    n, count = 9, 40009
+    for mode, alg, op in [(api.EXEC_FUSED, "InsAllReduceRing", T.MAX), (api.EXEC_STEP, "InsAllReduceMesh1DTwoShot", T.SUM)]:
         w = api.World(n, ccl_bytes=SMALL_CCL)
         try:
             w.set_mode(mode)
@@ -129,11 +129,11 @@ def test_step_by_step_plans_are_replayed_with_new_data(stream):
                     send[r].t[:count * 4] = torch.from_numpy(xs[r].view(np.uint8).copy()).to("cuda:0")
                 torch.cuda.synchronize()
                 for r in range(n):
-                    assert w.all_reduce(r, send[r].ptr, recv[r].ptr, count, T.FP32, T.SUM, stream.cuda_stream) == 0
+                    assert w.all_reduce(r, send[r].ptr, recv[r].ptr, count, T.FP32, op, stream.cuda_stream) == 0
                 stream.synchronize()
                 info = w.last_info()
                 assert info.fused == 0 and info.planCacheHit == (rep > 0) and info.launches >= info.levels > 1
-                want = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs, count, 4, alg, ccl_bytes=SMALL_CCL)
+                want = T.run_allreduce(T.NumericElems(T.FP32, op), xs, count, 4, alg, ccl_bytes=SMALL_CCL)
                 for r in range(n):
                     assert_same_bits(recv[r].get(np.float32), want[r], T.FP32, f"{alg} rep {rep} rank {r}")
         finally:
@@ -205,14 +205,14 @@ def test_reduce_scatter_both_templates_both_modes(stream, mode, alg, dtype, op, 
         w.close()
 
 
-@pytest.mark.parametrize("alg,fusable", [("InsAllReduceMesh1DTwoShot", True), ("InsAllReduceMesh1DOneShot", True),
-                                         ("InsAllReduceRing", True), ("InsAllReduceAicpuReduceNHR", True),
-                                         ("InsAllReduceNHR", False), ("InsAllReduceRHD", False)])
+@pytest.mark.parametrize("alg", ["InsAllReduceMesh1DTwoShot", "InsAllReduceMesh1DOneShot", "InsAllReduceRing",
+                                 "InsAllReduceAicpuReduceNHR", "InsAllReduceNHR", "InsAllReduceRHD"])
 @pytest.mark.parametrize("dtype,op,n,count", [(T.FP32, T.SUM, 24, 50021), (T.BFP16, T.SUM, 32, 70001),
-                                             (T.INT32, T.MAX, 40, 30011), (T.FP64, T.PROD, 17, 20000)])
-def test_allreduce_among_more_than_16_ranks(stream, alg, fusable, dtype, op, n, count):
-    """Chains over more than 16 sources take the wide fold kernel and stay one pass; the trees of the log-step
-    templates are deeper than four levels for floating types and are launched step by step."""
+                                             (T.INT32, T.MAX, 40, 30011), (T.FP64, T.PROD, 17, 20000),
+                                             (T.FP16, T.SUM, 64, 66001)])
+def test_allreduce_among_more_than_16_ranks(stream, alg, dtype, op, n, count):
+    """Chains over more than 16 sources and the trees of the log-step templates (up to six levels) take the wide
+    fold kernels and stay one pass."""
     rng = np.random.default_rng(n * 11 + count)
     kind = "prod" if op == T.PROD else "uniform" if dtype == T.FP32 else "normal"
     xs = [payload(rng, dtype, count, kind) for _ in range(n)]
@@ -221,7 +221,7 @@ def test_allreduce_among_more_than_16_ranks(stream, alg, fusable, dtype, op, n, 
         w.set_algorithm(api.CMD_ALLREDUCE, alg)
         got, bufs = run_allreduce(w, stream, xs, count, dtype, op)
         info = w.last_info()
-        assert bool(info.fused) == (fusable or dtype == T.INT32), alg
+        assert info.fused == 1, alg
         if info.fused and dtype in (T.FP16, T.BFP16) and op == T.SUM:
             want = wide_oracle_allreduce(xs, count, dtype, alg, SMALL_CCL)
         else:
@@ -249,7 +249,7 @@ def test_reduce_scatter_among_more_than_16_ranks(stream, alg, dtype, op, n, rc):
         stream.synchronize()
         info = w.last_info()
         esz = T.DTYPE_SIZE[dtype]
-        assert bool(info.fused) == (alg != "InsReduceScatterNHR" or dtype == T.INT8), alg
+        assert info.fused == 1, alg
         if info.fused and dtype in (T.FP16, T.BFP16) and op == T.SUM:
             wide = [T.widen16(x, dtype) for x in xs]
             want = [T.narrow16(o, dtype) for o in
@@ -264,8 +264,8 @@ def test_reduce_scatter_among_more_than_16_ranks(stream, alg, dtype, op, n, rc):
 
 
 def test_reduce_scatter_order_preserved_at_40_ranks(stream):
-    """The grouped variant for more than 32 ranks; its 40-leaf tree is deeper than the fold kernel's tree
-    mode takes, so the steps are launched one by one."""
+    """The grouped variant for more than 32 ranks; its 40-leaf tree of six levels is one pass of the wide tree
+    kernel."""
     n, rc, dtype = 40, 5003, T.FP32
     rng = np.random.default_rng(40)
     xs = [payload(rng, dtype, n * rc, "normal") for _ in range(n)]
@@ -278,7 +278,7 @@ def test_reduce_scatter_order_preserved_at_40_ranks(stream):
         for r in range(n):
             assert w.reduce_scatter(r, send[r].ptr, recv[r].ptr, rc, dtype, T.SUM, stream.cuda_stream) == 0
         stream.synchronize()
-        assert not w.last_info().fused
+        assert w.last_info().fused == 1
         want = T.run_reduce_scatter(T.NumericElems(dtype, T.SUM), xs, rc, 4, "ReduceScatterOrderPreservedGroup",
                                     ccl_bytes=SMALL_CCL)
         for r in range(n):

@@ -209,6 +209,67 @@ def test_tree_fold_keeps_the_association_of_the_program(nsrc, dtype, op):
             assert o.guard_intact()
 
 
+def split_tree(rng, nsrc, max_levels):
+    """A random program over nsrc registers whose tree has at most max_levels levels: the registers (0 first)
+    are split recursively into a dst side and a src side that both still fit."""
+    regs = [0] + [int(r) + 1 for r in rng.permutation(nsrc - 1)]
+    prog = []
+
+    def node(lst, levels):
+        if len(lst) == 1:
+            return lst[0]
+        half = 1 << (levels - 1)
+        lo, hi = max(1, len(lst) - half), min(half, len(lst) - 1)
+        k = int(rng.integers(lo, hi + 1))
+        d = node(lst[:k], levels - 1)
+        s_ = node(lst[k:], levels - 1)
+        prog.extend([d, s_])
+        return d
+
+    node(regs, max_levels)
+    return prog
+
+
+@pytest.mark.parametrize("nsrc,levels", [(6, 5), (7, 6), (17, 5), (20, 6), (33, 6), (40, 6), (64, 6)])
+@pytest.mark.parametrize("dtype,op", [(T.FP32, T.SUM), (T.BFP16, T.SUM), (T.FP16, T.PROD), (T.FP64, T.MAX),
+                                      (T.INT32, T.SUM)])
+def test_wide_tree_fold_up_to_six_levels(nsrc, levels, dtype, op):
+    """hcclx_fold_wide in tree mode: trees with more leaves or levels than the 16-slot kernel holds (the NHR and
+    halving-doubling schedules among 17 .. 64 ranks)."""
+    rng = np.random.default_rng(nsrc * 77 + dtype * 3 + op)
+    kind = "prod" if op == T.PROD else "uniform" if dtype in (T.FP32, T.FP64) else "normal"
+    esz = T.DTYPE_SIZE[dtype]
+    segs, cases = [], []
+    for si, count in enumerate((2 * 4096 // esz + 5, 3)):
+        xs = [payload(rng, dtype, count, kind) for _ in range(nsrc)]
+        prog = split_tree(rng, nsrc, levels)
+        bufs = [DevBuf(x, offset=(k % 4) * esz) for k, x in enumerate(xs)]
+        outs = [DevBuf(nbytes=xs[0].nbytes, offset=(si + 3 * k) % 5 * esz) for k in range(18)]
+        segs.append((count, [b.ptr for b in bufs], [o.ptr for o in outs], prog))
+        cases.append((xs, prog, outs, bufs))     # the sources must stay allocated until the launch has run
+    hcclx.fold_wide(segs, dtype, op, hcclx.FOLD_TREE)
+    sync()
+    for xs, prog, outs, _ in cases:
+        want = tree_oracle(xs, dtype, op, prog, fused_is_wide(dtype, op))
+        for o in outs:
+            assert_same_bits(o.get(T.NP_STORAGE[dtype]), want, dtype, f"program {prog}")
+            assert o.guard_intact()
+
+
+def test_wide_tree_fold_rejects_seven_levels_and_malformed_programs():
+    b = DevBuf(nbytes=64)
+    deep = [x for k in range(1, 8) for x in (0, k)]     # a spine of seven levels
+    with pytest.raises(HcclError) as e:
+        hcclx.fold_wide([(4, [b.ptr] * 8, [b.ptr], deep)], T.FP32, T.SUM, hcclx.FOLD_TREE)
+    assert e.value.code == 5
+    with pytest.raises(HcclError) as e:
+        hcclx.fold_wide([(4, [b.ptr] * 3, [b.ptr], [0, 1, 0, 1])], T.FP32, T.SUM, hcclx.FOLD_TREE)
+    assert e.value.code == 1
+    with pytest.raises(HcclError) as e:
+        hcclx.fold_wide([(4, [b.ptr] * 3, [b.ptr] * 3)], T.FP32, T.SUM, hcclx.FOLD_SELF_FIRST)
+    assert e.value.code == 5
+
+
 def test_tree_fold_in_place_and_chain_shaped_program():
     """The result may overwrite register 0's source; a left-deep program of up to four steps equals the
     chain fold of the same order."""
