@@ -346,6 +346,10 @@ WORKLOADS = {
     "all_reduce_sum_fp32_8x4MiB_ring_step_by_step": lambda *a: AllReduce(*a, count=1048576, alg="InsAllReduceRing",
                                                                          step_mode=True),
     "all_reduce_sum_fp32_8x64MiB_two_shot_step_by_step": lambda *a: AllReduce(*a, step_mode=True),
+    # communicators of more than 16 ranks: the wide chain kernel (two-shot mesh) and the wide tree kernel (NHR)
+    "all_reduce_sum_fp32_32x16MiB": lambda *a: AllReduce(*a, n=32, count=4 * 1024 * 1024),
+    "all_reduce_sum_fp32_32x16MiB_nhr": lambda *a: AllReduce(*a, n=32, count=4 * 1024 * 1024, alg="InsAllReduceNHR"),
+    "reduce_scatter_sum_bf16_mesh_32x32MiB": lambda *a: ReduceScatterMesh(*a, n=32, recv=512 * 1024),
     "moe_dispatch_pack_bf16_8x4096x7168": lambda *a: MoeDispatchPack(*a),
     "moe_combine_bf16_8x4096x7168": lambda *a: MoeDispatchPack(*a, combine=True),
 }
