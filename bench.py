@@ -258,7 +258,7 @@ class MoeDispatchPack(Workload):
     dtype = "u8"
     kernel = "k_moe_rows<true>"
 
-    def __init__(self, torch, api, T, n=8, tokens=4096, hidden=7168, seed=0, combine=False):
+    def __init__(self, torch, api, T, n=8, tokens=4096, hidden=7168, seed=0, combine=False, one_pass=False):
         import numpy as np
         from hccl_amd import hcclx
         self.torch, self.T, self.n, self.hx = torch, T, n, hcclx
@@ -266,7 +266,10 @@ class MoeDispatchPack(Workload):
         self.stream = self.stream_obj.cuda_stream
         self.world = _NoWorld()
         self.combine = combine
+        self.one_pass = one_pass    # route + dispatch straight into the receive buffers / combine straight out of them
         self.name = ("moe_combine_bf16_%dx%dx%d" if combine else "moe_dispatch_pack_bf16_%dx%dx%d") % (n, tokens, hidden)
+        if one_pass:
+            self.name = ("moe_gather_combine_bf16_%dx%dx%d" if combine else "moe_route_dispatch_bf16_%dx%dx%d") % (n, tokens, hidden)
         self.tokens, self.hidden = tokens, hidden
         rng = np.random.default_rng(seed)
         w = 1.0 / np.arange(1, n + 1) ** 1.2
@@ -281,6 +284,15 @@ class MoeDispatchPack(Workload):
         self.p = lambda ts: [t.data_ptr() for t in ts]
         self._route()
         self.hx.moe_pack(self.p(self.tok), self.p(self.perm), tokens, 1, hidden * 2, self.p(self.packed), stream=self.stream)
+        if one_pass:
+            # receive buffers sized for the worst case: every token of every rank
+            self.recv = [torch.empty(n * tokens * hidden, device="cuda:0", dtype=torch.int16) for _ in range(n)]
+            self._dispatch()
+
+    def _dispatch(self):
+        t = self.tabs
+        self.hx.moe_dispatch(self.p(self.tok), self.p(self.dest), self.p(self.perm), self.tokens, 1, self.hidden, self.T.BFP16,
+                             t[1].data_ptr(), t[3].data_ptr(), self.p(self.recv), stream=self.stream)
 
     def _route(self):
         t = self.tabs
@@ -288,7 +300,15 @@ class MoeDispatchPack(Workload):
                           t[3].data_ptr(), self.p(self.perm), self.ws.data_ptr(), stream=self.stream)
 
     def step(self):
-        if self.combine:
+        if self.one_pass:
+            if self.combine:
+                t = self.tabs
+                self.hx.moe_gather_combine(self.p(self.recv), self.p(self.dest), self.p(self.perm), self.tokens, 1, self.hidden,
+                                           self.T.BFP16, t[1].data_ptr(), t[3].data_ptr(), self.p(self.out), stream=self.stream)
+            else:
+                self._route()
+                self._dispatch()
+        elif self.combine:
             self.hx.moe_combine(self.p(self.packed), self.p(self.perm), self.tokens, 1, self.hidden, self.T.BFP16,
                                 self.p(self.out), stream=self.stream)
         else:
@@ -300,8 +320,11 @@ class MoeDispatchPack(Workload):
         return 2 * self.n * self.tokens * self.hidden * 2
 
     def info(self):
-        return {"algorithm": "moe combine (top-1)" if self.combine else "moe route + pack", "fused": True,
-                "launches": 1 if self.combine else 5, "plan_cache_hit": False}
+        if self.one_pass:
+            what = "AlltoAllV back + combine in one pass" if self.combine else "route + pack + AlltoAllV in one pass"
+        else:
+            what = "moe combine (top-1)" if self.combine else "moe route + pack"
+        return {"algorithm": what, "fused": True, "launches": 1 if self.combine else 5, "plan_cache_hit": False}
 
 
 class CopyCalibration(Workload):
@@ -352,6 +375,8 @@ WORKLOADS = {
     "reduce_scatter_sum_bf16_mesh_32x32MiB": lambda *a: ReduceScatterMesh(*a, n=32, recv=512 * 1024),
     "moe_dispatch_pack_bf16_8x4096x7168": lambda *a: MoeDispatchPack(*a),
     "moe_combine_bf16_8x4096x7168": lambda *a: MoeDispatchPack(*a, combine=True),
+    "moe_route_dispatch_bf16_8x4096x7168": lambda *a: MoeDispatchPack(*a, one_pass=True),
+    "moe_gather_combine_bf16_8x4096x7168": lambda *a: MoeDispatchPack(*a, combine=True, one_pass=True),
 }
 EXTRA_WORKLOADS = {"copy_calibration_1024MiB": lambda *a: CopyCalibration(*a)}
 

@@ -8,7 +8,9 @@
 //
 // Bound: HBM bandwidth (pack / combine move rows of several KiB); the routing kernels touch 4 bytes per
 // entry and are latency-bound.  Algorithmic bytes: pack 2 x entries x row bytes; combine (topk + 1) x
-// tokens x row bytes.
+// tokens x row bytes.  hcclx_moe_dispatch and hcclx_moe_gather_combine do pack + AlltoAllV, and AlltoAllV back
+// + combine, in one pass each: the rows go straight to (come straight from) the place the AlltoAllV would
+// have put them, which halves the traffic of either direction.
 #include "hcclx.h"
 #include "hcclx_internal.h"
 #include "kernels/elem.h"
@@ -30,6 +32,11 @@ struct MoeConstPtrs {
 struct MoePtrs {
     void *p[kMoeMaxRanks];
 };
+
+__device__ __forceinline__ const MoePtrs &as_mutable_dev(const MoeConstPtrs &c)
+{
+    return reinterpret_cast<const MoePtrs &>(c);   // same layout; the landing addresses are only read through
+}
 
 // Workspace layout (uint32): base[n][n][chunks] (chunk fastest) -- first the per-chunk histogram, then,
 // in place, its exclusive prefix over the chunks -- followed by row_start[n][n].
@@ -215,6 +222,194 @@ k_moe_combine(MoeConstPtrs packed, MoeConstPtrs perm, MoePtrs out, uint32_t toke
     st16(o + (static_cast<uint64_t>(t) * vpr + v) * 16, V::pack(acc));
 }
 
+// Where rank i's rows for destination j land: packed row p of rank i sits at landing(...) + p rows, i.e. at the
+// first row of the block from i in recv[j] minus the first row of the group for j in i's packed order.  The
+// tables are a few hundred bytes and stay in the caches.
+__device__ __forceinline__ char *landing(const MoePtrs &recv, uint32_t i, uint32_t j, uint32_t n, uint32_t esz,
+                                         const uint64_t *sdispls, const uint64_t *rdispls)
+{
+    const int64_t elems = static_cast<int64_t>(rdispls[j * n + i]) - static_cast<int64_t>(sdispls[i * n + j]);
+    return static_cast<char *>(recv.p[j]) + elems * static_cast<int64_t>(esz);
+}
+
+// Dispatch in one pass (what the pack kernel followed by the AlltoAllV kernel does in two):
+// recv[dest[e]] row (landing + perm[e]) = tokens[e / topk].
+__global__ void __launch_bounds__(256)
+k_moe_dispatch(MoeConstPtrs tokens, MoeConstPtrs dest, MoeConstPtrs perm, MoePtrs recv, uint32_t n, uint32_t entries,
+               uint32_t topk, uint32_t vpr, uint32_t esz, const uint64_t *sdispls, const uint64_t *rdispls)
+{
+    const uint32_t i = blockIdx.y;
+    const uint64_t total = static_cast<uint64_t>(entries) * vpr;
+    const uint32_t *pm = static_cast<const uint32_t *>(perm.p[i]);
+    const int32_t *dt = static_cast<const int32_t *>(dest.p[i]);
+    const char *s = static_cast<const char *>(tokens.p[i]);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const uint64_t g = static_cast<uint64_t>(blockIdx.x) * 512 + u * 256 + threadIdx.x;
+        if (g >= total) continue;
+        const uint32_t e = static_cast<uint32_t>(g / vpr);
+        const uint32_t v = static_cast<uint32_t>(g - static_cast<uint64_t>(e) * vpr);
+        const uint32_t p = pm[e];
+        const uint32_t j = static_cast<uint32_t>(dt[e]);
+        if (p == kDropped || j >= n) continue;   // perm marks entries with a destination outside 0 .. n-1 as dropped
+        char *o = landing(recv, i, j, n, esz, sdispls, rdispls);
+        st16(o + (static_cast<uint64_t>(p) * vpr + v) * 16, ld16(s + (static_cast<uint64_t>(e / topk) * vpr + v) * 16));
+    }
+}
+
+// The way back in one pass (what the AlltoAllV kernel followed by the combine kernel does in two):
+// out[t] = sum over j < topk of the row of entry t * topk + j where dispatch put it, in the buffers `expert`.
+// DT = int8 moves bytes (topk == 1: nothing is added).
+template <int DT>
+__global__ void __launch_bounds__(256)
+k_moe_gather_combine(MoeConstPtrs expert, MoeConstPtrs dest, MoeConstPtrs perm, MoePtrs out, uint32_t n, uint32_t tokens,
+                     uint32_t topk, uint32_t vpr, uint32_t esz, const uint64_t *sdispls, const uint64_t *rdispls)
+{
+    using V = Vec16<DT>;
+    using C = typename V::C;
+    constexpr int NE = V::NE;
+    const uint32_t i = blockIdx.y;
+    const uint64_t total = static_cast<uint64_t>(tokens) * vpr;
+    const uint32_t *pm = static_cast<const uint32_t *>(perm.p[i]);
+    const int32_t *dt = static_cast<const int32_t *>(dest.p[i]);
+    char *o = static_cast<char *>(out.p[i]);
+    const uint64_t g = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (g >= total) return;
+    const uint32_t t = static_cast<uint32_t>(g / vpr);
+    const uint32_t v = static_cast<uint32_t>(g - static_cast<uint64_t>(t) * vpr);
+    C acc[NE];
+    bool have = false;
+#pragma unroll
+    for (int e = 0; e < NE; ++e) acc[e] = C(0);
+    for (uint32_t j = 0; j < topk; ++j) {
+        const uint64_t e = static_cast<uint64_t>(t) * topk + j;
+        const uint32_t p = pm[e];
+        const uint32_t d = static_cast<uint32_t>(dt[e]);
+        if (p == kDropped || d >= n) continue;
+        const char *from = landing(as_mutable_dev(expert), i, d, n, esz, sdispls, rdispls);
+        C x[NE];
+        V::unpack(ld16(from + (static_cast<uint64_t>(p) * vpr + v) * 16), x);
+        if (!have) {
+#pragma unroll
+            for (int k = 0; k < NE; ++k) acc[k] = x[k];
+            have = true;
+        } else {
+#pragma unroll
+            for (int k = 0; k < NE; ++k) acc[k] = V::template combine<HCCL_REDUCE_SUM>(x[k], acc[k]);
+        }
+    }
+    st16(o + (static_cast<uint64_t>(t) * vpr + v) * 16, V::pack(acc));
+}
+
+// ---- rows of at least kLongRow vectors ----------------------------------------------------------------------
+// A workgroup moves one run of ONE row, so the entry, its destination and where it lands are the same for every
+// thread: they are fetched with scalar loads, and no thread divides or looks anything up.
+constexpr uint32_t kLongRow = 128;
+
+struct RowRuns {
+    uint32_t per_row;   // runs a row is cut into
+    uint32_t vecs;      // vectors per run (the last one may be shorter)
+};
+inline RowRuns row_runs(uint32_t vpr, uint32_t most)
+{
+    RowRuns r;
+    r.per_row = (vpr + most - 1) / most;
+    r.vecs = (vpr + r.per_row - 1) / r.per_row;
+    return r;
+}
+
+// Scatter one row per entry straight to where the AlltoAllV would put it in recv[dest[e]].  Runs of up to 512
+// vectors, two per thread.
+__global__ void __launch_bounds__(256)
+k_moe_scatter_long(MoeConstPtrs tokens, MoeConstPtrs dest, MoeConstPtrs perm, MoePtrs dst, uint32_t n, uint32_t topk, uint32_t vpr,
+                   RowRuns runs, uint32_t esz, const uint64_t *sdispls, const uint64_t *rdispls)
+{
+    const uint32_t i = blockIdx.y;
+    const uint32_t e = blockIdx.x / runs.per_row;
+    const uint32_t c = blockIdx.x - e * runs.per_row;
+    const uint32_t p = static_cast<const uint32_t *>(perm.p[i])[e];
+    if (p == kDropped) return;
+    const uint32_t j = static_cast<uint32_t>(static_cast<const int32_t *>(dest.p[i])[e]);
+    if (j >= n) return;
+    char *base = landing(dst, i, j, n, esz, sdispls, rdispls);
+    const char *from = static_cast<const char *>(tokens.p[i]) + static_cast<uint64_t>(e / topk) * vpr * 16;
+    char *to = base + static_cast<uint64_t>(p) * vpr * 16;
+    const uint32_t lo = c * runs.vecs;
+    const uint32_t hi = lo + runs.vecs < vpr ? lo + runs.vecs : vpr;
+    const uint32_t v0 = lo + threadIdx.x;
+    const uint32_t v1 = v0 + 256;
+    u32x4 x0, x1;
+    if (v0 < hi) x0 = ld16(from + static_cast<uint64_t>(v0) * 16);
+    if (v1 < hi) x1 = ld16(from + static_cast<uint64_t>(v1) * 16);
+    if (v0 < hi) st16(to + static_cast<uint64_t>(v0) * 16, x0);
+    if (v1 < hi) st16(to + static_cast<uint64_t>(v1) * 16, x1);
+}
+
+// Gather the rows of a token's entries from where dispatch put them in expert[dest[.]] and add them.  Runs of up
+// to 256 vectors, one per thread.  DT = int8 moves bytes (topk == 1).
+template <int DT>
+__global__ void __launch_bounds__(256)
+k_moe_gather_long(MoeConstPtrs rows, MoeConstPtrs dest, MoeConstPtrs perm, MoePtrs out, uint32_t n, uint32_t topk, uint32_t vpr,
+                  RowRuns runs, uint32_t esz, const uint64_t *sdispls, const uint64_t *rdispls)
+{
+    using V = Vec16<DT>;
+    using C = typename V::C;
+    constexpr int NE = V::NE;
+    const uint32_t i = blockIdx.y;
+    const uint32_t t = blockIdx.x / runs.per_row;
+    const uint32_t c = blockIdx.x - t * runs.per_row;
+    const uint32_t lo = c * runs.vecs;
+    const uint32_t hi = lo + runs.vecs < vpr ? lo + runs.vecs : vpr;
+    const uint32_t v = lo + threadIdx.x;
+    const uint32_t *pm = static_cast<const uint32_t *>(perm.p[i]);
+    const int32_t *dt = static_cast<const int32_t *>(dest.p[i]);
+    C acc[NE];
+    bool have = false;
+#pragma unroll
+    for (int k = 0; k < NE; ++k) acc[k] = C(0);
+    for (uint32_t j = 0; j < topk; ++j) {
+        const uint64_t e = static_cast<uint64_t>(t) * topk + j;
+        const uint32_t p = pm[e];
+        if (p == kDropped) continue;
+        const uint32_t d = static_cast<uint32_t>(dt[e]);
+        if (d >= n) continue;
+        const char *base = landing(as_mutable_dev(rows), i, d, n, esz, sdispls, rdispls);
+        if (v < hi) {
+            C x[NE];
+            V::unpack(ld16(base + (static_cast<uint64_t>(p) * vpr + v) * 16), x);
+            if (!have) {
+#pragma unroll
+                for (int k = 0; k < NE; ++k) acc[k] = x[k];
+            } else {
+#pragma unroll
+                for (int k = 0; k < NE; ++k) acc[k] = V::template combine<HCCL_REDUCE_SUM>(x[k], acc[k]);
+            }
+        }
+        have = true;
+    }
+    if (v < hi) st16(static_cast<char *>(out.p[i]) + (static_cast<uint64_t>(t) * vpr + v) * 16, V::pack(acc));
+}
+
+hipError_t launch_gather_long(int kind, dim3 grid, hipStream_t st, const MoeConstPtrs &rows, const MoeConstPtrs &dest,
+                              const MoeConstPtrs &perm, const MoePtrs &out, uint32_t n, uint32_t topk, uint32_t vpr, RowRuns runs,
+                              uint32_t esz, const uint64_t *sdispls, const uint64_t *rdispls)
+{
+    if (kind == HCCL_DATA_TYPE_FP32) {
+        hipLaunchKernelGGL(k_moe_gather_long<HCCL_DATA_TYPE_FP32>, grid, dim3(256), 0, st, rows, dest, perm, out, n, topk,
+                           vpr, runs, esz, sdispls, rdispls);
+    } else if (kind == HCCL_DATA_TYPE_FP16) {
+        hipLaunchKernelGGL(k_moe_gather_long<HCCL_DATA_TYPE_FP16>, grid, dim3(256), 0, st, rows, dest, perm, out, n, topk,
+                           vpr, runs, esz, sdispls, rdispls);
+    } else if (kind == HCCL_DATA_TYPE_BFP16) {
+        hipLaunchKernelGGL(k_moe_gather_long<HCCL_DATA_TYPE_BFP16>, grid, dim3(256), 0, st, rows, dest, perm, out, n, topk,
+                           vpr, runs, esz, sdispls, rdispls);
+    } else {
+        hipLaunchKernelGGL(k_moe_gather_long<HCCL_DATA_TYPE_INT8>, grid, dim3(256), 0, st, rows, dest, perm, out, n, topk,
+                           vpr, runs, esz, sdispls, rdispls);
+    }
+    return hipGetLastError();
+}
+
 int check_ranks(uint32_t n)
 {
     if (n == 0 || n > kMoeMaxRanks) return fail(HCCL_E_PARA, "rank count outside 1.." + std::to_string(kMoeMaxRanks));
@@ -350,6 +545,109 @@ int hcclx_moe_combine(const void *const *packed, const uint32_t *const *perm, ui
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail_hip(e, "moe combine kernel");
+    return HCCL_SUCCESS;
+}
+
+int hcclx_moe_dispatch(const void *const *tokens, const int32_t *const *dest, const uint32_t *const *perm, uint32_t n,
+                       uint32_t entries, uint32_t topk, uint64_t row_elems, int dtype, const uint64_t *sdispls,
+                       const uint64_t *rdispls, void *const *recv, void *stream)
+{
+    if (!device_ctx()) return HCCL_E_RUNTIME;
+    int rc = check_ranks(n);
+    if (rc != HCCL_SUCCESS) return rc;
+    const int esz = dtype_size(dtype);
+    if (esz == 0) return fail(HCCL_E_NOT_SUPPORT, "unknown data type " + std::to_string(dtype));
+    if (topk == 0 || entries == 0 || entries % topk != 0) return fail(HCCL_E_PARA, "entries must be a positive multiple of topk");
+    const uint64_t row_bytes = row_elems * esz;
+    if (row_bytes == 0 || row_bytes % 16 != 0) return fail(HCCL_E_PARA, "row size must be a positive multiple of 16 bytes");
+    if (row_bytes / 16 > 0xffffffffull) return fail(HCCL_E_PARA, "row too long");
+    if (!sdispls || !rdispls) return fail(HCCL_E_PTR, "displacement table is null");
+    MoeConstPtrs s, d, p, o;
+    rc = fill(tokens, n, &s, "tokens", true);
+    if (rc != HCCL_SUCCESS) return rc;
+    rc = fill(reinterpret_cast<const void *const *>(dest), n, &d, "dest", false);
+    if (rc != HCCL_SUCCESS) return rc;
+    rc = fill(reinterpret_cast<const void *const *>(perm), n, &p, "perm", false);
+    if (rc != HCCL_SUCCESS) return rc;
+    rc = fill(recv, n, &o, "recv", true);
+    if (rc != HCCL_SUCCESS) return rc;
+    const uint32_t vpr = static_cast<uint32_t>(row_bytes / 16);
+    if (vpr >= kLongRow) {
+        const RowRuns runs = row_runs(vpr, 512);
+        const uint64_t long_blocks = static_cast<uint64_t>(entries) * runs.per_row;
+        if (long_blocks > 0x7fffffffull) return fail(HCCL_E_PARA, "too much data for one launch");
+        hipLaunchKernelGGL(k_moe_scatter_long, dim3(static_cast<uint32_t>(long_blocks), n), dim3(256), 0,
+                           static_cast<hipStream_t>(stream), s, d, p, as_mutable(o), n, topk, vpr, runs, static_cast<uint32_t>(esz),
+                           sdispls, rdispls);
+        hipError_t le = hipGetLastError();
+        if (le != hipSuccess) return fail_hip(le, "moe dispatch kernel");
+        return HCCL_SUCCESS;
+    }
+    const uint64_t blocks = (static_cast<uint64_t>(entries) * vpr + 511) / 512;
+    if (blocks > 0x7fffffffull) return fail(HCCL_E_PARA, "too much data for one launch");
+    hipLaunchKernelGGL(k_moe_dispatch, dim3(static_cast<uint32_t>(blocks), n), dim3(256), 0, static_cast<hipStream_t>(stream), s, d,
+                       p, as_mutable(o), n, entries, topk, vpr, static_cast<uint32_t>(esz), sdispls, rdispls);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail_hip(e, "moe dispatch kernel");
+    return HCCL_SUCCESS;
+}
+
+int hcclx_moe_gather_combine(const void *const *expert, const int32_t *const *dest, const uint32_t *const *perm, uint32_t n,
+                             uint32_t tokens, uint32_t topk, uint64_t row_elems, int dtype, const uint64_t *sdispls,
+                             const uint64_t *rdispls, void *const *out, void *stream)
+{
+    if (!device_ctx()) return HCCL_E_RUNTIME;
+    int rc = check_ranks(n);
+    if (rc != HCCL_SUCCESS) return rc;
+    const int esz = dtype_size(dtype);
+    if (esz == 0) return fail(HCCL_E_NOT_SUPPORT, "unknown data type " + std::to_string(dtype));
+    if (topk == 0 || tokens == 0) return fail(HCCL_E_PARA, "tokens and topk must be positive");
+    const uint64_t row_bytes = row_elems * esz;
+    if (row_bytes == 0 || row_bytes % 16 != 0) return fail(HCCL_E_PARA, "row size must be a positive multiple of 16 bytes");
+    if (row_bytes / 16 > 0xffffffffull) return fail(HCCL_E_PARA, "row too long");
+    if (topk > 1 && dtype != HCCL_DATA_TYPE_FP32 && dtype != HCCL_DATA_TYPE_FP16 && dtype != HCCL_DATA_TYPE_BFP16) {
+        return fail(HCCL_E_NOT_SUPPORT, "combining several rows needs fp32, fp16 or bf16");
+    }
+    if (!sdispls || !rdispls) return fail(HCCL_E_PTR, "displacement table is null");
+    MoeConstPtrs s, d, p, o;
+    rc = fill(expert, n, &s, "expert", true);
+    if (rc != HCCL_SUCCESS) return rc;
+    rc = fill(reinterpret_cast<const void *const *>(dest), n, &d, "dest", false);
+    if (rc != HCCL_SUCCESS) return rc;
+    rc = fill(reinterpret_cast<const void *const *>(perm), n, &p, "perm", false);
+    if (rc != HCCL_SUCCESS) return rc;
+    rc = fill(out, n, &o, "out", true);
+    if (rc != HCCL_SUCCESS) return rc;
+    const uint32_t vpr = static_cast<uint32_t>(row_bytes / 16);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int kind = topk == 1 ? HCCL_DATA_TYPE_INT8 : dtype;
+    if (vpr >= kLongRow) {
+        const RowRuns runs = row_runs(vpr, 256);
+        const uint64_t long_blocks = static_cast<uint64_t>(tokens) * runs.per_row;
+        if (long_blocks > 0x7fffffffull) return fail(HCCL_E_PARA, "too much data for one launch");
+        const hipError_t le = launch_gather_long(kind, dim3(static_cast<uint32_t>(long_blocks), n), st, s, d, p, as_mutable(o), n,
+                                                       topk, vpr, runs, static_cast<uint32_t>(esz), sdispls, rdispls);
+        if (le != hipSuccess) return fail_hip(le, "moe gather-combine kernel");
+        return HCCL_SUCCESS;
+    }
+    const uint64_t blocks = (static_cast<uint64_t>(tokens) * vpr + 255) / 256;
+    if (blocks > 0x7fffffffull) return fail(HCCL_E_PARA, "too much data for one launch");
+    const dim3 grid(static_cast<uint32_t>(blocks), n);
+    if (kind == HCCL_DATA_TYPE_FP32) {
+        hipLaunchKernelGGL(k_moe_gather_combine<HCCL_DATA_TYPE_FP32>, grid, dim3(256), 0, st, s, d, p, as_mutable(o), n, tokens, topk,
+                           vpr, static_cast<uint32_t>(esz), sdispls, rdispls);
+    } else if (kind == HCCL_DATA_TYPE_FP16) {
+        hipLaunchKernelGGL(k_moe_gather_combine<HCCL_DATA_TYPE_FP16>, grid, dim3(256), 0, st, s, d, p, as_mutable(o), n, tokens, topk,
+                           vpr, static_cast<uint32_t>(esz), sdispls, rdispls);
+    } else if (kind == HCCL_DATA_TYPE_BFP16) {
+        hipLaunchKernelGGL(k_moe_gather_combine<HCCL_DATA_TYPE_BFP16>, grid, dim3(256), 0, st, s, d, p, as_mutable(o), n, tokens, topk,
+                           vpr, static_cast<uint32_t>(esz), sdispls, rdispls);
+    } else {
+        hipLaunchKernelGGL(k_moe_gather_combine<HCCL_DATA_TYPE_INT8>, grid, dim3(256), 0, st, s, d, p, as_mutable(o), n, tokens, topk,
+                           vpr, static_cast<uint32_t>(esz), sdispls, rdispls);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail_hip(e, "moe gather-combine kernel");
     return HCCL_SUCCESS;
 }
 

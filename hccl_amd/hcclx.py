@@ -142,3 +142,17 @@ def moe_pack(tokens, perm, entries, topk, row_bytes, packed, stream=0):
 def moe_combine(packed, perm, tokens, topk, row_elems, dtype, out, stream=0):
     check(_lib.load().hcclx_moe_combine(_ptr_array(packed), _ptr_array(perm), len(packed), tokens, topk, row_elems,
                                         int(dtype), _ptr_array(out), ctypes.c_void_p(stream)))
+
+
+def moe_dispatch(tokens, dest, perm, entries, topk, row_elems, dtype, sdispls, rdispls, recv, stream=0):
+    """Pack + AlltoAllV in one pass; sdispls / rdispls are the device tables moe_route wrote."""
+    check(_lib.load().hcclx_moe_dispatch(_ptr_array(tokens), _ptr_array(dest), _ptr_array(perm), len(tokens), entries, topk,
+                                         row_elems, int(dtype), ctypes.c_void_p(sdispls), ctypes.c_void_p(rdispls),
+                                         _ptr_array(recv), ctypes.c_void_p(stream)))
+
+
+def moe_gather_combine(expert, dest, perm, tokens, topk, row_elems, dtype, sdispls, rdispls, out, stream=0):
+    """AlltoAllV back + combine in one pass, reading the rows where moe_dispatch put them."""
+    check(_lib.load().hcclx_moe_gather_combine(_ptr_array(expert), _ptr_array(dest), _ptr_array(perm), len(expert), tokens,
+                                               topk, row_elems, int(dtype), ctypes.c_void_p(sdispls),
+                                               ctypes.c_void_p(rdispls), _ptr_array(out), ctypes.c_void_p(stream)))

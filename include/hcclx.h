@@ -158,6 +158,23 @@ int hcclx_moe_pack(const void *const *tokens, const uint32_t *const *perm, uint3
 int hcclx_moe_combine(const void *const *packed, const uint32_t *const *perm, uint32_t n, uint32_t tokens, uint32_t topk,
                       uint64_t row_elems, int dtype, void *const *out, void *stream);
 
+/* hcclx_moe_pack followed by hcclx_alltoallv(packed, recv, send_counts, sdispls, rdispls), in one pass and without
+ * the packed buffers: the row of entry e of rank i goes to
+ *   recv[j] + (rdispls[j*n + i] + perm[i][e] * row_elems - sdispls[i*n + j]) elements,  j = dest[i][e].
+ * sdispls / rdispls: the device tables hcclx_moe_route wrote.  Rows of row_elems elements of `dtype` (a multiple
+ * of 16 bytes; buffers 16-byte aligned). */
+int hcclx_moe_dispatch(const void *const *tokens, const int32_t *const *dest, const uint32_t *const *perm, uint32_t n,
+                       uint32_t entries, uint32_t topk, uint64_t row_elems, int dtype, const uint64_t *sdispls,
+                       const uint64_t *rdispls, void *const *recv, void *stream);
+
+/* The way back: hcclx_alltoallv(expert, back, recv_counts, rdispls, sdispls) followed by hcclx_moe_combine, in one
+ * pass and without the `back` buffers.  expert[j] holds one row per row of recv[j], in the same places;
+ * out[i][t] = sum over k < topk of the row of entry t*topk + k (k ascending, dropped entries skipped, all dropped:
+ * zeros).  Types as for hcclx_moe_combine. */
+int hcclx_moe_gather_combine(const void *const *expert, const int32_t *const *dest, const uint32_t *const *perm, uint32_t n,
+                             uint32_t tokens, uint32_t topk, uint64_t row_elems, int dtype, const uint64_t *sdispls,
+                             const uint64_t *rdispls, void *const *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
