@@ -78,7 +78,7 @@ class ReduceScatterMesh(Workload):
     r's own data, then ranks ascending (ins_temp_reduce_scatter_mesh_1D.cc:132-154), as one fused pass."""
     dtype = "bf16"
     kernel = "hcclx::k_fold<11, 0, 8, 0>"
-    traffic = 604081556
+    traffic = 604053285
     profile = "profiles/k_fold_reduce_scatter_bf16_8x64MiB.txt"
 
     def __init__(self, torch, api, T, n=8, recv=4 * 1024 * 1024):
@@ -121,7 +121,7 @@ class AllReduce(Workload):
     ranks, so each input is read once and the result is written to the eight outputs."""
     dtype = "f32"
     kernel = "hcclx::k_fold<4, 0, 8, 0>"
-    traffic = 1073843968
+    traffic = 1073639248
     profile = "profiles/k_fold_all_reduce_fp32_8x64MiB.txt"
 
     def __init__(self, torch, api, T, n=8, count=16 * 1024 * 1024, alg=None, step_mode=False):
@@ -156,7 +156,7 @@ class AllGather(Workload):
     output; each source byte is read once and written eight times."""
     dtype = "u8"
     kernel = "hcclx::(anonymous namespace)::k_allgatherv"
-    traffic = 4836742261
+    traffic = 4835368852
     profile = "profiles/k_allgatherv_fp16_8x64MiB.txt"
 
     def __init__(self, torch, api, T, n=8, count=32 * 1024 * 1024):
@@ -213,7 +213,7 @@ class AllToAllV(Workload):
     destination rank per token Zipf(s=1.2), tokens grouped by destination."""
     dtype = "u8"
     kernel = "hcclx::(anonymous namespace)::k_alltoallv_direct<2>"
-    traffic = 939581820
+    traffic = 939416174
     profile = "profiles/k_alltoallv_bf16_moe_8x4096x7168.txt"
 
     def __init__(self, torch, api, T, n=8, tokens=4096, hidden=7168, seed=0):
