@@ -5,6 +5,7 @@
 #include "kernels/vops.h"
 
 #include <cstring>
+#include <vector>
 
 using namespace hcclx;
 
@@ -60,79 +61,81 @@ int hcclx_alltoallv(const void *const *send, void *const *recv, const uint64_t *
     int rc = fill_ptrs(send, recv, n, &ptrs);
     if (rc != HCCL_SUCCESS) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    uint64_t grid = static_cast<uint64_t>(ctx->num_cus) * ctx->v_blocks_per_cu;
-    bool inline_ok = !tables_on_device && n <= kA2avInlineRanks;
     if (!tables_on_device) {
-        // host tables: the tile count is known here, so launch exactly one workgroup per tile
-        uint64_t total = 0;
-        for (uint32_t i = 0; i < n; ++i) {
-            for (uint32_t j = 0; j < n; ++j) {
-                const uint64_t dst = reinterpret_cast<uint64_t>(ptrs.recv[j]) + rdispls[j * n + i] * esz;
-                total += v_tiles_of(send_counts[i * n + j] * esz, dst, kA2avUnroll);
+        const int unroll = ctx->a2av_direct_unroll == 1 ? 1 : ctx->a2av_direct_unroll == 4 ? 4 : 2;
+        bool small = n <= kA2avDirectRanks && ctx->a2av_direct_unroll != 0;
+        for (size_t k = 0; k < static_cast<size_t>(n) * n && small; ++k) {
+            small = send_counts[k] <= 0xffffffffull && sdispls[k] <= 0xffffffffull && rdispls[k] <= 0xffffffffull;
+        }
+        if (small) {
+            // small host tables and their tile prefix ride in the kernel arguments: one small tile per workgroup,
+            // nothing is copied in front of the kernel
+            VRankPtrs16 p16;
+            A2avTablesDirect tabs;
+            std::memset(&p16, 0, sizeof(p16));
+            std::memset(&tabs, 0, sizeof(tabs));
+            for (uint32_t i = 0; i < n; ++i) {
+                p16.send[i] = ptrs.send[i];
+                p16.recv[i] = ptrs.recv[i];
+            }
+            uint64_t tiles = 0;
+            for (uint32_t i = 0; i < n; ++i) {
+                for (uint32_t j = 0; j < n; ++j) {
+                    const uint32_t k = i * n + j;
+                    const uint64_t dst = reinterpret_cast<uint64_t>(ptrs.recv[j]) + rdispls[j * n + i] * esz;
+                    tiles += v_tiles_of(send_counts[k] * esz, dst, unroll);
+                    tabs.send_counts[k] = static_cast<uint32_t>(send_counts[k]);
+                    tabs.sdispls[k] = static_cast<uint32_t>(sdispls[k]);
+                    tabs.rdispls[k] = static_cast<uint32_t>(rdispls[j * n + i]);
+                    tabs.tile_end[k] = static_cast<uint32_t>(tiles);
+                }
+            }
+            if (tiles == 0) return HCCL_SUCCESS;
+            if (tiles <= 0x7fffffffull) {
+                hipError_t e = launch_alltoallv_direct(p16, tabs, n, static_cast<uint32_t>(esz), static_cast<uint32_t>(tiles),
+                                                       unroll, st);
+                if (e != hipSuccess) return fail_hip(e, "alltoallv kernel launch");
+                return HCCL_SUCCESS;
             }
         }
-        if (total == 0) return HCCL_SUCCESS;
-        grid = (total + ctx->v_tiles_per_block - 1) / ctx->v_tiles_per_block;
-        if (grid > 0x7fffffffull) grid = 0x7fffffffull;
-        for (size_t k = 0; k < static_cast<size_t>(n) * n && inline_ok; ++k) {
-            inline_ok = send_counts[k] <= 0xffffffffull && sdispls[k] <= 0xffffffffull && rdispls[k] <= 0xffffffffull;
-        }
-    }
-    if (inline_ok && n <= kA2avDirectRanks && ctx->a2av_direct_unroll != 0) {
-        // small host tables and their tile prefix ride in the kernel arguments: one small tile per workgroup
-        const int unroll = ctx->a2av_direct_unroll == 1 ? 1 : ctx->a2av_direct_unroll == 2 ? 2 : 4;
-        VRankPtrs16 p16;
-        A2avTablesDirect tabs;
-        std::memset(&p16, 0, sizeof(p16));
-        std::memset(&tabs, 0, sizeof(tabs));
-        for (uint32_t i = 0; i < n; ++i) {
-            p16.send[i] = ptrs.send[i];
-            p16.recv[i] = ptrs.recv[i];
-        }
+        // any other host table: the non-empty blocks as a list in device memory, one small tile per workgroup
+        std::vector<CopyBlock> blocks;
+        blocks.reserve(static_cast<size_t>(n) * n);
         uint64_t tiles = 0;
         for (uint32_t i = 0; i < n; ++i) {
             for (uint32_t j = 0; j < n; ++j) {
-                const uint32_t k = i * n + j;
-                const uint64_t dst = reinterpret_cast<uint64_t>(ptrs.recv[j]) + rdispls[j * n + i] * esz;
-                tiles += v_tiles_of(send_counts[k] * esz, dst, unroll);
-                tabs.send_counts[k] = static_cast<uint32_t>(send_counts[k]);
-                tabs.sdispls[k] = static_cast<uint32_t>(sdispls[k]);
-                tabs.rdispls[k] = static_cast<uint32_t>(rdispls[j * n + i]);
-                tabs.tile_end[k] = static_cast<uint32_t>(tiles);
+                const uint64_t bytes = send_counts[i * n + j] * esz;
+                if (bytes == 0) continue;
+                CopyBlock b;
+                b.src = ptrs.send[i] + sdispls[i * n + j] * esz;
+                b.dst = ptrs.recv[j] + rdispls[j * n + i] * esz;
+                b.bytes = bytes;
+                tiles += v_tiles_of(bytes, reinterpret_cast<uint64_t>(b.dst), unroll);
+                b.tile_end = tiles;
+                blocks.push_back(b);
             }
         }
-        if (tiles <= 0x7fffffffull) {
-            hipError_t e = launch_alltoallv_direct(p16, tabs, n, static_cast<uint32_t>(esz), static_cast<uint32_t>(tiles),
-                                                   unroll, st);
-            if (e != hipSuccess) return fail_hip(e, "alltoallv kernel launch");
-            return HCCL_SUCCESS;
-        }
-    }
-    if (inline_ok) {
-        // small host tables ride in the kernel arguments: nothing is copied in front of the kernel
-        VRankPtrs16 p16;
-        A2avTablesInline tabs;
-        std::memset(&p16, 0, sizeof(p16));
-        for (uint32_t i = 0; i < n; ++i) {
-            p16.send[i] = ptrs.send[i];
-            p16.recv[i] = ptrs.recv[i];
-        }
-        for (size_t k = 0; k < static_cast<size_t>(n) * n; ++k) {
-            tabs.send_counts[k] = static_cast<uint32_t>(send_counts[k]);
-            tabs.sdispls[k] = static_cast<uint32_t>(sdispls[k]);
-            tabs.rdispls[k] = static_cast<uint32_t>(rdispls[k]);
-        }
-        hipError_t e = launch_alltoallv_inline(p16, tabs, n, static_cast<uint32_t>(esz), static_cast<uint32_t>(grid),
-                                               ctx->v_tiles_per_block, st);
+        if (blocks.empty()) return HCCL_SUCCESS;
+        if (tiles > 0x7fffffffull) return fail(HCCL_E_PARA, "too much data for one launch");
+        char *h = nullptr;
+        char *d = nullptr;
+        rc = ring_reserve(ctx, blocks.size() * sizeof(CopyBlock), st, &h, &d);
+        if (rc != HCCL_SUCCESS) return rc;
+        std::memcpy(h, blocks.data(), blocks.size() * sizeof(CopyBlock));
+        HCCLX_HIP(hipMemcpyAsync(d, h, blocks.size() * sizeof(CopyBlock), hipMemcpyHostToDevice, st));
+        hipError_t e = launch_copy_blocks(reinterpret_cast<const CopyBlock *>(d), static_cast<uint32_t>(blocks.size()),
+                                          static_cast<uint32_t>(tiles), unroll, st);
         if (e != hipSuccess) return fail_hip(e, "alltoallv kernel launch");
         return HCCL_SUCCESS;
     }
+    // tables on the device: the tile count is not known here, so a persistent grid derives its own tile map
+    const uint64_t grid = static_cast<uint64_t>(ctx->num_cus) * ctx->v_blocks_per_cu;
     const uint64_t *tabs[3] = {send_counts, sdispls, rdispls};
     const uint64_t *dev[3];
     rc = stage_tables(ctx, tabs, 3, static_cast<size_t>(n) * n, tables_on_device, st, dev);
     if (rc != HCCL_SUCCESS) return rc;
     hipError_t e = launch_alltoallv(ptrs, dev[0], dev[1], dev[2], n, static_cast<uint32_t>(esz),
-                                    static_cast<uint32_t>(grid), tables_on_device ? 1u : ctx->v_tiles_per_block, st);
+                                    static_cast<uint32_t>(grid), 1u, st);
     if (e != hipSuccess) return fail_hip(e, "alltoallv kernel launch");
     return HCCL_SUCCESS;
 }

@@ -49,22 +49,13 @@ struct VRankPtrs {
     char *recv[kMaxVRanks];
 };
 
-// Count / displacement tables as the kernels read them.  Tables that arrive as host arrays and are small
-// enough travel inside the kernel arguments (no host-to-device copy is queued in front of the kernel);
-// larger ones, and tables that already live on the device, are read through pointers.
+// Count / displacement tables as the kernels read them.  Host tables of up to 15 ranks travel inside the kernel
+// arguments (no host-to-device copy is queued in front of the kernel); larger host tables become a list of
+// blocks in device memory; tables that already live on the device are read through pointers.
 struct A2avTablesPtr {
     const uint64_t *send_counts;
     const uint64_t *sdispls;
     const uint64_t *rdispls;
-    __device__ uint64_t count(uint32_t p) const { return send_counts[p]; }
-    __device__ uint64_t sdispl(uint32_t p) const { return sdispls[p]; }
-    __device__ uint64_t rdispl(uint32_t p) const { return rdispls[p]; }
-};
-constexpr uint32_t kA2avInlineRanks = 16;  // 16 x 16 x 3 tables of uint32 = 3 KiB of kernel arguments
-struct A2avTablesInline {
-    uint32_t send_counts[kA2avInlineRanks * kA2avInlineRanks];
-    uint32_t sdispls[kA2avInlineRanks * kA2avInlineRanks];
-    uint32_t rdispls[kA2avInlineRanks * kA2avInlineRanks];
     __device__ uint64_t count(uint32_t p) const { return send_counts[p]; }
     __device__ uint64_t sdispl(uint32_t p) const { return sdispls[p]; }
     __device__ uint64_t rdispl(uint32_t p) const { return rdispls[p]; }
@@ -79,10 +70,18 @@ struct A2avTablesDirect {
     uint32_t rdispls[kA2avDirectRanks * kA2avDirectRanks];   // indexed like send_counts: block (i, j) at i * n + j
     uint32_t tile_end[kA2avDirectRanks * kA2avDirectRanks];  // inclusive prefix of tiles per block
 };
-// Base pointers for up to kA2avInlineRanks ranks, for the inline-table launch.
+// Base pointers for the launch with tables in the kernel arguments.
 struct VRankPtrs16 {
-    const char *send[kA2avInlineRanks];
-    char *recv[kA2avInlineRanks];
+    const char *send[16];
+    char *recv[16];
+};
+// One contiguous block to move, for host tables of any size: the host lists the non-empty blocks with the
+// inclusive prefix of their tiles; a workgroup finds its block with a binary search over that list (scalar loads).
+struct CopyBlock {
+    const char *src;
+    char *dst;
+    uint64_t bytes;
+    uint64_t tile_end;
 };
 struct AgvTablesPtr {
     const uint64_t *counts;
@@ -97,8 +96,8 @@ struct AgvTablesInline {
     __device__ uint64_t displ(uint32_t i) const { return displs[i]; }
 };
 
-hipError_t launch_alltoallv_inline(const VRankPtrs16 &ptrs, const A2avTablesInline &tabs, uint32_t n, uint32_t esz,
-                                   uint32_t grid, uint32_t tiles_per_block, hipStream_t stream);
+// blocks: device array of nblocks entries; unroll: 1, 2 or 4; grid = total number of tiles
+hipError_t launch_copy_blocks(const CopyBlock *blocks, uint32_t nblocks, uint32_t grid, int unroll, hipStream_t stream);
 // unroll: 1, 2 or 4 vectors per thread and tile; grid = total number of tiles
 hipError_t launch_alltoallv_direct(const VRankPtrs16 &ptrs, const A2avTablesDirect &tabs, uint32_t n, uint32_t esz,
                                    uint32_t grid, int unroll, hipStream_t stream);

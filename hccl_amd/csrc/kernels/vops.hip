@@ -185,6 +185,29 @@ k_alltoallv_direct(VRankPtrs16 ptrs, A2avTablesDirect tabs, uint32_t n, uint32_t
     copy_tile<UNROLL>(src, reinterpret_cast<uint64_t>(dst), bytes, tl, 1, [=](uint32_t) { return dst; });
 }
 
+// One tile per workgroup; its block is found in the host-made list (every index is wave-uniform: scalar loads).
+template <int UNROLL>
+__global__ void __launch_bounds__(kThreads)
+k_copy_blocks(const CopyBlock *__restrict__ blocks, uint32_t nblocks)
+{
+    const uint64_t t = blockIdx.x;
+    uint32_t lo = 0;
+    uint32_t hi = nblocks - 1;
+    while (lo < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (blocks[mid].tile_end > t) {
+            hi = mid;
+        } else {
+            lo = mid + 1;
+        }
+    }
+    const uint64_t tl = t - (lo ? blocks[lo - 1].tile_end : 0);
+    const char *src = blocks[lo].src;
+    char *dst = blocks[lo].dst;
+    const uint64_t bytes = blocks[lo].bytes;
+    copy_tile<UNROLL>(src, reinterpret_cast<uint64_t>(dst), bytes, tl, 1, [=](uint32_t) { return dst; });
+}
+
 template <typename Tabs>
 __global__ void __launch_bounds__(kThreads)
 k_allgatherv(VRankPtrs ptrs, Tabs tabs, uint32_t n, uint32_t esz, uint32_t tiles_per_block)
@@ -225,12 +248,15 @@ hipError_t launch_alltoallv(const VRankPtrs &ptrs, const uint64_t *send_counts, 
     return hipGetLastError();
 }
 
-hipError_t launch_alltoallv_inline(const VRankPtrs16 &ptrs, const A2avTablesInline &tabs, uint32_t n, uint32_t esz,
-                                   uint32_t grid, uint32_t tiles_per_block, hipStream_t stream)
+hipError_t launch_copy_blocks(const CopyBlock *blocks, uint32_t nblocks, uint32_t grid, int unroll, hipStream_t stream)
 {
-    const size_t lds = (static_cast<size_t>(n) * n + 4) * sizeof(uint64_t);
-    hipLaunchKernelGGL((k_alltoallv<VRankPtrs16, A2avTablesInline>), dim3(grid), dim3(kThreads), lds, stream, ptrs, tabs,
-                       n, esz, tiles_per_block);
+    if (unroll == 1) {
+        hipLaunchKernelGGL((k_copy_blocks<1>), dim3(grid), dim3(kThreads), 0, stream, blocks, nblocks);
+    } else if (unroll == 2) {
+        hipLaunchKernelGGL((k_copy_blocks<2>), dim3(grid), dim3(kThreads), 0, stream, blocks, nblocks);
+    } else {
+        hipLaunchKernelGGL((k_copy_blocks<4>), dim3(grid), dim3(kThreads), 0, stream, blocks, nblocks);
+    }
     return hipGetLastError();
 }
 
