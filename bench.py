@@ -385,7 +385,8 @@ def sweep_allreduce_12_ranks(torch, api, T, steps):
     """benchmark configuration 5: AllReduce on 12 ranks, 4 KiB ... 1 GiB per rank in powers of 4; int32 MAX through the
     NHR and halving-doubling templates, fp32 PROD through the CPU-reduce NHR template (what the selector
     takes for PROD) and halving-doubling.  Small sizes are bound by the launch, so microseconds are reported
-    beside GB/s (algorithmic bytes = 2 * 12 * size)."""
+    beside GB/s (algorithmic bytes = 2 * 12 * size); up to 1 MiB per rank also the time per collective when 20 of
+    them are replayed from one HIP graph."""
     n = 12
     cases = [("int32_max_nhr", T.INT32, T.MAX, "InsAllReduceNHR"), ("int32_max_rhd", T.INT32, T.MAX, "InsAllReduceRHD"),
              ("fp32_prod_aicpu_nhr", T.FP32, T.PROD, "InsAllReduceAicpuReduceNHR"),
@@ -417,6 +418,26 @@ def sweep_allreduce_12_ranks(torch, api, T, steps):
             info = w.last_info()
             row[name] = {"us": round(ms * 1e3, 1), "GB/s": round(2 * n * nbytes / (ms * 1e-3) / 1e9, 1),
                          "fused": bool(info.fused), "launches": info.launches}
+            if nbytes <= (1 << 20):
+                # launch-bound sizes: the warm collective captured 20 times into one HIP graph, so that the
+                # twelve host calls per collective drop out of the replayed time
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.stream(stream_obj):
+                    g.capture_begin()
+                    for _ in range(20):
+                        st.step()
+                    g.capture_end()
+                g.replay()
+                torch.cuda.synchronize()
+                e0 = torch.cuda.Event(enable_timing=True)
+                e1 = torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(5):
+                    g.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                row[name]["us_in_a_graph"] = round(e0.elapsed_time(e1) * 1e3 / 100, 2)
+                del g
             w.close()
         out["%d" % nbytes] = row
     del ins, outs
