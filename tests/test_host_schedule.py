@@ -139,6 +139,38 @@ def test_reduce_scatter_values_with_executor_chunks(alg):
         assert np.array_equal(got[r].view(np.uint32), want[r].view(np.uint32))
 
 
+def test_random_worlds_trace_equals_oracle():
+    """Seeded random (ranks, count, element size, template) draws up to 48 ranks, odd counts included: what the
+    recorded schedule computes for every output element is the oracle's expression, for AllReduce and
+    ReduceScatter alike."""
+    rng = np.random.default_rng(2024)
+    for _ in range(60):
+        n = int(rng.integers(1, 49))
+        dtype = [T.FP32, T.BFP16, T.FP64][int(rng.integers(3))]
+        esz = T.DTYPE_SIZE[dtype]
+        if rng.integers(2):
+            alg = AR_ALGS[int(rng.integers(len(AR_ALGS)))]
+            count = int(rng.integers(1, 4 * n + 40))
+            text, _ = dry_allreduce(n, count, dtype, T.SUM, alg)
+            want = T.run_allreduce(T.SymbolicElems(), sym_inputs(n, count), count, esz, alg, ccl_bytes=SMALL_CCL)
+            out_count = count
+        else:
+            alg = RS_ALGS[int(rng.integers(len(RS_ALGS)))]
+            rc = int(rng.integers(1, 60))
+            text, _ = dry_reduce_scatter(n, rc, dtype, T.SUM, alg)
+            want = T.run_reduce_scatter(T.SymbolicElems(), sym_inputs(n, n * rc), rc, esz, alg, ccl_bytes=SMALL_CCL)
+            out_count = rc
+        seen = [set() for _ in range(n)]
+        for rank, off, nbytes, expr in parse_trace(text):
+            tree = parse_expr(expr)
+            for e in range(nbytes // esz):
+                idx = off // esz + e
+                assert expr_to_oracle_string(tree, e, esz, off) == want[rank][idx], (alg, n, dtype, rank, idx)
+                seen[rank].add(idx)
+        if n > 1:
+            assert all(s_ == set(range(out_count)) for s_ in seen), (alg, n, out_count)
+
+
 def dry_reduce_scatter_v(counts, displs, dtype, op, ccl=SMALL_CCL):
     n = len(counts)
     w = api.World(n, ccl_bytes=ccl, dry=True)
