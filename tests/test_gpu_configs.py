@@ -314,3 +314,39 @@ def test_large_allreduce_takes_the_chunked_two_shot_template(stream):
             assert np.array_equal(take(outs[r], pos).view(np.uint32), want[r].val.view(np.uint32)), r
     finally:
         w.close()
+
+
+@pytest.mark.parametrize("n,alg,dtype,op", [(32, "InsAllReduceMesh1DTwoShot", T.FP32, T.SUM),     # wide chain kernel
+                                           (32, "InsAllReduceNHR", T.FP32, T.SUM),              # wide tree kernel
+                                           (64, "InsAllReduceRHD", T.FP32, T.PROD),
+                                           (40, "InsAllReduceNHR", T.INT32, T.MAX)])
+def test_allreduce_among_many_ranks_at_16MiB_per_rank(stream, n, alg, dtype, op):
+    """Communicators of more than 16 ranks at a size where the kernels run in their full-tile paths: all ranks
+    agree bit for bit, and 50,000 sampled columns equal the oracle's run of the same template."""
+    count = 4 * 1024 * 1024 + 3
+    if dtype == T.INT32:
+        xs = [torch.randint(-2**31, 2**31 - 1, (count,), device=DEV, dtype=torch.int32) for _ in range(n)]
+    elif op == T.PROD:
+        xs = [uniform(count, 900 + k, 0.97, 1.03) for k in range(n)]
+    else:
+        xs = [uniform(count, 900 + k, -1.0, 1.0) for k in range(n)]
+    outs = [torch.empty_like(x) for x in xs]
+    torch.cuda.synchronize()
+    w = api.World(n)
+    try:
+        w.set_algorithm(api.CMD_ALLREDUCE, alg)
+        for r in range(n):
+            assert w.all_reduce(r, xs[r].data_ptr(), outs[r].data_ptr(), count, dtype, op, stream.cuda_stream) == 0
+        stream.synchronize()
+        info = w.last_info()
+        assert info.fused == 1 and info.launches == 1
+        for r in range(1, n):
+            assert torch.equal(outs[r].view(torch.int32), outs[0].view(torch.int32)), r
+        rng = np.random.default_rng(n)
+        pos = sample_positions(rng, count, 50000, marks=[off for off, _ in T.split_data(count, n)][1:])
+        e = T.SampledElems(dtype, op)
+        want = T.run_allreduce(e, [e.sample(count, pos, take(x, pos)) for x in xs], count, 4, alg)
+        for r in (0, n // 2, n - 1):
+            assert np.array_equal(take(outs[r], pos).view(np.uint32), want[r].val.view(np.uint32)), r
+    finally:
+        w.close()
