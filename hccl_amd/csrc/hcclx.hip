@@ -376,8 +376,8 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
                                                 std::to_string(proto.maxn) + ") levels");
         }
         sd.head = fold_head_of(sd.count, proto.copy ? 1 : esz, sd.dst[0]);
-        sd.shift = fold_shift_of(sd.head, proto.copy ? 1 : esz, proto.maxn, sd.dst[0]);
-        const uint64_t tiles = fold_tiles_of(sd.count, ne, proto.maxn, sd.head, sd.shift);
+        sd.shift = fold_shift_of(sd.head, proto.copy ? 1 : esz, fold_tile_vecs(proto.maxn), sd.dst[0]);
+        const uint64_t tiles = fold_tiles_of(sd.count, ne, fold_tile_vecs(proto.maxn), sd.head, sd.shift);
         if (static_cast<int>(cur.segs.size()) == kMaxSegsPerLaunch) {
             out->batches.push_back(std::move(cur));
             cur = proto;
@@ -395,8 +395,8 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
 int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, Built *out)
 {
     if (nseg != 0 && segs == nullptr) return fail(HCCL_E_PTR, "segs is null");
-    if (mode != HCCLX_FOLD_CHAIN && mode != HCCLX_FOLD_TREE) {
-        return fail(mode == HCCLX_FOLD_SELF_FIRST ? HCCL_E_NOT_SUPPORT : HCCL_E_PARA, "wide segments fold as a chain or as a tree");
+    if (mode != HCCLX_FOLD_CHAIN && mode != HCCLX_FOLD_SELF_FIRST && mode != HCCLX_FOLD_TREE) {
+        return fail(HCCL_E_PARA, "unknown fold mode");
     }
     int esz = dtype_size(dtype);
     if (esz == 0) return fail(HCCL_E_NOT_SUPPORT, "unknown data type " + std::to_string(dtype));
@@ -415,6 +415,21 @@ int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, i
                 if (s.dst[k] == nullptr) return fail(HCCL_E_PTR, "segment " + std::to_string(i) + ": null destination");
             }
         }
+        if (mode == HCCLX_FOLD_SELF_FIRST) {
+            if (s.nsrc != s.ndst) return fail(HCCL_E_PARA, "self-first fold needs nsrc == ndst");
+            // the outputs are computed sixteen at a time by different workgroups: none may overwrite a source
+            // (integers have one value whatever the order and take the chain kernel: exempt)
+            const uint64_t bytes = is_float_dtype(dtype) ? s.count * static_cast<uint64_t>(esz) : 0;
+            for (uint32_t d = 0; d < s.ndst && bytes != 0; ++d) {
+                const uint64_t lo = reinterpret_cast<uint64_t>(s.dst[d]);
+                for (uint32_t k = 0; k < s.nsrc; ++k) {
+                    const uint64_t a = reinterpret_cast<uint64_t>(s.src[k]);
+                    if (lo < a + bytes && a < lo + bytes) {
+                        return fail(HCCL_E_PARA, "segment " + std::to_string(i) + ": a destination of a wide self-first fold overlaps a source");
+                    }
+                }
+            }
+        }
         if (mode == HCCLX_FOLD_TREE) {
             const int levels = tree_levels(s.nsrc, s.prog);
             if (levels < 0) return fail(HCCL_E_PARA, "segment " + std::to_string(i) + ": malformed tree program");
@@ -428,9 +443,10 @@ int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, i
     Batch proto;
     proto.dtype = dtype;
     proto.op = op;
-    // a tree over integers equals the chain of its leaves
-    proto.mode = (mode == HCCLX_FOLD_TREE && is_float_dtype(dtype) && max_src > 1) ? HCCLX_FOLD_TREE : HCCLX_FOLD_CHAIN;
+    // a tree over integers equals the chain of its leaves, and so does every self-first order
+    proto.mode = (mode != HCCLX_FOLD_CHAIN && is_float_dtype(dtype) && max_src > 1) ? mode : HCCLX_FOLD_CHAIN;
     proto.maxn = kMaxWideFan;
+    const uint64_t tile_vecs = wide_tile_vecs(proto.mode);
     uint64_t scale = 1;
     if (max_src <= 1) {
         // nothing is combined: any type is moved as bytes
@@ -468,16 +484,23 @@ int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, i
                 if (slot_reg[k] >= 0) sd.leaf_mask |= 1ull << k;
             }
         }
-        sd.head = fold_head_of(sd.count, esz, sd.dst[0]);
-        sd.shift = fold_shift_of(sd.head, esz, kMaxWideFan, sd.dst[0]);
-        const uint64_t tiles = fold_tiles_of(sd.count, ne, kMaxWideFan, sd.head, sd.shift);
-        if (static_cast<int>(cur.wide.size()) == kMaxWideSegsPerLaunch) {
-            out->batches.push_back(std::move(cur));
-            cur = proto;
+        // a self-first segment is entered once per group of kMaxFan outputs; its tiles follow that group's first
+        // destination
+        const uint32_t entries = proto.mode == HCCLX_FOLD_SELF_FIRST ? (s.nsrc + kMaxFan - 1) / kMaxFan : 1;
+        for (uint32_t g = 0; g < entries; ++g) {
+            sd.first_dst = g * kMaxFan;
+            char *lead = sd.dst[sd.first_dst];
+            sd.head = fold_head_of(sd.count, esz, lead);
+            sd.shift = fold_shift_of(sd.head, esz, tile_vecs, lead);
+            const uint64_t tiles = fold_tiles_of(sd.count, ne, tile_vecs, sd.head, sd.shift);
+            if (static_cast<int>(cur.wide.size()) == kMaxWideSegsPerLaunch) {
+                out->batches.push_back(std::move(cur));
+                cur = proto;
+            }
+            cur.total_tiles += tiles;
+            cur.tile_end.push_back(cur.total_tiles);
+            cur.wide.push_back(sd);
         }
-        cur.total_tiles += tiles;
-        cur.tile_end.push_back(cur.total_tiles);
-        cur.wide.push_back(sd);
         out->algo_bytes += static_cast<uint64_t>(s.nsrc + s.ndst) * sd.count * esz;
     }
     if (!cur.wide.empty()) out->batches.push_back(std::move(cur));

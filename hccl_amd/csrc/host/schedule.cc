@@ -479,6 +479,7 @@ struct FusedPlan {
     std::vector<hcclx_seg_t> treeSegs;
     std::vector<hcclx_wide_seg_t> wideSegs;       // chains over more than HCCLX_MAX_FAN sources
     std::vector<hcclx_wide_seg_t> wideTreeSegs;   // trees with more leaves or levels than the 16-slot kernel holds
+    std::vector<hcclx_wide_seg_t> wideSelfSegs;   // the per-rank orders of the one-shot templates among 17 .. 64 ranks
 };
 
 bool Overlaps(u64 a, u64 alen, u64 b, u64 blen) { return a < b + blen && b < a + alen; }
@@ -537,7 +538,7 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
     for (auto &kv : bySrc) {
         if (kv.second.size() != 1) continue;
         const Fold &f = folds[kv.second[0]];
-        if (!f.chain || f.src.size() < 2 || f.src.size() > HCCLX_MAX_FAN) continue;
+        if (!f.chain || f.src.size() < 2 || f.src.size() > HCCLX_MAX_WIDE_FAN) continue;
         std::vector<u64> key = f.src;
         std::sort(key.begin(), key.end());
         key.push_back(f.bytes);
@@ -570,6 +571,29 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
                 owner[j] = static_cast<int>(g);
             }
             if (!ok) continue;
+            if (n > HCCLX_MAX_FAN) {
+                // the wide kernel computes the outputs sixteen at a time in different workgroups, so none of
+                // them may overwrite a source (an in-place collective among more than 16 ranks is not grouped)
+                bool clash = false;
+                for (size_t j = 0; j < n && !clash; ++j) {
+                    for (size_t k = 0; k < n && !clash; ++k) {
+                        clash = Overlaps(folds[owner[j]].dst, folds[owner[j]].bytes, base[k], folds[cand].bytes);
+                    }
+                }
+                if (clash) break;
+                hcclx_wide_seg_t seg;
+                std::memset(&seg, 0, sizeof(seg));
+                seg.count = folds[cand].bytes / esz;
+                seg.nsrc = static_cast<uint32_t>(n);
+                seg.ndst = static_cast<uint32_t>(n);
+                for (size_t j = 0; j < n; ++j) {
+                    seg.src[j] = reinterpret_cast<const void *>(base[j]);
+                    seg.dst[j] = reinterpret_cast<void *>(folds[owner[j]].dst);
+                    taken[owner[j]] = true;
+                }
+                plan.wideSelfSegs.push_back(seg);
+                break;
+            }
             hcclx_seg_t seg;
             std::memset(&seg, 0, sizeof(seg));
             seg.count = folds[cand].bytes / esz;
@@ -1072,7 +1096,7 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
                                        (w->traceText || w->dryRun) ? &w->lastTrace : nullptr);
         w->lastFusedSegments =
             static_cast<u32>(plan.chainSegs.size() + plan.selfSegs.size() + plan.copySegs.size() + plan.treeSegs.size() +
-                             plan.wideSegs.size() + plan.wideTreeSegs.size());
+                             plan.wideSegs.size() + plan.wideTreeSegs.size() + plan.wideSelfSegs.size());
         if (w->dryRun) {
             w->lastWasFused = ok;
             return HCCL_SUCCESS;
@@ -1096,12 +1120,12 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
                 }
                 c.plans.push_back(hp);
             }
-            for (int i = 0; i < 2; ++i) {
-                const std::vector<hcclx_wide_seg_t> &segs = i == 0 ? plan.wideSegs : plan.wideTreeSegs;
+            for (int i = 0; i < 3; ++i) {
+                const std::vector<hcclx_wide_seg_t> &segs = i == 0 ? plan.wideSegs : i == 1 ? plan.wideTreeSegs : plan.wideSelfSegs;
                 if (segs.empty()) continue;
                 hcclx_plan *hp = nullptr;
                 const int rc = hcclx_plan_create_wide(segs.data(), static_cast<uint32_t>(segs.size()), foldType, op,
-                                                      i == 0 ? HCCLX_FOLD_CHAIN : HCCLX_FOLD_TREE, &hp);
+                                                      i == 0 ? HCCLX_FOLD_CHAIN : i == 1 ? HCCLX_FOLD_TREE : HCCLX_FOLD_SELF_FIRST, &hp);
                 if (rc != HCCL_SUCCESS) {
                     DropPlans(c.plans);
                     return static_cast<HcclResult>(rc);

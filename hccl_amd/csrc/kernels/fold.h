@@ -24,16 +24,31 @@ namespace hcclx {
 #define HCCLX_FOLD_THREADS 256
 #endif
 constexpr int kFoldThreads = HCCLX_FOLD_THREADS;
+// The wide kernels: vectors per thread and tile, and sources loaded before they are folded in.
+// Two vectors per thread with eight sources in flight measured 24 % faster on a 32-rank AllReduce than one
+// vector with sixteen (the same loads outstanding, twice the contiguous run per source).
+#ifndef HCCLX_WIDE_UNROLL
+#define HCCLX_WIDE_UNROLL 2
+#endif
+#ifndef HCCLX_WIDE_GROUP
+#define HCCLX_WIDE_GROUP 8
+#endif
+constexpr int kWideUnroll = HCCLX_WIDE_UNROLL;
+constexpr int kWideGroup = HCCLX_WIDE_GROUP;
 constexpr uint32_t kFoldDirectSegs = 64;   // up to this many segments the tile prefix is searched in place
 __host__ __device__ constexpr int fold_unroll(int maxn)
 {
     constexpr int u[5] = {HCCLX_FOLD_UNROLLS};
-    // more than kMaxFan sources: the wide kernel, which walks them in groups, one vector per thread
-    return maxn <= 1 ? u[0] : maxn <= 2 ? u[1] : maxn <= 4 ? u[2] : maxn <= 8 ? u[3] : maxn <= kMaxFan ? u[4] : 1;
+    return maxn <= 1 ? u[0] : maxn <= 2 ? u[1] : maxn <= 4 ? u[2] : maxn <= 8 ? u[3] : u[4];
 }
 __host__ __device__ constexpr uint64_t fold_tile_vecs(int maxn)
 {
     return static_cast<uint64_t>(kFoldThreads) * fold_unroll(maxn);
+}
+// Tiles of the wide kernels: the chain walks kWideUnroll vectors per thread, the self-first and tree orders one.
+__host__ __device__ constexpr uint64_t wide_tile_vecs(int mode)
+{
+    return static_cast<uint64_t>(kFoldThreads) * (mode == 0 ? kWideUnroll : 1);
 }
 
 #ifndef HCCLX_NT_LOAD
@@ -212,6 +227,17 @@ __device__ __forceinline__ void fold_tail(const SEG &sd, uint32_t nsrc, uint32_t
         }
         const S out = D::narrow(val[0][0]);
         for (uint32_t d = 0; d < ndst; ++d) reinterpret_cast<S *>(sd.dst[d])[idx] = out;
+    } else if constexpr (MAXN > kMaxFan) {
+        // The wide self-first order: the outputs of this entry's group, each from the sources as they lie in
+        // memory (no destination overlaps a source in this mode).
+        const uint32_t first = sd.first_dst;
+        for (uint32_t j = first; j < first + kMaxFan && j < nsrc; ++j) {
+            C acc = D::widen(reinterpret_cast<const S *>(sd.src[j])[idx]);
+            for (uint32_t k = 0; k < nsrc; ++k) {
+                if (k != j) acc = Op::run(D::widen(reinterpret_cast<const S *>(sd.src[k])[idx]), acc);
+            }
+            reinterpret_cast<S *>(sd.dst[j])[idx] = D::narrow(acc);
+        }
     } else {
         // Every source is read before the first destination is written: a destination may alias a source.
         C val[kMaxFan];
@@ -311,39 +337,59 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
 // each group loaded before it is folded in, so the loads in flight per thread stay what the 16-source kernel
 // has.  One vector per thread and tile.
 template <int DT, int OP, bool CHECK>
-__device__ __forceinline__ void fold_tile_wide(const SegWide &sd, uint32_t nsrc, uint32_t ndst, uint64_t v, uint64_t nvec,
+__device__ __forceinline__ void fold_tile_wide(const SegWide &sd, uint32_t nsrc, uint32_t ndst, uint64_t v0, uint64_t nvec,
                                                uint32_t head_bytes)
 {
     using V = Vec16<DT>;
     using C = typename V::C;
     constexpr int NE = V::NE;
-    if (CHECK && v >= nvec) {
-        return;
-    }
-    const uint64_t off = head_bytes + v * 16;
-    C acc[NE];
-    V::unpack(ld16(sd.src[0] + off), acc);
-    for (uint32_t base = 1; base < nsrc; base += kMaxFan) {
-        u32x4 raw[kMaxFan];
+    constexpr int U = kWideUnroll;
+    constexpr int G = kWideGroup;
+    bool ok[U];
+    uint64_t off[U];
+    C acc[U][NE];
 #pragma unroll
-        for (int k = 0; k < kMaxFan; ++k) {
-            if (base + k < nsrc) raw[k] = ld16(sd.src[base + k] + off);
+    for (int u = 0; u < U; ++u) {
+        const uint64_t v = v0 + static_cast<uint64_t>(u) * kFoldThreads;
+        ok[u] = !CHECK || v < nvec;
+        off[u] = head_bytes + v * 16;
+        if (ok[u]) V::unpack(ld16(sd.src[0] + off[u]), acc[u]);
+    }
+    for (uint32_t base = 1; base < nsrc; base += G) {
+        u32x4 raw[U][G];
+#pragma unroll
+        for (int k = 0; k < G; ++k) {
+            if (base + k < nsrc) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    if (ok[u]) raw[u][k] = ld16(sd.src[base + k] + off[u]);
+                }
+            }
         }
 #pragma unroll
-        for (int k = 0; k < kMaxFan; ++k) {
+        for (int k = 0; k < G; ++k) {
             if (base + k < nsrc) {
-                C x[NE];
-                V::unpack(raw[k], x);
 #pragma unroll
-                for (int e = 0; e < NE; ++e) acc[e] = V::template combine<OP>(x[e], acc[e]);
+                for (int u = 0; u < U; ++u) {
+                    if (ok[u]) {
+                        C x[NE];
+                        V::unpack(raw[u][k], x);
+#pragma unroll
+                        for (int e = 0; e < NE; ++e) acc[u][e] = V::template combine<OP>(x[e], acc[u][e]);
+                    }
+                }
             }
         }
     }
-    const u32x4 out = V::pack(acc);
     for (uint32_t base = 0; base < ndst; base += kMaxFan) {
 #pragma unroll
         for (int d = 0; d < kMaxFan; ++d) {
-            if (base + d < ndst) st16(sd.dst[base + d] + off, out);
+            if (base + d < ndst) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    if (ok[u]) st16(sd.dst[base + d] + off[u], V::pack(acc[u]));
+                }
+            }
         }
     }
 }
@@ -399,7 +445,7 @@ __device__ __forceinline__ void fold_tile_wide_tree(const SegWide &sd, uint32_t 
     wide_subtree<DT, OP, 1>(sd, off, mask, part[1]);
     wide_subtree<DT, OP, 2>(sd, off, mask, part[2]);
     wide_subtree<DT, OP, 3>(sd, off, mask, part[3]);
-    static_assert(kGroups == 4, "the subtree roots above are heap nodes 4 .. 7");
+    static_assert(kMaxFan == 16 && kGroups == 4, "the subtree roots above are heap nodes 4 .. 7");
     tree_eval_at<DT, OP, kGroups, 1, C, NE>(part, code);
     const u32x4 out = V::pack(part[0]);
     for (uint32_t base = 0; base < ndst; base += kMaxFan) {
@@ -410,13 +456,74 @@ __device__ __forceinline__ void fold_tile_wide_tree(const SegWide &sd, uint32_t 
     }
 }
 
+// The self-first order among more than kMaxFan ranks: this segment entry computes the kMaxFan outputs
+// first_dst .. first_dst + kMaxFan - 1 (a segment of n ranks is entered once per such group).  Output j starts
+// from src[j] and takes the other sources in ascending order; the sources are loaded in groups of kMaxFan and every
+// loaded vector goes into all accumulators but its own.  Destinations must not overlap sources: other workgroups
+// still read what this one would overwrite.
+template <int DT, int OP, bool CHECK>
+__device__ __forceinline__ void fold_tile_wide_self(const SegWide &sd, uint32_t nsrc, uint64_t v, uint64_t nvec,
+                                                    uint32_t head_bytes)
+{
+    using V = Vec16<DT>;
+    using C = typename V::C;
+    constexpr int NE = V::NE;
+    if (CHECK && v >= nvec) {
+        return;
+    }
+    const uint64_t off = head_bytes + v * 16;
+    const uint32_t first = sd.first_dst;
+    C acc[kMaxFan][NE];
+    {
+        u32x4 raw[kMaxFan];
+#pragma unroll
+        for (int j = 0; j < kMaxFan; ++j) {
+            if (first + j < nsrc) raw[j] = ld16(sd.src[first + j] + off);
+        }
+#pragma unroll
+        for (int j = 0; j < kMaxFan; ++j) {
+            if (first + j < nsrc) V::unpack(raw[j], acc[j]);
+        }
+    }
+    constexpr int G = 8;   // sources per load group: the unrolled body is G x kMaxFan updates
+    for (uint32_t base = 0; base < nsrc; base += G) {
+        u32x4 raw[G];
+#pragma unroll
+        for (int k = 0; k < G; ++k) {
+            if (base + k < nsrc) raw[k] = ld16(sd.src[base + k] + off);
+        }
+        // only the groups at first and first + G hold the outputs' own sources: source base + k is output
+        // j's own when j == k + (base - first)
+        const bool own_lo = (base == first);
+        const bool own_hi = (base == first + G);
+#pragma unroll
+        for (int k = 0; k < G; ++k) {
+            if (base + k < nsrc) {
+                C x[NE];
+                V::unpack(raw[k], x);
+#pragma unroll
+                for (int j = 0; j < kMaxFan; ++j) {
+                    const bool own = (own_lo && j == k) || (own_hi && j == k + G);
+                    if (first + j < nsrc && !own) {
+#pragma unroll
+                        for (int e = 0; e < NE; ++e) acc[j][e] = V::template combine<OP>(x[e], acc[j][e]);
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < kMaxFan; ++j) {
+        if (first + j < nsrc) st16(sd.dst[first + j] + off, V::pack(acc[j]));
+    }
+}
+
 template <int DT, int OP, int MODE>
 __global__ void __launch_bounds__(kFoldThreads)
 k_fold_wide(const uint64_t *__restrict__ tile_end, const SegWide *__restrict__ segs, uint32_t nseg, uint64_t total_tiles)
 {
     constexpr int NE = Vec16<DT>::kElems;
-    constexpr uint64_t TV = fold_tile_vecs(kMaxWideFan);
-    static_assert(TV == kFoldThreads, "the wide kernel moves one vector per thread and tile");
+    constexpr uint64_t TV = wide_tile_vecs(MODE);
     extern __shared__ uint64_t s_end[];
     const bool direct = nseg <= kFoldDirectSegs;
     if (!direct) {
@@ -442,12 +549,16 @@ k_fold_wide(const uint64_t *__restrict__ tile_end, const SegWide *__restrict__ s
         if (tl * TV >= shift && (tl + 1) * TV - shift <= nvec) {
             if constexpr (MODE == kFoldTree) {
                 fold_tile_wide_tree<DT, OP, false>(sd, ndst, v, nvec, head_bytes);
+            } else if constexpr (MODE == kFoldSelfFirst) {
+                fold_tile_wide_self<DT, OP, false>(sd, nsrc, v, nvec, head_bytes);
             } else {
                 fold_tile_wide<DT, OP, false>(sd, nsrc, ndst, v, nvec, head_bytes);
             }
         } else {
             if constexpr (MODE == kFoldTree) {
                 fold_tile_wide_tree<DT, OP, true>(sd, ndst, v, nvec, head_bytes);
+            } else if constexpr (MODE == kFoldSelfFirst) {
+                fold_tile_wide_self<DT, OP, true>(sd, nsrc, v, nvec, head_bytes);
             } else {
                 fold_tile_wide<DT, OP, true>(sd, nsrc, ndst, v, nvec, head_bytes);
             }
@@ -472,16 +583,16 @@ inline uint32_t fold_head_of(uint64_t count, int esz, const void *dst0)
 }
 
 // Vectors by which the tile grid is shifted so that tiles are aligned in the address space of dst0.
-inline uint32_t fold_shift_of(uint32_t head, int esz, int maxn, const void *dst0)
+inline uint32_t fold_shift_of(uint32_t head, int esz, uint64_t tile_vecs, const void *dst0)
 {
     const uint64_t body_addr = reinterpret_cast<uint64_t>(dst0) + static_cast<uint64_t>(head) * esz;
     if (body_addr % 16 != 0) {
         return 0;   // no aligned body (see fold_head_of)
     }
-    return static_cast<uint32_t>((body_addr % (fold_tile_vecs(maxn) * 16)) / 16);
+    return static_cast<uint32_t>((body_addr % (tile_vecs * 16)) / 16);
 }
 
-inline uint64_t fold_tiles_of(uint64_t count, int ne, int maxn, uint32_t head, uint32_t shift)
+inline uint64_t fold_tiles_of(uint64_t count, int ne, uint64_t tile_vecs, uint32_t head, uint32_t shift)
 {
     if (count == 0) {
         return 0;
@@ -489,8 +600,7 @@ inline uint64_t fold_tiles_of(uint64_t count, int ne, int maxn, uint32_t head, u
     const uint64_t body = count - head;
     const uint64_t nvec = body / ne;
     const uint64_t units = shift + nvec + ((head + body % ne) ? 1 : 0);
-    const uint64_t tv = fold_tile_vecs(maxn);
-    return (units + tv - 1) / tv;
+    return (units + tile_vecs - 1) / tile_vecs;
 }
 
 struct FoldLaunch {

@@ -40,12 +40,7 @@ static hipError_t by_fan(int maxn, const FoldLaunch &l)
         case 4: return launch_one<HCCLX_DT, OP, 4, MODE>(l);
         case 8: return launch_one<HCCLX_DT, OP, 8, MODE>(l);
         case 16: return launch_one<HCCLX_DT, OP, 16, MODE>(l);
-        case kMaxWideFan:
-            if constexpr (MODE == kFoldSelfFirst) {
-                return hipErrorInvalidValue;
-            } else {
-                return launch_wide<HCCLX_DT, OP, MODE>(l);
-            }
+        case kMaxWideFan: return launch_wide<HCCLX_DT, OP, MODE>(l);
         default: return hipErrorInvalidValue;
     }
 }

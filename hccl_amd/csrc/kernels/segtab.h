@@ -38,8 +38,9 @@ struct SegDev {
 
 // A segment of the wide kernels.  Chain: acc = src[0]; acc = src[k] (+) acc for k = 1 .. nsrc-1.  Tree: as in
 // SegDev, embedded in a complete binary tree with kMaxWideFan leaf slots; the 2-bit code of inner node i sits at
-// bit 2 * (i % 16) of tree_codes[i / 16].  The value goes to every dst.  head and shift as in SegDev, for tiles
-// of one vector per thread.
+// bit 2 * (i % 16) of tree_codes[i / 16].  In both the value goes to every dst.  Self-first: nsrc == ndst, and
+// the entry computes the outputs first_dst .. first_dst + kMaxFan - 1 only (the launcher enters a segment once per
+// such group).  head and shift as in SegDev, for the tile size of the mode.
 struct SegWide {
     uint64_t count;
     uint32_t nsrc;
@@ -48,6 +49,8 @@ struct SegWide {
     uint32_t shift;
     uint64_t leaf_mask;
     uint32_t tree_codes[4];
+    uint32_t first_dst;
+    uint32_t reserved;
     const char *src[kMaxWideFan];
     char *dst[kMaxWideFan];
 };

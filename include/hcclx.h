@@ -63,8 +63,10 @@ typedef struct {
 } hcclx_seg_t;
 
 /* A segment with up to HCCLX_MAX_WIDE_FAN sources and destinations, for communicators of more than
- * HCCLX_MAX_FAN ranks.  HCCLX_FOLD_CHAIN and HCCLX_FOLD_TREE as for hcclx_seg_t (a floating-point tree may have
- * up to six levels); HCCLX_FOLD_SELF_FIRST is not taken.  Aliasing rules as for hcclx_seg_t. */
+ * HCCLX_MAX_FAN ranks.  The modes are those of hcclx_seg_t; a floating-point tree may have up to six levels.
+ * Aliasing rules as for hcclx_seg_t, except HCCLX_FOLD_SELF_FIRST over floating-point types: there no
+ * destination may overlap a source (the outputs are computed sixteen at a time by different workgroups, each of
+ * which reads every source; such a call is rejected). */
 #define HCCLX_MAX_WIDE_FAN 64
 typedef struct {
     uint64_t count;

@@ -110,6 +110,26 @@ def test_checked_world_verifies_then_launches(stream):
         w.close()
 
 
+def test_one_shot_allreduce_in_place_among_24_ranks_runs_step_by_step(stream):
+    """sendBuf == recvBuf with the per-rank orders of the one-shot template: among more than 16 ranks the outputs
+    cannot be computed in one pass without overwriting inputs that other workgroups still read, so the steps run
+    one by one; the values are the template's."""
+    n, count = 24, 30011
+    rng = np.random.default_rng(24)
+    xs = [payload(rng, T.FP32, count, "uniform") for _ in range(n)]
+    w = api.World(n, ccl_bytes=SMALL_CCL)
+    try:
+        w.set_algorithm(api.CMD_ALLREDUCE, "InsAllReduceMesh1DOneShot")
+        got, bufs = run_allreduce(w, stream, xs, count, T.FP32, T.SUM, in_place=True)
+        assert w.last_info().fused == 0
+        want = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs, count, 4, "InsAllReduceMesh1DOneShot", ccl_bytes=SMALL_CCL)
+        for r in range(n):
+            assert_same_bits(got[r], want[r], T.FP32, f"rank {r}")
+            assert bufs[r].guard_intact()
+    finally:
+        w.close()
+
+
 def test_step_by_step_plans_are_replayed_with_new_data(stream):
     """A schedule that cannot be fused (among 9 ranks the ring's MAX fold is a spine of eight levels, and a
     floating-point MAX cannot be reordered) and the explicit step-by-step mode: the second identical call replays the per-level launches from the cache, on the

@@ -256,6 +256,46 @@ def test_wide_tree_fold_up_to_six_levels(nsrc, levels, dtype, op):
             assert o.guard_intact()
 
 
+@pytest.mark.parametrize("nsrc", [17, 24, 32, 33, 48, 64])
+@pytest.mark.parametrize("dtype,op", [(T.FP32, T.SUM), (T.BFP16, T.SUM), (T.FP16, T.PROD), (T.FP64, T.MAX), (T.INT32, T.SUM)])
+def test_wide_self_first_fold_gives_every_rank_its_own_order(nsrc, dtype, op):
+    """The per-rank orders of the one-shot templates among 17 .. 64 ranks: output j starts from source j and takes
+    the others ascending; outputs are computed sixteen at a time."""
+    rng = np.random.default_rng(nsrc * 13 + dtype + op)
+    esz = T.DTYPE_SIZE[dtype]
+    n = 2 * 4096 // esz + 11
+    kind = "prod" if op == T.PROD else "uniform" if dtype in (T.FP32, T.FP64) else "normal"
+    xs = [payload(rng, dtype, n, kind) for _ in range(nsrc)]
+    bufs = [DevBuf(x, offset=(k % 3) * esz) for k, x in enumerate(xs)]
+    outs = [DevBuf(nbytes=xs[0].nbytes, offset=(k % 5) * esz) for k in range(nsrc)]
+    hcclx.fold_wide([(n, [b.ptr for b in bufs], [o.ptr for o in outs])], dtype, op, hcclx.FOLD_SELF_FIRST)
+    sync()
+    for r in range(nsrc):
+        order = [r] + [k for k in range(nsrc) if k != r]
+        want = fold_oracle(xs, dtype, op, order, wide=fused_is_wide(dtype, op))
+        assert_same_bits(outs[r].get(T.NP_STORAGE[dtype]), want, dtype, f"rank {r}")
+        assert outs[r].guard_intact()
+
+
+def test_wide_self_first_fold_rejects_in_place():
+    x = np.arange(1024, dtype=np.float32)
+    bufs = [DevBuf(x + k) for k in range(20)]
+    outs = [DevBuf(nbytes=x.nbytes) for _ in range(20)]
+    with pytest.raises(HcclError) as e:
+        hcclx.fold_wide([(1024, [b.ptr for b in bufs], [b.ptr for b in bufs])], T.FP32, T.SUM, hcclx.FOLD_SELF_FIRST)
+    assert e.value.code == 1
+    with pytest.raises(HcclError) as e:
+        hcclx.fold_wide([(1024, [b.ptr for b in bufs], [o.ptr for o in outs[:19]])], T.FP32, T.SUM, hcclx.FOLD_SELF_FIRST)
+    assert e.value.code == 1
+    # integers have one value whatever the order, so in place is taken (one chain, twenty destinations)
+    xi = [np.arange(1024, dtype=np.int32) * (k + 1) for k in range(20)]
+    ib = [DevBuf(v) for v in xi]
+    hcclx.fold_wide([(1024, [b.ptr for b in ib], [b.ptr for b in ib])], T.INT32, T.SUM, hcclx.FOLD_SELF_FIRST)
+    sync()
+    for b in ib:
+        assert np.array_equal(b.get(np.int32), np.arange(1024, dtype=np.int32) * 210)
+
+
 def test_wide_tree_fold_rejects_seven_levels_and_malformed_programs():
     b = DevBuf(nbytes=64)
     deep = [x for k in range(1, 8) for x in (0, k)]     # a spine of seven levels
@@ -265,9 +305,6 @@ def test_wide_tree_fold_rejects_seven_levels_and_malformed_programs():
     with pytest.raises(HcclError) as e:
         hcclx.fold_wide([(4, [b.ptr] * 3, [b.ptr], [0, 1, 0, 1])], T.FP32, T.SUM, hcclx.FOLD_TREE)
     assert e.value.code == 1
-    with pytest.raises(HcclError) as e:
-        hcclx.fold_wide([(4, [b.ptr] * 3, [b.ptr] * 3)], T.FP32, T.SUM, hcclx.FOLD_SELF_FIRST)
-    assert e.value.code == 5
 
 
 def test_tree_fold_in_place_and_chain_shaped_program():
