@@ -69,6 +69,7 @@ void init_slot(DeviceSlot *s, int dev)
         c.blocks_per_cu = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
     }
     if (const char *v = std::getenv("HCCLX_A2AV_DIRECT")) c.a2av_direct_unroll = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
+    if (const char *v = std::getenv("HCCLX_WIDE_CHAIN_FROM")) c.wide_chain_from = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
     if (const char *v = std::getenv("HCCLX_V_BLOCKS_PER_CU")) {
         const uint32_t b = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
         if (b != 0) c.v_blocks_per_cu = b;
@@ -297,9 +298,34 @@ int tree_levels(uint32_t nsrc, const uint8_t *prog)
     return static_cast<int>(depth[0]);
 }
 
+int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, Built *out);
+
 int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, Built *out)
 {
     if (nseg != 0 && segs == nullptr) return fail(HCCL_E_PTR, "segs is null");
+    // Chains over many sources run faster on the wide chain kernel (sources in groups of eight, two vectors per
+    // thread) than on the kernel that holds every source in registers.
+    if (mode == HCCLX_FOLD_CHAIN && nseg != 0) {
+        const DeviceCtx *ctx = device_ctx();
+        uint32_t most = 0;
+        bool plain = true;
+        for (uint32_t i = 0; i < nseg; ++i) {
+            plain = plain && segs[i].nsrc <= HCCLX_MAX_FAN && segs[i].ndst <= HCCLX_MAX_FAN;
+            most = segs[i].nsrc > most ? segs[i].nsrc : most;
+        }
+        if (ctx && plain && most >= ctx->wide_chain_from) {
+            std::vector<hcclx_wide_seg_t> wide(nseg);
+            for (uint32_t i = 0; i < nseg; ++i) {
+                std::memset(&wide[i], 0, sizeof(wide[i]));
+                wide[i].count = segs[i].count;
+                wide[i].nsrc = segs[i].nsrc;
+                wide[i].ndst = segs[i].ndst;
+                for (uint32_t k = 0; k < segs[i].nsrc; ++k) wide[i].src[k] = segs[i].src[k];
+                for (uint32_t k = 0; k < segs[i].ndst; ++k) wide[i].dst[k] = segs[i].dst[k];
+            }
+            return build_wide_batches(wide.data(), nseg, dtype, op, HCCLX_FOLD_CHAIN, out);
+        }
+    }
     const int esz = dtype_size(dtype);
     if (esz == 0) return fail(HCCL_E_NOT_SUPPORT, "unknown data type " + std::to_string(dtype));
     if (mode != HCCLX_FOLD_CHAIN && mode != HCCLX_FOLD_SELF_FIRST && mode != HCCLX_FOLD_TREE) {
