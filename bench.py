@@ -75,11 +75,12 @@ def _randn_bits16(torch, n, seed, dt):
 class ReduceScatterMesh(Workload):
     """benchmark configuration 2: HcclReduceScatter SUM bf16, 8 ranks x 33,554,432 elements in (64 MiB per rank).
     The selector picks the mesh template; output shard r folds slice r of every rank starting from rank
-    r's own data, then ranks ascending (ins_temp_reduce_scatter_mesh_1D.cc:132-154), as one fused pass."""
+    r's own data, then ranks ascending (ins_temp_reduce_scatter_mesh_1D.cc:132-154), as one fused pass of the
+    chain kernel that moves four vectors per thread (eight sources, one destination per segment)."""
     dtype = "bf16"
-    kernel = "hcclx::k_fold<11, 0, 8, 0>"
-    traffic = 604053285
-    profile = "profiles/k_fold_reduce_scatter_bf16_8x64MiB.txt"
+    kernel = "hcclx::k_fold_wide<11, 0, 0, 4>"
+    traffic = 604101876
+    profile = "profiles/k_fold_wide_reduce_scatter_bf16_8x64MiB.txt"
 
     def __init__(self, torch, api, T, n=8, recv=4 * 1024 * 1024):
         super().__init__(torch, api, T, n)
@@ -122,7 +123,7 @@ class AllReduce(Workload):
     ranks, so each input is read once and the result is written to the eight outputs."""
     dtype = "f32"
     kernel = "hcclx::k_fold<4, 0, 8, 0>"
-    traffic = 1073639248
+    traffic = 1073659050
     profile = "profiles/k_fold_all_reduce_fp32_8x64MiB.txt"
 
     def __init__(self, torch, api, T, n=8, count=16 * 1024 * 1024, alg=None, step_mode=False):
@@ -157,7 +158,7 @@ class AllGather(Workload):
     output; each source byte is read once and written eight times."""
     dtype = "u8"
     kernel = "hcclx::(anonymous namespace)::k_allgatherv"
-    traffic = 4835368852
+    traffic = 4835342849
     profile = "profiles/k_allgatherv_fp16_8x64MiB.txt"
 
     def __init__(self, torch, api, T, n=8, count=32 * 1024 * 1024):
@@ -214,7 +215,7 @@ class AllToAllV(Workload):
     destination rank per token Zipf(s=1.2), tokens grouped by destination."""
     dtype = "u8"
     kernel = "hcclx::(anonymous namespace)::k_alltoallv_direct<2>"
-    traffic = 939416174
+    traffic = 939391554
     profile = "profiles/k_alltoallv_bf16_moe_8x4096x7168.txt"
 
     def __init__(self, torch, api, T, n=8, tokens=4096, hidden=7168, seed=0):

@@ -70,6 +70,9 @@ void init_slot(DeviceSlot *s, int dev)
     }
     if (const char *v = std::getenv("HCCLX_A2AV_DIRECT")) c.a2av_direct_unroll = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
     if (const char *v = std::getenv("HCCLX_WIDE_CHAIN_FROM")) c.wide_chain_from = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
+    if (const char *v = std::getenv("HCCLX_WIDE_CHAIN_FROM_ONE_DST")) {
+        c.wide_chain_from_one_dst = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
+    }
     if (const char *v = std::getenv("HCCLX_V_BLOCKS_PER_CU")) {
         const uint32_t b = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
         if (b != 0) c.v_blocks_per_cu = b;
@@ -204,6 +207,7 @@ struct Batch {
     std::vector<uint64_t> tile_end;
     std::vector<SegDev> segs;
     std::vector<SegWide> wide;   // instead of segs when maxn == kMaxWideFan
+    int wide_unroll = 1;         // vectors per thread of the wide kernel
     size_t nseg() const { return segs.size() + wide.size(); }
     size_t bytes() const
     {
@@ -308,12 +312,14 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
     if (mode == HCCLX_FOLD_CHAIN && nseg != 0) {
         const DeviceCtx *ctx = device_ctx();
         uint32_t most = 0;
+        uint32_t most_dst = 0;
         bool plain = true;
         for (uint32_t i = 0; i < nseg; ++i) {
             plain = plain && segs[i].nsrc <= HCCLX_MAX_FAN && segs[i].ndst <= HCCLX_MAX_FAN;
             most = segs[i].nsrc > most ? segs[i].nsrc : most;
+            most_dst = segs[i].ndst > most_dst ? segs[i].ndst : most_dst;
         }
-        if (ctx && plain && most >= ctx->wide_chain_from) {
+        if (ctx && plain && most >= (most_dst <= 1 ? ctx->wide_chain_from_one_dst : ctx->wide_chain_from)) {
             std::vector<hcclx_wide_seg_t> wide(nseg);
             for (uint32_t i = 0; i < nseg; ++i) {
                 std::memset(&wide[i], 0, sizeof(wide[i]));
@@ -472,7 +478,10 @@ int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, i
     // a tree over integers equals the chain of its leaves, and so does every self-first order
     proto.mode = (mode != HCCLX_FOLD_CHAIN && is_float_dtype(dtype) && max_src > 1) ? mode : HCCLX_FOLD_CHAIN;
     proto.maxn = kMaxWideFan;
-    const uint64_t tile_vecs = wide_tile_vecs(proto.mode);
+    uint32_t max_dst = 0;
+    for (uint32_t i = 0; i < nseg; ++i) max_dst = segs[i].ndst > max_dst ? segs[i].ndst : max_dst;
+    proto.wide_unroll = proto.mode != HCCLX_FOLD_CHAIN ? 1 : max_dst <= 1 ? kWideUnrollOne : kWideUnrollMany;
+    const uint64_t tile_vecs = wide_tile_vecs(proto.wide_unroll);
     uint64_t scale = 1;
     if (max_src <= 1) {
         // nothing is combined: any type is moved as bytes
@@ -549,6 +558,7 @@ int launch_batch(const DeviceCtx *ctx, const Batch &b, const char *d_table, hipS
     l.nseg = static_cast<uint32_t>(b.nseg());
     l.total_tiles = b.total_tiles;
     l.grid = grid_for(ctx, b.total_tiles);
+    l.wide_unroll = b.wide_unroll;
     l.stream = stream;
     hipError_t e;
     if (b.copy) {

@@ -29,6 +29,9 @@ struct DeviceCtx {
     // Chain folds whose largest fan-in reaches this go to the wide chain kernel (HCCLX_WIDE_CHAIN_FROM); with 9 to
     // 16 sources it measured 2 to 8 % faster than the kernel that holds all sources in registers, with 8 the same.
     uint32_t wide_chain_from = 9;
+    // The same for chains with a single destination (HCCLX_WIDE_CHAIN_FROM_ONE_DST): there the wide kernel moves
+    // four vectors per thread, and an 8-source ReduceScatter measured 5 % faster on it.
+    uint32_t wide_chain_from_one_dst = 5;
     uint32_t a2av_direct_unroll = 2;   // HCCLX_A2AV_DIRECT: 0 = off, 1 / 2 / 4 = vectors per thread and tile
     // V kernels whose tables live on the device cannot know their tile count on the host and run as a
     // persistent grid of this many workgroups per CU.

@@ -25,16 +25,13 @@ namespace hcclx {
 #endif
 constexpr int kFoldThreads = HCCLX_FOLD_THREADS;
 // The wide kernels: vectors per thread and tile, and sources loaded before they are folded in.
-// Two vectors per thread with eight sources in flight measured 24 % faster on a 32-rank AllReduce than one
-// vector with sixteen (the same loads outstanding, twice the contiguous run per source).
-#ifndef HCCLX_WIDE_UNROLL
-#define HCCLX_WIDE_UNROLL 2
-#endif
-#ifndef HCCLX_WIDE_GROUP
-#define HCCLX_WIDE_GROUP 8
-#endif
-constexpr int kWideUnroll = HCCLX_WIDE_UNROLL;
-constexpr int kWideGroup = HCCLX_WIDE_GROUP;
+// The wide chain kernel loads eight sources at a time for U vectors per thread.  U = 2 measured 24 % faster on a
+// 32-rank AllReduce than one vector with sixteen sources (the same loads outstanding, twice the contiguous run per
+// source); with a single destination (the ReduceScatter shape) U = 4 measured another 3 to 5 % faster, while it
+// costs 5 % where every result is written to many places.
+constexpr int kWideGroup = 8;
+constexpr int kWideUnrollMany = 2;   // several destinations
+constexpr int kWideUnrollOne = 4;    // one destination
 constexpr uint32_t kFoldDirectSegs = 64;   // up to this many segments the tile prefix is searched in place
 __host__ __device__ constexpr int fold_unroll(int maxn)
 {
@@ -45,10 +42,11 @@ __host__ __device__ constexpr uint64_t fold_tile_vecs(int maxn)
 {
     return static_cast<uint64_t>(kFoldThreads) * fold_unroll(maxn);
 }
-// Tiles of the wide kernels: the chain walks kWideUnroll vectors per thread, the self-first and tree orders one.
-__host__ __device__ constexpr uint64_t wide_tile_vecs(int mode)
+// Tiles of the wide kernels: `unroll` vectors per thread (the chain: kWideUnrollMany or kWideUnrollOne; the
+// self-first and tree orders: 1).
+__host__ __device__ constexpr uint64_t wide_tile_vecs(int unroll)
 {
-    return static_cast<uint64_t>(kFoldThreads) * (mode == 0 ? kWideUnroll : 1);
+    return static_cast<uint64_t>(kFoldThreads) * unroll;
 }
 
 #ifndef HCCLX_NT_LOAD
@@ -336,14 +334,13 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
 // More than kMaxFan sources or destinations, chain order: the sources are walked in groups of kMaxFan,
 // each group loaded before it is folded in, so the loads in flight per thread stay what the 16-source kernel
 // has.  One vector per thread and tile.
-template <int DT, int OP, bool CHECK>
+template <int DT, int OP, int U, bool CHECK>
 __device__ __forceinline__ void fold_tile_wide(const SegWide &sd, uint32_t nsrc, uint32_t ndst, uint64_t v0, uint64_t nvec,
                                                uint32_t head_bytes)
 {
     using V = Vec16<DT>;
     using C = typename V::C;
     constexpr int NE = V::NE;
-    constexpr int U = kWideUnroll;
     constexpr int G = kWideGroup;
     bool ok[U];
     uint64_t off[U];
@@ -518,12 +515,13 @@ __device__ __forceinline__ void fold_tile_wide_self(const SegWide &sd, uint32_t 
     }
 }
 
-template <int DT, int OP, int MODE>
+template <int DT, int OP, int MODE, int U>
 __global__ void __launch_bounds__(kFoldThreads)
 k_fold_wide(const uint64_t *__restrict__ tile_end, const SegWide *__restrict__ segs, uint32_t nseg, uint64_t total_tiles)
 {
     constexpr int NE = Vec16<DT>::kElems;
-    constexpr uint64_t TV = wide_tile_vecs(MODE);
+    static_assert(MODE == kFoldChain || U == 1, "only the chain moves several vectors per thread");
+    constexpr uint64_t TV = wide_tile_vecs(U);
     extern __shared__ uint64_t s_end[];
     const bool direct = nseg <= kFoldDirectSegs;
     if (!direct) {
@@ -552,7 +550,7 @@ k_fold_wide(const uint64_t *__restrict__ tile_end, const SegWide *__restrict__ s
             } else if constexpr (MODE == kFoldSelfFirst) {
                 fold_tile_wide_self<DT, OP, false>(sd, nsrc, v, nvec, head_bytes);
             } else {
-                fold_tile_wide<DT, OP, false>(sd, nsrc, ndst, v, nvec, head_bytes);
+                fold_tile_wide<DT, OP, U, false>(sd, nsrc, ndst, v, nvec, head_bytes);
             }
         } else {
             if constexpr (MODE == kFoldTree) {
@@ -560,7 +558,7 @@ k_fold_wide(const uint64_t *__restrict__ tile_end, const SegWide *__restrict__ s
             } else if constexpr (MODE == kFoldSelfFirst) {
                 fold_tile_wide_self<DT, OP, true>(sd, nsrc, v, nvec, head_bytes);
             } else {
-                fold_tile_wide<DT, OP, true>(sd, nsrc, ndst, v, nvec, head_bytes);
+                fold_tile_wide<DT, OP, U, true>(sd, nsrc, ndst, v, nvec, head_bytes);
             }
             if (tl == (nvec + shift) / TV && threadIdx.x < head + rem) {
                 const uint64_t idx = threadIdx.x < head ? threadIdx.x : head + nvec * NE + (threadIdx.x - head);
@@ -609,6 +607,7 @@ struct FoldLaunch {
     uint32_t nseg;
     uint64_t total_tiles;
     uint32_t grid;
+    int wide_unroll;           // the wide chain kernel: vectors per thread (kWideUnrollMany or kWideUnrollOne)
     hipStream_t stream;
 };
 

@@ -15,12 +15,23 @@ static hipError_t launch_one(const FoldLaunch &l)
     return hipGetLastError();
 }
 
+template <int DT, int OP, int MODE, int U>
+static hipError_t launch_wide_u(const FoldLaunch &l)
+{
+    hipLaunchKernelGGL((k_fold_wide<DT, OP, MODE, U>), dim3(l.grid), dim3(kFoldThreads), l.nseg * sizeof(uint64_t), l.stream,
+                       l.tile_end, static_cast<const SegWide *>(l.segs), l.nseg, l.total_tiles);
+    return hipGetLastError();
+}
+
 template <int DT, int OP, int MODE>
 static hipError_t launch_wide(const FoldLaunch &l)
 {
-    hipLaunchKernelGGL((k_fold_wide<DT, OP, MODE>), dim3(l.grid), dim3(kFoldThreads), l.nseg * sizeof(uint64_t), l.stream,
-                       l.tile_end, static_cast<const SegWide *>(l.segs), l.nseg, l.total_tiles);
-    return hipGetLastError();
+    if constexpr (MODE == kFoldChain) {
+        return l.wide_unroll == kWideUnrollOne ? launch_wide_u<DT, OP, MODE, kWideUnrollOne>(l)
+                                               : launch_wide_u<DT, OP, MODE, kWideUnrollMany>(l);
+    } else {
+        return launch_wide_u<DT, OP, MODE, 1>(l);
+    }
 }
 
 #ifdef HCCLX_COPY
