@@ -208,6 +208,7 @@ struct Batch {
     std::vector<SegDev> segs;
     std::vector<SegWide> wide;   // instead of segs when maxn == kMaxWideFan
     int wide_unroll = 1;         // vectors per thread of the wide kernel
+    uint32_t xcd_remap = 0;      // wide kernels: contiguous tile ranges per XCD (pays with 16 or more destinations)
     size_t nseg() const { return segs.size() + wide.size(); }
     size_t bytes() const
     {
@@ -481,6 +482,7 @@ int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, i
     uint32_t max_dst = 0;
     for (uint32_t i = 0; i < nseg; ++i) max_dst = segs[i].ndst > max_dst ? segs[i].ndst : max_dst;
     proto.wide_unroll = proto.mode != HCCLX_FOLD_CHAIN ? 1 : max_dst <= 1 ? kWideUnrollOne : kWideUnrollMany;
+    proto.xcd_remap = max_dst >= 16 ? 1u : 0u;
     const uint64_t tile_vecs = wide_tile_vecs(proto.wide_unroll);
     uint64_t scale = 1;
     if (max_src <= 1) {
@@ -559,6 +561,7 @@ int launch_batch(const DeviceCtx *ctx, const Batch &b, const char *d_table, hipS
     l.total_tiles = b.total_tiles;
     l.grid = grid_for(ctx, b.total_tiles);
     l.wide_unroll = b.wide_unroll;
+    l.xcd_remap = b.xcd_remap;
     l.stream = stream;
     hipError_t e;
     if (b.copy) {
