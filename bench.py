@@ -326,7 +326,7 @@ class MoeDispatchPack(Workload):
             what = "AlltoAllV back + combine in one pass" if self.combine else "route + pack + AlltoAllV in one pass"
         else:
             what = "moe combine (top-1)" if self.combine else "moe route + pack"
-        return {"algorithm": what, "fused": True, "launches": 1 if self.combine else 5, "plan_cache_hit": False}
+        return {"algorithm": what, "fused": True, "launches": 1 if self.combine else 4, "plan_cache_hit": False}
 
 
 class CopyCalibration(Workload):

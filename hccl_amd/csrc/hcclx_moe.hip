@@ -106,25 +106,22 @@ k_moe_scan(uint32_t n, uint32_t chunks, uint64_t row_elems, uint32_t *base, uint
     }
 }
 
-// rdispls[j][i] = what ranks 0 .. i-1 send to rank j.
-__global__ void __launch_bounds__(kMoeMaxRanks)
-k_moe_rdispls(uint32_t n, const uint64_t *send_counts, uint64_t *rdispls)
-{
-    const uint32_t j = threadIdx.x;
-    if (j >= n) return;
-    uint64_t run = 0;
-    for (uint32_t i = 0; i < n; ++i) {
-        rdispls[j * n + i] = run;
-        run += send_counts[i * n + j];
-    }
-}
-
 // perm[e] = first row of the destination's group + entries of earlier chunks with that destination + rank of
 // e among the entries of its own chunk with that destination (index order: the grouping is stable).
 __global__ void __launch_bounds__(kMoeChunk)
 k_moe_perm(MoeConstPtrs dest, MoePtrs perm, uint32_t n, uint32_t entries, uint32_t chunks, const uint32_t *base,
-           const uint32_t *row_start)
+           const uint32_t *row_start, const uint64_t *send_counts, uint64_t *rdispls)
 {
+    // one workgroup also writes rdispls[j][i] = what ranks 0 .. i-1 send to rank j (the send counts are complete:
+    // the scan kernel ran before this one)
+    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x < n) {
+        const uint32_t j = threadIdx.x;
+        uint64_t run = 0;
+        for (uint32_t i = 0; i < n; ++i) {
+            rdispls[j * n + i] = run;
+            run += send_counts[i * n + j];
+        }
+    }
     __shared__ uint32_t s_cnt[4][kMoeMaxRanks];
     const uint32_t c = blockIdx.x;
     const uint32_t i = blockIdx.y;
@@ -468,9 +465,8 @@ int hcclx_moe_route(const int32_t *const *dest, uint32_t n, uint32_t entries, ui
     hipLaunchKernelGGL(k_moe_hist, dim3(chunks, n), dim3(kMoeChunk), 0, st, d, n, entries, chunks, base);
     hipLaunchKernelGGL(k_moe_scan, dim3(n), dim3(256), 0, st, n, chunks, row_elems, base, row_start, send_counts, sdispls,
                        recv_counts);
-    hipLaunchKernelGGL(k_moe_rdispls, dim3(1), dim3(kMoeMaxRanks), 0, st, n, send_counts, rdispls);
     hipLaunchKernelGGL(k_moe_perm, dim3(chunks, n), dim3(kMoeChunk), 0, st, d, as_mutable(p), n, entries, chunks, base,
-                       row_start);
+                       row_start, send_counts, rdispls);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail_hip(e, "moe routing kernels");
     return HCCL_SUCCESS;
