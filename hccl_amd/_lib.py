@@ -74,6 +74,8 @@ def load():
     lib.hcclx_plan_destroy.argtypes = [ctypes.c_void_p]
     lib.hcclx_plan_bytes.restype = ctypes.c_uint64
     lib.hcclx_plan_bytes.argtypes = [ctypes.c_void_p]
+    lib.hcclx_plan_table_bytes.restype = ctypes.c_uint64
+    lib.hcclx_plan_table_bytes.argtypes = [ctypes.c_void_p]
     lib.hcclx_alltoallv.restype = ctypes.c_int
     lib.hcclx_alltoallv.argtypes = [vpp, vpp, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32,
                                     ctypes.c_int, ctypes.c_int, ctypes.c_void_p]

@@ -592,6 +592,7 @@ using namespace hcclx;
 struct hcclx_plan {
     int device = -1;
     char *d_table = nullptr;
+    uint64_t table_bytes = 0;
     uint64_t algo_bytes = 0;
     std::vector<Batch> batches;
     std::vector<size_t> offsets;
@@ -631,6 +632,7 @@ static int plan_from(DeviceCtx *ctx, Built &built, hcclx_plan_t **plan)
         p->offsets.push_back(total);
         total += b.bytes();
     }
+    p->table_bytes = total;
     if (total != 0) {
         std::vector<char> host(total);
         for (size_t i = 0; i < p->batches.size(); ++i) fill_table(p->batches[i], host.data() + p->offsets[i]);
@@ -713,5 +715,7 @@ int hcclx_plan_destroy(hcclx_plan_t *plan)
 }
 
 uint64_t hcclx_plan_bytes(const hcclx_plan_t *plan) { return plan ? plan->algo_bytes : 0; }
+
+uint64_t hcclx_plan_table_bytes(const hcclx_plan_t *plan) { return plan ? plan->table_bytes : 0; }
 
 }  // extern "C"

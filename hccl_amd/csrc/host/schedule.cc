@@ -855,27 +855,87 @@ void DropPlans(std::vector<hcclx_plan *> &plans)
     plans.clear();
 }
 
-// Launches a freshly built plan and, when it has a key, keeps it for the next identical collective (the least
-// recently used of 32 makes room).  A plan that is not kept is destroyed once its kernels have finished.
+u64 HashKey(const std::vector<u64> &key)
+{
+    u64 h = 1469598103934665603ull;   // FNV-1a over the words
+    for (u64 w : key) {
+        h ^= w;
+        h *= 1099511628211ull;
+    }
+    return h;
+}
+
+// Frees the retired plans whose kernels have finished.
+void ReapRetired(PlanCache &cache, bool wait)
+{
+    size_t kept = 0;
+    for (RetiredPlan &r : cache.retired) {
+        hipEvent_t ev = static_cast<hipEvent_t>(r.event);
+        bool done = (ev == nullptr);
+        if (!done) {
+            done = wait ? (hipEventSynchronize(ev) == hipSuccess) : (hipEventQuery(ev) == hipSuccess);
+        }
+        if (done) {
+            if (ev) (void)hipEventDestroy(ev);
+            DropPlans(r.plans);
+        } else {
+            cache.retired[kept++] = std::move(r);
+        }
+    }
+    cache.retired.resize(kept);
+}
+
+CachedPlan *FindPlan(PlanCache &cache, const std::vector<u64> &key)
+{
+    auto range = cache.index.equal_range(HashKey(key));
+    for (auto it = range.first; it != range.second; ++it) {
+        if (it->second->key == key) {
+            cache.lru.splice(cache.lru.begin(), cache.lru, it->second);   // most recently used first
+            return &*it->second;
+        }
+    }
+    return nullptr;
+}
+
+// Launches a freshly built plan and, when it has a key, keeps it for the next identical collective.  A plan that
+// is not kept is destroyed once its kernels have finished.
 HcclResult LaunchAndKeep(World *w, CachedPlan &&c, void *stream)
 {
+    PlanCache &cache = w->planCache;
     const HcclResult res = LaunchPlans(w, c.plans, stream);
-    if (!c.key.empty() && res == HCCL_SUCCESS) {
-        c.lastUse = ++w->useCounter;
-        if (w->planCache.size() >= 32) {
-            size_t victim = 0;
-            for (size_t i = 1; i < w->planCache.size(); ++i) {
-                if (w->planCache[i].lastUse < w->planCache[victim].lastUse) victim = i;
-            }
-            // its kernels may still be queued: wait for the device before the tables are freed
-            (void)hipDeviceSynchronize();
-            DropPlans(w->planCache[victim].plans);
-            w->planCache.erase(w->planCache.begin() + victim);
-        }
-        w->planCache.push_back(std::move(c));
-    } else {
+    if (c.key.empty() || res != HCCL_SUCCESS) {
         (void)hipDeviceSynchronize();
         DropPlans(c.plans);
+        return res;
+    }
+    c.lastStream = stream;
+    c.tableBytes = 0;
+    for (hcclx_plan *p : c.plans) c.tableBytes += hcclx_plan_table_bytes(p);
+    cache.bytes += c.tableBytes;
+    cache.lru.push_front(std::move(c));
+    cache.index.emplace(HashKey(cache.lru.front().key), cache.lru.begin());
+    while (cache.lru.size() > 1 && (cache.lru.size() > kPlanCacheEntries || cache.bytes > kPlanCacheBytes)) {
+        auto victim = std::prev(cache.lru.end());
+        auto range = cache.index.equal_range(HashKey(victim->key));
+        for (auto it = range.first; it != range.second; ++it) {
+            if (it->second == victim) {
+                cache.index.erase(it);
+                break;
+            }
+        }
+        RetiredPlan r;
+        r.plans = std::move(victim->plans);
+        hipEvent_t ev = nullptr;
+        if (!victim->manyStreams && hipEventCreateWithFlags(&ev, hipEventDisableTiming) == hipSuccess &&
+            hipEventRecord(ev, static_cast<hipStream_t>(victim->lastStream)) == hipSuccess) {
+            r.event = ev;
+        } else {
+            if (ev) (void)hipEventDestroy(ev);
+            (void)hipDeviceSynchronize();   // no single event covers it: make sure nothing still reads the tables
+        }
+        cache.bytes -= victim->tableBytes;
+        cache.lru.erase(victim);
+        cache.retired.push_back(std::move(r));
     }
     return res;
 }
@@ -1043,14 +1103,14 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
     if (!w->dryRun && !w->traceText && !w->check) {
         key = PlanKey(params, algName, w->cclBytes);
         key.push_back(fused ? 1 : 0);
-        for (CachedPlan &c : w->planCache) {
-            if (c.key == key) {
-                c.lastUse = ++w->useCounter;
-                w->lastWasFused = c.fused;
-                w->lastLevels = c.levels;
-                w->lastPlanCacheHit = true;
-                return LaunchPlans(w, c.plans, stream);
-            }
+        if (!w->planCache.retired.empty()) ReapRetired(w->planCache, false);
+        if (CachedPlan *c = FindPlan(w->planCache, key)) {
+            if (c->lastStream != stream) c->manyStreams = true;
+            c->lastStream = stream;
+            w->lastWasFused = c->fused;
+            w->lastLevels = c->levels;
+            w->lastPlanCacheHit = true;
+            return LaunchPlans(w, c->plans, stream);
         }
     }
 

@@ -71,7 +71,12 @@ World::~World()
     for (char *p : cclBuf) {
         if (p && !dryRun) (void)hipFree(p);
     }
-    for (CachedPlan &c : planCache) {
+    if (!dryRun && (!planCache.lru.empty() || !planCache.retired.empty())) (void)hipDeviceSynchronize();
+    for (RetiredPlan &r : planCache.retired) {
+        if (r.event) (void)hipEventDestroy(static_cast<hipEvent_t>(r.event));
+        for (hcclx_plan *p : r.plans) (void)hcclx_plan_destroy(p);
+    }
+    for (CachedPlan &c : planCache.lru) {
         for (hcclx_plan *p : c.plans) (void)hcclx_plan_destroy(p);
     }
 }

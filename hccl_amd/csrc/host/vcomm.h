@@ -6,8 +6,9 @@
 // and the recorded steps are launched on the GPU (schedule.h).
 #pragma once
 #include <condition_variable>
-#include <map>
 #include <deque>
+#include <list>
+#include <map>
 #include <memory>
 #include <mutex>
 #include <unordered_map>
@@ -70,9 +71,28 @@ struct QueuedOp {
 struct CachedPlan {
     std::vector<u64> key;
     std::vector<hcclx_plan *> plans;   // launched in this order
-    u64 lastUse = 0;
     bool fused = true;                 // false: the recorded steps, one or two plans per level
     u32 levels = 0;
+    u64 tableBytes = 0;                // device memory of the plans' tables
+    void *lastStream = nullptr;        // where it was launched last
+    bool manyStreams = false;          // it has been launched on more than one stream
+};
+
+// Plans of the collectives a world has run, most recently used first, found through a hash of the key.  What
+// falls out at the far end (more than kPlanCacheEntries plans, or more than kPlanCacheBytes of tables) is not
+// destroyed at once -- its kernels may still be queued -- but retired behind an event on its stream and freed
+// when a later collective finds that event complete.
+constexpr size_t kPlanCacheEntries = 1024;
+constexpr u64 kPlanCacheBytes = 256ull << 20;
+struct RetiredPlan {
+    std::vector<hcclx_plan *> plans;
+    void *event = nullptr;             // hipEvent_t
+};
+struct PlanCache {
+    std::list<CachedPlan> lru;
+    std::unordered_multimap<u64, std::list<CachedPlan>::iterator> index;
+    std::vector<RetiredPlan> retired;
+    u64 bytes = 0;
 };
 
 // What the schedule check found in the last collective (see hcclxCommSetCheck).
@@ -120,8 +140,7 @@ struct World {
     bool check = false;     // verify every schedule before it is launched
     CheckReport lastCheck;
 
-    std::vector<CachedPlan> planCache;
-    u64 useCounter = 0;
+    PlanCache planCache;
 
     // configuration
     std::map<int, std::string> forcedAlg;  // per HcclCMDType; empty = selector decides

@@ -79,6 +79,10 @@ class Plan:
     def bytes(self):
         return _lib.load().hcclx_plan_bytes(self._h)
 
+    @property
+    def table_bytes(self):
+        return _lib.load().hcclx_plan_table_bytes(self._h)
+
     def launch(self, stream=0):
         check(_lib.load().hcclx_plan_launch(self._h, ctypes.c_void_p(stream)))
 

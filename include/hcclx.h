@@ -106,6 +106,8 @@ int hcclx_plan_launch(const hcclx_plan_t *plan, void *stream);
 int hcclx_plan_destroy(hcclx_plan_t *plan);
 /* Algorithmic bytes one launch of the plan moves: sum over segments of (nsrc + ndst) * count * size. */
 uint64_t hcclx_plan_bytes(const hcclx_plan_t *plan);
+/* Bytes of device memory the plan's launch tables occupy. */
+uint64_t hcclx_plan_table_bytes(const hcclx_plan_t *plan);
 
 /* AlltoAllV among n virtual ranks whose buffers live in this GPU.
  *   send[i], recv[i]      device base pointers of rank i                               (host arrays, n)

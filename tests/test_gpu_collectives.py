@@ -500,3 +500,33 @@ def test_ranks_on_different_streams_and_threads():
             assert_same_bits(recv[r].get(np.float32), want[r], T.FP32, f"rank {r}")
     finally:
         w.close()
+
+
+def test_plan_cache_keeps_a_thousand_shapes_and_retires_the_oldest(stream):
+    """1100 different counts on one communicator (a training step has that many bucket sizes): the most recent
+    1024 plans stay cached, older ones are retired without stalling the device, and a retired shape is simply
+    planned again."""
+    n = 2
+    base = np.arange(1200, dtype=np.float32)
+    xs = [base + 1, base * 2]
+    w = api.World(n)
+    try:
+        send = [DevBuf(x) for x in xs]
+        recv = [DevBuf(nbytes=base.nbytes) for _ in range(n)]
+        torch.cuda.synchronize()
+
+        def run(count):
+            for r in range(n):
+                assert w.all_reduce(r, send[r].ptr, recv[r].ptr, count, T.FP32, T.SUM, stream.cuda_stream) == 0
+            return w.last_info().planCacheHit
+
+        for count in range(1, 1101):
+            assert run(count) == 0
+        assert run(1100) == 1 and run(77) == 1          # the newest 1024 are counts 77 .. 1100
+        assert run(76) == 0 and run(1) == 0             # retired; planned again
+        assert run(500) == 1
+        stream.synchronize()
+        got = recv[0].get(np.float32)
+        assert np.array_equal(got[:500], (xs[0] + xs[1])[:500])
+    finally:
+        w.close()
