@@ -33,11 +33,13 @@ def test_every_declared_function_is_exported():
                      "HcclAlltoAll", "HcclAlltoAllV", "HcclAlltoAllVC", "HcclCommInitAll", "hcclxCommInitAll",
                      "hcclxCommSetCheck", "HcommLocalCopyOnThread", "HcommLocalReduceOnThread", "HcommWriteReduceOnThread",
                      "HcommChannelNotifyWaitOnThread", "HcommThreadJoin", "hcclx_fold", "hcclx_plan_create",
-                     "hcclx_alltoallv", "hcclx_allgatherv", "hcclx_moe_route", "hcclx_moe_pack", "hcclx_moe_combine"):
+                     "hcclx_alltoallv", "hcclx_allgatherv", "hcclx_moe_route", "hcclx_moe_pack", "hcclx_moe_combine",
+                     "hcclx_fold_wide", "hcclx_plan_create_wide", "hcclx_plan_table_bytes", "hcclx_moe_dispatch",
+                     "hcclx_moe_gather_combine"):
         assert expected in names, f"{expected} is not declared in include/"
     missing = [f"{n} ({h})" for n, h in sorted(names.items()) if not hasattr(lib, n)]
     assert not missing, "declared but not exported: " + ", ".join(missing)
-    assert len(names) >= 45
+    assert len(names) >= 50
 
 
 C_PROGRAM = r'''
@@ -69,6 +71,15 @@ int main(void)
     hcclxCommGetLastTrace(comm[0], trace, sizeof(trace));
     printf("%s fused=%d steps=%u races=%u semantic=%u\n%.60s\n", info.algName, info.fused, rep.steps, rep.races, rep.semanticErrors, trace);
     if (HcclAllReduce(0, 0, 1000, HCCL_DATA_TYPE_FP32, HCCL_REDUCE_SUM, comm[0], (aclrtStream)1) != HCCL_E_PTR) return 5;
+    {
+        /* the kernel layer's structures as a C caller fills them; without a GPU the call reports an error */
+        hcclx_wide_seg_t wide = {0};
+        hcclx_seg_t seg = {0};
+        wide.count = 4; wide.nsrc = 20; wide.ndst = 1;
+        seg.count = 4; seg.nsrc = 2; seg.ndst = 1;
+        if (sizeof(wide.src) / sizeof(wide.src[0]) != HCCLX_MAX_WIDE_FAN || sizeof(seg.dst) / sizeof(seg.dst[0]) != HCCLX_MAX_FAN) return 7;
+        if (hcclx_plan_table_bytes(0) != 0 || hcclx_plan_bytes(0) != 0) return 8;
+    }
     for (int r = 0; r < 4; ++r) HcclCommDestroy(comm[r]);
     return (rep.races == 0 && rep.semanticErrors == 0) ? 0 : 6;
 }
