@@ -530,3 +530,31 @@ def test_plan_cache_keeps_a_thousand_shapes_and_retires_the_oldest(stream):
         assert np.array_equal(got[:500], (xs[0] + xs[1])[:500])
     finally:
         w.close()
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_a_communicator_of_one_rank(stream, mode):
+    """Every collective among one rank is a copy of the input (or nothing, in place)."""
+    count = 10007
+    x = np.arange(count, dtype=np.float32) - 5000
+    w = api.World(1, ccl_bytes=SMALL_CCL)
+    try:
+        w.set_mode(mode)
+        send = DevBuf(x)
+        for call in ("all_reduce", "reduce_scatter", "all_gather", "all_to_all", "in_place"):
+            recv = send if call == "in_place" else DevBuf(nbytes=x.nbytes)
+            torch.cuda.synchronize()
+            if call in ("all_reduce", "in_place"):
+                rc = w.all_reduce(0, send.ptr, recv.ptr, count, T.FP32, T.SUM, stream.cuda_stream)
+            elif call == "reduce_scatter":
+                rc = w.reduce_scatter(0, send.ptr, recv.ptr, count, T.FP32, T.MAX, stream.cuda_stream)
+            elif call == "all_gather":
+                rc = w.all_gather(0, send.ptr, recv.ptr, count, T.FP32, stream.cuda_stream)
+            else:
+                rc = w.all_to_all(0, send.ptr, count, recv.ptr, T.FP32, stream.cuda_stream)
+            assert rc == 0, call
+            stream.synchronize()
+            assert np.array_equal(recv.get(np.float32), x), call
+            assert recv.guard_intact(), call
+    finally:
+        w.close()
