@@ -12,6 +12,11 @@
  * events).  With one host thread driving all ranks the calls behave like a group: use the outputs after
  * the last rank's call.  With one host thread per rank set blocking mode, so that a call returns only
  * after the launch and the caller's later work on its stream is ordered after the collective.
+ *
+ * The first collective of a given kind (op, algorithm, type, count, buffers, mode) records the ranks' templates,
+ * plans the launch and keeps the plan (up to 1024 plans or 256 MiB of launch tables per communicator, least
+ * recently used out first); repeats only launch kernels -- no allocation, no copy -- and may therefore be issued
+ * on a stream that is being captured into a HIP graph.
  */
 #ifndef HCCL_AMD_HCCL_COMM_H_
 #define HCCL_AMD_HCCL_COMM_H_
