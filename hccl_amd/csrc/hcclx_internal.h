@@ -32,6 +32,9 @@ struct DeviceCtx {
     // The same for chains with a single destination (HCCLX_WIDE_CHAIN_FROM_ONE_DST): there the wide kernel moves
     // four vectors per thread, and an 8-source ReduceScatter measured 5 % faster on it.
     uint32_t wide_chain_from_one_dst = 5;
+    // Wide launches whose segments have this many destinations give each XCD a contiguous eighth of the tiles
+    // (HCCLX_WIDE_XCD_REMAP_FROM).
+    uint32_t wide_xcd_remap_from = 16;
     uint32_t a2av_direct_unroll = 2;   // HCCLX_A2AV_DIRECT: 0 = off, 1 / 2 / 4 = vectors per thread and tile
     // V kernels whose tables live on the device cannot know their tile count on the host and run as a
     // persistent grid of this many workgroups per CU.
