@@ -79,6 +79,9 @@ def load():
     lib.hcclx_alltoallv.restype = ctypes.c_int
     lib.hcclx_alltoallv.argtypes = [vpp, vpp, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32,
                                     ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    lib.hcclx_alltoallv_plan_create.restype = ctypes.c_int
+    lib.hcclx_alltoallv_plan_create.argtypes = [vpp, vpp, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32,
+                                                ctypes.c_int, ctypes.POINTER(ctypes.c_void_p)]
     lib.hcclx_moe_workspace_bytes.restype = ctypes.c_uint64
     lib.hcclx_moe_workspace_bytes.argtypes = [ctypes.c_uint32, ctypes.c_uint32]
     lib.hcclx_moe_route.restype = ctypes.c_int

@@ -2,6 +2,7 @@
 #include "hcclx.h"
 #include "hcclx_internal.h"
 #include "kernels/fold.h"
+#include "kernels/vops.h"
 
 #include <cstdlib>
 #include <cstring>
@@ -210,9 +211,12 @@ struct Batch {
     std::vector<SegWide> wide;   // instead of segs when maxn == kMaxWideFan
     int wide_unroll = 1;         // vectors per thread of the wide kernel
     uint32_t xcd_remap = 0;      // wide kernels: contiguous tile ranges per XCD (pays with 16 or more destinations)
+    std::vector<CopyBlock> blocks;   // instead of everything above: a list of blocks for the block copy kernel
+    int block_unroll = 2;
     size_t nseg() const { return segs.size() + wide.size(); }
     size_t bytes() const
     {
+        if (!blocks.empty()) return blocks.size() * sizeof(CopyBlock);
         return align256(tile_end.size() * 8) + segs.size() * sizeof(SegDev) + wide.size() * sizeof(SegWide);
     }
     static size_t align256(size_t x) { return (x + 255) & ~static_cast<size_t>(255); }
@@ -548,6 +552,10 @@ int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, i
 
 void fill_table(const Batch &b, char *h)
 {
+    if (!b.blocks.empty()) {
+        std::memcpy(h, b.blocks.data(), b.blocks.size() * sizeof(CopyBlock));
+        return;
+    }
     std::memcpy(h, b.tile_end.data(), b.tile_end.size() * 8);
     char *at = h + Batch::align256(b.tile_end.size() * 8);
     if (!b.segs.empty()) std::memcpy(at, b.segs.data(), b.segs.size() * sizeof(SegDev));
@@ -556,6 +564,12 @@ void fill_table(const Batch &b, char *h)
 
 int launch_batch(const DeviceCtx *ctx, const Batch &b, const char *d_table, hipStream_t stream)
 {
+    if (!b.blocks.empty()) {
+        const hipError_t be = launch_copy_blocks(reinterpret_cast<const CopyBlock *>(d_table), static_cast<uint32_t>(b.blocks.size()),
+                                                 static_cast<uint32_t>(b.total_tiles), b.block_unroll, stream);
+        if (be != hipSuccess) return fail_hip(be, "block copy kernel launch");
+        return HCCL_SUCCESS;
+    }
     FoldLaunch l;
     l.tile_end = reinterpret_cast<const uint64_t *>(d_table);
     l.segs = d_table + Batch::align256(b.tile_end.size() * 8);
@@ -692,6 +706,30 @@ int hcclx_plan_create_wide(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtyp
     Built built;
     int rc = build_wide_batches(segs, nseg, dtype, op, mode, &built);
     if (rc != HCCL_SUCCESS) return rc;
+    return plan_from(ctx, built, plan);
+}
+
+int hcclx_alltoallv_plan_create(const void *const *send, void *const *recv, const uint64_t *send_counts,
+                                const uint64_t *sdispls, const uint64_t *rdispls, uint32_t n, int dtype, hcclx_plan_t **plan)
+{
+    if (plan == nullptr) return fail(HCCL_E_PTR, "plan is null");
+    *plan = nullptr;
+    DeviceCtx *ctx = device_ctx();
+    if (!ctx) return HCCL_E_RUNTIME;
+    const int esz = dtype_size(dtype);
+    if (esz == 0) return fail(HCCL_E_NOT_SUPPORT, "unknown data type " + std::to_string(dtype));
+    if (!send || !recv) return fail(HCCL_E_PTR, "send/recv pointer array is null");
+    if (!send_counts || !sdispls || !rdispls) return fail(HCCL_E_PTR, "count/displacement table is null");
+    if (n == 0 || n > kMaxVRanks) return fail(HCCL_E_PARA, "rank count outside 1.." + std::to_string(kMaxVRanks));
+    Built built;
+    Batch b;
+    b.copy = true;
+    b.block_unroll = ctx->a2av_direct_unroll == 1 ? 1 : ctx->a2av_direct_unroll == 4 ? 4 : 2;
+    b.total_tiles = list_alltoallv_blocks(send, recv, send_counts, sdispls, rdispls, n, static_cast<uint32_t>(esz), b.block_unroll,
+                                          &b.blocks);
+    if (b.total_tiles > 0x7fffffffull) return fail(HCCL_E_PARA, "too much data for one launch");
+    for (const CopyBlock &c : b.blocks) built.algo_bytes += 2 * c.bytes;
+    if (!b.blocks.empty()) built.batches.push_back(std::move(b));
     return plan_from(ctx, built, plan);
 }
 

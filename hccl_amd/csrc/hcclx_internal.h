@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <string>
+#include <vector>
 #include "hccl_types.h"
 
 namespace hcclx {
@@ -56,5 +57,12 @@ DeviceCtx *device_ctx();
 int ring_reserve(DeviceCtx *ctx, size_t bytes, hipStream_t stream, char **h, char **d);
 
 uint32_t grid_for(const DeviceCtx *ctx, uint64_t total_tiles);
+
+struct CopyBlock;
+// The non-empty blocks of an AlltoAllV with host tables (row-major n x n, elements of esz bytes), with the
+// inclusive prefix of their tiles of `unroll` vectors per thread; returns the number of tiles.
+uint64_t list_alltoallv_blocks(const void *const *send, void *const *recv, const uint64_t *send_counts,
+                               const uint64_t *sdispls, const uint64_t *rdispls, uint32_t n, uint32_t esz, int unroll,
+                               std::vector<CopyBlock> *blocks);
 
 }  // namespace hcclx

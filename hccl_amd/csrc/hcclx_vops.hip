@@ -46,6 +46,33 @@ int fill_ptrs(const void *const *send, void *const *recv, uint32_t n, VRankPtrs 
 
 }  // namespace
 
+namespace hcclx {
+
+uint64_t list_alltoallv_blocks(const void *const *send, void *const *recv, const uint64_t *send_counts,
+                               const uint64_t *sdispls, const uint64_t *rdispls, uint32_t n, uint32_t esz, int unroll,
+                               std::vector<CopyBlock> *blocks)
+{
+    blocks->clear();
+    blocks->reserve(static_cast<size_t>(n) * n);
+    uint64_t tiles = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        for (uint32_t j = 0; j < n; ++j) {
+            const uint64_t bytes = send_counts[i * n + j] * esz;
+            if (bytes == 0) continue;
+            CopyBlock b;
+            b.src = static_cast<const char *>(send[i]) + sdispls[i * n + j] * esz;
+            b.dst = static_cast<char *>(recv[j]) + rdispls[j * n + i] * esz;
+            b.bytes = bytes;
+            tiles += v_tiles_of(bytes, reinterpret_cast<uint64_t>(b.dst), unroll);
+            b.tile_end = tiles;
+            blocks->push_back(b);
+        }
+    }
+    return tiles;
+}
+
+}  // namespace hcclx
+
 extern "C" {
 
 int hcclx_alltoallv(const void *const *send, void *const *recv, const uint64_t *send_counts,
@@ -100,21 +127,8 @@ int hcclx_alltoallv(const void *const *send, void *const *recv, const uint64_t *
         }
         // any other host table: the non-empty blocks as a list in device memory, one small tile per workgroup
         std::vector<CopyBlock> blocks;
-        blocks.reserve(static_cast<size_t>(n) * n);
-        uint64_t tiles = 0;
-        for (uint32_t i = 0; i < n; ++i) {
-            for (uint32_t j = 0; j < n; ++j) {
-                const uint64_t bytes = send_counts[i * n + j] * esz;
-                if (bytes == 0) continue;
-                CopyBlock b;
-                b.src = ptrs.send[i] + sdispls[i * n + j] * esz;
-                b.dst = ptrs.recv[j] + rdispls[j * n + i] * esz;
-                b.bytes = bytes;
-                tiles += v_tiles_of(bytes, reinterpret_cast<uint64_t>(b.dst), unroll);
-                b.tile_end = tiles;
-                blocks.push_back(b);
-            }
-        }
+        const uint64_t tiles = list_alltoallv_blocks(send, recv, send_counts, sdispls, rdispls, n, static_cast<uint32_t>(esz),
+                                                     unroll, &blocks);
         if (blocks.empty()) return HCCL_SUCCESS;
         if (tiles > 0x7fffffffull) return fail(HCCL_E_PARA, "too much data for one launch");
         char *h = nullptr;

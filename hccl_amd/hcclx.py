@@ -119,6 +119,20 @@ def alltoallv(send, recv, send_counts, sdispls, rdispls, dtype, on_device=False,
                                       1 if on_device else 0, ctypes.c_void_p(stream)))
 
 
+class AlltoAllVPlan(Plan):
+    """An AlltoAllV with host tables whose block list already sits in device memory: launch() is one kernel
+    launch with nothing copied in front of it."""
+
+    def __init__(self, send, recv, send_counts, sdispls, rdispls, dtype):
+        a, ka = _table(send_counts)
+        b, kb = _table(sdispls)
+        c, kc = _table(rdispls)
+        h = ctypes.c_void_p()
+        check(_lib.load().hcclx_alltoallv_plan_create(_ptr_array(send), _ptr_array(recv), a, b, c, len(send), int(dtype),
+                                                      ctypes.byref(h)))
+        self._h = h
+
+
 def allgatherv(send, recv, counts, displs, dtype, on_device=False, stream=0):
     n = len(send)
     a, ka = _table(counts)

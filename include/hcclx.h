@@ -120,6 +120,12 @@ int hcclx_alltoallv(const void *const *send, void *const *recv, const uint64_t *
                     const uint64_t *sdispls, const uint64_t *rdispls, uint32_t n, int dtype,
                     int tables_on_device, void *stream);
 
+/* The same AlltoAllV with host tables as a plan: the tables are read once and turned into a block list in device
+ * memory; hcclx_plan_launch then moves the data with no table travelling at launch time (a repeated exchange,
+ * or one that is captured into a HIP graph).  Launched, measured and destroyed like any other plan. */
+int hcclx_alltoallv_plan_create(const void *const *send, void *const *recv, const uint64_t *send_counts,
+                                const uint64_t *sdispls, const uint64_t *rdispls, uint32_t n, int dtype, hcclx_plan_t **plan);
+
 /* AllGatherV among n virtual ranks: recv[j][displs[i] .. displs[i]+counts[i]) = send[i][0 .. counts[i])
  * for every i and j; each source element is read once and written n times.  counts/displs as above. */
 int hcclx_allgatherv(const void *const *send, void *const *recv, const uint64_t *counts,

@@ -61,6 +61,53 @@ def test_alltoallv_odd_counts_and_misaligned_blocks():
         run_a2av(m, T.BFP16, rng)
 
 
+@pytest.mark.parametrize("n", [2, 8, 16, 24, 40, 64])
+def test_alltoallv_host_tables_of_any_rank_count_and_as_a_plan(n):
+    """Up to 15 ranks the tables ride in the kernel arguments; beyond, the non-empty blocks become a list in device
+    memory.  The same exchange as a plan moves new data at every launch, also from a captured graph."""
+    rng = np.random.default_rng(n)
+    m = rng.integers(0, 3000, size=(n, n))
+    m[rng.random((n, n)) < 0.3] = 0                     # empty blocks
+    m = m.tolist()
+    run_a2av(m, T.BFP16, rng, send_pad=2)
+    run_a2av(m, T.INT8, rng, send_pad=1)
+    v = [T.alltoallvc_to_v(m, r) for r in range(n)]
+    sc = np.array([x[0] for x in v], dtype=np.uint64).ravel()
+    sd = np.array([x[1] for x in v], dtype=np.uint64).ravel()
+    rd = np.array([x[3] for x in v], dtype=np.uint64).ravel()
+    send = [DevBuf(nbytes=max(1, sum(m[i])) * 4) for i in range(n)]
+    recv = [DevBuf(nbytes=max(1, sum(x[2])) * 4) for x in v]
+    plan = hcclx.AlltoAllVPlan([s.ptr for s in send], [r.ptr for r in recv], sc, sd, rd, T.FP32)
+    assert plan.bytes == 2 * 4 * int(sc.sum()) and plan.table_bytes > 0
+    stream = torch.cuda.Stream()
+    graph = None
+    for rep in range(4):
+        ins = [rng.integers(0, 2**32 - 1, size=max(1, sum(m[i])), dtype=np.uint32) for i in range(n)]
+        for i in range(n):
+            send[i].t[:ins[i].nbytes] = torch.from_numpy(ins[i].view(np.uint8).copy()).to("cuda:0")
+        for r in recv:
+            r.t.fill_(0xA5)
+        torch.cuda.synchronize()
+        if rep < 2:
+            plan.launch(stream.cuda_stream)
+        else:
+            if graph is None:
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.stream(stream):
+                    graph.capture_begin()
+                    plan.launch(stream.cuda_stream)
+                    graph.capture_end()
+            graph.replay()
+        torch.cuda.synchronize()
+        want = T.run_alltoallv([x[:sum(m[i])] for i, x in enumerate(ins)], [x[0] for x in v], [x[1] for x in v],
+                               [x[2] for x in v], [x[3] for x in v], [sum(x[2]) for x in v])
+        for j in range(n):
+            assert np.array_equal(recv[j].get(np.uint32)[:sum(v[j][2])], want[j]), (rep, j)
+            assert recv[j].guard_intact()
+    del graph
+    plan.close()
+
+
 def test_alltoallv_all_zero_and_single_rank():
     rng = np.random.default_rng(1)
     run_a2av([[0, 0], [0, 0]], T.FP32, rng)
