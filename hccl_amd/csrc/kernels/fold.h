@@ -24,7 +24,6 @@ namespace hcclx {
 #define HCCLX_FOLD_THREADS 256
 #endif
 constexpr int kFoldThreads = HCCLX_FOLD_THREADS;
-// The wide kernels: vectors per thread and tile, and sources loaded before they are folded in.
 // The wide chain kernel loads eight sources at a time for U vectors per thread.  U = 2 measured 24 % faster on a
 // 32-rank AllReduce than one vector with sixteen sources (the same loads outstanding, twice the contiguous run per
 // source); with a single destination (the ReduceScatter shape) U = 4 measured another 3 to 5 % faster, while it
