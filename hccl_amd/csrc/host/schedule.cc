@@ -480,6 +480,17 @@ struct FusedPlan {
     std::vector<hcclx_wide_seg_t> wideSegs;       // chains over more than HCCLX_MAX_FAN sources
     std::vector<hcclx_wide_seg_t> wideTreeSegs;   // trees with more leaves or levels than the 16-slot kernel holds
     std::vector<hcclx_wide_seg_t> wideSelfSegs;   // the per-rank orders of the one-shot templates among 17 .. 64 ranks
+    // The same in place (outputs overwrite inputs): the wide kernel computes its outputs sixteen at a time in
+    // different workgroups, so they go to a staging buffer first (dst[] hold byte offsets into it) and are copied
+    // to their places by a second launch.
+    struct StagedCopy {
+        u64 offset;
+        u64 dst;
+        u64 bytes;
+    };
+    std::vector<hcclx_wide_seg_t> stagedSelfSegs;
+    std::vector<StagedCopy> stagedCopies;
+    u64 stagingBytes = 0;
 };
 
 bool Overlaps(u64 a, u64 alen, u64 b, u64 blen) { return a < b + blen && b < a + alen; }
@@ -545,6 +556,7 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
         bySet[key].push_back(kv.second[0]);
     }
     std::vector<bool> taken(folds.size(), false);
+    std::vector<bool> staged(folds.size(), false);   // written by the second launch: cannot race with what the first reads
     std::vector<int> group(folds.size(), -1);
     for (auto &kv : bySet) {
         const std::vector<size_t> &grp = kv.second;
@@ -573,14 +585,13 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
             if (!ok) continue;
             if (n > HCCLX_MAX_FAN) {
                 // the wide kernel computes the outputs sixteen at a time in different workgroups, so none of
-                // them may overwrite a source (an in-place collective among more than 16 ranks is not grouped)
+                // them may overwrite a source: an in-place collective writes to a staging buffer first
                 bool clash = false;
                 for (size_t j = 0; j < n && !clash; ++j) {
                     for (size_t k = 0; k < n && !clash; ++k) {
                         clash = Overlaps(folds[owner[j]].dst, folds[owner[j]].bytes, base[k], folds[cand].bytes);
                     }
                 }
-                if (clash) break;
                 hcclx_wide_seg_t seg;
                 std::memset(&seg, 0, sizeof(seg));
                 seg.count = folds[cand].bytes / esz;
@@ -590,6 +601,16 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
                     seg.src[j] = reinterpret_cast<const void *>(base[j]);
                     seg.dst[j] = reinterpret_cast<void *>(folds[owner[j]].dst);
                     taken[owner[j]] = true;
+                    if (clash) {
+                        seg.dst[j] = reinterpret_cast<void *>(plan.stagingBytes);
+                        plan.stagedCopies.push_back({plan.stagingBytes, folds[owner[j]].dst, folds[owner[j]].bytes});
+                        plan.stagingBytes += (folds[owner[j]].bytes + 255) & ~static_cast<u64>(255);
+                        staged[owner[j]] = true;
+                    }
+                }
+                if (clash) {
+                    plan.stagedSelfSegs.push_back(seg);
+                    break;
                 }
                 plan.wideSelfSegs.push_back(seg);
                 break;
@@ -627,6 +648,7 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
         }
         std::sort(reads.begin(), reads.end(), [](const Read &x, const Read &y) { return x.addr < y.addr; });
         for (size_t i = 0; i < folds.size(); ++i) {
+            if (staged[i]) continue;
             // reads that can reach into [dst, dst + bytes) start after dst - longest
             const u64 from = folds[i].dst > longest ? folds[i].dst - longest : 0;
             auto it = std::lower_bound(reads.begin(), reads.end(), from,
@@ -849,10 +871,12 @@ HcclResult LaunchPlans(World *w, const std::vector<hcclx_plan *> &plans, void *s
     return HCCL_SUCCESS;
 }
 
-void DropPlans(std::vector<hcclx_plan *> &plans)
+void DropPlans(std::vector<hcclx_plan *> &plans, std::vector<void *> &buffers)
 {
     for (hcclx_plan *q : plans) (void)hcclx_plan_destroy(q);
     plans.clear();
+    for (void *b : buffers) (void)hipFree(b);
+    buffers.clear();
 }
 
 u64 HashKey(const std::vector<u64> &key)
@@ -877,7 +901,7 @@ void ReapRetired(PlanCache &cache, bool wait)
         }
         if (done) {
             if (ev) (void)hipEventDestroy(ev);
-            DropPlans(r.plans);
+            DropPlans(r.plans, r.buffers);
         } else {
             cache.retired[kept++] = std::move(r);
         }
@@ -905,7 +929,7 @@ HcclResult LaunchAndKeep(World *w, CachedPlan &&c, void *stream)
     const HcclResult res = LaunchPlans(w, c.plans, stream);
     if (c.key.empty() || res != HCCL_SUCCESS) {
         (void)hipDeviceSynchronize();
-        DropPlans(c.plans);
+        DropPlans(c.plans, c.buffers);
         return res;
     }
     c.lastStream = stream;
@@ -925,6 +949,7 @@ HcclResult LaunchAndKeep(World *w, CachedPlan &&c, void *stream)
         }
         RetiredPlan r;
         r.plans = std::move(victim->plans);
+        r.buffers = std::move(victim->buffers);
         hipEvent_t ev = nullptr;
         if (!victim->manyStreams && hipEventCreateWithFlags(&ev, hipEventDisableTiming) == hipSuccess &&
             hipEventRecord(ev, static_cast<hipStream_t>(victim->lastStream)) == hipSuccess) {
@@ -1156,7 +1181,8 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
                                        (w->traceText || w->dryRun) ? &w->lastTrace : nullptr);
         w->lastFusedSegments =
             static_cast<u32>(plan.chainSegs.size() + plan.selfSegs.size() + plan.copySegs.size() + plan.treeSegs.size() +
-                             plan.wideSegs.size() + plan.wideTreeSegs.size() + plan.wideSelfSegs.size());
+                             plan.wideSegs.size() + plan.wideTreeSegs.size() + plan.wideSelfSegs.size() +
+                             plan.stagedSelfSegs.size());
         if (w->dryRun) {
             w->lastWasFused = ok;
             return HCCL_SUCCESS;
@@ -1175,7 +1201,7 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
                 const int rc = hcclx_plan_create(parts[i].first->data(), static_cast<uint32_t>(parts[i].first->size()),
                                                  dt, op, parts[i].second, &hp);
                 if (rc != HCCL_SUCCESS) {
-                    DropPlans(c.plans);
+                    DropPlans(c.plans, c.buffers);
                     return static_cast<HcclResult>(rc);
                 }
                 c.plans.push_back(hp);
@@ -1187,10 +1213,46 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
                 const int rc = hcclx_plan_create_wide(segs.data(), static_cast<uint32_t>(segs.size()), foldType, op,
                                                       i == 0 ? HCCLX_FOLD_CHAIN : i == 1 ? HCCLX_FOLD_TREE : HCCLX_FOLD_SELF_FIRST, &hp);
                 if (rc != HCCL_SUCCESS) {
-                    DropPlans(c.plans);
+                    DropPlans(c.plans, c.buffers);
                     return static_cast<HcclResult>(rc);
                 }
                 c.plans.push_back(hp);
+            }
+            if (!plan.stagedSelfSegs.empty()) {
+                char *staging = nullptr;
+                if (hipMalloc(reinterpret_cast<void **>(&staging), plan.stagingBytes) != hipSuccess) {
+                    DropPlans(c.plans, c.buffers);
+                    return HCCL_E_RUNTIME;
+                }
+                c.buffers.push_back(staging);
+                std::vector<hcclx_seg_t> copies;
+                for (hcclx_wide_seg_t &seg : plan.stagedSelfSegs) {
+                    for (uint32_t j = 0; j < seg.ndst; ++j) seg.dst[j] = staging + reinterpret_cast<u64>(seg.dst[j]);
+                }
+                for (const FusedPlan::StagedCopy &sc : plan.stagedCopies) {
+                    hcclx_seg_t cp;
+                    std::memset(&cp, 0, sizeof(cp));
+                    cp.count = sc.bytes;
+                    cp.nsrc = 1;
+                    cp.ndst = 1;
+                    cp.src[0] = staging + sc.offset;
+                    cp.dst[0] = reinterpret_cast<void *>(sc.dst);
+                    copies.push_back(cp);
+                }
+                hcclx_plan *first = nullptr;
+                hcclx_plan *second = nullptr;
+                int rc = hcclx_plan_create_wide(plan.stagedSelfSegs.data(), static_cast<uint32_t>(plan.stagedSelfSegs.size()),
+                                                foldType, op, HCCLX_FOLD_SELF_FIRST, &first);
+                if (rc == HCCL_SUCCESS) {
+                    c.plans.push_back(first);
+                    rc = hcclx_plan_create(copies.data(), static_cast<uint32_t>(copies.size()), HCCL_DATA_TYPE_INT8, 0,
+                                           HCCLX_FOLD_CHAIN, &second);
+                }
+                if (rc != HCCL_SUCCESS) {
+                    DropPlans(c.plans, c.buffers);
+                    return static_cast<HcclResult>(rc);
+                }
+                c.plans.push_back(second);   // launched last: every read of the inputs is queued in front of it
             }
             w->lastWasFused = true;
             return LaunchAndKeep(w, std::move(c), stream);
@@ -1202,7 +1264,7 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
     c.levels = numLevels;
     const HcclResult built = BuildStepPlans(order, numLevels, foldType, op, c.plans);
     if (built != HCCL_SUCCESS) {
-        DropPlans(c.plans);
+        DropPlans(c.plans, c.buffers);
         return built;
     }
     return LaunchAndKeep(w, std::move(c), stream);

@@ -75,9 +75,11 @@ World::~World()
     for (RetiredPlan &r : planCache.retired) {
         if (r.event) (void)hipEventDestroy(static_cast<hipEvent_t>(r.event));
         for (hcclx_plan *p : r.plans) (void)hcclx_plan_destroy(p);
+        for (void *b : r.buffers) (void)hipFree(b);
     }
     for (CachedPlan &c : planCache.lru) {
         for (hcclx_plan *p : c.plans) (void)hcclx_plan_destroy(p);
+        for (void *b : c.buffers) (void)hipFree(b);
     }
 }
 

@@ -71,6 +71,7 @@ struct QueuedOp {
 struct CachedPlan {
     std::vector<u64> key;
     std::vector<hcclx_plan *> plans;   // launched in this order
+    std::vector<void *> buffers;       // device memory the plans use besides their tables (staged outputs)
     bool fused = true;                 // false: the recorded steps, one or two plans per level
     u32 levels = 0;
     u64 tableBytes = 0;                // device memory of the plans' tables
@@ -86,6 +87,7 @@ constexpr size_t kPlanCacheEntries = 1024;
 constexpr u64 kPlanCacheBytes = 256ull << 20;
 struct RetiredPlan {
     std::vector<hcclx_plan *> plans;
+    std::vector<void *> buffers;
     void *event = nullptr;             // hipEvent_t
 };
 struct PlanCache {

@@ -110,22 +110,33 @@ def test_checked_world_verifies_then_launches(stream):
         w.close()
 
 
-def test_one_shot_allreduce_in_place_among_24_ranks_runs_step_by_step(stream):
+@pytest.mark.parametrize("n,alg,dtype,op", [(24, "InsAllReduceMesh1DOneShot", T.FP32, T.SUM),
+                                           (40, "InsAllReduceMesh1DOneShot", T.BFP16, T.SUM),
+                                           (17, "InsAllReduceAicpuReduceNHR", T.FP64, T.PROD),
+                                           (64, "InsAllReduceMesh1DOneShot", T.FP16, T.MAX)])
+def test_one_shot_allreduce_in_place_among_many_ranks(stream, n, alg, dtype, op):
     """sendBuf == recvBuf with the per-rank orders of the one-shot template: among more than 16 ranks the outputs
-    cannot be computed in one pass without overwriting inputs that other workgroups still read, so the steps run
-    one by one; the values are the template's."""
-    n, count = 24, 30011
-    rng = np.random.default_rng(24)
-    xs = [payload(rng, T.FP32, count, "uniform") for _ in range(n)]
+    are computed sixteen at a time by different workgroups, so they go to a staging buffer and a second launch
+    copies them over the inputs; repeated, on new data."""
+    count = 30011
+    rng = np.random.default_rng(n)
+    esz = T.DTYPE_SIZE[dtype]
     w = api.World(n, ccl_bytes=SMALL_CCL)
     try:
-        w.set_algorithm(api.CMD_ALLREDUCE, "InsAllReduceMesh1DOneShot")
-        got, bufs = run_allreduce(w, stream, xs, count, T.FP32, T.SUM, in_place=True)
-        assert w.last_info().fused == 0
-        want = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs, count, 4, "InsAllReduceMesh1DOneShot", ccl_bytes=SMALL_CCL)
-        for r in range(n):
-            assert_same_bits(got[r], want[r], T.FP32, f"rank {r}")
-            assert bufs[r].guard_intact()
+        w.set_algorithm(api.CMD_ALLREDUCE, alg)
+        for rep in range(2):
+            kind = "prod" if op == T.PROD else "uniform" if dtype in (T.FP32, T.FP64) else "normal"
+            xs = [payload(rng, dtype, count, kind) for _ in range(n)]
+            got, bufs = run_allreduce(w, stream, xs, count, dtype, op, in_place=True)
+            info = w.last_info()
+            assert info.fused == 1 and info.launches == 2 and info.planCacheHit == 0   # new buffers: a new plan
+            if dtype in (T.FP16, T.BFP16) and op == T.SUM:
+                want = wide_oracle_allreduce(xs, count, dtype, alg, SMALL_CCL)
+            else:
+                want = T.run_allreduce(T.NumericElems(dtype, op), xs, count, esz, alg, ccl_bytes=SMALL_CCL)
+            for r in range(n):
+                assert_same_bits(got[r], want[r], dtype, f"rep {rep} rank {r}")
+                assert bufs[r].guard_intact()
     finally:
         w.close()
 
