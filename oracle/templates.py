@@ -21,8 +21,11 @@ Reference followed (paths relative to the reference tree, src/ops/...):
   allreduce_aicpu_reduce_nhr   all_reduce/template/aicpu/ins_temp_all_reduce_aicpu_reduce_nhr.cc:65-271
   reduce_scatter_mesh          reduce_scatter/template/aicpu/ins_temp_reduce_scatter_mesh_1D.cc:65-227
   reduce_scatter_nhr           reduce_scatter/template/aicpu/ins_temp_reduce_scatter_nhr.cc:77-425
+  reduce_scatter_aicpu_reduce_nhr  reduce_scatter/template/aicpu/ins_temp_reduce_scatter_aicpu_reduce_nhr.cc:52-240
   reduce_scatter_order_preserved  reduce_scatter/template/aicpu/ins_temp_reduce_scatter_order_preserved_level1.cc:52-330,
-                               executor reduce_scatter/executor/ins_v2_reduce_scatter_order_preserved_executor.cc:77-186
+                               executor reduce_scatter/executor/ins_v2_reduce_scatter_order_preserved_executor.cc:77-186;
+                               the same result stands for ins_temp_reduce_scatter_order_preserved_group.cc, which
+                               only changes which peer sends when (its sends are whole-slot copies)
   reduce_scatter_mesh_chunk    reduce_scatter/template/aicpu/ins_temp_reduce_scatter_mesh_1D_meshchunk.cc:69-263
   allreduce_mesh_two_shot_mesh_chunk  all_reduce/template/aicpu/ins_temp_all_reduce_mesh_1D_two_shot_mesh_chunk.cc:49-336
   reduce_scatter_v_mesh        reduce_scatter_v/template/aicpu/ins_temp_reduce_scatter_v_mesh_1D.cc:50-179,
