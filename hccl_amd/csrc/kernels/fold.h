@@ -122,12 +122,13 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
 #pragma unroll
     for (int k = 0; k < MAXN; ++k) {
         if ((present >> k) & 1u) {
-            const char *p = sd.src[k] + head_bytes + v0 * 16;
+            const char *p = sd.src[k] + head_bytes;
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
-                if (!CHECK || v0 + static_cast<uint64_t>(u) * kFoldThreads < nvec) {
-                    raw[u][k] = ld16(p + static_cast<uint64_t>(u) * kFoldThreads * 16);
-                }
+                // A lane outside the segment loads the segment's first vector and stores nothing: the loads
+                // stay unconditional, so all of them are in flight at once as in the unchecked tile.
+                const uint64_t vi = v0 + static_cast<uint64_t>(u) * kFoldThreads;
+                raw[u][k] = ld16(p + ((!CHECK || vi < nvec) ? vi : 0) * 16);
             }
         }
     }
@@ -333,7 +334,7 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
         if (tl * TV >= shift && (tl + 1) * TV - shift <= nvec) {
             fold_tile<DT, OP, MAXN, MODE, false>(sd, nsrc, ndst, v0, nvec, head_bytes);
         } else {
-            fold_tile<DT, OP, MAXN, MODE, true>(sd, nsrc, ndst, v0, nvec, head_bytes);
+            if (nvec != 0) fold_tile<DT, OP, MAXN, MODE, true>(sd, nsrc, ndst, v0, nvec, head_bytes);
             // the last tile also takes the elements in front of and behind the vector body, one per thread
             if (tl == (nvec + shift) / TV && threadIdx.x < head + rem) {
                 const uint64_t idx = threadIdx.x < head ? threadIdx.x : head + nvec * NE + (threadIdx.x - head);
@@ -360,9 +361,11 @@ __device__ __forceinline__ void fold_tile_wide(const SegWide &sd, uint32_t nsrc,
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const uint64_t v = v0 + static_cast<uint64_t>(u) * kFoldThreads;
+        // A lane outside the segment loads the segment's first vector and stores nothing: the loads stay
+        // unconditional, so all of a group are in flight at once as in the unchecked tile.
         ok[u] = !CHECK || v < nvec;
-        off[u] = head_bytes + v * 16;
-        if (ok[u]) V::unpack(ld16(sd.src[0] + off[u]), acc[u]);
+        off[u] = head_bytes + (ok[u] ? v : 0) * 16;
+        V::unpack(ld16(sd.src[0] + off[u]), acc[u]);
     }
     for (uint32_t base = 1; base < nsrc; base += G) {
         u32x4 raw[U][G];
@@ -370,9 +373,7 @@ __device__ __forceinline__ void fold_tile_wide(const SegWide &sd, uint32_t nsrc,
         for (int k = 0; k < G; ++k) {
             if (base + k < nsrc) {
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    if (ok[u]) raw[u][k] = ld16(sd.src[base + k] + off[u]);
-                }
+                for (int u = 0; u < U; ++u) raw[u][k] = ld16(sd.src[base + k] + off[u]);
             }
         }
 #pragma unroll
@@ -380,12 +381,10 @@ __device__ __forceinline__ void fold_tile_wide(const SegWide &sd, uint32_t nsrc,
             if (base + k < nsrc) {
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    if (ok[u]) {
-                        C x[NE];
-                        V::unpack(raw[u][k], x);
+                    C x[NE];
+                    V::unpack(raw[u][k], x);
 #pragma unroll
-                        for (int e = 0; e < NE; ++e) acc[u][e] = V::template combine<OP>(x[e], acc[u][e]);
-                    }
+                    for (int e = 0; e < NE; ++e) acc[u][e] = V::template combine<OP>(x[e], acc[u][e]);
                 }
             }
         }
@@ -571,7 +570,7 @@ k_fold_wide(const uint64_t *__restrict__ tile_end, const SegWide *__restrict__ s
             } else if constexpr (MODE == kFoldSelfFirst) {
                 fold_tile_wide_self<DT, OP, true>(sd, nsrc, v, nvec, head_bytes);
             } else {
-                fold_tile_wide<DT, OP, U, true>(sd, nsrc, ndst, v, nvec, head_bytes);
+                if (nvec != 0) fold_tile_wide<DT, OP, U, true>(sd, nsrc, ndst, v, nvec, head_bytes);
             }
             if (tl == (nvec + shift) / TV && threadIdx.x < head + rem) {
                 const uint64_t idx = threadIdx.x < head ? threadIdx.x : head + nvec * NE + (threadIdx.x - head);
