@@ -72,6 +72,8 @@ void init_slot(DeviceSlot *s, int dev)
     if (const char *v = std::getenv("HCCLX_A2AV_DIRECT")) c.a2av_direct_unroll = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
     if (const char *v = std::getenv("HCCLX_WIDE_CHAIN_FROM")) c.wide_chain_from = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
     if (const char *v = std::getenv("HCCLX_WIDE_XCD_REMAP_FROM")) c.wide_xcd_remap_from = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
+    c.wide_min_tiles = 2u * static_cast<uint32_t>(c.num_cus);
+    if (const char *v = std::getenv("HCCLX_WIDE_MIN_TILES")) c.wide_min_tiles = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
     if (const char *v = std::getenv("HCCLX_WIDE_CHAIN_FROM_ONE_DST")) {
         c.wide_chain_from_one_dst = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
     }
@@ -488,6 +490,11 @@ int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, i
     for (uint32_t i = 0; i < nseg; ++i) max_dst = segs[i].ndst > max_dst ? segs[i].ndst : max_dst;
     proto.wide_unroll = proto.mode != HCCLX_FOLD_CHAIN ? 1 : max_dst <= 1 ? kWideUnrollOne : kWideUnrollMany;
     const DeviceCtx *dctx = device_ctx();
+    if (proto.wide_unroll == kWideUnrollOne && dctx) {
+        uint64_t bytes = 0;
+        for (uint32_t i = 0; i < nseg; ++i) bytes += segs[i].count * static_cast<uint64_t>(esz);
+        if (bytes / (16 * wide_tile_vecs(kWideUnrollOne)) < dctx->wide_min_tiles) proto.wide_unroll = kWideUnrollMany;
+    }
     proto.xcd_remap = (dctx && max_dst >= dctx->wide_xcd_remap_from) ? 1u : 0u;
     const uint64_t tile_vecs = wide_tile_vecs(proto.wide_unroll);
     uint64_t scale = 1;

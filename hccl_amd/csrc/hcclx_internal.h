@@ -36,6 +36,9 @@ struct DeviceCtx {
     // Wide launches whose segments have this many destinations give each XCD a contiguous eighth of the tiles
     // (HCCLX_WIDE_XCD_REMAP_FROM).
     uint32_t wide_xcd_remap_from = 16;
+    // A single-destination chain launch that would have fewer four-vector tiles than this takes two vectors per
+    // thread instead, to spread a small job over more CUs (HCCLX_WIDE_MIN_TILES; set from the CU count).
+    uint32_t wide_min_tiles = 0;
     uint32_t a2av_direct_unroll = 2;   // HCCLX_A2AV_DIRECT: 0 = off, 1 / 2 / 4 = vectors per thread and tile
     // V kernels whose tables live on the device cannot know their tile count on the host and run as a
     // persistent grid of this many workgroups per CU.
