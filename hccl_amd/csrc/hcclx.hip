@@ -336,6 +336,7 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
                 wide[i].ndst = segs[i].ndst;
                 for (uint32_t k = 0; k < segs[i].nsrc; ++k) wide[i].src[k] = segs[i].src[k];
                 for (uint32_t k = 0; k < segs[i].ndst; ++k) wide[i].dst[k] = segs[i].dst[k];
+                for (uint32_t k = 1; k < segs[i].nsrc; ++k) wide[i].prog[k] = segs[i].prog[k];   // operand order per step
             }
             return build_wide_batches(wide.data(), nseg, dtype, op, HCCLX_FOLD_CHAIN, out);
         }
@@ -411,6 +412,9 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
         sd.ndst = s.ndst;
         for (uint32_t k = 0; k < s.nsrc; ++k) sd.src[k] = static_cast<const char *>(s.src[k]);
         for (uint32_t k = 0; k < s.ndst; ++k) sd.dst[k] = static_cast<char *>(s.dst[k]);
+        if (mode == HCCLX_FOLD_CHAIN) {
+            for (uint32_t k = 1; k < s.nsrc; ++k) sd.tree_codes |= (s.prog[k] ? 1u : 0u) << k;   // acc (+) src[k] steps
+        }
         if (proto.mode == HCCLX_FOLD_TREE && !embed_tree(s, static_cast<uint32_t>(proto.maxn), &sd)) {
             return fail(HCCL_E_NOT_SUPPORT, "segment " + std::to_string(i) + ": tree deeper than log2(" +
                                                 std::to_string(proto.maxn) + ") levels");
@@ -520,6 +524,9 @@ int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, i
         sd.ndst = s.ndst;
         for (uint32_t k = 0; k < s.nsrc; ++k) sd.src[k] = static_cast<const char *>(s.src[k]);
         for (uint32_t k = 0; k < s.ndst; ++k) sd.dst[k] = static_cast<char *>(s.dst[k]);
+        if (mode == HCCLX_FOLD_CHAIN) {
+            for (uint32_t k = 1; k < s.nsrc; ++k) sd.leaf_mask |= static_cast<uint64_t>(s.prog[k] ? 1 : 0) << k;
+        }
         if (proto.mode == HCCLX_FOLD_TREE) {
             std::vector<uint8_t> code;
             std::vector<int> slot_reg;

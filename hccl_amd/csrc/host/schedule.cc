@@ -370,7 +370,8 @@ struct Fold {
     bool chain = true;        // false: a tree that no chain reproduces
     bool fits = true;         // false: a tree too large for the tree kernels
     u32 levels = 0;           // tree: levels below the root
-    std::vector<u8> prog;     // tree: (dst register, src register) per step over src[] as registers
+    std::vector<u8> prog;     // tree: (dst register, src register) per step over src[] as registers;
+                              // chain: empty, or one byte per source, non-zero = that step is acc (+) src
 };
 
 bool IsFloatType(int dt)
@@ -434,7 +435,7 @@ u32 EmitTree(const Tracer &tr, int e, u64 shift, Fold &f, u32 *levels)
 // any tree equals the chain of its leaves.  For floating types IEEE addition and multiplication are
 // commutative but not associative: "acc (+) leaf" still equals "leaf (+) acc" bit for bit (NaN payloads
 // aside), other tree shapes do not flatten; max/min additionally depend on operand order for NaN and
-// signed zeros, so only the exact spine is taken.
+// signed zeros: there a step "acc (+) leaf" is marked, and the chain kernels swap its operands.
 Fold Flatten(const Tracer &tr, int e, u64 shift, int dtype, int op)
 {
     Fold f;
@@ -444,16 +445,21 @@ Fold Flatten(const Tracer &tr, int e, u64 shift, int dtype, int op)
     }
     const bool commutes = (op == HCCL_REDUCE_SUM || op == HCCL_REDUCE_PROD);
     std::vector<u64> rev;  // leaves from the outermost step inwards
+    std::vector<u8> revSwap;
+    bool anySwap = false;
     int cur = e;
     u64 sh = shift;
     while (cur != 0) {
         const Expr &x = tr.At(cur);
         if (x.src == 0) {
             rev.push_back(sh + x.srcShift);
+            revSwap.push_back(0);
             sh += x.dstShift;
             cur = x.dst;
-        } else if (x.dst == 0 && commutes) {
+        } else if (x.dst == 0) {
             rev.push_back(sh + x.dstShift);
+            revSwap.push_back(commutes ? 0 : 1);
+            anySwap = anySwap || !commutes;
             sh += x.srcShift;
             cur = x.src;
         } else {
@@ -469,6 +475,10 @@ Fold Flatten(const Tracer &tr, int e, u64 shift, int dtype, int op)
     }
     f.src.push_back(sh);
     for (auto it = rev.rbegin(); it != rev.rend(); ++it) f.src.push_back(*it);
+    if (anySwap) {
+        f.prog.push_back(0);
+        for (auto it = revSwap.rbegin(); it != revSwap.rend(); ++it) f.prog.push_back(*it);
+    }
     return f;
 }
 
@@ -549,7 +559,7 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
     for (auto &kv : bySrc) {
         if (kv.second.size() != 1) continue;
         const Fold &f = folds[kv.second[0]];
-        if (!f.chain || f.src.size() < 2 || f.src.size() > HCCLX_MAX_WIDE_FAN) continue;
+        if (!f.chain || !f.prog.empty() || f.src.size() < 2 || f.src.size() > HCCLX_MAX_WIDE_FAN) continue;
         std::vector<u64> key = f.src;
         std::sort(key.begin(), key.end());
         key.push_back(f.bytes);
@@ -681,6 +691,7 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
                     seg.dst[seg.ndst++] = reinterpret_cast<void *>(folds[rest[d]].dst);
                 }
                 if (f.chain) {
+                    if (!f.prog.empty()) std::memcpy(seg.prog, f.prog.data(), f.prog.size());
                     plan.wideSegs.push_back(seg);
                 } else {
                     std::memcpy(seg.prog, f.prog.data(), f.prog.size());
@@ -707,6 +718,7 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
                 plan.treeSegs.push_back(seg);
             } else {
                 seg.count = f.bytes / esz;
+                if (!f.prog.empty()) std::memcpy(seg.prog, f.prog.data(), f.prog.size());
                 plan.chainSegs.push_back(seg);
             }
         }

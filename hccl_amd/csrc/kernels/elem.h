@@ -217,6 +217,14 @@ template <> struct Vec16<HCCL_DATA_TYPE_INT8> {
     }
 };
 
+// Floating-point max and min select one operand, so  a (+) b  and  b (+) a  differ for signed zeros and NaNs;
+// every other type and op gives the same bits either way.
+template <int DT, int OP> struct OperandOrderMatters {
+    static constexpr bool value =
+        (OP == HCCL_REDUCE_MAX || OP == HCCL_REDUCE_MIN) &&
+        (DT == HCCL_DATA_TYPE_FP16 || DT == HCCL_DATA_TYPE_FP32 || DT == HCCL_DATA_TYPE_FP64 || DT == HCCL_DATA_TYPE_BFP16);
+};
+
 __host__ __device__ constexpr int dtype_size(int dt)
 {
     // DATATYPE_SIZE_TABLE, src/ops/op_common/inc/alg_param.h:43-45

@@ -142,13 +142,19 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
         if constexpr (MODE == kFoldChain) {
             C acc[NE];
             V::unpack(raw[u][0], acc);
+            const uint32_t flips = sd.tree_codes;
 #pragma unroll
             for (int k = 1; k < MAXN; ++k) {
                 if (k < static_cast<int>(nsrc)) {
                     C x[NE];
                     V::unpack(raw[u][k], x);
+                    if (OperandOrderMatters<DT, OP>::value && ((flips >> k) & 1u)) {
 #pragma unroll
-                    for (int e = 0; e < NE; ++e) acc[e] = V::template combine<OP>(x[e], acc[e]);
+                        for (int e = 0; e < NE; ++e) acc[e] = V::template combine<OP>(acc[e], x[e]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < NE; ++e) acc[e] = V::template combine<OP>(x[e], acc[e]);
+                    }
                 }
             }
             const u32x4 out = V::pack(acc);
@@ -198,6 +204,10 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
     }
 }
 
+// Chain mode: bit k set = step k takes the accumulated value as its source operand.
+__device__ __forceinline__ uint64_t chain_flips(const SegDev &sd) { return sd.tree_codes; }
+__device__ __forceinline__ uint64_t chain_flips(const SegWide &sd) { return sd.leaf_mask; }
+
 // The last (count % NE) elements of a segment, one per thread.
 template <int DT, int OP, int MAXN, int MODE, typename SEG>
 __device__ __forceinline__ void fold_tail(const SEG &sd, uint32_t nsrc, uint32_t ndst, uint64_t idx)
@@ -208,8 +218,10 @@ __device__ __forceinline__ void fold_tail(const SEG &sd, uint32_t nsrc, uint32_t
     using Op = Combine<DT, OP>;
     if constexpr (MODE == kFoldChain) {
         C acc = D::widen(reinterpret_cast<const S *>(sd.src[0])[idx]);
+        const uint64_t flips = chain_flips(sd);
         for (uint32_t k = 1; k < nsrc; ++k) {
-            acc = Op::run(D::widen(reinterpret_cast<const S *>(sd.src[k])[idx]), acc);
+            const C x = D::widen(reinterpret_cast<const S *>(sd.src[k])[idx]);
+            acc = (OperandOrderMatters<DT, OP>::value && ((flips >> k) & 1u)) ? Op::run(acc, x) : Op::run(x, acc);
         }
         const S out = D::narrow(acc);
         for (uint32_t d = 0; d < ndst; ++d) reinterpret_cast<S *>(sd.dst[d])[idx] = out;
@@ -367,6 +379,7 @@ __device__ __forceinline__ void fold_tile_wide(const SegWide &sd, uint32_t nsrc,
         off[u] = head_bytes + (ok[u] ? v : 0) * 16;
         V::unpack(ld16(sd.src[0] + off[u]), acc[u]);
     }
+    const uint64_t flips = sd.leaf_mask;
     for (uint32_t base = 1; base < nsrc; base += G) {
         u32x4 raw[U][G];
 #pragma unroll
@@ -383,8 +396,13 @@ __device__ __forceinline__ void fold_tile_wide(const SegWide &sd, uint32_t nsrc,
                 for (int u = 0; u < U; ++u) {
                     C x[NE];
                     V::unpack(raw[u][k], x);
+                    if (OperandOrderMatters<DT, OP>::value && ((flips >> (base + k)) & 1u)) {
 #pragma unroll
-                    for (int e = 0; e < NE; ++e) acc[u][e] = V::template combine<OP>(x[e], acc[u][e]);
+                        for (int e = 0; e < NE; ++e) acc[u][e] = V::template combine<OP>(acc[u][e], x[e]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < NE; ++e) acc[u][e] = V::template combine<OP>(x[e], acc[u][e]);
+                    }
                 }
             }
         }

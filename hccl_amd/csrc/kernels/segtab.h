@@ -25,6 +25,8 @@ struct SegDev {
     // 1, children of i are 2i = the step's dst side and 2i+1 = its src side, leaf slots MAXN .. 2*MAXN-1
     // hold src[slot - MAXN]).  Two bits per inner node i at bit 2*i: 0 = nothing below, 1 = take the dst
     // child unchanged, 2 = child(2i+1) (+) child(2i).  leaf_mask has bit k set when src[k] is present.
+    // Chain mode: bit k of tree_codes set = step k is  acc = acc (+) src[k]  instead of  src[k] (+) acc  (only
+    // floating-point max and min tell the two apart).
     uint32_t tree_codes;
     uint32_t leaf_mask;
     // Elements in front of the first 16-byte boundary of dst[0]; they are handled one by one so that the
@@ -36,7 +38,8 @@ struct SegDev {
     uint32_t shift;
 };
 
-// A segment of the wide kernels.  Chain: acc = src[0]; acc = src[k] (+) acc for k = 1 .. nsrc-1.  Tree: as in
+// A segment of the wide kernels.  Chain: acc = src[0]; acc = src[k] (+) acc for k = 1 .. nsrc-1, or
+// acc (+) src[k] where bit k of leaf_mask is set.  Tree: as in
 // SegDev, embedded in a complete binary tree with kMaxWideFan leaf slots; the 2-bit code of inner node i sits at
 // bit 2 * (i % 16) of tree_codes[i / 16].  In both the value goes to every dst.  Self-first: nsrc == ndst, and
 // the entry computes the outputs first_dst .. first_dst + kMaxFan - 1 only (the launcher enters a segment once per

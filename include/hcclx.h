@@ -36,7 +36,9 @@ extern "C" {
 /* How the sources of a segment are folded; every step is  acc = src (+) acc  (operand order of
  * AicpuReduceTemplate, alg_data_trans_wrapper.cc:1226-1243). */
 typedef enum {
-    /* acc = src[0]; for k = 1 .. nsrc-1: acc = src[k] (+) acc; the result goes to dst[0 .. ndst-1]. */
+    /* acc = src[0]; for k = 1 .. nsrc-1: acc = src[k] (+) acc; the result goes to dst[0 .. ndst-1].
+     * A non-zero prog[k] turns step k into  acc = acc (+) src[k]  (a ring hands the accumulated value on as the
+     * source operand); only floating-point MAX and MIN tell the two apart, for signed zeros and NaNs. */
     HCCLX_FOLD_CHAIN = 0,
     /* nsrc == ndst; dst[j] = fold that starts from src[j] and then takes src[k], k ascending, k != j:
      * the per-rank order of the one-shot AllReduce and of the CPU-reduce NHR AllReduce
@@ -59,7 +61,8 @@ typedef struct {
     uint32_t ndst;
     const void *src[HCCLX_MAX_FAN];
     void *dst[HCCLX_MAX_FAN];
-    uint8_t prog[2 * HCCLX_MAX_FAN]; /* HCCLX_FOLD_TREE only: (dst register, src register) per step */
+    uint8_t prog[2 * HCCLX_MAX_FAN]; /* HCCLX_FOLD_TREE: (dst register, src register) per step;
+                                        HCCLX_FOLD_CHAIN: prog[k] != 0 swaps the operands of step k; else unused */
 } hcclx_seg_t;
 
 /* A segment with up to HCCLX_MAX_WIDE_FAN sources and destinations, for communicators of more than
@@ -74,7 +77,7 @@ typedef struct {
     uint32_t ndst;
     const void *src[HCCLX_MAX_WIDE_FAN];
     void *dst[HCCLX_MAX_WIDE_FAN];
-    uint8_t prog[2 * HCCLX_MAX_WIDE_FAN]; /* HCCLX_FOLD_TREE only */
+    uint8_t prog[2 * HCCLX_MAX_WIDE_FAN]; /* as in hcclx_seg_t */
 } hcclx_wide_seg_t;
 
 /* Library set-up for the current device: creates the descriptor arena.  Idempotent.  Called lazily by the

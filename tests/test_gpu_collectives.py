@@ -141,12 +141,39 @@ def test_one_shot_allreduce_in_place_among_many_ranks(stream, n, alg, dtype, op)
         w.close()
 
 
+@pytest.mark.parametrize("n", [3, 9, 12, 20])
+@pytest.mark.parametrize("dtype,op", [(T.FP32, T.MAX), (T.FP32, T.MIN), (T.BFP16, T.MIN), (T.FP64, T.MAX)])
+def test_ring_max_min_keep_the_operand_order_in_one_pass(stream, n, dtype, op):
+    """The ring hands the accumulated value on as the source operand (acc (+) x), and a floating-point MAX / MIN of
+    signed zeros or NaNs depends on which operand comes first: the fused pass marks those steps and must give the
+    bits of the step-by-step order, among any number of ranks."""
+    rng = np.random.default_rng(n * 13 + dtype + op)
+    count = 20011
+    pool = np.array([0.0, -0.0, np.nan, 1.0, -1.0, np.inf, -np.inf, 0.5], dtype=np.float32)
+    xs = []
+    for _ in range(n):
+        f = pool[rng.integers(0, pool.size, size=count)]
+        xs.append(T.narrow16(f, dtype) if dtype == T.BFP16 else f.astype(T.NP_STORAGE[dtype]))
+    w = api.World(n, ccl_bytes=SMALL_CCL)
+    try:
+        w.set_algorithm(api.CMD_ALLREDUCE, "InsAllReduceRing")
+        got, bufs = run_allreduce(w, stream, xs, count, dtype, op)
+        info = w.last_info()
+        assert info.fused == 1 and info.launches == 1
+        want = T.run_allreduce(T.NumericElems(dtype, op), xs, count, T.DTYPE_SIZE[dtype], "InsAllReduceRing",
+                               ccl_bytes=SMALL_CCL)
+        for r in range(n):
+            assert_same_bits(got[r], want[r], dtype, f"rank {r}")
+            assert bufs[r].guard_intact()
+    finally:
+        w.close()
+
+
 def test_step_by_step_plans_are_replayed_with_new_data(stream):
-    """A schedule that cannot be fused (among 9 ranks the ring's MAX fold is a spine of eight levels, and a
-    floating-point MAX cannot be reordered) and the explicit step-by-step mode: the second identical call replays the per-level launches from the cache, on the
-    data the buffers hold then."""
+    """The step-by-step mode: the second identical call replays the per-level launches from the cache, on the data
+    the buffers hold then."""
     n, count = 9, 40009
-    for mode, alg, op in [(api.EXEC_FUSED, "InsAllReduceRing", T.MAX), (api.EXEC_STEP, "InsAllReduceMesh1DTwoShot", T.SUM)]:
+    for mode, alg, op in [(api.EXEC_STEP, "InsAllReduceRing", T.MAX), (api.EXEC_STEP, "InsAllReduceMesh1DTwoShot", T.SUM)]:
         w = api.World(n, ccl_bytes=SMALL_CCL)
         try:
             w.set_mode(mode)

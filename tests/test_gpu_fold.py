@@ -359,6 +359,52 @@ def test_float_max_min_nan_and_zero_operand_order():
         assert_same_bits(dd.get(np.float32), fold_oracle([dst, src], T.FP32, op, [0, 1], False), T.FP32)
 
 
+def special_floats(rng, dtype, n):
+    """Values whose max / min depends on which operand comes first: signed zeros, NaNs, repeated values."""
+    pool = np.array([0.0, -0.0, np.nan, 1.0, -1.0, np.inf, -np.inf, 0.5], dtype=np.float32)
+    f = pool[rng.integers(0, pool.size, size=n)]
+    if dtype in (T.FP16, T.BFP16):
+        return T.narrow16(f, dtype)
+    return f.astype(T.NP_STORAGE[dtype])
+
+
+@pytest.mark.parametrize("nsrc", [2, 3, 8, 9, 16, 23, 64])
+@pytest.mark.parametrize("dtype,op", [(T.FP32, T.MAX), (T.FP32, T.MIN), (T.BFP16, T.MAX), (T.FP16, T.MIN),
+                                      (T.FP64, T.MAX), (T.FP32, T.SUM), (T.INT32, T.MAX)])
+def test_chain_steps_with_swapped_operands(nsrc, dtype, op):
+    """A chain step marked in prog[] computes acc (+) src[k] instead of src[k] (+) acc: what a ring does when it
+    hands the accumulated value on.  Floating-point max and min tell the two apart for signed zeros and NaNs."""
+    rng = np.random.default_rng(nsrc * 31 + dtype * 7 + op)
+    n = 4096 + 13
+    is_float = dtype in (T.FP16, T.BFP16, T.FP32, T.FP64)
+    if is_float and op != T.SUM:
+        xs = [special_floats(rng, dtype, n) for _ in range(nsrc)]
+    else:
+        xs = [payload(rng, dtype, n, "uniform" if is_float else "normal") for _ in range(nsrc)]
+    swaps = [0] + [int(b) for b in rng.integers(0, 2, size=nsrc - 1)]
+    swaps[-1] = 1
+    e = T.NumericElems(dtype, op)
+    acc = xs[0].copy()
+    for k in range(1, nsrc):
+        if swaps[k]:                       # acc is the source operand: the value lands where src[k] was
+            nxt = xs[k].copy()
+            e.reduce(nxt, 0, acc, 0, n)
+            acc = nxt
+        else:
+            e.reduce(acc, 0, xs[k], 0, n)
+    bufs = [DevBuf(x) for x in xs]
+    outs = [DevBuf(nbytes=xs[0].nbytes) for _ in range(2)]
+    seg = (n, [b.ptr for b in bufs], [o.ptr for o in outs], swaps)
+    if nsrc <= 16:
+        hcclx.fold([seg], dtype, op)
+    else:
+        hcclx.fold_wide([seg], dtype, op)
+    sync()
+    for o in outs:
+        assert_same_bits(o.get(T.NP_STORAGE[dtype]), acc, dtype)
+        assert o.guard_intact()
+
+
 def test_many_ragged_segments_and_empty_ones():
     rng = np.random.default_rng(8)
     counts = [0, 1, 3, 4, 5, 255, 256, 257, 1023, 1024, 4099, 0, 8191, 65537] + list(rng.integers(0, 3000, 2200))

@@ -280,12 +280,14 @@ def test_which_templates_fuse():
     # the one-shot order of all 12 ranks is one segment: 12 sources read once, 12 outputs
     _, info = dry_allreduce(12, 1200, T.FP32, T.SUM, "InsAllReduceMesh1DOneShot")
     assert info.fusedSegments == 1
-    # float max keeps operand order: the ring's "acc (+) leaf" steps are not swapped into a chain.  With 4
-    # ranks the 3-level tree still fits the tree kernel; with 12 ranks (11 levels) the steps run one by one
+    # float max keeps operand order: the ring's "acc (+) leaf" steps stay a chain whose marked steps swap their
+    # operands, among any number of ranks
     _, info = dry_allreduce(4, 64, T.FP32, T.MAX, "InsAllReduceRing")
     assert info.fused == 1
     _, info = dry_allreduce(12, 1200, T.FP32, T.MAX, "InsAllReduceRing")
-    assert info.fused == 0
+    assert info.fused == 1
+    _, info = dry_allreduce(40, 4000, T.FP32, T.MIN, "InsAllReduceRing")
+    assert info.fused == 1
 
 
 def test_selector_choices_follow_the_reference_thresholds():
