@@ -128,6 +128,15 @@ int ring_reserve(DeviceCtx *ctx, size_t bytes, hipStream_t stream, char **h, cha
     if (bytes > kSliceBytes) {
         return fail(HCCL_E_PARA, "descriptor table larger than one ring slice");
     }
+    // A captured copy would read its ring slot again at every replay, long after the slot has been reused.
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) {
+        (void)hipGetLastError();
+    } else if (capturing != hipStreamCaptureStatusNone) {
+        return fail(HCCL_E_NOT_SUPPORT,
+                    "this launch uploads its tables at call time and cannot be captured into a HIP graph: create a plan "
+                    "outside the capture and capture hcclx_plan_launch");
+    }
     Ring &r = g_slots[ctx->device].ring;
     std::lock_guard<std::mutex> lock(r.mu);
     if (r.off + bytes > kSliceBytes) {

@@ -94,7 +94,9 @@ uint32_t hcclx_dtype_size(int dtype);
  * dtype: HcclDataType of the elements; reduce types are int8 int16 int32 int64 uint64 fp16 fp32 fp64 bf16.
  * For nsrc == 1 everywhere any dtype with a known size is accepted (pure copy).  op: HcclReduceOp.
  * All segments of a call share nsrc's upper bound HCCLX_MAX_FAN.  segs is a host array, copied before
- * return. */
+ * return.  The launch table is uploaded at call time through a ring of pinned slots, so this call (like every
+ * entry point that takes host tables and is not a plan) returns HCCL_E_NOT_SUPPORT on a stream that is being
+ * captured into a HIP graph: create a plan outside the capture and capture hcclx_plan_launch. */
 int hcclx_fold(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, void *stream);
 /* The same for wide segments. */
 int hcclx_fold_wide(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, void *stream);

@@ -62,3 +62,31 @@ def test_warm_allreduce_captured_into_a_graph_and_replayed(n, count, dtype, op, 
                 assert recv[r].guard_intact()
     finally:
         w.close()
+
+
+def test_a_launch_that_uploads_its_tables_refuses_to_be_captured():
+    """A one-shot launch copies its table through a ring of pinned slots that later calls reuse; captured, the copy
+    would read a stale slot at every replay.  It must fail loudly instead, and leave the capture usable."""
+    from hccl_amd import hcclx
+    from hccl_amd._lib import HcclError
+    x = np.arange(5000, dtype=np.float32)
+    src, dst = DevBuf(x), DevBuf(nbytes=x.nbytes)
+    s = torch.cuda.Stream()
+    hcclx.fold([(x.size, [src.ptr], [dst.ptr])], T.FP32, stream=s.cuda_stream)    # eagerly: fine
+    s.synchronize()
+    assert np.array_equal(dst.get(np.float32), x)
+    plan = hcclx.Plan([(x.size, [src.ptr], [dst.ptr])], T.FP32)
+    dst.t[dst.offset:dst.offset + dst.nbytes] = 0
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(s):
+        g.capture_begin()
+        with pytest.raises(HcclError):
+            hcclx.fold([(x.size, [src.ptr], [dst.ptr])], T.FP32, stream=s.cuda_stream)
+        plan.launch(s.cuda_stream)                                                 # the capturable form
+        g.capture_end()
+    g.replay()
+    torch.cuda.synchronize()
+    assert np.array_equal(dst.get(np.float32), x) and dst.guard_intact()
+    del g
+    plan.close()
