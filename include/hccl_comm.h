@@ -16,7 +16,10 @@
  * The first collective of a given kind (op, algorithm, type, count, buffers, mode) records the ranks' templates,
  * plans the launch and keeps the plan (up to 1024 plans or 256 MiB of launch tables per communicator, least
  * recently used out first); repeats only launch kernels -- no allocation, no copy -- and may therefore be issued
- * on a stream that is being captured into a HIP graph.
+ * on a stream that is being captured into a HIP graph.  AllGather(V) and AlltoAll(V, VC) among up to 15 ranks carry
+ * their tables in the kernel arguments and can be captured from the first call on; AlltoAll(V, VC) among more ranks
+ * uploads a block list at call time and returns HCCL_E_NOT_SUPPORT on a capturing stream (a graph needs
+ * hcclx_alltoallv_plan_create of hcclx.h there).
  */
 #ifndef HCCL_AMD_HCCL_COMM_H_
 #define HCCL_AMD_HCCL_COMM_H_
