@@ -90,3 +90,53 @@ def test_a_launch_that_uploads_its_tables_refuses_to_be_captured():
     assert np.array_equal(dst.get(np.float32), x) and dst.guard_intact()
     del g
     plan.close()
+
+
+def test_data_movement_collectives_captured_from_their_first_call():
+    """AllGatherV and AlltoAllV among 8 ranks carry their tables in the kernel arguments: they can be captured without
+    a warm-up, and a replay moves what the buffers hold then."""
+    n = 8
+    rng = np.random.default_rng(5)
+    counts = [int(c) for c in rng.integers(0, 3000, size=n)]
+    displs = [int(d) for d in np.concatenate([[0], np.cumsum(counts)[:-1]])]
+    total = sum(counts)
+    m = rng.integers(0, 900, size=(n, n)).tolist()
+    v = [T.alltoallvc_to_v(m, r) for r in range(n)]
+    ag_in = [DevBuf(nbytes=max(counts) * 2) for _ in range(n)]
+    ag_out = [DevBuf(nbytes=total * 2) for _ in range(n)]
+    aa_in = [DevBuf(nbytes=max(1, sum(m[i])) * 2) for i in range(n)]
+    aa_out = [DevBuf(nbytes=max(1, sum(x[2])) * 2) for x in v]
+    s = torch.cuda.Stream()
+    w1, w2 = api.World(n), api.World(n)
+    try:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(s):
+            g.capture_begin()
+            for r in range(n):
+                assert w1.all_gather_v(r, ag_in[r].ptr, counts[r], ag_out[r].ptr, counts, displs, T.FP16, s.cuda_stream) == 0
+            for r in range(n):
+                sc, sd, rc, rd = v[r]
+                assert w2.all_to_all_v(r, aa_in[r].ptr, sc, sd, aa_out[r].ptr, rc, rd, T.BFP16, s.cuda_stream) == 0
+            g.capture_end()
+        for rep in range(2):
+            xs = [rng.integers(0, 65536, size=max(counts), dtype=np.uint16) for _ in range(n)]
+            ys = [rng.integers(0, 65536, size=max(1, sum(m[i])), dtype=np.uint16) for i in range(n)]
+            for r in range(n):
+                ag_in[r].t[ag_in[r].offset:ag_in[r].offset + xs[r].nbytes] = torch.from_numpy(xs[r].view(np.uint8).copy()).to("cuda:0")
+                aa_in[r].t[aa_in[r].offset:aa_in[r].offset + ys[r].nbytes] = torch.from_numpy(ys[r].view(np.uint8).copy()).to("cuda:0")
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            want = T.run_allgatherv(xs, counts, displs, total, 0)
+            for r in range(n):
+                assert np.array_equal(ag_out[r].get(np.uint16)[:total], want[r]), f"AllGatherV replay {rep} rank {r}"
+                assert ag_out[r].guard_intact()
+            want = T.run_alltoallv([y[:sum(m[i])] for i, y in enumerate(ys)], [x[0] for x in v], [x[1] for x in v],
+                                   [x[2] for x in v], [x[3] for x in v], [sum(x[2]) for x in v])
+            for r in range(n):
+                assert np.array_equal(aa_out[r].get(np.uint16)[:sum(v[r][2])], want[r]), f"AlltoAllV replay {rep} rank {r}"
+                assert aa_out[r].guard_intact()
+        del g
+    finally:
+        w1.close()
+        w2.close()
