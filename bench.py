@@ -79,7 +79,7 @@ class ReduceScatterMesh(Workload):
     chain kernel that moves four vectors per thread (eight sources, one destination per segment)."""
     dtype = "bf16"
     kernel = "hcclx::k_fold_wide<11, 0, 0, 4>"
-    traffic = 604140165
+    traffic = 604142658
     profile = "profiles/k_fold_wide_reduce_scatter_bf16_8x64MiB.txt"
 
     def __init__(self, torch, api, T, n=8, recv=4 * 1024 * 1024):
@@ -123,7 +123,7 @@ class AllReduce(Workload):
     ranks, so each input is read once and the result is written to the eight outputs."""
     dtype = "f32"
     kernel = "hcclx::k_fold<4, 0, 8, 0>"
-    traffic = 1073834160
+    traffic = 1073743637
     profile = "profiles/k_fold_all_reduce_fp32_8x64MiB.txt"
 
     def __init__(self, torch, api, T, n=8, count=16 * 1024 * 1024, alg=None, step_mode=False):
@@ -158,7 +158,7 @@ class AllGather(Workload):
     output; each source byte is read once and written eight times."""
     dtype = "u8"
     kernel = "hcclx::(anonymous namespace)::k_allgatherv"
-    traffic = 4833547094
+    traffic = 4835777689
     profile = "profiles/k_allgatherv_fp16_8x64MiB.txt"
 
     def __init__(self, torch, api, T, n=8, count=32 * 1024 * 1024):
@@ -215,7 +215,7 @@ class AllToAllV(Workload):
     destination rank per token Zipf(s=1.2), tokens grouped by destination."""
     dtype = "u8"
     kernel = "hcclx::(anonymous namespace)::k_alltoallv_direct<2>"
-    traffic = 939549414
+    traffic = 939493444
     profile = "profiles/k_alltoallv_bf16_moe_8x4096x7168.txt"
 
     def __init__(self, torch, api, T, n=8, tokens=4096, hidden=7168, seed=0):
