@@ -520,3 +520,34 @@ def test_alltoallv_count_mismatch_between_ranks_is_rejected():
         assert w.all_to_all_v(1, ins[1], [3, 1], [0, 3], outs[1], [4, 1], [0, 4], T.INT8, FAKE_STREAM) == 1
     finally:
         w.close()
+
+
+def test_one_host_thread_per_rank_meets_at_every_collective():
+    """The reference's test style (one host thread per rank, all_reduce_testcase.cc:73-107) on a world without a
+    device: in blocking mode a call returns when the last rank has arrived, whatever the order of arrival, and a
+    thread that runs ahead queues its next collective behind the one in flight."""
+    import threading
+    n, rounds = 8, 40
+    w = api.World(n, ccl_bytes=SMALL_CCL, dry=True)
+    try:
+        w.set_blocking(True)
+        ins, outs = fake_ptrs(n)
+        rcs = [[] for _ in range(n)]
+
+        def body(r):
+            for k in range(rounds):
+                if k % 2 == 0:
+                    rcs[r].append(w.all_reduce(r, ins[r], outs[r], 100 + k, T.FP32, T.SUM, FAKE_STREAM))
+                else:
+                    rcs[r].append(w.reduce_scatter(r, ins[r], outs[r], 10 + k, T.INT32, T.MAX, FAKE_STREAM))
+
+        ts = [threading.Thread(target=body, args=(r,)) for r in range(n)]
+        for t in ts:
+            t.start()
+        for t in ts:
+            t.join(timeout=60)
+        assert all(not t.is_alive() for t in ts)
+        assert rcs == [[0] * rounds for _ in range(n)]
+        assert w.last_info().algName.decode().startswith("InsReduceScatter")
+    finally:
+        w.close()
