@@ -101,6 +101,9 @@ def load():
     lib.hcclx_moe_gather_combine.argtypes = [vpp, vpp, vpp, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32,
                                              ctypes.c_uint64, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, vpp,
                                              ctypes.c_void_p]
+    lib.hcclx_displs_from_counts.restype = ctypes.c_int
+    lib.hcclx_displs_from_counts.argtypes = [ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p,
+                                             ctypes.c_void_p, ctypes.c_void_p]
     lib.hcclx_allgatherv.restype = ctypes.c_int
     lib.hcclx_allgatherv.argtypes = [vpp, vpp, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_int,
                                      ctypes.c_int, ctypes.c_void_p]

@@ -192,4 +192,17 @@ int hcclx_allgatherv(const void *const *send, void *const *recv, const uint64_t 
     return HCCL_SUCCESS;
 }
 
+int hcclx_displs_from_counts(const uint64_t *counts, uint32_t rows, uint32_t n, uint64_t *displs, uint64_t *totals,
+                             void *stream)
+{
+    if (!device_ctx()) return HCCL_E_RUNTIME;
+    if (!counts || !displs) return fail(HCCL_E_PTR, "counts or displs is null");
+    if (n == 0 || n > kMaxVRanks) return fail(HCCL_E_PARA, "rank count outside 1.." + std::to_string(kMaxVRanks));
+    if (rows == 0) return HCCL_SUCCESS;
+    if (rows > 0x7fffffffu) return fail(HCCL_E_PARA, "too many rows");
+    hipError_t e = launch_displs_from_counts(counts, rows, n, displs, totals, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail_hip(e, "displacement kernel launch");
+    return HCCL_SUCCESS;
+}
+
 }  // extern "C"

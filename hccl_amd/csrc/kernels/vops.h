@@ -110,6 +110,8 @@ hipError_t launch_alltoallv(const VRankPtrs &ptrs, const uint64_t *send_counts, 
                             hipStream_t stream);
 
 // counts / displs: device pointers, uint64 elements, n entries.
+hipError_t launch_displs_from_counts(const uint64_t *counts, uint32_t rows, uint32_t n, uint64_t *displs, uint64_t *totals,
+                                     hipStream_t stream);
 hipError_t launch_allgatherv(const VRankPtrs &ptrs, const uint64_t *counts, const uint64_t *displs, uint32_t n,
                              uint32_t esz, uint32_t grid, uint32_t tiles_per_block, hipStream_t stream);
 

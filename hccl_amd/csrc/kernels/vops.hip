@@ -273,6 +273,26 @@ hipError_t launch_alltoallv_direct(const VRankPtrs16 &ptrs, const A2avTablesDire
     return hipGetLastError();
 }
 
+// One wavefront per row of n <= 64 counts: displs = exclusive prefix sum, totals[row] = the row's sum.
+__global__ void __launch_bounds__(64)
+k_displs_from_counts(const uint64_t *__restrict__ counts, uint32_t n, uint64_t *__restrict__ displs,
+                     uint64_t *__restrict__ totals)
+{
+    const uint64_t row = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    const uint64_t c = lane < n ? counts[row * n + lane] : 0;
+    const uint64_t incl = wave_inclusive_scan(c);
+    if (lane < n) displs[row * n + lane] = incl - c;
+    if (totals != nullptr && lane == n - 1) totals[row] = incl;
+}
+
+hipError_t launch_displs_from_counts(const uint64_t *counts, uint32_t rows, uint32_t n, uint64_t *displs, uint64_t *totals,
+                                     hipStream_t stream)
+{
+    hipLaunchKernelGGL(k_displs_from_counts, dim3(rows), dim3(64), 0, stream, counts, n, displs, totals);
+    return hipGetLastError();
+}
+
 hipError_t launch_allgatherv(const VRankPtrs &ptrs, const uint64_t *counts, const uint64_t *displs, uint32_t n,
                              uint32_t esz, uint32_t grid, uint32_t tiles_per_block, hipStream_t stream)
 {

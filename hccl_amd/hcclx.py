@@ -141,6 +141,12 @@ def allgatherv(send, recv, counts, displs, dtype, on_device=False, stream=0):
                                        1 if on_device else 0, ctypes.c_void_p(stream)))
 
 
+def displs_from_counts(counts, rows, n, displs, totals=0, stream=0):
+    """counts, displs, totals: device addresses of uint64 arrays (rows x n, rows x n, rows; totals may be 0)."""
+    check(_lib.load().hcclx_displs_from_counts(ctypes.c_void_p(counts), rows, n, ctypes.c_void_p(displs),
+                                               ctypes.c_void_p(totals) if totals else None, ctypes.c_void_p(stream)))
+
+
 def moe_workspace_bytes(n, entries):
     return _lib.load().hcclx_moe_workspace_bytes(n, entries)
 

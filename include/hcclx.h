@@ -136,6 +136,15 @@ int hcclx_alltoallv_plan_create(const void *const *send, void *const *recv, cons
 int hcclx_allgatherv(const void *const *send, void *const *recv, const uint64_t *counts,
                      const uint64_t *displs, uint32_t n, int dtype, int tables_on_device, void *stream);
 
+/* Displacements that pack ragged blocks back to back, computed on the device by a wavefront prefix sum:
+ * displs[r*n + i] = counts[r*n + 0] + ... + counts[r*n + i-1] for each of `rows` rows of n <= 64 counts, and, if
+ * totals is not null, totals[r] = the row's sum.  All three are device arrays of uint64.  One row gives the recvDispls
+ * of an AllGatherV whose counts were produced on the device (then hcclx_allgatherv with tables_on_device = 1); the
+ * n rows of an AlltoAllV's send counts give its sdispls.  No counterpart in the reference, whose callers pass
+ * finished displacement arrays (include/hccl.h:134-135). */
+int hcclx_displs_from_counts(const uint64_t *counts, uint32_t rows, uint32_t n, uint64_t *displs, uint64_t *totals,
+                             void *stream);
+
 /* ---- The caller side of an MoE AlltoAllV, for n virtual ranks at once -------------------------------------
  * No counterpart in the reference, whose AlltoAllV takes finished send buffers and tables; the nearest code is
  * the staging either side of the transfer (PreCopy / PostCopy,

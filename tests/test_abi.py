@@ -35,7 +35,7 @@ def test_every_declared_function_is_exported():
                      "HcommChannelNotifyWaitOnThread", "HcommThreadJoin", "hcclx_fold", "hcclx_plan_create",
                      "hcclx_alltoallv", "hcclx_allgatherv", "hcclx_moe_route", "hcclx_moe_pack", "hcclx_moe_combine",
                      "hcclx_fold_wide", "hcclx_plan_create_wide", "hcclx_plan_table_bytes", "hcclx_moe_dispatch",
-                     "hcclx_moe_gather_combine"):
+                     "hcclx_moe_gather_combine", "hcclx_displs_from_counts"):
         assert expected in names, f"{expected} is not declared in include/"
     missing = [f"{n} ({h})" for n, h in sorted(names.items()) if not hasattr(lib, n)]
     assert not missing, "declared but not exported: " + ", ".join(missing)

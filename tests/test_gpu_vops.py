@@ -174,6 +174,50 @@ def test_allgatherv_16_ranks_random_counts():
     run_agv(counts, displs, T.FP16, rng, on_device=True)
 
 
+@pytest.mark.parametrize("rows,n", [(1, 1), (1, 16), (8, 8), (64, 64), (5, 37)])
+def test_displacements_from_counts_on_the_device(rows, n):
+    """The exclusive prefix sum per row, by one wavefront: against numpy, with zeros and counts beyond 32 bits."""
+    rng = np.random.default_rng(rows * 100 + n)
+    counts = rng.integers(0, 1 << 20, size=(rows, n)).astype(np.uint64)
+    counts[rng.random((rows, n)) < 0.2] = 0
+    counts[0, n // 2] = (1 << 35) + 7
+    dc = torch.from_numpy(counts.view(np.int64)).to("cuda:0")
+    dd = torch.full((rows, n), -1, dtype=torch.int64, device="cuda:0")
+    dt = torch.full((rows,), -1, dtype=torch.int64, device="cuda:0")
+    hcclx.displs_from_counts(dc.data_ptr(), rows, n, dd.data_ptr(), dt.data_ptr())
+    torch.cuda.synchronize()
+    want = np.cumsum(counts, axis=1) - counts
+    assert np.array_equal(dd.cpu().numpy().view(np.uint64), want)
+    assert np.array_equal(dt.cpu().numpy().view(np.uint64), counts.sum(axis=1))
+    dd.fill_(-1)
+    hcclx.displs_from_counts(dc.data_ptr(), rows, n, dd.data_ptr())          # totals are optional
+    torch.cuda.synchronize()
+    assert np.array_equal(dd.cpu().numpy().view(np.uint64), want)
+
+
+def test_allgatherv_with_counts_and_displacements_that_never_leave_the_device():
+    """Config 3 of the baseline in small: 16 ranks, ragged fp16 blocks packed back to back; the displacements come
+    from the counts by the device prefix sum and feed hcclx_allgatherv with tables_on_device."""
+    rng = np.random.default_rng(3)
+    n = 16
+    counts = rng.integers(0, 50000, size=n).astype(np.uint64)
+    counts[5] = 0
+    ins = [rng.integers(0, 65536, size=int(c), dtype=np.uint16) for c in counts]
+    total = int(counts.sum())
+    send = [DevBuf(x) if x.size else DevBuf(nbytes=2) for x in ins]
+    recv = [DevBuf(nbytes=total * 2) for _ in range(n)]
+    dc = torch.from_numpy(counts.view(np.int64)).to("cuda:0")
+    dd = torch.empty(n, dtype=torch.int64, device="cuda:0")
+    hcclx.displs_from_counts(dc.data_ptr(), 1, n, dd.data_ptr())
+    hcclx.allgatherv([s.ptr for s in send], [r.ptr for r in recv], dc.data_ptr(), dd.data_ptr(), T.FP16, on_device=True)
+    torch.cuda.synchronize()
+    displs = (np.cumsum(counts) - counts).astype(np.int64).tolist()
+    want = T.run_allgatherv(ins, [int(c) for c in counts], displs, total, 0)
+    for j in range(n):
+        assert np.array_equal(recv[j].get(np.uint16), want[j]), f"rank {j}"
+        assert recv[j].guard_intact()
+
+
 def test_v_ops_reject_bad_arguments():
     b = DevBuf(nbytes=64)
     with pytest.raises(HcclError) as e:
