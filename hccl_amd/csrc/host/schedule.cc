@@ -155,6 +155,9 @@ HcclResult BuildOrder(World *w, std::vector<Node> &order, u32 &numLevels, CheckR
         for (int id : dataFlat) {
             const TaskItem &it = *flat[id].item;
             if (it.bytes == 0) continue;
+            // a copy onto itself (the first step of an in-place collective) changes no byte: neither a read
+            // nor a write that could race
+            if (it.kind == ItemKind::COPY && it.dst == it.src) continue;
             const u64 d = reinterpret_cast<u64>(it.dst);
             const u64 sA = reinterpret_cast<u64>(it.src);
             acc.push_back({d, d + it.bytes, id, true});

@@ -38,6 +38,24 @@ def test_allreduce_templates_pass_the_check(alg, n):
         w.close()
 
 
+@pytest.mark.parametrize("n", [2, 3, 8, 12])
+@pytest.mark.parametrize("alg", list(T.ALLREDUCE_TEMPLATES))
+def test_in_place_allreduce_passes_the_check(alg, n):
+    """sendBuf == recvBuf: the template's first step copies the input onto itself, which changes no byte and so
+    races with no reader; every other pair of steps on the shared buffer must still be ordered."""
+    w = checked_world(n)
+    try:
+        w.set_algorithm(api.CMD_ALLREDUCE, alg)
+        ins, _ = fake_ptrs(n)
+        for count, dtype, op in ((n * 1000 + 3, T.FP32, T.SUM), (7, T.INT32, T.MAX)):
+            for r in range(n):
+                assert w.all_reduce(r, ins[r], ins[r], count, dtype, op, FAKE_STREAM) == 0, (alg, count)
+            rep = w.last_check()
+            assert rep.races == 0 and rep.semanticErrors == 0, rep.firstProblem
+    finally:
+        w.close()
+
+
 @pytest.mark.parametrize("n", [2, 4, 7, 8, 13])
 def test_the_other_collectives_pass_the_check(n):
     w = checked_world(n)
