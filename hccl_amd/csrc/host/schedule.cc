@@ -394,21 +394,57 @@ void CollectLeaves(const Tracer &tr, int e, u64 shift, std::vector<u64> &out)
     CollectLeaves(tr, x.src, shift + x.srcShift, out);
 }
 
-std::string ExprText(const Tracer &tr, int e, u64 shift, const std::vector<OpParam> &params)
+// The ranks' input buffers sorted by address, to find the one an address lies in without walking all ranks.
+struct InputRanges {
+    struct Range {
+        u64 base;
+        u64 size;
+        u32 rank;
+    };
+    std::vector<Range> sorted;
+    u64 longest = 1;   // no buffer that starts more than this below an address can hold it
+    explicit InputRanges(const std::vector<OpParam> &params)
+    {
+        for (size_t r = 0; r < params.size(); ++r) {
+            sorted.push_back({reinterpret_cast<u64>(params[r].inputPtr), params[r].inputSize, static_cast<u32>(r)});
+            longest = std::max<u64>(longest, params[r].inputSize);
+        }
+        std::sort(sorted.begin(), sorted.end(), [](const Range &a, const Range &b) { return a.base < b.base; });
+    }
+    // The input buffer that holds [addr, addr + bytes), or nullptr.  Buffers that start at or below addr are
+    // tried from the nearest one down (in-place and overlapping operands may nest).
+    const Range *Find(u64 addr, u64 bytes) const
+    {
+        auto it = std::upper_bound(sorted.begin(), sorted.end(), addr,
+                                   [](u64 v, const Range &x) { return v < x.base; });
+        while (it != sorted.begin()) {
+            --it;
+            if (it->base + longest <= addr) break;
+            if (addr + bytes <= it->base + it->size) return &*it;
+        }
+        return nullptr;
+    }
+};
+
+std::string ExprText(const Tracer &tr, int e, u64 shift, const InputRanges &inputs)
 {
     if (e == 0) {
-        for (size_t r = 0; r < params.size(); ++r) {
-            const u64 base = reinterpret_cast<u64>(params[r].inputPtr);
-            if (shift >= base && shift < base + std::max<u64>(params[r].inputSize, 1)) {
-                std::ostringstream os;
-                os << "x" << r << "@" << (shift - base);
-                return os.str();
-            }
+        // the lowest rank whose input holds the address, as a reader of the trace expects for shared buffers
+        const InputRanges::Range *best = nullptr;
+        auto it = std::upper_bound(inputs.sorted.begin(), inputs.sorted.end(), shift,
+                                   [](u64 v, const InputRanges::Range &x) { return v < x.base; });
+        while (it != inputs.sorted.begin()) {
+            --it;
+            if (it->base + inputs.longest <= shift) break;
+            if (shift < it->base + std::max<u64>(it->size, 1) && (best == nullptr || it->rank < best->rank)) best = &*it;
         }
-        return "?";
+        if (best == nullptr) return "?";
+        std::ostringstream os;
+        os << "x" << best->rank << "@" << (shift - best->base);
+        return os.str();
     }
     const Expr &x = tr.At(e);
-    return "(" + ExprText(tr, x.src, shift + x.srcShift, params) + "+" + ExprText(tr, x.dst, shift + x.dstShift, params) +
+    return "(" + ExprText(tr, x.src, shift + x.srcShift, inputs) + "+" + ExprText(tr, x.dst, shift + x.dstShift, inputs) +
            ")";
 }
 
@@ -516,6 +552,7 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
 {
     std::vector<Fold> folds;
     bool allFit = true;
+    const InputRanges inputs(params);
     for (size_t r = 0; r < params.size(); ++r) {
         const u64 out = reinterpret_cast<u64>(params[r].outputPtr);
         if (params[r].outputSize == 0) continue;
@@ -527,7 +564,7 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
             if (text) {
                 std::ostringstream os;
                 os << "rank " << r << " out[" << (s.start - out) << "," << s.len << ") = "
-                   << ExprText(tr, s.expr, s.shift, params) << "\n";
+                   << ExprText(tr, s.expr, s.shift, inputs) << "\n";
                 *text += os.str();
             }
             if (!f.fits) allFit = false;
@@ -535,18 +572,13 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
         }
     }
     if (!allFit) return false;
+    if (folds.size() > 100000) return false;
     // every source must be input data (or an output that the same fold overwrites in place)
     for (const Fold &f : folds) {
         for (u64 a : f.src) {
-            bool ok = false;
-            for (const OpParam &p : params) {
-                const u64 in = reinterpret_cast<u64>(p.inputPtr);
-                if (a >= in && a + f.bytes <= in + p.inputSize) ok = true;
-            }
-            if (!ok) return false;
+            if (inputs.Find(a, f.bytes) == nullptr) return false;
         }
     }
-    if (folds.size() > 100000) return false;
 
     // group folds with the same sources in the same order: one segment, several destinations
     std::map<std::vector<u64>, std::vector<size_t>> bySrc;
