@@ -439,9 +439,7 @@ std::string ExprText(const Tracer &tr, int e, u64 shift, const InputRanges &inpu
             if (shift < it->base + std::max<u64>(it->size, 1) && (best == nullptr || it->rank < best->rank)) best = &*it;
         }
         if (best == nullptr) return "?";
-        std::ostringstream os;
-        os << "x" << best->rank << "@" << (shift - best->base);
-        return os.str();
+        return "x" + std::to_string(best->rank) + "@" + std::to_string(shift - best->base);
     }
     const Expr &x = tr.At(e);
     return "(" + ExprText(tr, x.src, shift + x.srcShift, inputs) + "+" + ExprText(tr, x.dst, shift + x.dstShift, inputs) +
@@ -569,10 +567,10 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
             }
             if (!f.fits) allFit = false;
             folds.push_back(std::move(f));
+            if (folds.size() > 100000) return false;   // more pieces than one pass is worth planning for
         }
     }
     if (!allFit) return false;
-    if (folds.size() > 100000) return false;
     // every source must be input data (or an output that the same fold overwrites in place)
     for (const Fold &f : folds) {
         for (u64 a : f.src) {
