@@ -4,6 +4,7 @@
 #include "kernels/fold.h"
 #include "kernels/vops.h"
 
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -85,6 +86,12 @@ void init_slot(DeviceSlot *s, int dev)
         const uint32_t b = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
         if (b != 0) c.v_tiles_per_block = b;
     }
+    if (const char *v = std::getenv("HCCLX_FANOUT_FROM")) c.fanout_from = std::strtoull(v, nullptr, 10);
+    if (const char *v = std::getenv("HCCLX_FANOUT_RUN")) {
+        const uint64_t b = std::strtoull(v, nullptr, 10);
+        if (b >= 65536) c.fanout_run = b & ~static_cast<uint64_t>(4095);
+    }
+    if (const char *v = std::getenv("HCCLX_AGV_PHASED_FROM")) c.agv_phased_from = std::strtoull(v, nullptr, 10);
     c.ring_bytes = kSliceBytes * kSlices;
     e = hipHostMalloc(reinterpret_cast<void **>(&c.h_ring), c.ring_bytes, hipHostMallocDefault);
     if (e != hipSuccess) {
@@ -181,6 +188,92 @@ uint32_t grid_for(const DeviceCtx *ctx, uint64_t total_tiles)
 }
 
 // ---------------------------------------------------------------------------------------------------
+// copies that write one output at a time
+// ---------------------------------------------------------------------------------------------------
+size_t PhasedLaunch::jobs_bytes() const { return (jobs.size() * sizeof(PhasedJob) + 255) & ~static_cast<size_t>(255); }
+size_t PhasedLaunch::bytes() const { return jobs_bytes() + dsts.size() * sizeof(char *); }
+void PhasedLaunch::fill(char *h) const
+{
+    std::memcpy(h, jobs.data(), jobs.size() * sizeof(PhasedJob));
+    std::memcpy(h + jobs_bytes(), dsts.data(), dsts.size() * sizeof(char *));
+}
+
+void build_phased(std::vector<PhasedStream> &streams, uint64_t run_bytes, std::vector<PhasedLaunch> *out)
+{
+    // join streams that continue each other: the slices of a two-shot AllReduce lie back to back in every buffer
+    std::vector<PhasedStream> joined;
+    for (PhasedStream &st : streams) {
+        if (st.bytes == 0 || st.dst.empty()) continue;
+        bool cont = !joined.empty() && joined.back().dst.size() == st.dst.size() &&
+                    joined.back().src + joined.back().bytes == st.src;
+        for (size_t d = 0; cont && d < st.dst.size(); ++d) cont = joined.back().dst[d] + joined.back().bytes == st.dst[d];
+        if (cont) {
+            joined.back().bytes += st.bytes;
+        } else {
+            joined.push_back(std::move(st));
+        }
+    }
+    struct Run {
+        const PhasedStream *st;
+        uint64_t at, len;
+        uint32_t tiles;
+    };
+    // runs of equal length per stream, a multiple of the tile size; then launches by length class (powers of four)
+    constexpr uint64_t kTile = 256ull * 16 * kPhasedUnroll;
+    std::vector<Run> runs;
+    for (const PhasedStream &st : joined) {
+        const uint64_t n = (st.bytes + run_bytes - 1) / run_bytes;
+        const uint64_t len = ((st.bytes + n - 1) / n + kTile - 1) / kTile * kTile;
+        for (uint64_t at = 0; at < st.bytes; at += len) {
+            Run r{&st, at, st.bytes - at < len ? st.bytes - at : len, 0};
+            r.tiles = static_cast<uint32_t>(v_tiles_of(r.len, reinterpret_cast<uint64_t>(st.dst[0]) + at, kPhasedUnroll));
+            runs.push_back(r);
+        }
+    }
+    constexpr size_t kMaxJobs = 4096;   // per launch: the table stays well inside one slice of the descriptor ring
+    for (int cls = 15; cls >= 0; --cls) {
+        PhasedLaunch cur;
+        auto flush = [&]() {
+            if (cur.jobs.empty()) return;
+            // Workgroups go to the eight XCDs in turn, each with an L2 of its own: with a multiple of eight slots per
+            // destination a tile is copied to all its destinations by the same XCD, whose L2 then serves the re-reads.
+            cur.slots = (cur.slots + 7) & ~7u;
+            // the pointer array is laid out once the widest job is known
+            std::vector<char *> flat(cur.jobs.size() * cur.nd, nullptr);
+            size_t at = 0;
+            for (size_t j = 0; j < cur.jobs.size(); ++j) {
+                for (uint32_t d = 0; d < cur.jobs[j].ndst; ++d) flat[j * cur.nd + d] = cur.dsts[at++];
+            }
+            cur.dsts = std::move(flat);
+            out->push_back(std::move(cur));
+            cur = PhasedLaunch();
+        };
+        for (const Run &r : runs) {
+            int c = 0;
+            for (uint32_t t = r.tiles; t > 1; t = (t + 3) / 4) ++c;
+            if (c != cls) continue;
+            const uint32_t nd = static_cast<uint32_t>(r.st->dst.size());
+            const uint64_t grid_x = (static_cast<uint64_t>(std::max(cur.slots, r.tiles)) + 7) * std::max(cur.nd, nd);
+            if (cur.jobs.size() == kMaxJobs || grid_x > 0x7fffffffull ||
+                (cur.jobs.size() + 1) * (sizeof(PhasedJob) + 8ull * std::max(cur.nd, nd)) > (1u << 19)) {
+                flush();
+            }
+            PhasedJob j;
+            j.src = r.st->src + r.at;
+            j.bytes = r.len;
+            j.dst0 = reinterpret_cast<uint64_t>(r.st->dst[0]) + r.at;
+            j.ndst = nd;
+            j.tiles = r.tiles;
+            cur.jobs.push_back(j);
+            for (char *p : r.st->dst) cur.dsts.push_back(p + r.at);   // packed for now, see flush()
+            cur.slots = std::max(cur.slots, r.tiles);
+            cur.nd = std::max(cur.nd, nd);
+        }
+        flush();
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
 // fold tables
 // ---------------------------------------------------------------------------------------------------
 namespace {
@@ -224,9 +317,12 @@ struct Batch {
     uint32_t xcd_remap = 0;      // wide kernels: contiguous tile ranges per XCD (pays with 16 or more destinations)
     std::vector<CopyBlock> blocks;   // instead of everything above: a list of blocks for the block copy kernel
     int block_unroll = 2;
+    PhasedLaunch phased;         // instead of everything above: jobs of the copy kernel that writes one output at a time
+    uint32_t plain_store = 0;    // fold results are stored the ordinary way: the next batch fans them out
     size_t nseg() const { return segs.size() + wide.size(); }
     size_t bytes() const
     {
+        if (!phased.jobs.empty()) return phased.bytes();
         if (!blocks.empty()) return blocks.size() * sizeof(CopyBlock);
         return align256(tile_end.size() * 8) + segs.size() * sizeof(SegDev) + wide.size() * sizeof(SegWide);
     }
@@ -319,9 +415,99 @@ int tree_levels(uint32_t nsrc, const uint8_t *prog)
     return static_cast<int>(depth[0]);
 }
 
-int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, Built *out);
+int build_wide_batches_impl(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, uint32_t plain_store,
+                            Built *out);
+
+// Results that go to several places, from fanout_from bytes of them on: the fold stores each result once (to
+// dst[0], with ordinary stores) and a second launch copies it to the other places, one place at a time in runs
+// that the L2 still holds; segments that only copy go to that second launch whole (their source is the run).
+// Fills `one` (the segments of the first launch, one destination each) and `fan` (what the second launch copies)
+// and returns true; returns false when the launch stays as it is.  max_fan: the segment type's array size.
+template <typename SEG>
+bool split_fanout(const DeviceCtx *ctx, const SEG *segs, uint32_t nseg, int esz, int mode, uint32_t max_fan,
+                  std::vector<SEG> *one, std::vector<PhasedStream> *fan)
+{
+    if (ctx == nullptr || mode == HCCLX_FOLD_SELF_FIRST || esz == 0) return false;
+    uint64_t fold_traffic = 0;   // bytes read and written by the folds whose result goes to several places
+    uint64_t copy_payload = 0;   // bytes of the sources that are only copied to several places
+    for (uint32_t i = 0; i < nseg; ++i) {
+        const SEG &g = segs[i];
+        if (g.nsrc == 0 || g.nsrc > max_fan || g.ndst == 0 || g.ndst > max_fan) return false;   // rejected later
+        if (g.count == 0 || g.ndst < 2) continue;
+        for (uint32_t d = 0; d < g.ndst; ++d) {
+            if (g.dst[d] == nullptr) return false;
+        }
+        if (g.src[0] == nullptr) return false;
+        const uint64_t bytes = g.count * static_cast<uint64_t>(esz);
+        if (g.nsrc == 1) {
+            copy_payload += bytes;
+        } else {
+            fold_traffic += bytes * (g.nsrc + g.ndst);
+        }
+    }
+    const bool split_folds = ctx->fanout_from != 0 && fold_traffic >= ctx->fanout_from;
+    const bool split_copies = ctx->agv_phased_from != 0 && copy_payload >= ctx->agv_phased_from;
+    if (!split_folds && !split_copies) return false;
+    one->clear();
+    fan->clear();
+    for (uint32_t i = 0; i < nseg; ++i) {
+        const SEG &g = segs[i];
+        if (g.count == 0 || g.ndst < 2 || !(g.nsrc == 1 ? split_copies : split_folds)) {
+            one->push_back(g);
+            continue;
+        }
+        const bool copy = g.nsrc == 1;
+        PhasedStream st;
+        st.src = copy ? static_cast<const char *>(g.src[0]) : static_cast<const char *>(g.dst[0]);
+        st.bytes = g.count * static_cast<uint64_t>(esz);
+        for (uint32_t d = copy ? 0 : 1; d < g.ndst; ++d) st.dst.push_back(static_cast<char *>(g.dst[d]));
+        fan->push_back(std::move(st));
+        if (!copy) {
+            SEG f = g;
+            f.ndst = 1;
+            one->push_back(f);
+        }
+    }
+    return true;
+}
+
+// Appends the second launch (or launches) of a split fold.
+void append_fanout(const DeviceCtx *ctx, std::vector<PhasedStream> &fan, Built *out)
+{
+    std::vector<PhasedLaunch> launches;
+    build_phased(fan, ctx->fanout_run, &launches);
+    for (PhasedLaunch &l : launches) {
+        Batch b;
+        b.copy = true;
+        b.phased = std::move(l);
+        out->batches.push_back(std::move(b));
+    }
+}
+
+int build_batches_impl(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, uint32_t plain_store, Built *out);
 
 int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, Built *out)
+{
+    if (nseg != 0 && segs == nullptr) return fail(HCCL_E_PTR, "segs is null");
+    std::vector<hcclx_seg_t> one;
+    std::vector<PhasedStream> fan;
+    const DeviceCtx *fctx = device_ctx();
+    if (!split_fanout(fctx, segs, nseg, dtype_size(dtype), mode, HCCLX_MAX_FAN, &one, &fan)) {
+        return build_batches_impl(segs, nseg, dtype, op, mode, 0, out);
+    }
+    const uint64_t algo_before = out->algo_bytes;
+    const int rc = build_batches_impl(one.data(), static_cast<uint32_t>(one.size()), dtype, op, mode, 1, out);
+    if (rc != HCCL_SUCCESS) return rc;
+    // the algorithmic bytes are those of the segments as the caller gave them, however the work is split
+    out->algo_bytes = algo_before;
+    for (uint32_t i = 0; i < nseg; ++i) {
+        out->algo_bytes += static_cast<uint64_t>(segs[i].nsrc + segs[i].ndst) * segs[i].count * dtype_size(dtype);
+    }
+    append_fanout(fctx, fan, out);
+    return HCCL_SUCCESS;
+}
+
+int build_batches_impl(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, uint32_t plain_store, Built *out)
 {
     if (nseg != 0 && segs == nullptr) return fail(HCCL_E_PTR, "segs is null");
     // Chains over many sources run faster on the wide chain kernel (sources in groups of eight, two vectors per
@@ -347,7 +533,7 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
                 for (uint32_t k = 0; k < segs[i].ndst; ++k) wide[i].dst[k] = segs[i].dst[k];
                 for (uint32_t k = 1; k < segs[i].nsrc; ++k) wide[i].prog[k] = segs[i].prog[k];   // operand order per step
             }
-            return build_wide_batches(wide.data(), nseg, dtype, op, HCCLX_FOLD_CHAIN, out);
+            return build_wide_batches_impl(wide.data(), nseg, dtype, op, HCCLX_FOLD_CHAIN, plain_store, out);
         }
     }
     const int esz = dtype_size(dtype);
@@ -392,6 +578,7 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
     proto.dtype = dtype;
     proto.op = op;
     proto.mode = mode;
+    proto.plain_store = plain_store;
     if (!proto.copy) {
         if (!is_reduce_dtype(dtype)) return fail(HCCL_E_NOT_SUPPORT, "data type cannot be reduced");
         if (op < HCCL_REDUCE_SUM || op > HCCL_REDUCE_MIN) return fail(HCCL_E_NOT_SUPPORT, "unknown reduce op");
@@ -444,8 +631,29 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
     return HCCL_SUCCESS;
 }
 
-// Wide segments: chain order, up to kMaxWideFan sources and destinations, one kernel for every fan-in.
 int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, Built *out)
+{
+    if (nseg != 0 && segs == nullptr) return fail(HCCL_E_PTR, "segs is null");
+    std::vector<hcclx_wide_seg_t> one;
+    std::vector<PhasedStream> fan;
+    const DeviceCtx *fctx = device_ctx();
+    if (!split_fanout(fctx, segs, nseg, dtype_size(dtype), mode, HCCLX_MAX_WIDE_FAN, &one, &fan)) {
+        return build_wide_batches_impl(segs, nseg, dtype, op, mode, 0, out);
+    }
+    const uint64_t algo_before = out->algo_bytes;
+    const int rc = build_wide_batches_impl(one.data(), static_cast<uint32_t>(one.size()), dtype, op, mode, 1, out);
+    if (rc != HCCL_SUCCESS) return rc;
+    out->algo_bytes = algo_before;
+    for (uint32_t i = 0; i < nseg; ++i) {
+        out->algo_bytes += static_cast<uint64_t>(segs[i].nsrc + segs[i].ndst) * segs[i].count * dtype_size(dtype);
+    }
+    append_fanout(fctx, fan, out);
+    return HCCL_SUCCESS;
+}
+
+// Wide segments: chain order, up to kMaxWideFan sources and destinations, one kernel for every fan-in.
+int build_wide_batches_impl(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, uint32_t plain_store,
+                            Built *out)
 {
     if (nseg != 0 && segs == nullptr) return fail(HCCL_E_PTR, "segs is null");
     if (mode != HCCLX_FOLD_CHAIN && mode != HCCLX_FOLD_SELF_FIRST && mode != HCCLX_FOLD_TREE) {
@@ -496,6 +704,7 @@ int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, i
     Batch proto;
     proto.dtype = dtype;
     proto.op = op;
+    proto.plain_store = plain_store;
     // a tree over integers equals the chain of its leaves, and so does every self-first order
     proto.mode = (mode != HCCLX_FOLD_CHAIN && is_float_dtype(dtype) && max_src > 1) ? mode : HCCLX_FOLD_CHAIN;
     proto.maxn = kMaxWideFan;
@@ -575,6 +784,10 @@ int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, i
 
 void fill_table(const Batch &b, char *h)
 {
+    if (!b.phased.jobs.empty()) {
+        b.phased.fill(h);
+        return;
+    }
     if (!b.blocks.empty()) {
         std::memcpy(h, b.blocks.data(), b.blocks.size() * sizeof(CopyBlock));
         return;
@@ -587,6 +800,13 @@ void fill_table(const Batch &b, char *h)
 
 int launch_batch(const DeviceCtx *ctx, const Batch &b, const char *d_table, hipStream_t stream)
 {
+    if (!b.phased.jobs.empty()) {
+        const hipError_t pe = launch_phased_copy(reinterpret_cast<const PhasedJob *>(d_table),
+                                                 reinterpret_cast<char *const *>(d_table + b.phased.jobs_bytes()),
+                                                 static_cast<uint32_t>(b.phased.jobs.size()), b.phased.slots, b.phased.nd, stream);
+        if (pe != hipSuccess) return fail_hip(pe, "phased copy kernel launch");
+        return HCCL_SUCCESS;
+    }
     if (!b.blocks.empty()) {
         const hipError_t be = launch_copy_blocks(reinterpret_cast<const CopyBlock *>(d_table), static_cast<uint32_t>(b.blocks.size()),
                                                  static_cast<uint32_t>(b.total_tiles), b.block_unroll, stream);
@@ -601,6 +821,7 @@ int launch_batch(const DeviceCtx *ctx, const Batch &b, const char *d_table, hipS
     l.grid = grid_for(ctx, b.total_tiles);
     l.wide_unroll = b.wide_unroll;
     l.xcd_remap = b.xcd_remap;
+    l.plain_store = b.plain_store;
     l.stream = stream;
     hipError_t e;
     if (b.copy) {

@@ -45,6 +45,17 @@ struct DeviceCtx {
     uint32_t v_blocks_per_cu = 2;
     // With host tables the V kernels launch one workgroup per run of this many consecutive tiles.
     uint32_t v_tiles_per_block = 1;
+    // Writing n outputs at once runs HBM a third slower than writing them one after the other (the banks see n
+    // streams of row misses).  A fold whose result goes to several places therefore stores it once, with ordinary
+    // stores, and a second launch copies it to the other places, one place at a time in runs of fanout_run bytes
+    // (HCCLX_FANOUT_RUN) that the L2 still holds: 8 x 64 MiB fp32 AllReduce 204 -> 176 us.  It pays from about
+    // 640 MiB read and written by such folds in one launch (HCCLX_FANOUT_FROM, 0 = never): below that the
+    // Infinity Cache (256 MiB) absorbs enough of the writes for the single pass to win (8 x 32 MiB: 89 against 93 us).
+    uint64_t fanout_from = 640ull << 20;
+    uint64_t fanout_run = 8ull << 20;
+    // AllGather(V) with host tables: from this many bytes of payload on (HCCLX_AGV_PHASED_FROM, 0 = never) the outputs
+    // of a run of a source are written one after the other, each workgroup writing one output.
+    uint64_t agv_phased_from = 4ull << 20;
     // Descriptor ring: tables of one-shot launches are written to pinned host memory and copied to the
     // device ring on the launch stream just before the kernel.
     char *h_ring = nullptr;
@@ -62,6 +73,28 @@ int ring_reserve(DeviceCtx *ctx, size_t bytes, hipStream_t stream, char **h, cha
 uint32_t grid_for(const DeviceCtx *ctx, uint64_t total_tiles);
 
 struct CopyBlock;
+struct PhasedJob;
+
+// One launch of the copy kernel that writes one output at a time.
+struct PhasedLaunch {
+    std::vector<PhasedJob> jobs;
+    std::vector<char *> dsts;   // jobs.size() * nd pointers, job j's at [j * nd, j * nd + ndst)
+    uint32_t slots = 0;         // tiles of the longest job
+    uint32_t nd = 0;            // destinations of the widest job
+    size_t jobs_bytes() const;  // size of the job array, rounded up to 256
+    size_t bytes() const;       // job array + pointer array as they lie in the launch table
+    void fill(char *h) const;
+};
+// A contiguous source that goes to several places whole.
+struct PhasedStream {
+    const char *src;
+    uint64_t bytes;
+    std::vector<char *> dst;
+};
+// Turns streams into launches: streams that continue each other (source and every destination) are joined, each
+// is cut into runs of at most run_bytes of equal length, and runs of similar length share a launch (a launch's
+// grid is sized for its longest run; shorter ones leave workgroups that exit at once).
+void build_phased(std::vector<PhasedStream> &streams, uint64_t run_bytes, std::vector<PhasedLaunch> *out);
 // The non-empty blocks of an AlltoAllV with host tables (row-major n x n, elements of esz bytes), with the
 // inclusive prefix of their tiles of `unroll` vectors per thread; returns the number of tiles.
 uint64_t list_alltoallv_blocks(const void *const *send, void *const *recv, const uint64_t *send_counts,

@@ -168,6 +168,38 @@ int hcclx_allgatherv(const void *const *send, void *const *recv, const uint64_t 
     hipStream_t st = static_cast<hipStream_t>(stream);
     uint64_t grid = static_cast<uint64_t>(ctx->num_cus) * ctx->v_blocks_per_cu;
     if (!tables_on_device) {
+        uint64_t payload = 0;
+        for (uint32_t i = 0; i < n; ++i) payload += counts[i] * esz;
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(st, &capturing) != hipSuccess) (void)hipGetLastError();
+        // Large, and not being captured into a graph (the job table is uploaded at call time): the outputs of a run of
+        // a source are written one after the other.
+        if (n > 1 && ctx->agv_phased_from != 0 && payload >= ctx->agv_phased_from && capturing == hipStreamCaptureStatusNone) {
+            std::vector<PhasedStream> streams;
+            for (uint32_t i = 0; i < n; ++i) {
+                if (counts[i] == 0) continue;
+                PhasedStream s;
+                s.src = ptrs.send[i];
+                s.bytes = counts[i] * esz;
+                for (uint32_t d = 0; d < n; ++d) s.dst.push_back(ptrs.recv[d] + displs[i] * esz);
+                streams.push_back(std::move(s));
+            }
+            std::vector<PhasedLaunch> launches;
+            build_phased(streams, ctx->fanout_run, &launches);
+            for (const PhasedLaunch &l : launches) {
+                char *h = nullptr;
+                char *d = nullptr;
+                rc = ring_reserve(ctx, l.bytes(), st, &h, &d);
+                if (rc != HCCL_SUCCESS) return rc;
+                l.fill(h);
+                HCCLX_HIP(hipMemcpyAsync(d, h, l.bytes(), hipMemcpyHostToDevice, st));
+                hipError_t e = launch_phased_copy(reinterpret_cast<const PhasedJob *>(d),
+                                                  reinterpret_cast<char *const *>(d + l.jobs_bytes()),
+                                                  static_cast<uint32_t>(l.jobs.size()), l.slots, l.nd, st);
+                if (e != hipSuccess) return fail_hip(e, "allgatherv kernel launch");
+            }
+            return HCCL_SUCCESS;
+        }
         uint64_t total = 0;
         for (uint32_t i = 0; i < n; ++i) {
             total += v_tiles_of(counts[i] * esz, reinterpret_cast<uint64_t>(ptrs.recv[0]) + displs[i] * esz, kAgvUnroll);

@@ -71,6 +71,16 @@ __device__ __forceinline__ void st16(char *p, u32x4 v)
     *reinterpret_cast<u32x4_u *>(p) = v;
 #endif
 }
+// A result that a second launch fans out to its other destinations is stored the ordinary way, so that it is
+// still in the L2 / Infinity Cache when that launch reads it; everything else streams past the caches.
+__device__ __forceinline__ void st16x(char *p, u32x4 v, bool plain)
+{
+    if (plain) {
+        *reinterpret_cast<u32x4_u *>(p) = v;
+    } else {
+        st16(p, v);
+    }
+}
 __device__ __forceinline__ uint64_t uniform64(uint64_t x)
 {
     uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(x));
@@ -111,7 +121,7 @@ __device__ __forceinline__ void tree_eval(C (&leaf)[MAXN][NE], uint32_t codes)
 
 template <int DT, int OP, int MAXN, int MODE, bool CHECK>
 __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint32_t ndst, uint64_t v0, uint64_t nvec,
-                                          uint32_t head_bytes)
+                                          uint32_t head_bytes, bool plain)
 {
     constexpr int UNROLL = fold_unroll(MAXN);
     using V = Vec16<DT>;
@@ -162,7 +172,7 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
             // batch of scalar loads instead of one dependent load per iteration
 #pragma unroll
             for (int d = 0; d < kMaxFan; ++d) {
-                if (d < static_cast<int>(ndst)) st16(sd.dst[d] + head_bytes + vi * 16, out);
+                if (d < static_cast<int>(ndst)) st16x(sd.dst[d] + head_bytes + vi * 16, out, plain);
             }
         } else if constexpr (MODE == kFoldTree) {
             C val[MAXN][NE];
@@ -176,7 +186,7 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
             // batch of scalar loads instead of one dependent load per iteration
 #pragma unroll
             for (int d = 0; d < kMaxFan; ++d) {
-                if (d < static_cast<int>(ndst)) st16(sd.dst[d] + head_bytes + vi * 16, out);
+                if (d < static_cast<int>(ndst)) st16x(sd.dst[d] + head_bytes + vi * 16, out, plain);
             }
         } else {
             C val[MAXN][NE];
@@ -310,8 +320,10 @@ __device__ __forceinline__ void locate_tile(const uint64_t *__restrict__ tile_en
 
 template <int DT, int OP, int MAXN, int MODE>
 __global__ void __launch_bounds__(kFoldThreads)
-k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, uint32_t nseg, uint64_t total_tiles)
+k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, uint32_t nseg, uint64_t total_tiles,
+       uint32_t plain_store)
 {
+    const bool plain = plain_store != 0;
     constexpr int NE = Vec16<DT>::kElems;   // elements per 16-byte vector
     constexpr uint64_t TV = fold_tile_vecs(MAXN);
     extern __shared__ uint64_t s_end[];  // nseg entries, sized by the launcher
@@ -344,9 +356,9 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
         // they fail the bound check of the checked path like the ones behind its end.
         const uint64_t v0 = tl * TV + threadIdx.x - shift;
         if (tl * TV >= shift && (tl + 1) * TV - shift <= nvec) {
-            fold_tile<DT, OP, MAXN, MODE, false>(sd, nsrc, ndst, v0, nvec, head_bytes);
+            fold_tile<DT, OP, MAXN, MODE, false>(sd, nsrc, ndst, v0, nvec, head_bytes, plain);
         } else {
-            if (nvec != 0) fold_tile<DT, OP, MAXN, MODE, true>(sd, nsrc, ndst, v0, nvec, head_bytes);
+            if (nvec != 0) fold_tile<DT, OP, MAXN, MODE, true>(sd, nsrc, ndst, v0, nvec, head_bytes, plain);
             // the last tile also takes the elements in front of and behind the vector body, one per thread
             if (tl == (nvec + shift) / TV && threadIdx.x < head + rem) {
                 const uint64_t idx = threadIdx.x < head ? threadIdx.x : head + nvec * NE + (threadIdx.x - head);
@@ -361,7 +373,7 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
 // has.  One vector per thread and tile.
 template <int DT, int OP, int U, bool CHECK>
 __device__ __forceinline__ void fold_tile_wide(const SegWide &sd, uint32_t nsrc, uint32_t ndst, uint64_t v0, uint64_t nvec,
-                                               uint32_t head_bytes)
+                                               uint32_t head_bytes, bool plain)
 {
     using V = Vec16<DT>;
     using C = typename V::C;
@@ -413,7 +425,7 @@ __device__ __forceinline__ void fold_tile_wide(const SegWide &sd, uint32_t nsrc,
             if (base + d < ndst) {
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    if (ok[u]) st16(sd.dst[base + d] + off[u], V::pack(acc[u]));
+                    if (ok[u]) st16x(sd.dst[base + d] + off[u], V::pack(acc[u]), plain);
                 }
             }
         }
@@ -454,7 +466,7 @@ __device__ __forceinline__ void wide_subtree(const SegWide &sd, uint64_t off, ui
 // through the two top levels.
 template <int DT, int OP, bool CHECK>
 __device__ __forceinline__ void fold_tile_wide_tree(const SegWide &sd, uint32_t ndst, uint64_t v, uint64_t nvec,
-                                                    uint32_t head_bytes)
+                                                    uint32_t head_bytes, bool plain)
 {
     using V = Vec16<DT>;
     using C = typename V::C;
@@ -477,7 +489,7 @@ __device__ __forceinline__ void fold_tile_wide_tree(const SegWide &sd, uint32_t 
     for (uint32_t base = 0; base < ndst; base += kMaxFan) {
 #pragma unroll
         for (int d = 0; d < kMaxFan; ++d) {
-            if (base + d < ndst) st16(sd.dst[base + d] + off, out);
+            if (base + d < ndst) st16x(sd.dst[base + d] + off, out, plain);
         }
     }
 }
@@ -547,9 +559,10 @@ __device__ __forceinline__ void fold_tile_wide_self(const SegWide &sd, uint32_t 
 template <int DT, int OP, int MODE, int U>
 __global__ void __launch_bounds__(kFoldThreads)
 k_fold_wide(const uint64_t *__restrict__ tile_end, const SegWide *__restrict__ segs, uint32_t nseg, uint64_t total_tiles,
-            uint32_t xcd_remap)
+            uint32_t xcd_remap, uint32_t plain_store)
 {
     constexpr int NE = Vec16<DT>::kElems;
+    const bool plain = plain_store != 0;
     static_assert(MODE == kFoldChain || U == 1, "only the chain moves several vectors per thread");
     constexpr uint64_t TV = wide_tile_vecs(U);
     extern __shared__ uint64_t s_end[];
@@ -576,19 +589,19 @@ k_fold_wide(const uint64_t *__restrict__ tile_end, const SegWide *__restrict__ s
         const uint64_t v = tl * TV + threadIdx.x - shift;   // wraps in front of a shifted segment: fails the check
         if (tl * TV >= shift && (tl + 1) * TV - shift <= nvec) {
             if constexpr (MODE == kFoldTree) {
-                fold_tile_wide_tree<DT, OP, false>(sd, ndst, v, nvec, head_bytes);
+                fold_tile_wide_tree<DT, OP, false>(sd, ndst, v, nvec, head_bytes, plain);
             } else if constexpr (MODE == kFoldSelfFirst) {
                 fold_tile_wide_self<DT, OP, false>(sd, nsrc, v, nvec, head_bytes);
             } else {
-                fold_tile_wide<DT, OP, U, false>(sd, nsrc, ndst, v, nvec, head_bytes);
+                fold_tile_wide<DT, OP, U, false>(sd, nsrc, ndst, v, nvec, head_bytes, plain);
             }
         } else {
             if constexpr (MODE == kFoldTree) {
-                fold_tile_wide_tree<DT, OP, true>(sd, ndst, v, nvec, head_bytes);
+                fold_tile_wide_tree<DT, OP, true>(sd, ndst, v, nvec, head_bytes, plain);
             } else if constexpr (MODE == kFoldSelfFirst) {
                 fold_tile_wide_self<DT, OP, true>(sd, nsrc, v, nvec, head_bytes);
             } else {
-                if (nvec != 0) fold_tile_wide<DT, OP, U, true>(sd, nsrc, ndst, v, nvec, head_bytes);
+                if (nvec != 0) fold_tile_wide<DT, OP, U, true>(sd, nsrc, ndst, v, nvec, head_bytes, plain);
             }
             if (tl == (nvec + shift) / TV && threadIdx.x < head + rem) {
                 const uint64_t idx = threadIdx.x < head ? threadIdx.x : head + nvec * NE + (threadIdx.x - head);
@@ -639,6 +652,7 @@ struct FoldLaunch {
     uint32_t grid;
     int wide_unroll;           // the wide chain kernel: vectors per thread (kWideUnrollMany or kWideUnrollOne)
     uint32_t xcd_remap;        // the wide kernels: give each XCD a contiguous eighth of the tiles
+    uint32_t plain_store;      // chain and tree: results are stored the ordinary way (a fan-out launch reads them next)
     hipStream_t stream;
 };
 

@@ -19,6 +19,8 @@ constexpr uint32_t kMaxVRanks = 64;
 #endif
 constexpr int kA2avUnroll = HCCLX_A2AV_UNROLL;
 constexpr int kAgvUnroll = HCCLX_AGV_UNROLL;
+// The copies that write one output at a time (large AllGatherV, fan-out of a fold's result): 8 KiB tiles.
+constexpr int kPhasedUnroll = 2;
 
 // Tiles of a block of `bytes` bytes whose first destination byte sits at address `dst`.  Stores are
 // aligned: the bytes before the first 16-byte boundary of dst (head) and after the last whole vector
@@ -89,6 +91,16 @@ struct AgvTablesPtr {
     __device__ uint64_t count(uint32_t i) const { return counts[i]; }
     __device__ uint64_t displ(uint32_t i) const { return displs[i]; }
 };
+// One job of the copy kernel that writes one output at a time: `bytes` bytes from src to ndst places (the
+// launch's pointer array holds them at [job * nd, job * nd + ndst)), cut into `tiles` tiles laid out for the
+// alignment of the first place, whose address is dst0.
+struct PhasedJob {
+    const char *src;
+    uint64_t bytes;
+    uint64_t dst0;
+    uint32_t ndst;
+    uint32_t tiles;
+};
 struct AgvTablesInline {
     uint64_t counts[kMaxVRanks];
     uint64_t displs[kMaxVRanks];
@@ -98,6 +110,10 @@ struct AgvTablesInline {
 
 // blocks: device array of nblocks entries; unroll: 1, 2 or 4; grid = total number of tiles
 hipError_t launch_copy_blocks(const CopyBlock *blocks, uint32_t nblocks, uint32_t grid, int unroll, hipStream_t stream);
+// jobs, dsts: device arrays of njobs and njobs * nd entries; slots: tiles of the longest job; slots * nd < 2^31,
+// njobs < 65536
+hipError_t launch_phased_copy(const PhasedJob *jobs, char *const *dsts, uint32_t njobs, uint32_t slots, uint32_t nd,
+                              hipStream_t stream);
 // unroll: 1, 2 or 4 vectors per thread and tile; grid = total number of tiles
 hipError_t launch_alltoallv_direct(const VRankPtrs16 &ptrs, const A2avTablesDirect &tabs, uint32_t n, uint32_t esz,
                                    uint32_t grid, int unroll, hipStream_t stream);
@@ -114,5 +130,4 @@ hipError_t launch_displs_from_counts(const uint64_t *counts, uint32_t rows, uint
                                      hipStream_t stream);
 hipError_t launch_allgatherv(const VRankPtrs &ptrs, const uint64_t *counts, const uint64_t *displs, uint32_t n,
                              uint32_t esz, uint32_t grid, uint32_t tiles_per_block, hipStream_t stream);
-
 }  // namespace hcclx

@@ -42,8 +42,22 @@ Reference followed (paths relative to the reference tree, src/ops/...):
   moe_route / moe_pack / moe_combine  no reference code; the contract of include/hcclx.h (stable grouping by
                                destination rank, its inverse, fp32-accumulated combine)
 
-PARITY UNPINNED: allreduce_ring and allreduce_rhd restate documentation prose only; no reference code,
-test or fixture fixes their step order.
+What pins each function (tests/test_oracle_templates.py, fixtures in tests/golden/st_cases.json):
+  * every template: the predicates of the reference's semantics checkers on the symbolic run (each output
+    element reduces every rank exactly once at its own offset), equality with numpy folds on integers with
+    executor chunking, two ranks = one pairwise op;
+  * association order, as expression strings worked by hand from the cited lines: one-shot / two-shot /
+    CPU-reduce NHR (self-first and chain orders), NHR (N = 5, 12 and the rank-0-of-12 step table), order-preserved
+    tree (3, 8, 12 ranks), mesh-chunk ReduceScatter and AllReduce (N = 3, 4, every owner and chunk, and the
+    4 KiB / by-element chunk cuts), ReduceScatter CPU-reduce NHR (N = 3, 5), ring (N = 3, 5, 8, every slice, plus
+    the chain written out in fp32) and halving-doubling (p = 5, the document's own example, and p = 12, every
+    slice, plus p = 5 written out in fp32).
+  * ring and halving-doubling have no executable form in the reference (its AICPU templates are mesh and NHR);
+    their step order follows Ring.md:5-15 and RHD.md:11-17, and where the prose leaves a choice (which half of
+    its range a rank keeps, which operand is the source) the fixture states the rule used.
+PARITY UNPINNED, by nature: the rounding of Ascend's inline reduce for 16-bit floats (external hardware; the
+tests allow 1 ULP of an fp32-accumulated result) and NaN payloads (the reference's host FPU decides them; the
+tests compare NaN positions).
 """
 import ctypes
 import os

@@ -103,3 +103,45 @@ def fold_oracle(srcs, dtype, op, order, wide):
 def fused_is_wide(dtype, op):
     """16-bit float SUM accumulates in fp32 inside a fused fold; PROD narrows every step; MAX/MIN select."""
     return dtype in (T.FP16, T.BFP16) and op == T.SUM
+
+
+def sample_positions(rng, length, k, marks=()):
+    """k random positions plus the first and last 70 and 8 either side of every mark (slice boundaries)."""
+    parts = [rng.integers(0, length, k), np.arange(min(70, length)), np.arange(max(0, length - 70), length)]
+    for m in marks:
+        parts.append(np.arange(max(0, m - 8), min(length, m + 8)))
+    return np.unique(np.concatenate(parts)).astype(np.int64)
+
+
+def take(t, pos):
+    """The elements of device tensor t at the (sorted) host positions pos, as a numpy array."""
+    return t[torch.from_numpy(pos).to(t.device)].cpu().numpy()
+
+
+TORCH_STORAGE = {T.INT8: torch.int8, T.INT16: torch.int16, T.INT32: torch.int32, T.INT64: torch.int64,
+                 T.FP16: torch.float16, T.BFP16: torch.bfloat16, T.FP32: torch.float32, T.FP64: torch.float64}
+
+
+def device_payload(dtype, n, seed):
+    """Seeded payload made on the GPU (sizes where a host-made one would take minutes): integers over their whole
+    range, floats standard normal.  Returns the tensor in its storage type."""
+    g = torch.Generator(device="cuda:0")
+    g.manual_seed(seed)
+    td = TORCH_STORAGE[dtype]
+    if td in (torch.int8, torch.int16, torch.int32):
+        ii = torch.iinfo(td)
+        return torch.randint(ii.min, ii.max + 1, (n,), device="cuda:0", generator=g, dtype=td)
+    if td == torch.int64:
+        return torch.randint(-2**62, 2**62, (n,), device="cuda:0", generator=g, dtype=td)
+    out = torch.empty(n, device="cuda:0", dtype=td)
+    step = 1 << 28                      # through fp32 in pieces: no second full-size buffer
+    for at in range(0, n, step):
+        m = min(step, n - at)
+        out[at:at + m] = torch.randn(m, device="cuda:0", generator=g, dtype=torch.float32).to(td)
+    return out
+
+
+def host_sample(t, pos, dtype):
+    """Sampled elements of a device tensor as the oracle's storage type (16-bit floats as bit patterns)."""
+    v = take(t.view(torch.int16) if dtype in (T.FP16, T.BFP16) else t, pos)
+    return v.view(np.uint16) if dtype in (T.FP16, T.BFP16) else v

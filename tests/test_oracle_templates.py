@@ -402,3 +402,125 @@ def test_order_preserved_tree_is_the_same_on_every_rank():
     b[0] = f"({b[1]}+{b[0]})"
     for r in range(12):
         assert outs[r][0] == b[0]
+
+
+# ------------------------------------------------------------------------------------------------
+# Association orders worked by hand from the sources named in tests/golden/st_cases.json
+# ------------------------------------------------------------------------------------------------
+
+def run_lengths(seq):
+    out = []
+    for x in seq:
+        if out and out[-1][0] == x:
+            out[-1][1] += 1
+        else:
+            out.append([x, 1])
+    return [(a, b) for a, b in out]
+
+
+@pytest.mark.parametrize("n", [3, 5, 8])
+def test_ring_association_order_matches_the_hand_worked_chains(n):
+    want = GOLD["ring"]["slices"][str(n)]
+    outs = T.run_allreduce(T.SymbolicElems(), sym_inputs(n, n), n, 4, "InsAllReduceRing")   # one element per slice
+    for r in range(n):
+        assert list(outs[r]) == want, (n, r)
+    # ragged slices keep the order: 2n + 3 elements, slices of ceil(count / n)
+    count = 2 * n + 3
+    outs = T.run_allreduce(T.SymbolicElems(), sym_inputs(n, count), count, 4, "InsAllReduceRing")
+    per = -(-count // n)
+    for r in range(n):
+        for i in range(count):
+            assert outs[r][i] == want[i // per], (n, r, i)
+
+
+@pytest.mark.parametrize("n", [3, 5, 8])
+def test_ring_fp32_equals_the_plain_chain_along_the_ring(n):
+    """The closed form stated without the oracle's machinery: slice c = ((x_c + x_{c+1}) + x_{c+2}) + ... in fp32."""
+    rng = np.random.default_rng(50 + n)
+    count = 16 * n
+    xs = [(rng.random(count, dtype=np.float32) * 2 - 1) for _ in range(n)]
+    outs = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs, count, 4, "InsAllReduceRing")
+    for c in range(n):
+        lo, hi = c * 16, (c + 1) * 16
+        acc = xs[c][lo:hi].copy()
+        for k in range(1, n):
+            acc = acc + xs[(c + k) % n][lo:hi]
+        for r in range(n):
+            assert np.array_equal(outs[r][lo:hi].view(np.uint32), acc.view(np.uint32)), (n, c, r)
+
+
+@pytest.mark.parametrize("n", [5, 12])
+def test_rhd_association_order_matches_the_hand_worked_trees(n):
+    want = GOLD["rhd"]["slices"][str(n)]
+    extra, block = T.rhd_block(n)
+    assert block == GOLD["rhd"]["block"][str(n)] and extra == n - len(block)
+    p2 = len(want)
+    outs = T.run_allreduce(T.SymbolicElems(), sym_inputs(n, p2), p2, 4, "InsAllReduceRHD")  # one element per slice
+    for r in range(n):
+        assert list(outs[r]) == want, (n, r)
+
+
+def test_rhd_fp32_of_five_ranks_equals_the_tree_written_out():
+    rng = np.random.default_rng(55)
+    xs = [(0.9 + 0.2 * rng.random(4)).astype(np.float32) for _ in range(5)]
+    outs = T.run_allreduce(T.NumericElems(T.FP32, T.PROD), xs, 4, 4, "InsAllReduceRHD")
+    a = xs[1] * xs[0]                 # rank 1 folded into rank 0
+    want = [(xs[4] * xs[3]) * (xs[2] * a), (xs[2] * a) * (xs[4] * xs[3]), (xs[3] * xs[4]) * (a * xs[2]),
+            (a * xs[2]) * (xs[3] * xs[4])]
+    for r in range(5):
+        for k in range(4):
+            assert outs[r][k].view(np.uint32) == want[k][k].view(np.uint32), (r, k)
+
+
+@pytest.mark.parametrize("n", [3, 4])
+def test_mesh_chunk_rotation_matches_the_hand_worked_orders(n):
+    want = GOLD["mesh_chunk"]["by_owner_chunk"][str(n)]
+    parts = n - 1
+    # ReduceScatter: one element per chunk of every shard
+    outs = T.run_reduce_scatter(T.SymbolicElems(), sym_inputs(n, n * parts), parts, 4, "InsReduceScatterMesh1DMeshChunk")
+    for f in range(n):
+        assert list(outs[f]) == want[f], (n, f)
+    # AllReduce: slice f = elements [f * parts, (f + 1) * parts), the same on every rank
+    outs = T.run_allreduce(T.SymbolicElems(), sym_inputs(n, n * parts), n * parts, 4, "InsAllReduceMesh1DTwoShotMeshChunk")
+    flat = [s for f in range(n) for s in want[f]]
+    for r in range(n):
+        assert list(outs[r]) == flat, (n, r)
+
+
+@pytest.mark.parametrize("case", GOLD["mesh_chunk"]["reduce_scatter_split"]["cases"],
+                         ids=lambda c: "%dx%d" % (c["ranks"], c["recv_count"]))
+def test_mesh_chunk_reduce_scatter_cuts_shards_at_4_kib(case):
+    n, rc, esz = case["ranks"], case["recv_count"], case["esz"]
+    outs = T.run_reduce_scatter(T.SymbolicElems(), sym_inputs(n, n * rc), rc, esz, "InsReduceScatterMesh1DMeshChunk")
+    for f in range(n):
+        assert [b for _, b in run_lengths(outs[f])] == case["chunk_elems"], (f, run_lengths(outs[f])[:4])
+    assert sum(case["chunk_elems"]) == rc
+
+
+@pytest.mark.parametrize("case", GOLD["mesh_chunk"]["all_reduce_split"]["cases"],
+                         ids=lambda c: "%dx%d" % (c["ranks"], c["count"]))
+def test_mesh_chunk_allreduce_cuts_slices_by_elements(case):
+    n, count = case["ranks"], case["count"]
+    assert [c for _, c in T.split_data(count, n)] == case["slice_elems"]
+    outs = T.run_allreduce(T.SymbolicElems(), sym_inputs(n, count), count, 4, "InsAllReduceMesh1DTwoShotMeshChunk")
+    want = [c for row in case["chunk_elems"] for c in row if c]
+    for r in range(n):
+        assert [b for _, b in run_lengths(outs[r])] == want, r
+
+
+@pytest.mark.parametrize("n", [3, 5])
+def test_reduce_scatter_cpu_reduce_nhr_starts_from_the_own_shard(n):
+    want = GOLD["reduce_scatter_aicpu_reduce_nhr"]["by_rank"][str(n)]
+    outs = T.run_reduce_scatter(T.SymbolicElems(), sym_inputs(n, n * 2), 2, 8, "InsReduceScatterAicpuReduceNHR")
+    for r in range(n):
+        assert list(outs[r]) == [want[r]] * 2, (n, r)
+
+
+def test_reference_system_test_tuples_are_well_formed():
+    names = {"int8", "int16", "int32", "fp16", "fp32", "bfp16"}
+    ar = GOLD["allreduce_st"]["cases"]
+    assert len(ar) == 18 and all(c["dtype"] in names and c["op"] in ("sum", "max", "min") for c in ar)
+    assert [c["count"] for c in ar if c["name"] == "2shot_upper_boundary_data"] == [32 * 1024 * 1024 - 1]
+    rs = GOLD["reducescatter_st"]["cases"]
+    assert len(rs) == 27 and all(c["dtype"] in names for c in rs)
+    assert sum(next(c for c in rs if c["name"].startswith("nhr_asymmetric"))["servers"]) == 17
