@@ -59,6 +59,9 @@ def load():
     lib.hcclx_fold.restype = ctypes.c_int
     lib.hcclx_fold.argtypes = [ctypes.POINTER(Seg), ctypes.c_uint32, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                ctypes.c_void_p]
+    lib.hcclx_fold_static.restype = ctypes.c_int
+    lib.hcclx_fold_static.argtypes = [ctypes.POINTER(Seg), ctypes.c_uint32, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                      ctypes.c_void_p]
     lib.hcclx_plan_create.restype = ctypes.c_int
     lib.hcclx_plan_create.argtypes = [ctypes.POINTER(Seg), ctypes.c_uint32, ctypes.c_int, ctypes.c_int,
                                       ctypes.c_int, ctypes.POINTER(ctypes.c_void_p)]

@@ -10,7 +10,24 @@
 #include <mutex>
 #include <vector>
 
+// The launch table of hcclx_fold_static: a fixed array in every GPU's memory that the library runs on, so that the
+// entry point has nothing to allocate.  In host code this name is only a handle for hipGetSymbolAddress (done once
+// per device in init_slot below); everything else uses the device address kept in DeviceCtx::static_table.
+static __device__ __align__(256) unsigned char scratch[HCCLX_STATIC_TABLE_BYTES];
+
 namespace hcclx {
+
+// One piece of a launch table, carried in the kernel arguments and stored to `dst`: how hcclx_fold_static gets its
+// table into device memory without a staging buffer or a copy engine.
+constexpr uint32_t kPutBytes = 3584;   // kernel arguments hold up to 4 KiB
+struct TablePiece {
+    u32x4 v[kPutBytes / 16];
+};
+__global__ void __launch_bounds__(256) k_put_table(TablePiece piece, char *dst, uint32_t bytes)
+{
+    const uint32_t i = threadIdx.x;
+    if (i * 16 < bytes) *reinterpret_cast<u32x4 *>(dst + i * 16) = piece.v[i];
+}
 
 static thread_local std::string g_err;
 
@@ -101,6 +118,12 @@ void init_slot(DeviceSlot *s, int dev)
     e = hipMalloc(reinterpret_cast<void **>(&c.d_ring), c.ring_bytes);
     if (e != hipSuccess) {
         s->err = std::string("hipMalloc(descriptor ring): ") + hipGetErrorString(e);
+        return;
+    }
+    // init_slot runs with `dev` current (device_ctx() asks for the current device): this is that device's copy
+    e = hipGetSymbolAddress(reinterpret_cast<void **>(&c.static_table), HIP_SYMBOL(scratch));
+    if (e != hipSuccess || c.static_table == nullptr) {
+        s->err = std::string("hipGetSymbolAddress(launch table): ") + hipGetErrorString(e);
         return;
     }
     s->ok = true;
@@ -338,13 +361,15 @@ struct Built {
 // leaf slots: code[i] of inner heap node i (0 = nothing below, 1 = take the dst child, 2 = combine) and, per
 // leaf slot, the register whose source sits there (-1 = empty).  Returns false when the tree is deeper than
 // log2(slots).
-bool embed_tree(uint32_t nsrc, const uint8_t *prog, uint32_t slots, std::vector<uint8_t> *code, std::vector<int> *slot_reg)
+// code and slot_reg hold `slots` <= kMaxWideFan entries; nothing is allocated.
+bool embed_tree(uint32_t nsrc, const uint8_t *prog, uint32_t slots, uint8_t *code, int *slot_reg)
 {
     struct N {
         int dst = -1, src = -1, leaf = -1;
     };
-    std::vector<N> nodes(nsrc);
-    std::vector<int> holder(nsrc);  // node currently held by each register
+    N nodes[2 * kMaxWideFan];
+    int holder[kMaxWideFan];  // node currently held by each register
+    uint32_t nnodes = nsrc;
     for (uint32_t k = 0; k < nsrc; ++k) {
         nodes[k].leaf = static_cast<int>(k);
         holder[k] = static_cast<int>(k);
@@ -353,30 +378,38 @@ bool embed_tree(uint32_t nsrc, const uint8_t *prog, uint32_t slots, std::vector<
         N n;
         n.dst = holder[prog[2 * t]];
         n.src = holder[prog[2 * t + 1]];
-        nodes.push_back(n);
-        holder[prog[2 * t]] = static_cast<int>(nodes.size()) - 1;
+        nodes[nnodes] = n;
+        holder[prog[2 * t]] = static_cast<int>(nnodes++);
     }
-    code->assign(slots, 0);
-    slot_reg->assign(slots, -1);
+    for (uint32_t k = 0; k < slots; ++k) {
+        code[k] = 0;
+        slot_reg[k] = -1;
+    }
     // place(node, heap index): inner nodes combine their two children; a leaf above the bottom level is
     // passed up from the left-most slot below it
-    std::vector<std::pair<int, uint32_t>> stack{{holder[0], 1u}};
-    while (!stack.empty()) {
-        const int id = stack.back().first;
-        uint32_t at = stack.back().second;
-        stack.pop_back();
+    struct Todo {
+        int id;
+        uint32_t at;
+    };
+    Todo stack[2 * kMaxWideFan];
+    uint32_t top = 0;
+    stack[top++] = {holder[0], 1u};
+    while (top != 0) {
+        const int id = stack[top - 1].id;
+        uint32_t at = stack[top - 1].at;
+        --top;
         const N &n = nodes[id];
         if (n.leaf >= 0) {
             while (at < slots) {
-                (*code)[at] = 1;
+                code[at] = 1;
                 at *= 2;
             }
-            (*slot_reg)[at - slots] = n.leaf;
+            slot_reg[at - slots] = n.leaf;
         } else {
             if (at >= slots) return false;
-            (*code)[at] = 2;
-            stack.push_back({n.dst, 2 * at});
-            stack.push_back({n.src, 2 * at + 1});
+            code[at] = 2;
+            stack[top++] = {n.dst, 2 * at};
+            stack[top++] = {n.src, 2 * at + 1};
         }
     }
     return true;
@@ -384,9 +417,9 @@ bool embed_tree(uint32_t nsrc, const uint8_t *prog, uint32_t slots, std::vector<
 
 bool embed_tree(const hcclx_seg_t &s, uint32_t slots, SegDev *sd)
 {
-    std::vector<uint8_t> code;
-    std::vector<int> slot_reg;
-    if (!embed_tree(s.nsrc, s.prog, slots, &code, &slot_reg)) return false;
+    uint8_t code[kMaxWideFan];
+    int slot_reg[kMaxWideFan];
+    if (!embed_tree(s.nsrc, s.prog, slots, code, slot_reg)) return false;
     sd->tree_codes = 0;
     sd->leaf_mask = 0;
     for (uint32_t k = 0; k < kMaxFan; ++k) sd->src[k] = nullptr;
@@ -403,8 +436,8 @@ bool embed_tree(const hcclx_seg_t &s, uint32_t slots, SegDev *sd)
 // step on a consumed register.  Returns the number of levels of the tree, or -1 when it is malformed.
 int tree_levels(uint32_t nsrc, const uint8_t *prog)
 {
-    std::vector<bool> dead(nsrc, false);
-    std::vector<uint32_t> depth(nsrc, 0);
+    bool dead[kMaxWideFan] = {};
+    uint32_t depth[kMaxWideFan] = {};
     for (uint32_t t = 0; t + 1 < nsrc; ++t) {
         const uint32_t rd = prog[2 * t];
         const uint32_t rs = prog[2 * t + 1];
@@ -417,6 +450,93 @@ int tree_levels(uint32_t nsrc, const uint8_t *prog)
 
 int build_wide_batches_impl(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, uint32_t plain_store,
                             Built *out);
+
+// What the segments of one launch of the register-resident kernels have in common.
+struct SegProto {
+    bool copy = false;   // no segment combines anything: the byte copy kernel
+    int mode = 0;        // the kernel's mode (integers take the chain kernel whatever order is asked for)
+    int maxn = 1;        // source slots of the kernel instance
+    int esz = 1;
+};
+
+// Checks the segments of a call and works out the kernel instance they need.  Allocates nothing unless it fails.
+int check_segs(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, SegProto *sp)
+{
+    const int esz = dtype_size(dtype);
+    if (esz == 0) return fail(HCCL_E_NOT_SUPPORT, "unknown data type " + std::to_string(dtype));
+    if (mode != HCCLX_FOLD_CHAIN && mode != HCCLX_FOLD_SELF_FIRST && mode != HCCLX_FOLD_TREE) {
+        return fail(HCCL_E_PARA, "unknown fold mode");
+    }
+    uint32_t max_src = 0;
+    uint32_t max_depth = 0;  // tree mode: levels of the deepest tree
+    for (uint32_t i = 0; i < nseg; ++i) {
+        const hcclx_seg_t &s = segs[i];
+        if (s.nsrc == 0 || s.nsrc > HCCLX_MAX_FAN || s.ndst == 0 || s.ndst > HCCLX_MAX_FAN) {
+            return fail(HCCL_E_PARA, "segment " + std::to_string(i) + ": nsrc/ndst outside 1.." +
+                                         std::to_string(HCCLX_MAX_FAN));
+        }
+        if (mode == HCCLX_FOLD_SELF_FIRST && s.nsrc != s.ndst) {
+            return fail(HCCL_E_PARA, "self-first fold needs nsrc == ndst");
+        }
+        if (s.count != 0) {
+            for (uint32_t k = 0; k < s.nsrc; ++k) {
+                if (s.src[k] == nullptr) return fail(HCCL_E_PTR, "segment " + std::to_string(i) + ": null source");
+            }
+            for (uint32_t k = 0; k < s.ndst; ++k) {
+                if (s.dst[k] == nullptr) return fail(HCCL_E_PTR, "segment " + std::to_string(i) + ": null destination");
+            }
+        }
+        if (mode == HCCLX_FOLD_TREE) {
+            const int levels = tree_levels(s.nsrc, s.prog);
+            if (levels < 0) return fail(HCCL_E_PARA, "segment " + std::to_string(i) + ": malformed tree program");
+            if (is_float_dtype(dtype) && (1u << levels) > HCCLX_MAX_FAN) {
+                return fail(HCCL_E_NOT_SUPPORT, "segment " + std::to_string(i) + ": tree has " + std::to_string(levels) +
+                                                    " levels, the kernel holds 4");
+            }
+            if (static_cast<uint32_t>(levels) > max_depth) max_depth = static_cast<uint32_t>(levels);
+        }
+        if (s.nsrc > max_src) max_src = s.nsrc;
+    }
+    sp->copy = (max_src <= 1);
+    sp->mode = mode;
+    sp->esz = esz;
+    if (!sp->copy) {
+        if (!is_reduce_dtype(dtype)) return fail(HCCL_E_NOT_SUPPORT, "data type cannot be reduced");
+        if (op < HCCL_REDUCE_SUM || op > HCCL_REDUCE_MIN) return fail(HCCL_E_NOT_SUPPORT, "unknown reduce op");
+        sp->maxn = max_src <= 2 ? 2 : max_src <= 4 ? 4 : max_src <= 8 ? 8 : 16;
+        // a tree needs one leaf slot per position of the complete tree of its depth
+        if (mode == HCCLX_FOLD_TREE && is_float_dtype(dtype) && (1 << max_depth) > sp->maxn) sp->maxn = 1 << max_depth;
+        // Integer folds are association-free: the self-first order and every tree give the bits of the plain
+        // chain.  The kernels for those orders exist only for floating types, so integers take the chain kernel.
+        if (mode != HCCLX_FOLD_CHAIN && !is_float_dtype(dtype)) sp->mode = HCCLX_FOLD_CHAIN;
+    } else {
+        sp->maxn = 1;
+        sp->mode = HCCLX_FOLD_CHAIN;
+    }
+    return HCCL_SUCCESS;
+}
+
+// The device descriptor of one segment and its number of tiles; false when a tree does not fit the kernel instance.
+bool make_segdev(const hcclx_seg_t &s, const SegProto &sp, int mode, SegDev *out, uint64_t *tiles)
+{
+    SegDev sd;
+    std::memset(&sd, 0, sizeof(sd));
+    sd.count = sp.copy ? s.count * sp.esz : s.count;  // the copy kernel counts bytes
+    sd.nsrc = s.nsrc;
+    sd.ndst = s.ndst;
+    for (uint32_t k = 0; k < s.nsrc; ++k) sd.src[k] = static_cast<const char *>(s.src[k]);
+    for (uint32_t k = 0; k < s.ndst; ++k) sd.dst[k] = static_cast<char *>(s.dst[k]);
+    if (mode == HCCLX_FOLD_CHAIN) {
+        for (uint32_t k = 1; k < s.nsrc; ++k) sd.tree_codes |= (s.prog[k] ? 1u : 0u) << k;   // acc (+) src[k] steps
+    }
+    if (sp.mode == HCCLX_FOLD_TREE && !embed_tree(s, static_cast<uint32_t>(sp.maxn), &sd)) return false;
+    const int ne = sp.copy ? 16 : 16 / sp.esz;
+    sd.head = fold_head_of(sd.count, sp.copy ? 1 : sp.esz, sd.dst[0]);
+    sd.shift = fold_shift_of(sd.head, sp.copy ? 1 : sp.esz, fold_tile_vecs(sp.maxn), sd.dst[0]);
+    *tiles = fold_tiles_of(sd.count, ne, fold_tile_vecs(sp.maxn), sd.head, sd.shift);
+    *out = sd;
+    return true;
+}
 
 // Results that go to several places, from fanout_from bytes of them on: the fold stores each result once (to
 // dst[0], with ordinary stores) and a second launch copies it to the other places, one place at a time in runs
@@ -536,88 +656,26 @@ int build_batches_impl(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op
             return build_wide_batches_impl(wide.data(), nseg, dtype, op, HCCLX_FOLD_CHAIN, plain_store, out);
         }
     }
-    const int esz = dtype_size(dtype);
-    if (esz == 0) return fail(HCCL_E_NOT_SUPPORT, "unknown data type " + std::to_string(dtype));
-    if (mode != HCCLX_FOLD_CHAIN && mode != HCCLX_FOLD_SELF_FIRST && mode != HCCLX_FOLD_TREE) {
-        return fail(HCCL_E_PARA, "unknown fold mode");
-    }
-
-    uint32_t max_src = 0;
-    uint32_t max_depth = 0;  // tree mode: levels of the deepest tree
-    for (uint32_t i = 0; i < nseg; ++i) {
-        const hcclx_seg_t &s = segs[i];
-        if (s.nsrc == 0 || s.nsrc > HCCLX_MAX_FAN || s.ndst == 0 || s.ndst > HCCLX_MAX_FAN) {
-            return fail(HCCL_E_PARA, "segment " + std::to_string(i) + ": nsrc/ndst outside 1.." +
-                                         std::to_string(HCCLX_MAX_FAN));
-        }
-        if (mode == HCCLX_FOLD_SELF_FIRST && s.nsrc != s.ndst) {
-            return fail(HCCL_E_PARA, "self-first fold needs nsrc == ndst");
-        }
-        if (s.count != 0) {
-            for (uint32_t k = 0; k < s.nsrc; ++k) {
-                if (s.src[k] == nullptr) return fail(HCCL_E_PTR, "segment " + std::to_string(i) + ": null source");
-            }
-            for (uint32_t k = 0; k < s.ndst; ++k) {
-                if (s.dst[k] == nullptr) return fail(HCCL_E_PTR, "segment " + std::to_string(i) + ": null destination");
-            }
-        }
-        if (mode == HCCLX_FOLD_TREE) {
-            const int levels = tree_levels(s.nsrc, s.prog);
-            if (levels < 0) return fail(HCCL_E_PARA, "segment " + std::to_string(i) + ": malformed tree program");
-            if (is_float_dtype(dtype) && (1u << levels) > HCCLX_MAX_FAN) {
-                return fail(HCCL_E_NOT_SUPPORT, "segment " + std::to_string(i) + ": tree has " + std::to_string(levels) +
-                                                    " levels, the kernel holds 4");
-            }
-            if (static_cast<uint32_t>(levels) > max_depth) max_depth = static_cast<uint32_t>(levels);
-        }
-        if (s.nsrc > max_src) max_src = s.nsrc;
-    }
-
+    SegProto sp;
+    const int rc = check_segs(segs, nseg, dtype, op, mode, &sp);
+    if (rc != HCCL_SUCCESS) return rc;
     Batch proto;
-    proto.copy = (max_src <= 1);
+    proto.copy = sp.copy;
     proto.dtype = dtype;
     proto.op = op;
-    proto.mode = mode;
+    proto.mode = sp.mode;
+    proto.maxn = sp.maxn;
     proto.plain_store = plain_store;
-    if (!proto.copy) {
-        if (!is_reduce_dtype(dtype)) return fail(HCCL_E_NOT_SUPPORT, "data type cannot be reduced");
-        if (op < HCCL_REDUCE_SUM || op > HCCL_REDUCE_MIN) return fail(HCCL_E_NOT_SUPPORT, "unknown reduce op");
-        proto.maxn = max_src <= 2 ? 2 : max_src <= 4 ? 4 : max_src <= 8 ? 8 : 16;
-        // a tree needs one leaf slot per position of the complete tree of its depth
-        if (mode == HCCLX_FOLD_TREE && is_float_dtype(dtype) && (1 << max_depth) > proto.maxn) proto.maxn = 1 << max_depth;
-        // Integer folds are association-free: the self-first order gives the bits of the plain chain.
-        // The kernel for it exists only for floating types, so integers take the chain kernel with the
-        // self-first segment rewritten below.
-    } else {
-        proto.maxn = 1;
-        proto.mode = HCCLX_FOLD_CHAIN;
-    }
-    // likewise a tree over integers equals the chain of its leaves
-    const bool rewrite_self = (!proto.copy && mode != HCCLX_FOLD_CHAIN && !is_float_dtype(dtype));
-    if (rewrite_self) proto.mode = HCCLX_FOLD_CHAIN;
-
-    const int ne = proto.copy ? 16 : 16 / esz;
     Batch cur = proto;
     for (uint32_t i = 0; i < nseg; ++i) {
         const hcclx_seg_t &s = segs[i];
         if (s.count == 0) continue;
         SegDev sd;
-        std::memset(&sd, 0, sizeof(sd));
-        sd.count = proto.copy ? s.count * esz : s.count;  // the copy kernel counts bytes
-        sd.nsrc = s.nsrc;
-        sd.ndst = s.ndst;
-        for (uint32_t k = 0; k < s.nsrc; ++k) sd.src[k] = static_cast<const char *>(s.src[k]);
-        for (uint32_t k = 0; k < s.ndst; ++k) sd.dst[k] = static_cast<char *>(s.dst[k]);
-        if (mode == HCCLX_FOLD_CHAIN) {
-            for (uint32_t k = 1; k < s.nsrc; ++k) sd.tree_codes |= (s.prog[k] ? 1u : 0u) << k;   // acc (+) src[k] steps
-        }
-        if (proto.mode == HCCLX_FOLD_TREE && !embed_tree(s, static_cast<uint32_t>(proto.maxn), &sd)) {
+        uint64_t tiles = 0;
+        if (!make_segdev(s, sp, mode, &sd, &tiles)) {
             return fail(HCCL_E_NOT_SUPPORT, "segment " + std::to_string(i) + ": tree deeper than log2(" +
-                                                std::to_string(proto.maxn) + ") levels");
+                                                std::to_string(sp.maxn) + ") levels");
         }
-        sd.head = fold_head_of(sd.count, proto.copy ? 1 : esz, sd.dst[0]);
-        sd.shift = fold_shift_of(sd.head, proto.copy ? 1 : esz, fold_tile_vecs(proto.maxn), sd.dst[0]);
-        const uint64_t tiles = fold_tiles_of(sd.count, ne, fold_tile_vecs(proto.maxn), sd.head, sd.shift);
         if (static_cast<int>(cur.segs.size()) == kMaxSegsPerLaunch) {
             out->batches.push_back(std::move(cur));
             cur = proto;
@@ -625,7 +683,7 @@ int build_batches_impl(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op
         cur.total_tiles += tiles;
         cur.tile_end.push_back(cur.total_tiles);
         cur.segs.push_back(sd);
-        out->algo_bytes += static_cast<uint64_t>(s.nsrc + s.ndst) * s.count * esz;
+        out->algo_bytes += static_cast<uint64_t>(s.nsrc + s.ndst) * s.count * sp.esz;
     }
     if (!cur.segs.empty()) out->batches.push_back(std::move(cur));
     return HCCL_SUCCESS;
@@ -746,9 +804,9 @@ int build_wide_batches_impl(const hcclx_wide_seg_t *segs, uint32_t nseg, int dty
             for (uint32_t k = 1; k < s.nsrc; ++k) sd.leaf_mask |= static_cast<uint64_t>(s.prog[k] ? 1 : 0) << k;
         }
         if (proto.mode == HCCLX_FOLD_TREE) {
-            std::vector<uint8_t> code;
-            std::vector<int> slot_reg;
-            if (!embed_tree(s.nsrc, s.prog, kMaxWideFan, &code, &slot_reg)) {
+            uint8_t code[kMaxWideFan];
+            int slot_reg[kMaxWideFan];
+            if (!embed_tree(s.nsrc, s.prog, kMaxWideFan, code, slot_reg)) {
                 return fail(HCCL_E_NOT_SUPPORT, "segment " + std::to_string(i) + ": tree deeper than 6 levels");
             }
             for (uint32_t node = 1; node < static_cast<uint32_t>(kMaxWideFan); ++node) {
@@ -798,6 +856,22 @@ void fill_table(const Batch &b, char *h)
     if (!b.wide.empty()) std::memcpy(at, b.wide.data(), b.wide.size() * sizeof(SegWide));
 }
 
+hipError_t dispatch_fold(int dtype, int op, int maxn, int mode, const FoldLaunch &l)
+{
+    switch (dtype) {
+        case HCCL_DATA_TYPE_INT8: return fold_dispatch_i8(op, maxn, mode, l);
+        case HCCL_DATA_TYPE_INT16: return fold_dispatch_i16(op, maxn, mode, l);
+        case HCCL_DATA_TYPE_INT32: return fold_dispatch_i32(op, maxn, mode, l);
+        case HCCL_DATA_TYPE_INT64: return fold_dispatch_i64(op, maxn, mode, l);
+        case HCCL_DATA_TYPE_UINT64: return fold_dispatch_u64(op, maxn, mode, l);
+        case HCCL_DATA_TYPE_FP16: return fold_dispatch_f16(op, maxn, mode, l);
+        case HCCL_DATA_TYPE_FP32: return fold_dispatch_f32(op, maxn, mode, l);
+        case HCCL_DATA_TYPE_FP64: return fold_dispatch_f64(op, maxn, mode, l);
+        case HCCL_DATA_TYPE_BFP16: return fold_dispatch_bf16(op, maxn, mode, l);
+        default: return hipErrorInvalidValue;
+    }
+}
+
 int launch_batch(const DeviceCtx *ctx, const Batch &b, const char *d_table, hipStream_t stream)
 {
     if (!b.phased.jobs.empty()) {
@@ -823,23 +897,7 @@ int launch_batch(const DeviceCtx *ctx, const Batch &b, const char *d_table, hipS
     l.xcd_remap = b.xcd_remap;
     l.plain_store = b.plain_store;
     l.stream = stream;
-    hipError_t e;
-    if (b.copy) {
-        e = fold_dispatch_copy(l);
-    } else {
-        switch (b.dtype) {
-            case HCCL_DATA_TYPE_INT8: e = fold_dispatch_i8(b.op, b.maxn, b.mode, l); break;
-            case HCCL_DATA_TYPE_INT16: e = fold_dispatch_i16(b.op, b.maxn, b.mode, l); break;
-            case HCCL_DATA_TYPE_INT32: e = fold_dispatch_i32(b.op, b.maxn, b.mode, l); break;
-            case HCCL_DATA_TYPE_INT64: e = fold_dispatch_i64(b.op, b.maxn, b.mode, l); break;
-            case HCCL_DATA_TYPE_UINT64: e = fold_dispatch_u64(b.op, b.maxn, b.mode, l); break;
-            case HCCL_DATA_TYPE_FP16: e = fold_dispatch_f16(b.op, b.maxn, b.mode, l); break;
-            case HCCL_DATA_TYPE_FP32: e = fold_dispatch_f32(b.op, b.maxn, b.mode, l); break;
-            case HCCL_DATA_TYPE_FP64: e = fold_dispatch_f64(b.op, b.maxn, b.mode, l); break;
-            case HCCL_DATA_TYPE_BFP16: e = fold_dispatch_bf16(b.op, b.maxn, b.mode, l); break;
-            default: e = hipErrorInvalidValue; break;
-        }
-    }
+    const hipError_t e = b.copy ? fold_dispatch_copy(l) : dispatch_fold(b.dtype, b.op, b.maxn, b.mode, l);
     if (e != hipSuccess) return fail_hip(e, "fold kernel launch");
     return HCCL_SUCCESS;
 }
@@ -916,6 +974,72 @@ int hcclx_fold(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mo
     int rc = build_batches(segs, nseg, dtype, op, mode, &built);
     if (rc != HCCL_SUCCESS) return rc;
     return launch_built(ctx, built, static_cast<hipStream_t>(stream));
+}
+
+int hcclx_fold_static(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, void *stream)
+{
+    DeviceCtx *ctx = device_ctx();
+    if (!ctx) return HCCL_E_RUNTIME;
+    if (nseg != 0 && segs == nullptr) return fail(HCCL_E_PTR, "segs is null");
+    if (nseg > HCCLX_STATIC_MAX_SEGS) {
+        return fail(HCCL_E_PARA, "hcclx_fold_static takes at most " + std::to_string(HCCLX_STATIC_MAX_SEGS) +
+                                     " segments per call (its launch table is a fixed array); got " + std::to_string(nseg));
+    }
+    SegProto sp;
+    int rc = check_segs(segs, nseg, dtype, op, mode, &sp);
+    if (rc != HCCL_SUCCESS) return rc;
+    // the table as the kernels read it: tile_end[] (rounded up to 256 bytes), then the segment descriptors
+    alignas(16) char table[HCCLX_STATIC_TABLE_BYTES];
+    uint64_t *tile_end = reinterpret_cast<uint64_t *>(table);
+    uint32_t live = 0;
+    for (uint32_t i = 0; i < nseg; ++i) live += segs[i].count != 0 ? 1 : 0;
+    if (live == 0) return HCCL_SUCCESS;
+    const size_t seg_off = (static_cast<size_t>(live) * 8 + 255) & ~static_cast<size_t>(255);
+    const size_t bytes = seg_off + static_cast<size_t>(live) * sizeof(SegDev);
+    static_assert(((HCCLX_STATIC_MAX_SEGS * 8 + 255) & ~255) + HCCLX_STATIC_MAX_SEGS * sizeof(SegDev) <= HCCLX_STATIC_TABLE_BYTES,
+                  "the fixed launch table holds HCCLX_STATIC_MAX_SEGS segments");
+    std::memset(table, 0, seg_off);
+    SegDev *descs = reinterpret_cast<SegDev *>(table + seg_off);
+    uint64_t total = 0;
+    uint32_t at = 0;
+    for (uint32_t i = 0; i < nseg; ++i) {
+        if (segs[i].count == 0) continue;
+        uint64_t tiles = 0;
+        if (!make_segdev(segs[i], sp, mode, &descs[at], &tiles)) {
+            return fail(HCCL_E_NOT_SUPPORT, "segment " + std::to_string(i) + ": tree deeper than the kernel holds");
+        }
+        total += tiles;
+        tile_end[at++] = total;
+    }
+    if (total > 0x7fffffffull) return fail(HCCL_E_PARA, "too much data for one launch");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // the table travels in kernel arguments, piece by piece; the fold kernel follows on the same stream
+    for (size_t off = 0; off < bytes; off += kPutBytes) {
+        TablePiece piece;
+        const uint32_t n = static_cast<uint32_t>(bytes - off < kPutBytes ? bytes - off : kPutBytes);
+        std::memcpy(&piece, table + off, n);
+        hipLaunchKernelGGL(k_put_table, dim3(1), dim3(256), 0, st, piece, ctx->static_table + off, n);
+        const hipError_t pe = hipGetLastError();
+        if (pe != hipSuccess) return fail_hip(pe, "launch table upload");
+    }
+    FoldLaunch l;
+    l.tile_end = reinterpret_cast<const uint64_t *>(ctx->static_table);
+    l.segs = ctx->static_table + seg_off;
+    l.nseg = live;
+    l.total_tiles = total;
+    l.grid = grid_for(ctx, total);
+    l.wide_unroll = 1;
+    l.xcd_remap = 0;
+    l.plain_store = 0;
+    l.stream = st;
+    hipError_t e;
+    if (sp.copy) {
+        e = fold_dispatch_copy(l);
+    } else {
+        e = dispatch_fold(dtype, op, sp.maxn, sp.mode, l);
+    }
+    if (e != hipSuccess) return fail_hip(e, "fold kernel launch");
+    return HCCL_SUCCESS;
 }
 
 int hcclx_fold_wide(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, void *stream)

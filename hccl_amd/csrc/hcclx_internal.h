@@ -61,6 +61,9 @@ struct DeviceCtx {
     char *h_ring = nullptr;
     char *d_ring = nullptr;
     size_t ring_bytes = 0;
+    // Device address, on this GPU, of the library's fixed launch-table array (hcclx_fold_static): looked up once
+    // when the context is made.
+    char *static_table = nullptr;
 };
 
 // Returns the context of the current device, creating it on first use (nullptr + error set on failure).

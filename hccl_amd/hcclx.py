@@ -56,6 +56,16 @@ def fold(segs, dtype, op=0, mode=FOLD_CHAIN, stream=0):
     check(_lib.load().hcclx_fold(arr, n, int(dtype), int(op), int(mode), ctypes.c_void_p(stream)))
 
 
+STATIC_MAX_SEGS = 128
+
+
+def fold_static(segs, dtype, op=0, mode=FOLD_CHAIN, stream=0):
+    """fold() through the entry point that allocates nothing (hcclx_fold_static): at most STATIC_MAX_SEGS segments,
+    launch table in the library's fixed device array."""
+    arr, n = make_segs(segs)
+    check(_lib.load().hcclx_fold_static(arr, n, int(dtype), int(op), int(mode), ctypes.c_void_p(stream)))
+
+
 def fold_wide(segs, dtype, op=0, mode=FOLD_CHAIN, stream=0):
     """Fold of segments with up to 64 sources and destinations (chain or tree order)."""
     arr, n = make_wide_segs(segs)

@@ -101,6 +101,19 @@ int hcclx_fold(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mo
 /* The same for wide segments. */
 int hcclx_fold_wide(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, void *stream);
 
+/* hcclx_fold for callers that cannot allocate: code that runs under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments, same results bit for bit, but
+ * the launch table lives in a fixed array of HCCLX_STATIC_TABLE_BYTES bytes that every GPU the library runs on
+ * holds until the process ends, and reaches it through kernel arguments: the call makes no hipMalloc, hipFree,
+ * hipHostMalloc or copy, also on its first use (hcclx_init() on the device beforehand does the one-time set-up).
+ * At most HCCLX_STATIC_MAX_SEGS segments of at most HCCLX_MAX_FAN sources and destinations per call (more:
+ * HCCL_E_PARA); always the register-resident kernels, one launch, so large many-destination folds run slower than
+ * through hcclx_fold.  Every call on a GPU uses that GPU's one table: calls on the same stream follow each other
+ * safely, calls on different streams that may overlap in time race and must be ordered by the caller. */
+#define HCCLX_STATIC_MAX_SEGS 128
+#define HCCLX_STATIC_TABLE_BYTES 40960
+int hcclx_fold_static(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, void *stream);
+
 /* The same, split in two so that a repeated collective uploads its table once. */
 typedef struct hcclx_plan hcclx_plan_t;
 int hcclx_plan_create(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, hcclx_plan_t **plan);
