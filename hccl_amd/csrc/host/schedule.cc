@@ -902,6 +902,20 @@ std::vector<u64> PlanKey(const std::vector<OpParam> &params, const std::string &
         key.push_back(reinterpret_cast<u64>(p.outputPtr));
         key.push_back(p.inputSize);
     }
+    // The AlltoAll family: what moves is in every rank's tables, not in the extents above (an expert router
+    // changes the counts every step while the buffers stay where they are).
+    if (p0.opType == HcclCMDType::HCCL_CMD_ALLTOALL || p0.opType == HcclCMDType::HCCL_CMD_ALLTOALLV ||
+        p0.opType == HcclCMDType::HCCL_CMD_ALLTOALLVC) {
+        key.push_back(static_cast<u64>(p0.all2AllVDataDes.sendType));
+        for (const OpParam &p : params) {
+            const auto &d = p.all2AllVDataDes;
+            key.push_back(d.sendCounts.size());
+            key.insert(key.end(), d.sendCounts.begin(), d.sendCounts.end());
+            key.insert(key.end(), d.sdispls.begin(), d.sdispls.end());
+            key.insert(key.end(), d.recvCounts.begin(), d.recvCounts.end());
+            key.insert(key.end(), d.rdispls.begin(), d.rdispls.end());
+        }
+    }
     return key;
 }
 

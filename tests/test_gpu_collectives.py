@@ -596,3 +596,74 @@ def test_a_communicator_of_one_rank(stream, mode):
             assert recv.guard_intact(), call
     finally:
         w.close()
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_alltoallv_same_buffers_new_tables_every_step(stream, mode):
+    """An expert router changes the counts every step while the buffers stay where they are: the second call must
+    move what ITS tables say (step plans are cached, and the tables are part of what they are cached under)."""
+    n = 4
+    rows = 3000
+    rng = np.random.default_rng(33)
+    xs = [rng.integers(0, 65535, size=rows, dtype=np.uint16) for _ in range(n)]
+    send = [DevBuf(x) for x in xs]
+    recv = [DevBuf(nbytes=2 * n * rows) for _ in range(n)]
+    w = api.World(n, ccl_bytes=SMALL_CCL)
+    try:
+        w.set_mode(mode)
+        for step in range(3):
+            # every rank sends all its rows each step, split differently: same extents, different blocks
+            m = []
+            for i in range(n):
+                cut = np.sort(rng.integers(0, rows + 1, size=n - 1))
+                m.append([int(c) for c in np.diff(np.concatenate([[0], cut, [rows]]))])
+            v = [T.alltoallvc_to_v(m, r) for r in range(n)]
+            for b in recv:
+                b.t.fill_(0xA5)
+            torch.cuda.synchronize()
+            for r in range(n):
+                sc, sd, rc, rd = v[r]
+                assert w.all_to_all_v(r, send[r].ptr, sc, sd, recv[r].ptr, rc, rd, T.BFP16, stream.cuda_stream) == 0
+            stream.synchronize()
+            info = w.last_info()
+            assert bool(info.fused) == (mode == api.EXEC_FUSED)
+            want = T.run_alltoallv(xs, [x[0] for x in v], [x[1] for x in v], [x[2] for x in v], [x[3] for x in v],
+                                   [sum(x[2]) for x in v])
+            for r in range(n):
+                got = recv[r].get(np.uint16)[:len(want[r])]
+                assert np.array_equal(got, want[r]), (mode, step, r)
+    finally:
+        w.close()
+
+
+def test_ranks_on_different_streams_one_host_thread(stream):
+    """One host thread issues every rank's call, each on that rank's own stream (the default, non-blocking
+    rendezvous).  The collective enters every rank's stream when the LAST rank calls: what a stream holds before
+    that moment (here: the kernels that produce the inputs) runs before it, what is enqueued afterwards (here: the
+    consumers) runs after it."""
+    n, count = 6, 200000
+    w = api.World(n)
+    try:
+        streams = [torch.cuda.Stream() for _ in range(n)]
+        base = [torch.arange(count, device="cuda:0", dtype=torch.float32) * (r + 1) for r in range(n)]
+        send = [torch.zeros(count, device="cuda:0") for _ in range(n)]
+        recv = [torch.zeros(count, device="cuda:0") for _ in range(n)]
+        seen = [torch.zeros(count, device="cuda:0") for _ in range(n)]
+        torch.cuda.synchronize()
+        for it in range(1, 4):
+            for r in range(n):
+                with torch.cuda.stream(streams[r]):
+                    for _ in range(20):                      # a producer that takes a while
+                        send[r].copy_(base[r] * it)
+                assert w.all_reduce(r, send[r].data_ptr(), recv[r].data_ptr(), count, T.FP32, T.SUM,
+                                    streams[r].cuda_stream) == 0
+            for r in range(n):                               # consumers, after every rank has called
+                with torch.cuda.stream(streams[r]):
+                    seen[r].copy_(recv[r])
+            for s in streams:
+                s.synchronize()
+            want = torch.arange(count, device="cuda:0", dtype=torch.float32) * (it * n * (n + 1) // 2)
+            for r in range(n):
+                assert torch.equal(seen[r], want), (it, r)     # exact: small integers in fp32
+    finally:
+        w.close()
