@@ -856,6 +856,16 @@ void fill_table(const Batch &b, char *h)
     if (!b.wide.empty()) std::memcpy(at, b.wide.data(), b.wide.size() * sizeof(SegWide));
 }
 
+// The common tile count of the segments of a launch, or 0 when they differ (or it does not fit 32 bits).
+uint32_t uniform_tiles_of(const uint64_t *tile_end, size_t nseg)
+{
+    if (nseg < 2 || tile_end[0] == 0 || tile_end[0] > 0xffffffffull) return 0;
+    for (size_t i = 1; i < nseg; ++i) {
+        if (tile_end[i] != tile_end[0] * (i + 1)) return 0;
+    }
+    return static_cast<uint32_t>(tile_end[0]);
+}
+
 hipError_t dispatch_fold(int dtype, int op, int maxn, int mode, const FoldLaunch &l)
 {
     switch (dtype) {
@@ -896,6 +906,7 @@ int launch_batch(const DeviceCtx *ctx, const Batch &b, const char *d_table, hipS
     l.wide_unroll = b.wide_unroll;
     l.xcd_remap = b.xcd_remap;
     l.plain_store = b.plain_store;
+    l.uniform_tiles = uniform_tiles_of(b.tile_end.data(), b.tile_end.size());
     l.stream = stream;
     const hipError_t e = b.copy ? fold_dispatch_copy(l) : dispatch_fold(b.dtype, b.op, b.maxn, b.mode, l);
     if (e != hipSuccess) return fail_hip(e, "fold kernel launch");
@@ -1031,6 +1042,7 @@ int hcclx_fold_static(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op,
     l.wide_unroll = 1;
     l.xcd_remap = 0;
     l.plain_store = 0;
+    l.uniform_tiles = uniform_tiles_of(tile_end, live);
     l.stream = st;
     hipError_t e;
     if (sp.copy) {

@@ -211,6 +211,94 @@ HcclResult SendRecvReadReduce(const SendRecvReduceInfo &info, const ThreadHandle
     return R(HcommChannelNotifyWaitOnThread(thread, tx.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
 }
 
+// ---- batch verbs: every slice of the call in one descriptor array (wrapper.cc:99-125), between the handshakes of
+//      the per-slice verbs (DoSendBatchTx :151-168, DoSendRecvBatchTx :127-149, DoRecvBatchRx :171-187)
+
+namespace {
+
+HcclResult RunBatch(const ThreadHandle &thread, const ChannelInfo &ch, const std::vector<DataSlice> &src,
+                    const std::vector<DataSlice> &dst, HcclHcommTransferType type, bool reduce, HcclDataType dataType,
+                    HcclReduceOp reduceOp)
+{
+    std::vector<HcclHcommBatchTransferDesc> descs;
+    for (size_t i = 0; i < src.size(); ++i) {
+        if (src[i].size_ == 0) continue;   // :110-113
+        HcclHcommBatchTransferDesc d = {};
+        d.transType = type;
+        if (reduce) {
+            CHK_RET(CheckReduceSlices(src[i], dst[i], dataType));
+            d.transferInfo.reduce.count = src[i].count_;
+            d.transferInfo.reduce.dst = GetSliceAddr(dst[i]);
+            d.transferInfo.reduce.src = GetSliceAddr(src[i]);
+            d.transferInfo.reduce.dataType = dataType;
+            d.transferInfo.reduce.reduceOp = reduceOp;
+        } else {
+            d.transferInfo.write.len = src[i].size_;
+            d.transferInfo.write.dst = GetSliceAddr(dst[i]);
+            d.transferInfo.write.src = GetSliceAddr(src[i]);
+        }
+        descs.push_back(d);
+    }
+    if (descs.empty()) return HCCL_SUCCESS;
+    return R(HcommBatchTransferOnThread(thread, ch.handle, descs.data(), static_cast<uint32_t>(descs.size())));
+}
+
+}  // namespace
+
+HcclResult SendBatchWrite(const DataInfo &sendInfo, const ThreadHandle &thread)
+{
+    const ChannelInfo &ch = sendInfo.channel_;
+    CHK_RET(HcommChannelNotifyWaitOnThread(thread, ch.handle, NOTIFY_IDX_ACK, kTimeout));
+    CHK_RET(RunBatch(thread, ch, sendInfo.slices_.srcSlices_, sendInfo.slices_.dstSlices_, HCCL_HCOMM_TRANSFER_TYPE_WRITE,
+                     false, HCCL_DATA_TYPE_INT8, HCCL_REDUCE_SUM));
+    return R(HcommChannelNotifyRecordOnThread(thread, ch.handle, NOTIFY_IDX_DATA_SIGNAL));
+}
+
+HcclResult SendRecvBatchWrite(const SendRecvInfo &info, const ThreadHandle &thread)
+{
+    const ChannelInfo &tx = info.sendRecvChannels_.txChannel_;
+    const ChannelInfo &rx = info.sendRecvChannels_.rxChannel_;
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, rx.handle, NOTIFY_IDX_ACK));
+    CHK_RET(HcommChannelNotifyWaitOnThread(thread, tx.handle, NOTIFY_IDX_ACK, kTimeout));
+    CHK_RET(RunBatch(thread, tx, info.sendRecvSlices_.txSlicesList_.srcSlices_, info.sendRecvSlices_.txSlicesList_.dstSlices_,
+                     HCCL_HCOMM_TRANSFER_TYPE_WRITE, false, HCCL_DATA_TYPE_INT8, HCCL_REDUCE_SUM));
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, tx.handle, NOTIFY_IDX_DATA_SIGNAL));
+    return R(HcommChannelNotifyWaitOnThread(thread, rx.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+}
+
+HcclResult SendRecvBatchWriteReduce(const SendRecvReduceInfo &info, const ThreadHandle &thread)
+{
+    const ChannelInfo &tx = info.sendRecvChannels_.txChannel_;
+    const ChannelInfo &rx = info.sendRecvChannels_.rxChannel_;
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, rx.handle, NOTIFY_IDX_ACK));
+    CHK_RET(HcommChannelNotifyWaitOnThread(thread, tx.handle, NOTIFY_IDX_ACK, kTimeout));
+    CHK_RET(RunBatch(thread, tx, info.sendRecvSlices_.txSlicesList_.srcSlices_, info.sendRecvSlices_.txSlicesList_.dstSlices_,
+                     HCCL_HCOMM_TRANSFER_TYPE_WRITE_REDUCE, true, info.dataType_, info.reduceType_));
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, tx.handle, NOTIFY_IDX_DATA_SIGNAL));
+    return R(HcommChannelNotifyWaitOnThread(thread, rx.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+}
+
+HcclResult RecvBatchRead(const DataInfo &recvInfo, const ThreadHandle &thread)
+{
+    const ChannelInfo &ch = recvInfo.channel_;
+    CHK_RET(HcommChannelNotifyWaitOnThread(thread, ch.handle, NOTIFY_IDX_ACK, kTimeout));
+    CHK_RET(RunBatch(thread, ch, recvInfo.slices_.srcSlices_, recvInfo.slices_.dstSlices_, HCCL_HCOMM_TRANSFER_TYPE_READ,
+                     false, HCCL_DATA_TYPE_INT8, HCCL_REDUCE_SUM));
+    return R(HcommChannelNotifyRecordOnThread(thread, ch.handle, NOTIFY_IDX_DATA_SIGNAL));
+}
+
+HcclResult SendRecvBatchRead(const SendRecvInfo &info, const ThreadHandle &thread)
+{
+    const ChannelInfo &tx = info.sendRecvChannels_.txChannel_;
+    const ChannelInfo &rx = info.sendRecvChannels_.rxChannel_;
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, tx.handle, NOTIFY_IDX_ACK));
+    CHK_RET(HcommChannelNotifyWaitOnThread(thread, rx.handle, NOTIFY_IDX_ACK, kTimeout));
+    CHK_RET(RunBatch(thread, rx, info.sendRecvSlices_.rxSlicesList_.srcSlices_, info.sendRecvSlices_.rxSlicesList_.dstSlices_,
+                     HCCL_HCOMM_TRANSFER_TYPE_READ, false, HCCL_DATA_TYPE_INT8, HCCL_REDUCE_SUM));
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, rx.handle, NOTIFY_IDX_DATA_SIGNAL));
+    return R(HcommChannelNotifyWaitOnThread(thread, tx.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+}
+
 // ---- main thread <-> sub threads
 
 HcclResult PreSyncInterThreads(const ThreadHandle &mainThread, const std::vector<ThreadHandle> &subThreads,

@@ -1,7 +1,7 @@
 // The data-movement verbs the templates call (reference: src/ops/op_common/template/wrapper/
 // alg_data_trans_wrapper.{h,cc}).  Each verb checks its slices and expands to the primitive calls and the
-// ACK / DATA_SIGNAL handshakes of the reference, in the reference's order; the *Batch* names take the
-// reference's per-slice fall-back path (wrapper.cc:127-226), which is what its system tests run.
+// ACK / DATA_SIGNAL handshakes of the reference, in the reference's order.  The *Batch* verbs hand all slices of a
+// call to HcommBatchTransferOnThread in one descriptor array, between the same handshakes (wrapper.cc:99-226).
 #pragma once
 #include "alg_param.h"
 
@@ -23,14 +23,11 @@ HcclResult SendRecvRead(const SendRecvInfo &sendRecvInfo, const ThreadHandle &th
 HcclResult SendRecvWriteReduce(const SendRecvReduceInfo &sendRecvInfo, const ThreadHandle &thread);
 HcclResult SendRecvReadReduce(const SendRecvReduceInfo &sendRecvInfo, const ThreadHandle &thread);
 
-inline HcclResult SendBatchWrite(const DataInfo &i, const ThreadHandle &t) { return SendWrite(i, t); }
-inline HcclResult SendRecvBatchWrite(const SendRecvInfo &i, const ThreadHandle &t) { return SendRecvWrite(i, t); }
-inline HcclResult RecvBatchRead(const DataInfo &i, const ThreadHandle &t) { return RecvRead(i, t); }
-inline HcclResult SendRecvBatchRead(const SendRecvInfo &i, const ThreadHandle &t) { return SendRecvRead(i, t); }
-inline HcclResult SendRecvBatchWriteReduce(const SendRecvReduceInfo &i, const ThreadHandle &t)
-{
-    return SendRecvWriteReduce(i, t);
-}
+HcclResult SendBatchWrite(const DataInfo &sendInfo, const ThreadHandle &thread);
+HcclResult SendRecvBatchWrite(const SendRecvInfo &sendRecvInfo, const ThreadHandle &thread);
+HcclResult RecvBatchRead(const DataInfo &recvInfo, const ThreadHandle &thread);
+HcclResult SendRecvBatchRead(const SendRecvInfo &sendRecvInfo, const ThreadHandle &thread);
+HcclResult SendRecvBatchWriteReduce(const SendRecvReduceInfo &sendRecvInfo, const ThreadHandle &thread);
 
 HcclResult PreSyncInterThreads(const ThreadHandle &mainThread, const std::vector<ThreadHandle> &subThreads,
                                const std::vector<u32> &notifyIdxMainToSub);

@@ -346,6 +346,65 @@ int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, u
     return RecordNotify(t, ItemKind::NOTIFY_WAIT, ThreadKey(t, notifyIdx));
 }
 
+int32_t HcommBatchTransferOnThread(ThreadHandle thread, ChannelHandle channel,
+                                   const HcclHcommBatchTransferDesc *transferDescs, uint32_t transferDescNum)
+{
+    if (AsThread(thread) == nullptr || AsChannel(channel) == nullptr) return HCCL_E_PTR;
+    if (transferDescNum != 0 && transferDescs == nullptr) return HCCL_E_PTR;
+    for (uint32_t i = 0; i < transferDescNum; ++i) {
+        const HcclHcommBatchTransferDesc &d = transferDescs[i];
+        int32_t rc = HCCL_SUCCESS;
+        switch (d.transType) {
+            case HCCL_HCOMM_TRANSFER_TYPE_WRITE:
+                rc = HcommWriteOnThread(thread, channel, d.transferInfo.write.dst, d.transferInfo.write.src,
+                                        d.transferInfo.write.len);
+                break;
+            case HCCL_HCOMM_TRANSFER_TYPE_READ:
+                rc = HcommReadOnThread(thread, channel, d.transferInfo.read.dst, d.transferInfo.read.src,
+                                       d.transferInfo.read.len);
+                break;
+            case HCCL_HCOMM_TRANSFER_TYPE_WRITE_REDUCE:
+                rc = HcommWriteReduceOnThread(thread, channel, d.transferInfo.reduce.dst, d.transferInfo.reduce.src,
+                                              d.transferInfo.reduce.count, d.transferInfo.reduce.dataType,
+                                              d.transferInfo.reduce.reduceOp);
+                break;
+            case HCCL_HCOMM_TRANSFER_TYPE_READ_REDUCE:
+                rc = HcommReadReduceOnThread(thread, channel, d.transferInfo.reduce.dst, d.transferInfo.reduce.src,
+                                             d.transferInfo.reduce.count, d.transferInfo.reduce.dataType,
+                                             d.transferInfo.reduce.reduceOp);
+                break;
+            case HCCL_HCOMM_TRANSFER_TYPE_WRITE_WITH_NOTIFY:
+                rc = HcommWriteOnThread(thread, channel, d.transferInfo.writeWithNotify.dst,
+                                        d.transferInfo.writeWithNotify.src, d.transferInfo.writeWithNotify.len);
+                if (rc == HCCL_SUCCESS) {
+                    rc = HcommChannelNotifyRecordOnThread(thread, channel, d.transferInfo.writeWithNotify.notifyIdx);
+                }
+                break;
+            case HCCL_HCOMM_TRANSFER_TYPE_WRITE_REDUCE_WITH_NOTIFY:
+                rc = HcommWriteReduceOnThread(thread, channel, d.transferInfo.writeReduceWithNotify.dst,
+                                              d.transferInfo.writeReduceWithNotify.src,
+                                              d.transferInfo.writeReduceWithNotify.count,
+                                              d.transferInfo.writeReduceWithNotify.dataType,
+                                              d.transferInfo.writeReduceWithNotify.reduceOp);
+                if (rc == HCCL_SUCCESS) {
+                    rc = HcommChannelNotifyRecordOnThread(thread, channel, d.transferInfo.writeReduceWithNotify.notifyIdx);
+                }
+                break;
+            case HCCL_HCOMM_TRANSFER_TYPE_NOTIFY_RECORD:
+                rc = HcommChannelNotifyRecordOnThread(thread, channel, d.transferInfo.notifyRecord.notifyIdx);
+                break;
+            case HCCL_HCOMM_TRANSFER_TYPE_NOTIFY_WAIT:
+            case HCCL_HCOMM_TRANSFER_TYPE_NOTIFY_WAIT_WITH_DEFAULT_TIMEOUT:
+                rc = HcommChannelNotifyWaitOnThread(thread, channel, d.transferInfo.notifyRecord.notifyIdx, 0);
+                break;
+            default:
+                return HCCL_E_PARA;
+        }
+        if (rc != HCCL_SUCCESS) return rc;
+    }
+    return HCCL_SUCCESS;
+}
+
 int32_t HcommBatchModeStart(const char *batchTag)
 {
     (void)batchTag;

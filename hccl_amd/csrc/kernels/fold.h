@@ -288,8 +288,17 @@ __device__ __forceinline__ uint64_t remap_tile(uint64_t t, uint64_t total)
 // Maps tile number t of a launch to its segment (the first one whose inclusive tile prefix exceeds t) and
 // to the tile's number inside that segment.  Every value is wave-uniform.
 __device__ __forceinline__ void locate_tile(const uint64_t *__restrict__ tile_end, const uint64_t *s_end, uint32_t nseg,
-                                            bool direct, uint64_t t, uint32_t *seg, uint64_t *tile_in_seg)
+                                            bool direct, uint32_t uniform_tiles, uint64_t t, uint32_t *seg,
+                                            uint64_t *tile_in_seg)
 {
+    if (uniform_tiles != 0) {
+        // every segment has this many tiles (the slices of a two-shot, ring or NHR AllReduce): no table to search.
+        // A search is a chain of dependent loads, which a launch of a few hundred workgroups cannot hide.
+        const uint64_t s = t / uniform_tiles;
+        *seg = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(s));
+        *tile_in_seg = uniform64(t - s * uniform_tiles);
+        return;
+    }
     uint32_t lo = 0;
     uint32_t hi = nseg - 1;
     uint64_t before = 0;   // tiles of the segments in front of the one found
@@ -321,7 +330,7 @@ __device__ __forceinline__ void locate_tile(const uint64_t *__restrict__ tile_en
 template <int DT, int OP, int MAXN, int MODE>
 __global__ void __launch_bounds__(kFoldThreads)
 k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, uint32_t nseg, uint64_t total_tiles,
-       uint32_t plain_store)
+       uint32_t plain_store, uint32_t uniform_tiles)
 {
     const bool plain = plain_store != 0;
     constexpr int NE = Vec16<DT>::kElems;   // elements per 16-byte vector
@@ -330,7 +339,7 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
     // Few segments: the prefix is searched where it lies (every index is wave-uniform, so these are scalar
     // loads that hit the constant cache after the first workgroup); staging it in LDS would cost a barrier
     // before the first data load.  Many segments: staged once per workgroup.
-    const bool direct = nseg <= kFoldDirectSegs;
+    const bool direct = nseg <= kFoldDirectSegs || uniform_tiles != 0;
     if (!direct) {
         for (uint32_t i = threadIdx.x; i < nseg; i += kFoldThreads) {
             s_end[i] = tile_end[i];
@@ -341,7 +350,7 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
     for (uint64_t t = blockIdx.x; t < total_tiles; t += gridDim.x) {
         uint32_t s;
         uint64_t tl;
-        locate_tile(tile_end, s_end, nseg, direct, t, &s, &tl);
+        locate_tile(tile_end, s_end, nseg, direct, uniform_tiles, t, &s, &tl);
         const SegDev &sd = segs[s];
         const uint32_t nsrc = sd.nsrc;
         const uint32_t ndst = sd.ndst;
@@ -559,14 +568,14 @@ __device__ __forceinline__ void fold_tile_wide_self(const SegWide &sd, uint32_t 
 template <int DT, int OP, int MODE, int U>
 __global__ void __launch_bounds__(kFoldThreads)
 k_fold_wide(const uint64_t *__restrict__ tile_end, const SegWide *__restrict__ segs, uint32_t nseg, uint64_t total_tiles,
-            uint32_t xcd_remap, uint32_t plain_store)
+            uint32_t xcd_remap, uint32_t plain_store, uint32_t uniform_tiles)
 {
     constexpr int NE = Vec16<DT>::kElems;
     const bool plain = plain_store != 0;
     static_assert(MODE == kFoldChain || U == 1, "only the chain moves several vectors per thread");
     constexpr uint64_t TV = wide_tile_vecs(U);
     extern __shared__ uint64_t s_end[];
-    const bool direct = nseg <= kFoldDirectSegs;
+    const bool direct = nseg <= kFoldDirectSegs || uniform_tiles != 0;
     if (!direct) {
         for (uint32_t i = threadIdx.x; i < nseg; i += kFoldThreads) {
             s_end[i] = tile_end[i];
@@ -576,7 +585,7 @@ k_fold_wide(const uint64_t *__restrict__ tile_end, const SegWide *__restrict__ s
     for (uint64_t t = blockIdx.x; t < total_tiles; t += gridDim.x) {
         uint32_t s;
         uint64_t tl;
-        locate_tile(tile_end, s_end, nseg, direct, xcd_remap ? remap_tile(t, total_tiles) : t, &s, &tl);
+        locate_tile(tile_end, s_end, nseg, direct, uniform_tiles, xcd_remap ? remap_tile(t, total_tiles) : t, &s, &tl);
         const SegWide &sd = segs[s];
         const uint32_t nsrc = sd.nsrc;
         const uint32_t ndst = sd.ndst;
@@ -653,6 +662,7 @@ struct FoldLaunch {
     int wide_unroll;           // the wide chain kernel: vectors per thread (kWideUnrollMany or kWideUnrollOne)
     uint32_t xcd_remap;        // the wide kernels: give each XCD a contiguous eighth of the tiles
     uint32_t plain_store;      // chain and tree: results are stored the ordinary way (a fan-out launch reads them next)
+    uint32_t uniform_tiles;    // non-zero: every segment has this many tiles, tile t belongs to segment t / uniform_tiles
     hipStream_t stream;
 };
 

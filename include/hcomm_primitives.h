@@ -44,6 +44,44 @@ int32_t HcommChannelNotifyWaitOnThread(ThreadHandle thread, ChannelHandle channe
 /* Main thread <-> sub thread fan-out / fan-in inside one rank.          hccl_stub.cc:449, :397 */
 int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThread, uint32_t dstNotifyIdx);
 int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, uint32_t timeout);
+/* Several transfers and handshakes on one channel in one call: what every *Batch* verb of the wrapper issues first
+ * (src/ops/op_common/template/wrapper/alg_data_trans_wrapper.cc:99-125) and falls back from, slice by slice, when
+ * libhcomm does not export it.  The reference resolves the symbol by this name
+ * (src/common/hcomm_dlsym/hcomm_primitives_dl.cc:115-116); the descriptor is its ABI-compatible mirror
+ * (src/common/hcomm_dlsym/hcomm_primitives_dl.h:26-79).  Descriptors are carried out in array order: WRITE / READ
+ * copy `len` bytes, the *_REDUCE kinds do dst = src (+) dst on `count` elements, NOTIFY_RECORD / NOTIFY_WAIT are the
+ * channel handshakes, and the *_WITH_NOTIFY kinds record the notify after their transfer. */
+typedef enum {
+    HCCL_HCOMM_TRANSFER_TYPE_INVALID = -1,
+    HCCL_HCOMM_TRANSFER_TYPE_WRITE = 0,
+    HCCL_HCOMM_TRANSFER_TYPE_WRITE_REDUCE = 1,
+    HCCL_HCOMM_TRANSFER_TYPE_WRITE_WITH_NOTIFY = 2,
+    HCCL_HCOMM_TRANSFER_TYPE_WRITE_REDUCE_WITH_NOTIFY = 3,
+    HCCL_HCOMM_TRANSFER_TYPE_READ = 4,
+    HCCL_HCOMM_TRANSFER_TYPE_READ_REDUCE = 5,
+    HCCL_HCOMM_TRANSFER_TYPE_NOTIFY_RECORD = 6,
+    HCCL_HCOMM_TRANSFER_TYPE_NOTIFY_WAIT = 7,
+    HCCL_HCOMM_TRANSFER_TYPE_NOTIFY_WAIT_WITH_DEFAULT_TIMEOUT = 8
+} HcclHcommTransferType;
+
+typedef struct {
+    HcclHcommTransferType transType;
+    uint8_t reserved[4];
+    union {
+        uint8_t raws[56];
+        struct { uint64_t len; void *dst; void *src; } write;
+        struct { uint64_t len; void *dst; void *src; } read;
+        struct { uint64_t count; void *dst; void *src; HcommReduceOp reduceOp; HcommDataType dataType; } reduce;
+        struct { uint32_t notifyIdx; } notifyRecord;
+        struct { uint64_t len; void *dst; void *src; uint32_t notifyIdx; } writeWithNotify;
+        struct { uint64_t count; void *dst; void *src; HcommReduceOp reduceOp; HcommDataType dataType;
+                 uint32_t notifyIdx; } writeReduceWithNotify;
+    } transferInfo;
+} HcclHcommBatchTransferDesc;
+
+int32_t HcommBatchTransferOnThread(ThreadHandle thread, ChannelHandle channel,
+                                   const HcclHcommBatchTransferDesc *transferDescs, uint32_t transferDescNum);
+
 /* Flush / join before CPU-side work.  Stream order already gives that here.   hccl_stub.cc:799, :805, :937 */
 int32_t HcommBatchModeStart(const char *batchTag);
 int32_t HcommBatchModeEnd(const char *batchTag);
