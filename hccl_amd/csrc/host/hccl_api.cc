@@ -226,7 +226,7 @@ HcclResult hcclxCommGetLastOpInfo(HcclComm comm, hcclxLastOpInfo *info)
     info->launches = w->lastLaunches;
     info->fusedSegments = w->lastFusedSegments;
     info->fused = w->lastWasFused ? 1 : 0;
-    info->planCacheHit = w->lastPlanCacheHit ? 1 : 0;
+    info->planCacheHit = w->lastPlanCacheHit;
     return HCCL_SUCCESS;
 }
 

@@ -1,6 +1,9 @@
 #include "schedule.h"
 
 #include <algorithm>
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <functional>
 #include <map>
@@ -193,13 +196,17 @@ HcclResult BuildOrder(World *w, std::vector<Node> &order, u32 &numLevels, CheckR
 // ---------------------------------------------------------------------------------------------------
 // STEP mode: the recorded steps as they are, level by level; the copies of a level are one launch and its
 // reduce steps another.  The launches are built as plans so that a repeated collective only replays them.
-HcclResult BuildStepPlans(const std::vector<Node> &order, u32 numLevels, int dtype, int op,
-                          std::vector<hcclx_plan *> &plans)
+void BuildStepParts(const std::vector<Node> &order, u32 numLevels, int dtype, int op, std::vector<HostPart> &parts)
 {
     size_t i = 0;
     for (u32 level = 0; level < numLevels; ++level) {
-        std::vector<hcclx_seg_t> copies;
-        std::vector<hcclx_seg_t> reduces;
+        HostPart copies;
+        copies.dtype = HCCL_DATA_TYPE_INT8;
+        copies.mode = HCCLX_FOLD_CHAIN;
+        HostPart reduces;
+        reduces.dtype = dtype;
+        reduces.op = op;
+        reduces.mode = HCCLX_FOLD_CHAIN;
         for (; i < order.size() && order[i].level == level; ++i) {
             const TaskItem &it = *order[i].item;
             hcclx_seg_t s;
@@ -210,7 +217,7 @@ HcclResult BuildStepPlans(const std::vector<Node> &order, u32 numLevels, int dty
                 s.ndst = 1;
                 s.src[0] = it.src;
                 s.dst[0] = it.dst;
-                copies.push_back(s);
+                copies.segs.push_back(s);
             } else {
                 s.count = it.count;
                 s.nsrc = 2;  // dst = src (+) dst: the accumulator comes first in fold order
@@ -218,20 +225,12 @@ HcclResult BuildStepPlans(const std::vector<Node> &order, u32 numLevels, int dty
                 s.src[0] = it.dst;
                 s.src[1] = it.src;
                 s.dst[0] = it.dst;
-                reduces.push_back(s);
+                reduces.segs.push_back(s);
             }
         }
-        for (int part = 0; part < 2; ++part) {
-            const std::vector<hcclx_seg_t> &segs = part == 0 ? copies : reduces;
-            if (segs.empty()) continue;
-            hcclx_plan *hp = nullptr;
-            const int rc = hcclx_plan_create(segs.data(), static_cast<uint32_t>(segs.size()),
-                                             part == 0 ? HCCL_DATA_TYPE_INT8 : dtype, part == 0 ? 0 : op, HCCLX_FOLD_CHAIN, &hp);
-            if (rc != HCCL_SUCCESS) return static_cast<HcclResult>(rc);
-            plans.push_back(hp);
-        }
+        if (!copies.segs.empty()) parts.push_back(std::move(copies));
+        if (!reduces.segs.empty()) parts.push_back(std::move(reduces));
     }
-    return HCCL_SUCCESS;
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -882,12 +881,13 @@ void CheckSemantics(const Tracer &tr, const std::vector<OpParam> &params, CheckR
     }
 }
 
-// What a cached plan depends on, as plain numbers (a string would cost more to build than the launch).
-std::vector<u64> PlanKey(const std::vector<OpParam> &params, const std::string &alg, u64 cclBytes)
+// What the plan of a collective depends on apart from where the buffers lie, as plain numbers (a string would cost
+// more to build than the launch).  The last words say which ranks run in place.
+std::vector<u64> ShapeKey(const std::vector<OpParam> &params, const std::string &alg, u64 cclBytes)
 {
     const OpParam &p0 = params[0];
     std::vector<u64> key;
-    key.reserve(8 + 2 * p0.vDataDes.counts.size() + 3 * params.size());
+    key.reserve(10 + 2 * p0.vDataDes.counts.size() + 2 * params.size());
     key.push_back(static_cast<u64>(p0.opType));
     key.push_back(std::hash<std::string>()(alg));
     key.push_back(static_cast<u64>(p0.DataDes.dataType));
@@ -897,13 +897,8 @@ std::vector<u64> PlanKey(const std::vector<OpParam> &params, const std::string &
     key.push_back(p0.vDataDes.counts.size());
     key.insert(key.end(), p0.vDataDes.counts.begin(), p0.vDataDes.counts.end());
     key.insert(key.end(), p0.vDataDes.displs.begin(), p0.vDataDes.displs.end());
-    for (const OpParam &p : params) {
-        key.push_back(reinterpret_cast<u64>(p.inputPtr));
-        key.push_back(reinterpret_cast<u64>(p.outputPtr));
-        key.push_back(p.inputSize);
-    }
-    // The AlltoAll family: what moves is in every rank's tables, not in the extents above (an expert router
-    // changes the counts every step while the buffers stay where they are).
+    // The AlltoAll family: what moves is in every rank's tables, not in the extents (an expert router changes the
+    // counts every step while the buffers stay where they are).
     if (p0.opType == HcclCMDType::HCCL_CMD_ALLTOALL || p0.opType == HcclCMDType::HCCL_CMD_ALLTOALLV ||
         p0.opType == HcclCMDType::HCCL_CMD_ALLTOALLVC) {
         key.push_back(static_cast<u64>(p0.all2AllVDataDes.sendType));
@@ -916,7 +911,124 @@ std::vector<u64> PlanKey(const std::vector<OpParam> &params, const std::string &
             key.insert(key.end(), d.rdispls.begin(), d.rdispls.end());
         }
     }
+    for (const OpParam &p : params) {
+        key.push_back(p.inputSize);
+        key.push_back(p.outputSize);
+        key.push_back(p.inputPtr == p.outputPtr ? 1 : 0);
+    }
     return key;
+}
+
+// The shape and the addresses: what a plan with its tables in device memory is found by.
+std::vector<u64> PlanKey(const std::vector<u64> &shape, const std::vector<OpParam> &params)
+{
+    std::vector<u64> key = shape;
+    for (const OpParam &p : params) {
+        key.push_back(reinterpret_cast<u64>(p.inputPtr));
+        key.push_back(reinterpret_cast<u64>(p.outputPtr));
+    }
+    return key;
+}
+
+// True when no two of the ranks' buffers overlap, a rank's input being the same as its own output aside: then the
+// recorded schedule, its trace and the plan made from it are the same wherever the buffers lie, and a plan made for
+// one set of addresses serves another by shifting every pointer with its buffer.
+bool BuffersAreSeparate(const std::vector<OpParam> &params)
+{
+    struct R {
+        u64 lo, hi;
+    };
+    std::vector<R> r;
+    r.reserve(2 * params.size());
+    for (const OpParam &p : params) {
+        const u64 in = reinterpret_cast<u64>(p.inputPtr);
+        const u64 out = reinterpret_cast<u64>(p.outputPtr);
+        if (in == out) {
+            const u64 size = std::max(p.inputSize, p.outputSize);
+            if (size) r.push_back({in, in + size});
+            continue;
+        }
+        if (p.inputSize != 0) r.push_back({in, in + p.inputSize});
+        if (p.outputSize != 0) r.push_back({out, out + p.outputSize});
+    }
+    std::sort(r.begin(), r.end(), [](const R &a, const R &b) { return a.lo < b.lo; });
+    for (size_t i = 1; i < r.size(); ++i) {
+        if (r[i].lo < r[i - 1].hi) return false;
+    }
+    return true;
+}
+
+// Moves the pointers of a shape plan's parts from the buffers it was made for to those of `params`.  Pointers
+// outside the ranks' buffers (the scratch buffers of step plans, which belong to the world) stay.
+void Rebase(const ShapePlan &sp, const std::vector<OpParam> &params, std::vector<HostPart> &parts)
+{
+    struct Move {
+        u64 lo, hi;
+        int64_t delta;
+    };
+    std::vector<Move> moves;
+    for (size_t r = 0; r < params.size(); ++r) {
+        const ShapePlan::Buffer &in = sp.buffers[2 * r];
+        const ShapePlan::Buffer &out = sp.buffers[2 * r + 1];
+        const u64 newIn = reinterpret_cast<u64>(params[r].inputPtr);
+        const u64 newOut = reinterpret_cast<u64>(params[r].outputPtr);
+        if (in.base == out.base) {   // in place: one buffer, as long as the longer of the two
+            const u64 size = std::max(in.size, out.size);
+            if (size) moves.push_back({in.base, in.base + size, static_cast<int64_t>(newIn - in.base)});
+            continue;
+        }
+        if (in.size) moves.push_back({in.base, in.base + in.size, static_cast<int64_t>(newIn - in.base)});
+        if (out.size) moves.push_back({out.base, out.base + out.size, static_cast<int64_t>(newOut - out.base)});
+    }
+    std::sort(moves.begin(), moves.end(), [](const Move &a, const Move &b) { return a.lo < b.lo; });
+    auto shift = [&](const void *p) -> void * {
+        const u64 a = reinterpret_cast<u64>(p);
+        auto it = std::upper_bound(moves.begin(), moves.end(), a, [](u64 v, const Move &m) { return v < m.lo; });
+        if (it == moves.begin()) return const_cast<void *>(p);
+        --it;
+        return a < it->hi ? reinterpret_cast<void *>(a + it->delta) : const_cast<void *>(p);
+    };
+    parts = sp.parts;
+    for (HostPart &hp : parts) {
+        for (hcclx_seg_t &g : hp.segs) {
+            for (uint32_t k = 0; k < g.nsrc; ++k) g.src[k] = shift(g.src[k]);
+            for (uint32_t k = 0; k < g.ndst; ++k) g.dst[k] = shift(g.dst[k]);
+        }
+        for (hcclx_wide_seg_t &g : hp.wideSegs) {
+            for (uint32_t k = 0; k < g.nsrc; ++k) g.src[k] = shift(g.src[k]);
+            for (uint32_t k = 0; k < g.ndst; ++k) g.dst[k] = shift(g.dst[k]);
+        }
+    }
+}
+
+// Device-resident plans of a list of parts.
+HcclResult CreatePlans(const std::vector<HostPart> &parts, std::vector<hcclx_plan *> &plans)
+{
+    for (const HostPart &hp : parts) {
+        hcclx_plan *p = nullptr;
+        const int rc = hp.wide ? hcclx_plan_create_wide(hp.wideSegs.data(), static_cast<uint32_t>(hp.wideSegs.size()), hp.dtype,
+                                                        hp.op, hp.mode, &p)
+                               : hcclx_plan_create(hp.segs.data(), static_cast<uint32_t>(hp.segs.size()), hp.dtype, hp.op,
+                                                   hp.mode, &p);
+        if (rc != HCCL_SUCCESS) return static_cast<HcclResult>(rc);
+        plans.push_back(p);
+    }
+    return HCCL_SUCCESS;
+}
+
+// The same parts launched once, their tables travelling through the descriptor ring: no allocation, no plan kept.
+HcclResult LaunchParts(World *w, const std::vector<HostPart> &parts, void *stream)
+{
+    w->lastLaunches = 0;
+    for (const HostPart &hp : parts) {
+        const int rc = hp.wide ? hcclx_fold_wide(hp.wideSegs.data(), static_cast<uint32_t>(hp.wideSegs.size()), hp.dtype, hp.op,
+                                                 hp.mode, stream)
+                               : hcclx_fold(hp.segs.data(), static_cast<uint32_t>(hp.segs.size()), hp.dtype, hp.op, hp.mode,
+                                            stream);
+        if (rc != HCCL_SUCCESS) return static_cast<HcclResult>(rc);
+        w->lastLaunches++;
+    }
+    return HCCL_SUCCESS;
 }
 
 HcclResult LaunchPlans(World *w, const std::vector<hcclx_plan *> &plans, void *stream)
@@ -978,6 +1090,70 @@ CachedPlan *FindPlan(PlanCache &cache, const std::vector<u64> &key)
         }
     }
     return nullptr;
+}
+
+ShapePlan *FindShape(PlanCache &cache, const std::vector<u64> &shape)
+{
+    auto range = cache.shapeIndex.equal_range(HashKey(shape));
+    for (auto it = range.first; it != range.second; ++it) {
+        if (it->second->key == shape) {
+            cache.shapes.splice(cache.shapes.begin(), cache.shapes, it->second);
+            return &*it->second;
+        }
+    }
+    return nullptr;
+}
+
+// True when this address key was launched from a shape plan before (among the last few dozen such launches);
+// remembers it otherwise.
+bool SeenBefore(PlanCache &cache, u64 hash)
+{
+    constexpr size_t kRemembered = 64;
+    if (std::find(cache.seenOnce.begin(), cache.seenOnce.end(), hash) != cache.seenOnce.end()) return true;
+    if (cache.seenOnce.size() < kRemembered) {
+        cache.seenOnce.push_back(hash);
+    } else {
+        cache.seenOnce[cache.seenAt] = hash;
+        cache.seenAt = (cache.seenAt + 1) % kRemembered;
+    }
+    return false;
+}
+
+// Keeps the host side of a plan so that the same collective on other buffers need not be planned again.
+void KeepShape(PlanCache &cache, const std::vector<u64> &shape, std::vector<HostPart> &&parts,
+               const std::vector<OpParam> &params, bool fused, u32 levels, u32 segments)
+{
+    if (shape.empty() || FindShape(cache, shape) != nullptr) return;
+    ShapePlan sp;
+    sp.key = shape;
+    sp.parts = std::move(parts);
+    sp.fused = fused;
+    sp.levels = levels;
+    sp.segments = segments;
+    sp.hostBytes = shape.size() * sizeof(u64);
+    for (const HostPart &hp : sp.parts) {
+        sp.hostBytes += hp.segs.size() * sizeof(hcclx_seg_t) + hp.wideSegs.size() * sizeof(hcclx_wide_seg_t);
+    }
+    if (sp.hostBytes > kShapeCacheBytes / 4) return;   // one plan must not push most of the others out
+    for (const OpParam &p : params) {
+        sp.buffers.push_back({reinterpret_cast<u64>(p.inputPtr), p.inputSize});
+        sp.buffers.push_back({reinterpret_cast<u64>(p.outputPtr), p.outputSize});
+    }
+    cache.shapeBytes += sp.hostBytes;
+    cache.shapes.push_front(std::move(sp));
+    cache.shapeIndex.emplace(HashKey(shape), cache.shapes.begin());
+    while (cache.shapes.size() > 1 && (cache.shapes.size() > kShapeCacheEntries || cache.shapeBytes > kShapeCacheBytes)) {
+        auto victim = std::prev(cache.shapes.end());
+        auto range = cache.shapeIndex.equal_range(HashKey(victim->key));
+        for (auto it = range.first; it != range.second; ++it) {
+            if (it->second == victim) {
+                cache.shapeIndex.erase(it);
+                break;
+            }
+        }
+        cache.shapeBytes -= victim->hostBytes;
+        cache.shapes.erase(victim);
+    }
 }
 
 // Launches a freshly built plan and, when it has a key, keeps it for the next identical collective.  A plan that
@@ -1171,7 +1347,7 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
     }
     w->lastAlgName = algName;
     w->lastWasFused = false;
-    w->lastPlanCacheHit = false;
+    w->lastPlanCacheHit = 0;
     w->lastFusedSegments = 0;
     w->lastLevels = 0;
     void *stream = params[n - 1].stream;
@@ -1183,22 +1359,59 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
         w->lastWasFused = true;
         return LaunchDataMove(w, params, stream);
     }
+    std::vector<u64> shape;
     std::vector<u64> key;
+    bool separate = false;
     if (!w->dryRun && !w->traceText && !w->check) {
-        key = PlanKey(params, algName, w->cclBytes);
-        key.push_back(fused ? 1 : 0);
-        if (!w->planCache.retired.empty()) ReapRetired(w->planCache, false);
-        if (CachedPlan *c = FindPlan(w->planCache, key)) {
+        PlanCache &cache = w->planCache;
+        shape = ShapeKey(params, algName, w->cclBytes);
+        shape.push_back(fused ? 1 : 0);
+        key = PlanKey(shape, params);
+        if (!cache.retired.empty()) ReapRetired(cache, false);
+        if (CachedPlan *c = FindPlan(cache, key)) {
             if (c->lastStream != stream) c->manyStreams = true;
             c->lastStream = stream;
             w->lastWasFused = c->fused;
             w->lastLevels = c->levels;
-            w->lastPlanCacheHit = true;
+            w->lastFusedSegments = c->segments;
+            w->lastPlanCacheHit = 1;
             return LaunchPlans(w, c->plans, stream);
+        }
+        separate = BuffersAreSeparate(params);
+        if (ShapePlan *sp = separate ? FindShape(cache, shape) : nullptr) {
+            // The same collective on other buffers: the plan it had, with every pointer moved along with its buffer.
+            std::vector<HostPart> parts;
+            Rebase(*sp, params, parts);
+            w->lastWasFused = sp->fused;
+            w->lastLevels = sp->levels;
+            w->lastFusedSegments = sp->segments;
+            w->lastPlanCacheHit = 2;
+            if (!SeenBefore(cache, HashKey(key))) return LaunchParts(w, parts, stream);
+            // these buffers have come by before: they are worth tables of their own in device memory
+            CachedPlan c;
+            c.key = key;
+            c.fused = sp->fused;
+            c.levels = sp->levels;
+            c.segments = sp->segments;
+            const HcclResult made = CreatePlans(parts, c.plans);
+            if (made != HCCL_SUCCESS) {
+                DropPlans(c.plans, c.buffers);
+                return made;
+            }
+            return LaunchAndKeep(w, std::move(c), stream);
         }
     }
 
     // expand: every rank's executor + template records its steps
+    static const bool kTiming = std::getenv("HCCL_VRANK_TIMING") != nullptr;
+    auto tnow = [] { return std::chrono::steady_clock::now(); };
+    auto t0 = tnow();
+    auto lap = [&](const char *what) {
+        if (!kTiming) return;
+        auto t1 = tnow();
+        std::fprintf(stderr, "[timing] %-12s %8.3f ms\n", what, std::chrono::duration<double, std::milli>(t1 - t0).count());
+        t0 = t1;
+    };
     CHK_RET(w->EnsureScratch());
     w->ResetRecording();
     for (u32 r = 0; r < n; ++r) {
@@ -1211,11 +1424,13 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
         FillResources(w, r, static_cast<u32>(threadNum), resCtx);
         CHK_RET(exec->Orchestrate(params[r], resCtx));
     }
+    lap("record");
     std::vector<Node> order;
     u32 numLevels = 0;
     w->lastCheck = CheckReport();
     CHK_RET(BuildOrder(w, order, numLevels, w->check ? &w->lastCheck : nullptr));
     w->lastLevels = numLevels;
+    lap("order");
 
     const u32 esz = IsDataMove(type) ? 1 : DATATYPE_SIZE_TABLE[dtype];
     const int foldType = IsDataMove(type) ? HCCL_DATA_TYPE_INT8 : dtype;
@@ -1229,6 +1444,7 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
                 tr.Reduce(reinterpret_cast<u64>(it.dst), reinterpret_cast<u64>(it.src), it.bytes);
             }
         }
+        lap("trace");
         if (w->check) {
             CheckSemantics(tr, params, w->lastCheck);
             CHK_PRT_RET(w->lastCheck.races != 0 || w->lastCheck.semanticErrors != 0,
@@ -1238,6 +1454,7 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
         w->lastTrace.clear();
         const bool ok = BuildFusedPlan(w, tr, params, foldType, op, esz, plan,
                                        (w->traceText || w->dryRun) ? &w->lastTrace : nullptr);
+        lap("fusedplan");
         w->lastFusedSegments =
             static_cast<u32>(plan.chainSegs.size() + plan.selfSegs.size() + plan.copySegs.size() + plan.treeSegs.size() +
                              plan.wideSegs.size() + plan.wideTreeSegs.size() + plan.wideSelfSegs.size() +
@@ -1247,47 +1464,46 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
             return HCCL_SUCCESS;
         }
         if (ok && fused) {
+            std::vector<HostPart> parts;
+            auto add = [&](std::vector<hcclx_seg_t> &segs, int dt, int mode) {
+                if (segs.empty()) return;
+                parts.emplace_back();
+                parts.back().dtype = dt;
+                parts.back().op = op;
+                parts.back().mode = mode;
+                parts.back().segs = std::move(segs);
+            };
+            auto addWide = [&](std::vector<hcclx_wide_seg_t> &segs, int mode) {
+                if (segs.empty()) return;
+                parts.emplace_back();
+                parts.back().wide = true;
+                parts.back().dtype = foldType;
+                parts.back().op = op;
+                parts.back().mode = mode;
+                parts.back().wideSegs = std::move(segs);
+            };
+            add(plan.selfSegs, foldType, HCCLX_FOLD_SELF_FIRST);
+            add(plan.chainSegs, foldType, HCCLX_FOLD_CHAIN);
+            add(plan.copySegs, HCCL_DATA_TYPE_INT8, HCCLX_FOLD_CHAIN);
+            add(plan.treeSegs, foldType, HCCLX_FOLD_TREE);
+            addWide(plan.wideSegs, HCCLX_FOLD_CHAIN);
+            addWide(plan.wideTreeSegs, HCCLX_FOLD_TREE);
+            addWide(plan.wideSelfSegs, HCCLX_FOLD_SELF_FIRST);
             CachedPlan c;
             c.key = key;
             c.levels = numLevels;
-            const std::pair<std::vector<hcclx_seg_t> *, int> parts[4] = {
-                {&plan.selfSegs, HCCLX_FOLD_SELF_FIRST}, {&plan.chainSegs, HCCLX_FOLD_CHAIN},
-                {&plan.copySegs, HCCLX_FOLD_CHAIN}, {&plan.treeSegs, HCCLX_FOLD_TREE}};
-            for (int i = 0; i < 4; ++i) {
-                if (parts[i].first->empty()) continue;
-                hcclx_plan *hp = nullptr;
-                const int dt = (i == 2) ? HCCL_DATA_TYPE_INT8 : foldType;
-                const int rc = hcclx_plan_create(parts[i].first->data(), static_cast<uint32_t>(parts[i].first->size()),
-                                                 dt, op, parts[i].second, &hp);
-                if (rc != HCCL_SUCCESS) {
-                    DropPlans(c.plans, c.buffers);
-                    return static_cast<HcclResult>(rc);
-                }
-                c.plans.push_back(hp);
-            }
-            for (int i = 0; i < 3; ++i) {
-                const std::vector<hcclx_wide_seg_t> &segs = i == 0 ? plan.wideSegs : i == 1 ? plan.wideTreeSegs : plan.wideSelfSegs;
-                if (segs.empty()) continue;
-                hcclx_plan *hp = nullptr;
-                const int rc = hcclx_plan_create_wide(segs.data(), static_cast<uint32_t>(segs.size()), foldType, op,
-                                                      i == 0 ? HCCLX_FOLD_CHAIN : i == 1 ? HCCLX_FOLD_TREE : HCCLX_FOLD_SELF_FIRST, &hp);
-                if (rc != HCCL_SUCCESS) {
-                    DropPlans(c.plans, c.buffers);
-                    return static_cast<HcclResult>(rc);
-                }
-                c.plans.push_back(hp);
-            }
-            if (!plan.stagedSelfSegs.empty()) {
+            c.segments = w->lastFusedSegments;
+            const bool stagedOutputs = !plan.stagedSelfSegs.empty();
+            if (stagedOutputs) {
+                // outputs that go through a staging buffer of the plan's own: kept with its addresses only
                 char *staging = nullptr;
-                if (hipMalloc(reinterpret_cast<void **>(&staging), plan.stagingBytes) != hipSuccess) {
-                    DropPlans(c.plans, c.buffers);
-                    return HCCL_E_RUNTIME;
-                }
+                if (hipMalloc(reinterpret_cast<void **>(&staging), plan.stagingBytes) != hipSuccess) return HCCL_E_RUNTIME;
                 c.buffers.push_back(staging);
-                std::vector<hcclx_seg_t> copies;
                 for (hcclx_wide_seg_t &seg : plan.stagedSelfSegs) {
                     for (uint32_t j = 0; j < seg.ndst; ++j) seg.dst[j] = staging + reinterpret_cast<u64>(seg.dst[j]);
                 }
+                addWide(plan.stagedSelfSegs, HCCLX_FOLD_SELF_FIRST);
+                std::vector<hcclx_seg_t> copies;
                 for (const FusedPlan::StagedCopy &sc : plan.stagedCopies) {
                     hcclx_seg_t cp;
                     std::memset(&cp, 0, sizeof(cp));
@@ -1298,35 +1514,37 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
                     cp.dst[0] = reinterpret_cast<void *>(sc.dst);
                     copies.push_back(cp);
                 }
-                hcclx_plan *first = nullptr;
-                hcclx_plan *second = nullptr;
-                int rc = hcclx_plan_create_wide(plan.stagedSelfSegs.data(), static_cast<uint32_t>(plan.stagedSelfSegs.size()),
-                                                foldType, op, HCCLX_FOLD_SELF_FIRST, &first);
-                if (rc == HCCL_SUCCESS) {
-                    c.plans.push_back(first);
-                    rc = hcclx_plan_create(copies.data(), static_cast<uint32_t>(copies.size()), HCCL_DATA_TYPE_INT8, 0,
-                                           HCCLX_FOLD_CHAIN, &second);
-                }
-                if (rc != HCCL_SUCCESS) {
-                    DropPlans(c.plans, c.buffers);
-                    return static_cast<HcclResult>(rc);
-                }
-                c.plans.push_back(second);   // launched last: every read of the inputs is queued in front of it
+                // launched last: every read of the inputs is queued in front of it
+                add(copies, HCCL_DATA_TYPE_INT8, HCCLX_FOLD_CHAIN);
             }
+            const HcclResult made = CreatePlans(parts, c.plans);
+            if (made != HCCL_SUCCESS) {
+                DropPlans(c.plans, c.buffers);
+                return made;
+            }
+            lap("tables");
             w->lastWasFused = true;
-            return LaunchAndKeep(w, std::move(c), stream);
+            const HcclResult res = LaunchAndKeep(w, std::move(c), stream);
+            if (res == HCCL_SUCCESS && separate && !stagedOutputs) {
+                KeepShape(w->planCache, shape, std::move(parts), params, true, numLevels, w->lastFusedSegments);
+            }
+            return res;
         }
     }
+    std::vector<HostPart> parts;
+    BuildStepParts(order, numLevels, foldType, op, parts);
     CachedPlan c;
     c.key = key;
     c.fused = false;
     c.levels = numLevels;
-    const HcclResult built = BuildStepPlans(order, numLevels, foldType, op, c.plans);
-    if (built != HCCL_SUCCESS) {
+    const HcclResult made = CreatePlans(parts, c.plans);
+    if (made != HCCL_SUCCESS) {
         DropPlans(c.plans, c.buffers);
-        return built;
+        return made;
     }
-    return LaunchAndKeep(w, std::move(c), stream);
+    const HcclResult res = LaunchAndKeep(w, std::move(c), stream);
+    if (res == HCCL_SUCCESS && separate) KeepShape(w->planCache, shape, std::move(parts), params, false, numLevels, 0);
+    return res;
 }
 
 }  // namespace

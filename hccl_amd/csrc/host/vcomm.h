@@ -19,6 +19,8 @@
 #include "alg_env_config.h"
 #include "alg_param.h"
 
+#include "hcclx.h"
+
 struct hcclx_plan;
 
 namespace ops_hccl {
@@ -74,6 +76,7 @@ struct CachedPlan {
     std::vector<void *> buffers;       // device memory the plans use besides their tables (staged outputs)
     bool fused = true;                 // false: the recorded steps, one or two plans per level
     u32 levels = 0;
+    u32 segments = 0;                  // segments of the fused plan
     u64 tableBytes = 0;                // device memory of the plans' tables
     void *lastStream = nullptr;        // where it was launched last
     bool manyStreams = false;          // it has been launched on more than one stream
@@ -90,11 +93,43 @@ struct RetiredPlan {
     std::vector<void *> buffers;
     void *event = nullptr;             // hipEvent_t
 };
+// One launch of a planned collective as the host keeps it: the segment list of one hcclx_plan_create /
+// hcclx_fold call.  A shape's list of these is independent of where the ranks' buffers lie, up to a shift of every
+// pointer by the distance its buffer has moved.
+struct HostPart {
+    bool wide = false;
+    int dtype = 0;
+    int op = 0;
+    int mode = 0;
+    std::vector<hcclx_seg_t> segs;
+    std::vector<hcclx_wide_seg_t> wideSegs;
+};
+// The plan of a collective without its addresses: found by (op, algorithm, types, counts, tables, which ranks run in
+// place), it is moved to the buffers of the call at hand by shifting pointers, with no template run and no trace.
+struct ShapePlan {
+    std::vector<u64> key;
+    std::vector<HostPart> parts;     // launched in this order
+    struct Buffer {
+        u64 base, size;
+    };
+    std::vector<Buffer> buffers;     // the ranks' input and output buffers the parts' pointers refer to (2 per rank)
+    bool fused = true;
+    u32 levels = 0;
+    u32 segments = 0;
+    u64 hostBytes = 0;
+};
+constexpr size_t kShapeCacheEntries = 256;
+constexpr u64 kShapeCacheBytes = 128ull << 20;
 struct PlanCache {
     std::list<CachedPlan> lru;
     std::unordered_multimap<u64, std::list<CachedPlan>::iterator> index;
     std::vector<RetiredPlan> retired;
     u64 bytes = 0;
+    std::list<ShapePlan> shapes;     // most recently used first
+    std::unordered_multimap<u64, std::list<ShapePlan>::iterator> shapeIndex;
+    u64 shapeBytes = 0;
+    std::vector<u64> seenOnce;       // hashes of address keys that were launched from a shape plan once (a ring)
+    size_t seenAt = 0;
 };
 
 // What the schedule check found in the last collective (see hcclxCommSetCheck).
@@ -136,7 +171,7 @@ struct World {
     u32 lastLaunches = 0;
     u32 lastFusedSegments = 0;
     bool lastWasFused = false;
-    bool lastPlanCacheHit = false;
+    int lastPlanCacheHit = 0;  // 0 planned, 1 a plan with these addresses replayed, 2 a plan of this shape moved to them
     std::string lastTrace;  // expression of every output piece, filled when traceText is set
     bool traceText = false;
     bool check = false;     // verify every schedule before it is launched

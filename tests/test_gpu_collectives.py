@@ -129,7 +129,8 @@ def test_one_shot_allreduce_in_place_among_many_ranks(stream, n, alg, dtype, op)
             xs = [payload(rng, dtype, count, kind) for _ in range(n)]
             got, bufs = run_allreduce(w, stream, xs, count, dtype, op, in_place=True)
             info = w.last_info()
-            assert info.fused == 1 and info.launches == 2 and info.planCacheHit == 0   # new buffers: a new plan
+            assert info.fused == 1 and info.launches == 2
+            assert info.planCacheHit == 0   # new buffers: a plan with a staging buffer of its own is made for its addresses
             if dtype in (T.FP16, T.BFP16) and op == T.SUM:
                 want = wide_oracle_allreduce(xs, count, dtype, alg, SMALL_CCL)
             else:
@@ -665,5 +666,107 @@ def test_ranks_on_different_streams_one_host_thread(stream):
             want = torch.arange(count, device="cuda:0", dtype=torch.float32) * (it * n * (n + 1) // 2)
             for r in range(n):
                 assert torch.equal(seen[r], want), (it, r)     # exact: small integers in fp32
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("alg,dtype,op,n,count", [("InsAllReduceMesh1DTwoShot", T.FP32, T.SUM, 8, 70003),
+                                                  ("InsAllReduceRing", T.BFP16, T.SUM, 5, 40001),
+                                                  ("InsAllReduceNHR", T.INT32, T.MAX, 12, 50021),
+                                                  ("InsAllReduceAicpuReduceNHR", T.FP32, T.PROD, 12, 30011),
+                                                  ("InsAllReduceMesh1DOneShot", T.FP16, T.SUM, 24, 9001),
+                                                  ("InsAllReduceMesh1DTwoShotMeshChunk", T.FP32, T.SUM, 6, 60007)])
+def test_a_plan_follows_its_collective_to_other_buffers(stream, mode, alg, dtype, op, n, count):
+    """The same collective on buffers somewhere else (and differently aligned) is not planned again: the plan of the
+    first call is moved there pointer by pointer, gets device tables of its own when the same buffers come a second
+    time, and is replayed from then on.  Every call's result is the oracle's.  Running in place is another shape."""
+    rng = np.random.default_rng(count)
+    esz = T.DTYPE_SIZE[dtype]
+    kind = "prod" if op == T.PROD else "uniform" if dtype == T.FP32 else "normal"
+    w = api.World(n, ccl_bytes=SMALL_CCL)
+    try:
+        w.set_mode(mode)
+        w.set_algorithm(api.CMD_ALLREDUCE, alg)
+
+        def call(send, recv, xs):
+            for r in range(n):
+                send[r].t[send[r].offset:send[r].offset + send[r].nbytes] = torch.from_numpy(
+                    xs[r].view(np.uint8).reshape(-1).copy()).to("cuda:0")
+            torch.cuda.synchronize()
+            for r in range(n):
+                assert w.all_reduce(r, send[r].ptr, recv[r].ptr, count, dtype, op, stream.cuda_stream) == 0
+            stream.synchronize()
+            info = w.last_info()
+            if info.fused and dtype in (T.FP16, T.BFP16) and op == T.SUM:
+                want = wide_oracle_allreduce(xs, count, dtype, alg, SMALL_CCL)
+            else:
+                want = T.run_allreduce(T.NumericElems(dtype, op), xs, count, esz, alg, ccl_bytes=SMALL_CCL)
+            for r in range(n):
+                assert_same_bits(recv[r].get(T.NP_STORAGE[dtype]), want[r], dtype, f"{alg} rank {r}")
+                assert recv[r].guard_intact()
+            return info.planCacheHit, info.fused, info.launches
+
+        def buffers(offsets):
+            send = [DevBuf(nbytes=count * esz, offset=offsets[r % len(offsets)]) for r in range(n)]
+            recv = [DevBuf(nbytes=count * esz, offset=offsets[(r + 1) % len(offsets)]) for r in range(n)]
+            return send, recv
+
+        first = buffers([0])
+        second = buffers([esz, 0, 3 * esz, 128 + esz])   # other places, other alignments
+        fresh = lambda: [payload(rng, dtype, count, kind) for _ in range(n)]
+        hit0, fused0, launches0 = call(*first, fresh())
+        assert hit0 == 0
+        assert call(*second, fresh()) == (2, fused0, launches0)    # moved, launched from host tables
+        assert call(*second, fresh()) == (2, fused0, launches0)    # moved, tables now in device memory
+        assert call(*second, fresh()) == (1, fused0, launches0)    # replayed
+        assert call(*first, fresh()) == (1, fused0, launches0)     # the first plan is still there
+        hit, _, _ = call(first[0], first[0], fresh())              # in place: not the same collective
+        assert hit == 0
+        mixed = (first[0], second[1])                              # known buffers in a new combination
+        assert call(*mixed, fresh())[0] == 2
+    finally:
+        w.close()
+
+
+def test_overlapping_buffers_are_planned_for_their_addresses(stream):
+    """When ranks' buffers overlap each other (here every rank receives into a slice of one allocation that is also a
+    rank's input), what the plan may fuse depends on where they lie: such calls never borrow another call's plan."""
+    n, count = 4, 4099
+    rng = np.random.default_rng(5)
+    xs = [payload(rng, T.FP32, count, "uniform") for _ in range(n)]
+    w = api.World(n, ccl_bytes=SMALL_CCL)
+    try:
+        send = [DevBuf(x) for x in xs]
+        recv = [DevBuf(nbytes=count * 4) for _ in range(n)]
+        for r in range(n):
+            assert w.all_reduce(r, send[r].ptr, recv[r].ptr, count, T.FP32, T.SUM, stream.cuda_stream) == 0
+        stream.synchronize()
+        assert w.last_info().planCacheHit == 0
+        want = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs, count, 4, w.last_info().algName.decode(),
+                               ccl_bytes=SMALL_CCL)
+        # rank 1 now sends what rank 0 received: its input buffer is rank 0's old output, still apart from the rest
+        xs2 = [xs[0], want[0], xs[2], xs[3]]
+        send2 = [send[0], recv[0], send[2], send[3]]
+        recv2 = [DevBuf(nbytes=count * 4) for _ in range(n)]
+        for r in range(n):
+            assert w.all_reduce(r, send2[r].ptr, recv2[r].ptr, count, T.FP32, T.SUM, stream.cuda_stream) == 0
+        stream.synchronize()
+        assert w.last_info().planCacheHit == 2
+        want2 = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs2, count, 4, w.last_info().algName.decode(),
+                                ccl_bytes=SMALL_CCL)
+        for r in range(n):
+            assert_same_bits(recv2[r].get(np.float32), want2[r], T.FP32, f"rank {r}")
+        # two ranks share one input buffer: overlapping, so planned for these addresses
+        send3 = [send[0], send[0], send[2], send[3]]
+        xs3 = [xs[0], xs[0], xs[2], xs[3]]
+        for r in range(n):
+            assert w.all_reduce(r, send3[r].ptr, recv2[r].ptr, count, T.FP32, T.SUM, stream.cuda_stream) == 0
+        stream.synchronize()
+        assert w.last_info().planCacheHit == 0
+        want3 = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs3, count, 4, w.last_info().algName.decode(),
+                                ccl_bytes=SMALL_CCL)
+        for r in range(n):
+            assert_same_bits(recv2[r].get(np.float32), want3[r], T.FP32, f"shared input, rank {r}")
     finally:
         w.close()
