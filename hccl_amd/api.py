@@ -45,6 +45,7 @@ def lib():
             "hcclxCommGetLastOpInfo": [vp, ctypes.POINTER(LastOpInfo)],
             "hcclxCommSetTrace": [vp, ci],
             "hcclxCommSetCheck": [vp, ci],
+            "hcclxCommSetClosedForm": [vp, ci],
             "hcclxCommGetLastCheck": [vp, ctypes.POINTER(CheckReport)],
             "HcclAllReduce": [vp, vp, u64, ci, ci, vp, vp],
             "HcclReduceScatter": [vp, vp, u64, ci, ci, vp, vp],
@@ -109,6 +110,10 @@ class World:
 
     def set_trace(self, on):
         check(lib().hcclxCommSetTrace(self.comms[0], 1 if on else 0))
+
+    def set_closed_form(self, mode):
+        """0 = record every template's steps, 1 = closed forms for plain launches, 2 = also when tracing / dry."""
+        check(lib().hcclxCommSetClosedForm(self.comms[0], int(mode)))
 
     def set_check(self, on):
         check(lib().hcclxCommSetCheck(self.comms[0], 1 if on else 0))

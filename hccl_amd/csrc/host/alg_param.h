@@ -213,6 +213,20 @@ struct SliceInfo {
     SliceInfo(u64 o, u64 s, u64 c = 0) : offset(o), size(s), count(c) {}
 };
 
+// One piece of a collective's result in closed form: `bytes` bytes that are the fold of the ranks' input pieces
+// src[0], src[1], ... (src[0] is what the others are reduced onto, one after the other, each as the source operand
+// of its step), delivered to every piece in dst.  A piece is (rank, byte offset in that rank's input -- for src --
+// or output -- for dst).  What a template's recorded steps amount to when they are traced, written down directly.
+struct ClosedFold {
+    struct Ref {
+        u32 rank;
+        u64 offset;
+    };
+    std::vector<Ref> src;
+    std::vector<Ref> dst;
+    u64 bytes = 0;
+};
+
 u32 GetNHRStepNum(u32 rankSize);
 HcclResult GetAlgRank(u32 virtRank, const std::vector<u32> &rankIds, u32 &algRank);
 

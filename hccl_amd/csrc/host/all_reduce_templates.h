@@ -16,6 +16,20 @@ namespace ops_hccl {
                              TemplateResource &templateResource) override;                                \
     }
 
+// The same for a template that also states its result in closed form.
+#define HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(CLASS, NAME, THREADS, SCRATCH)                             \
+    class CLASS : public InsAlgTemplateBase {                                                             \
+    public:                                                                                               \
+        using InsAlgTemplateBase::InsAlgTemplateBase;                                                     \
+        std::string Describe() const override { return NAME; }                                            \
+        u64 GetThreadNum() const override { return THREADS; }                                             \
+        u64 CalcScratchMultiple(BufferType, BufferType) override { return SCRATCH; }                      \
+        HcclResult KernelRun(const OpParam &param, const TemplateDataParams &tempAlgParams,               \
+                             TemplateResource &templateResource) override;                                \
+        bool ClosedForm(const TemplateDataParams &tempAlgParams, u64 dataTypeSize,                        \
+                        std::vector<ClosedFold> &out) const override;                                     \
+    }
+
 // scratch multiples: one_shot.cc:42-48 (N), two_shot.cc:20-27 (2), nhr.cc:20-26 (1), aicpu_reduce_nhr.cc:22-28 (N)
 HCCL_DECLARE_TEMPLATE(InsTempAllReduceMesh1DOneShot, "AllReduce mesh 1D one-shot",
                       (templateRankSize_ > 1 ? templateRankSize_ : 1), templateRankSize_);

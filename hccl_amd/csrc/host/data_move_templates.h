@@ -10,15 +10,15 @@ HCCL_DECLARE_TEMPLATE(InsTempReduceScatterMesh1D, "ReduceScatter mesh 1D",
                       (templateRankSize_ > 1 ? templateRankSize_ : 1), templateRankSize_);
 HCCL_DECLARE_TEMPLATE(InsTempReduceScatterNHR, "ReduceScatter NHR", 1, templateRankSize_);
 // reduce_scatter aicpu_reduce_nhr.cc:46-50, :242-249: one thread, N scratch slots
-HCCL_DECLARE_TEMPLATE(InsTempReduceScatterAicpuReduceNHR, "ReduceScatter NHR gather + local reduce", 1, templateRankSize_);
+HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempReduceScatterAicpuReduceNHR, "ReduceScatter NHR gather + local reduce", 1, templateRankSize_);
 // reduce_scatter_v mesh_1D.cc:26-48: N-1 threads (the main thread sends too), N scratch slots
 HCCL_DECLARE_TEMPLATE(InsTempReduceScatterVMesh1D, "ReduceScatterV mesh 1D",
                       (templateRankSize_ > 1 ? templateRankSize_ - 1 : 1), templateRankSize_);
 // mesh-chunk templates (mesh_chunk_templates.cc): reduce_scatter meshchunk.cc:25-52 (N-1 threads, N-1 scratch
 // multiple); all_reduce two_shot_mesh_chunk.cc:17-38 (N threads, scratch multiple 2)
-HCCL_DECLARE_TEMPLATE(InsTempReduceScatterMesh1DMeshChunk, "ReduceScatter mesh 1D, chunked",
+HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempReduceScatterMesh1DMeshChunk, "ReduceScatter mesh 1D, chunked",
                       (templateRankSize_ > 1 ? templateRankSize_ - 1 : 1), (templateRankSize_ > 0 ? templateRankSize_ - 1 : 0));
-HCCL_DECLARE_TEMPLATE(InsTempAllReduceMesh1DTwoShotMeshChunk, "AllReduce mesh 1D two-shot, chunked",
+HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempAllReduceMesh1DTwoShotMeshChunk, "AllReduce mesh 1D two-shot, chunked",
                       (templateRankSize_ > 1 ? templateRankSize_ : 1), 2);
 // Where each rank's block sits in the scratch buffer during one loop of the order-preserved ReduceScatter
 // (ins_v2_reduce_scatter_order_preserved_executor.h:37-42).

@@ -35,6 +35,16 @@ public:
     // Threads the template of this executor needs on one rank.
     virtual u64 CalcThreadNum(const OpParam &param, u32 rank, u32 rankSize) = 0;
     virtual HcclResult Orchestrate(const OpParam &param, const AlgResourceCtxSerializable &resCtx) = 0;
+    // The whole collective among `rankSize` ranks in closed form (see ClosedFold), when the template has one: the
+    // same chunk loop as Orchestrate, asking the template for the net effect of each chunk instead of its steps.
+    virtual bool ClosedForm(const OpParam &param, u32 rankSize, u64 cclBytes, std::vector<ClosedFold> &out)
+    {
+        (void)param;
+        (void)rankSize;
+        (void)cclBytes;
+        (void)out;
+        return false;
+    }
 
 protected:
     u32 myRank_ = INVALID_VALUE_RANKID;

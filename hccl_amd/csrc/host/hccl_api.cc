@@ -239,6 +239,16 @@ HcclResult hcclxCommSetTrace(HcclComm comm, int on)
     return HCCL_SUCCESS;
 }
 
+HcclResult hcclxCommSetClosedForm(HcclComm comm, int mode)
+{
+    RankComm *rc = AsRankComm(comm);
+    CHK_PTR_NULL(rc);
+    CHK_PRT_RET(mode < 0 || mode > 2, HCCL_ERROR("[hcclxCommSetClosedForm] mode %d is not 0, 1 or 2", mode), HCCL_E_PARA);
+    std::lock_guard<std::mutex> lock(rc->world->mu);
+    rc->world->closedForm = mode;
+    return HCCL_SUCCESS;
+}
+
 HcclResult hcclxCommSetCheck(HcclComm comm, int on)
 {
     RankComm *rc = AsRankComm(comm);

@@ -45,6 +45,28 @@ std::vector<u64> SplitEven(u64 count, u64 parts, u64 esz)
     return sizes;
 }
 
+// A ReduceScatter shard of `size` bytes in N-1 chunks: all but the last rounded down to 4 KiB, the last takes the
+// rest; shards too small for that are cut evenly by elements (mesh_1D_meshchunk.cc:139-162).
+std::vector<u64> ShardChunks(u64 size, u32 n, u64 esz)
+{
+    const u64 parts = n - 1;
+    const u64 aligned = (size / parts) / AICPU_ALIGN_SIZE * AICPU_ALIGN_SIZE;
+    if (parts >= 2 && aligned > 0) {
+        std::vector<u64> chunk(parts - 1, aligned);
+        chunk.push_back(size - aligned * (parts - 1));
+        return chunk;
+    }
+    return SplitEven(size / esz, parts, esz);
+}
+
+// The ranks whose data chunk `chunk` of `owner`'s shard takes, in the order it takes them: the owner's own first,
+// then the writer of step 0, 1, ... N-2.
+void ChunkOrder(u32 owner, u32 chunk, u32 n, std::vector<u32> &ranks)
+{
+    ranks.assign(1, owner);
+    for (u32 step = 0; step + 1 < n; ++step) ranks.push_back((owner + ChunkDistance(step, chunk, n)) % n);
+}
+
 }  // namespace
 
 HcclResult InsTempReduceScatterMesh1DMeshChunk::KernelRun(const OpParam &param, const TemplateDataParams &p,
@@ -72,17 +94,7 @@ HcclResult InsTempReduceScatterMesh1DMeshChunk::KernelRun(const OpParam &param, 
     CHK_RET(PreSync(threads));
 
     if (n > 1) {
-        // N-1 chunks: all but the last rounded down to 4 KiB, the last takes the rest; shards too small for
-        // that are cut evenly by elements (mesh_1D_meshchunk.cc:139-162)
-        const u64 parts = n - 1;
-        std::vector<u64> chunk;
-        const u64 aligned = (size / parts) / AICPU_ALIGN_SIZE * AICPU_ALIGN_SIZE;
-        if (parts >= 2 && aligned > 0) {
-            chunk.assign(parts - 1, aligned);
-            chunk.push_back(size - aligned * (parts - 1));
-        } else {
-            chunk = SplitEven(size / esz, parts, esz);
-        }
+        const std::vector<u64> chunk = ShardChunks(size, n, esz);
         for (u32 step = 0; step + 1 < n; ++step) {
             u64 off = 0;
             for (u32 i = 0; i + 1 < n; ++i) {
@@ -114,6 +126,34 @@ HcclResult InsTempReduceScatterMesh1DMeshChunk::KernelRun(const OpParam &param, 
                           DataSlice(p.buffInfo.outputPtr, p.buffInfo.outBuffBaseOff, size)));
     }
     return HCCL_SUCCESS;
+}
+
+// What the steps above amount to: chunk i of rank r's shard is r's own data with the peers' reduced onto it in the
+// rotation of ChunkOrder, and lands in r's output.
+bool InsTempReduceScatterMesh1DMeshChunk::ClosedForm(const TemplateDataParams &p, u64 esz, std::vector<ClosedFold> &out) const
+{
+    const u32 n = templateRankSize_;
+    if (n == 0 || p.repeatNum != 1) return false;
+    const u64 size = p.sliceSize;
+    if (size == 0) return true;
+    std::vector<u64> chunk(1, size);
+    if (n > 1) chunk = ShardChunks(size, n, esz);
+    std::vector<u32> order;
+    for (u32 r = 0; r < n; ++r) {
+        u64 off = 0;
+        for (u32 i = 0; i < chunk.size(); ++i) {
+            if (chunk[i] != 0) {
+                ClosedFold f;
+                f.bytes = chunk[i];
+                ChunkOrder(r, i, n, order);
+                for (u32 from : order) f.src.push_back({from, p.buffInfo.inBuffBaseOff + r * p.inputSliceStride + off});
+                f.dst.push_back({r, p.buffInfo.outBuffBaseOff + off});
+                out.push_back(std::move(f));
+            }
+            off += chunk[i];
+        }
+    }
+    return true;
 }
 
 HcclResult InsTempAllReduceMesh1DTwoShotMeshChunk::KernelRun(const OpParam &param, const TemplateDataParams &p,
@@ -200,6 +240,36 @@ HcclResult InsTempAllReduceMesh1DTwoShotMeshChunk::KernelRun(const OpParam &para
         CHK_RET(PostSyncInterThreads(res.threads[0], subs, up));
     }
     return HCCL_SUCCESS;
+}
+
+// What the steps above amount to: chunk c of owner k's slice is k's own data with the peers' reduced onto it in the
+// rotation of ChunkOrder, and every rank reads it into the same place of its output.
+bool InsTempAllReduceMesh1DTwoShotMeshChunk::ClosedForm(const TemplateDataParams &p, u64 esz,
+                                                        std::vector<ClosedFold> &out) const
+{
+    const u32 n = templateRankSize_;
+    if (n == 0) return false;
+    if (p.count == 0) return true;
+    const std::vector<SliceInfo> sl = SplitDataByRank(p.count, n, esz);
+    std::vector<u32> order;
+    for (u32 k = 0; k < n; ++k) {
+        if (sl[k].size == 0) continue;
+        std::vector<u64> chunk(1, sl[k].size);
+        if (n > 1) chunk = SplitEven(sl[k].size / esz, n - 1, esz);
+        u64 off = 0;
+        for (u32 c = 0; c < chunk.size(); ++c) {
+            if (chunk[c] != 0) {
+                ClosedFold f;
+                f.bytes = chunk[c];
+                ChunkOrder(k, c, n, order);
+                for (u32 from : order) f.src.push_back({from, p.buffInfo.inBuffBaseOff + sl[k].offset + off});
+                for (u32 r = 0; r < n; ++r) f.dst.push_back({r, p.buffInfo.outBuffBaseOff + sl[k].offset + off});
+                out.push_back(std::move(f));
+            }
+            off += chunk[c];
+        }
+    }
+    return true;
 }
 
 }  // namespace ops_hccl

@@ -159,6 +159,29 @@ HcclResult InsTempReduceScatterAicpuReduceNHR::KernelRun(const OpParam &param, c
     return HCCL_SUCCESS;
 }
 
+// What the rounds above amount to: the all-gather of round k puts every rank's shard k into rank k's scratch, and
+// rank k folds them onto its own in ascending rank order.  (The N rounds of N log N forwarded copies are what makes
+// the recorded schedule grow with the cube of the rank count.)
+bool InsTempReduceScatterAicpuReduceNHR::ClosedForm(const TemplateDataParams &p, u64 esz, std::vector<ClosedFold> &out) const
+{
+    (void)esz;
+    const u32 n = templateRankSize_;
+    if (n == 0 || p.repeatNum > 1) return false;
+    if (p.sliceSize == 0) return true;
+    for (u32 k = 0; k < n; ++k) {
+        ClosedFold f;
+        f.bytes = p.sliceSize;
+        const u64 inOff = p.buffInfo.inBuffBaseOff + k * p.inputSliceStride;
+        f.src.push_back({k, inOff});
+        for (u32 q = 0; q < n; ++q) {
+            if (q != k) f.src.push_back({q, inOff});
+        }
+        f.dst.push_back({k, p.buffInfo.outBuffBaseOff});
+        out.push_back(std::move(f));
+    }
+    return true;
+}
+
 // Shards are copied into scratch slots (slot k = shard k), the NHR reduce-scatter steps fold them across
 // ranks, and the own slot is copied out.  The slices a rank sends in step 0 go straight from its input
 // (ins_temp_reduce_scatter_nhr.cc:98-101, :329-332), so they are not pre-copied.

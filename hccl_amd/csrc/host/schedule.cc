@@ -38,6 +38,21 @@ void SetWorldTopo(World *w, u32 levels, Level0Shape shape, u32 devicesPerServer)
 
 namespace {
 
+// HCCL_VRANK_TIMING=1 prints what each phase of planning a collective took (stderr).
+struct PhaseTimer {
+    const bool on = std::getenv("HCCL_VRANK_TIMING") != nullptr;
+    std::chrono::steady_clock::time_point last = std::chrono::steady_clock::now();
+    void Start() { if (on) last = std::chrono::steady_clock::now(); }
+    void Lap(const char *what)
+    {
+        if (!on) return;
+        const auto now = std::chrono::steady_clock::now();
+        std::fprintf(stderr, "[timing] %-12s %8.3f ms\n", what, std::chrono::duration<double, std::milli>(now - last).count());
+        last = now;
+    }
+};
+PhaseTimer g_phase;
+
 bool IsDataOp(const TaskItem &it) { return it.kind == ItemKind::COPY || it.kind == ItemKind::REDUCE; }
 
 // ---------------------------------------------------------------------------------------------------
@@ -56,6 +71,28 @@ struct Node {
 // for a dependency path; beyond that only steps of the same level (which are unordered by construction).
 constexpr size_t kExhaustiveSteps = 4096;
 
+// A step is followed by the next one of its thread and, when it is a record, by the wait it releases: records
+// and waits of one identity pair up one to one.
+struct Succ {
+    int n = 0;
+    int to[2] = {-1, -1};
+    std::vector<int> more;   // a record that several waits matched (a malformed schedule): kept so that it is reported
+    void Add(int id)
+    {
+        if (n < 2) {
+            to[n] = id;
+        } else {
+            more.push_back(id);
+        }
+        ++n;
+    }
+    template <typename F> void Each(F &&f) const
+    {
+        for (int k = 0; k < n && k < 2; ++k) f(to[k]);
+        for (int id : more) f(id);
+    }
+};
+
 HcclResult BuildOrder(World *w, std::vector<Node> &order, u32 &numLevels, CheckReport *report = nullptr)
 {
     struct Flat {
@@ -66,31 +103,42 @@ HcclResult BuildOrder(World *w, std::vector<Node> &order, u32 &numLevels, CheckR
         u32 indeg;
     };
     std::vector<Flat> flat;
-    std::map<std::pair<u64, u32>, int> records;
+    size_t total = 0;
+    for (auto &perRank : w->threads) {
+        for (auto &t : perRank) total += t->items.size();
+    }
+    flat.reserve(total);
     for (auto &perRank : w->threads) {
         for (auto &t : perRank) {
             int prev = -1;
             for (const TaskItem &it : t->items) {
                 const int id = static_cast<int>(flat.size());
                 flat.push_back({&it, prev, -1, 0, 0});
-                if (it.kind == ItemKind::NOTIFY_RECORD) records[{it.key, it.seq}] = id;
                 prev = id;
             }
         }
     }
-    std::vector<std::vector<int>> succ(flat.size());
+    // The records of one notify identity in the order they were made: recordAt[first[identity] + n] is the n-th.
+    const size_t identities = w->recordSeq.size();
+    std::vector<u32> first(identities + 1, 0);
+    for (size_t k = 0; k < identities; ++k) first[k + 1] = first[k] + w->recordSeq[k];
+    std::vector<int> recordAt(first[identities], -1);
+    for (int id = 0; id < static_cast<int>(flat.size()); ++id) {
+        const TaskItem &it = *flat[id].item;
+        if (it.kind == ItemKind::NOTIFY_RECORD) recordAt[first[it.key] + it.seq] = id;
+    }
+    std::vector<Succ> succ(flat.size());
     for (int id = 0; id < static_cast<int>(flat.size()); ++id) {
         Flat &f = flat[id];
         if (f.prev >= 0) {
-            succ[f.prev].push_back(id);
+            succ[f.prev].Add(id);
             f.indeg++;
         }
         if (f.item->kind == ItemKind::NOTIFY_WAIT) {
-            auto it = records.find({f.item->key, f.item->seq});
-            CHK_PRT_RET(it == records.end(), HCCL_ERROR("[schedule] a notify wait has no matching record"),
-                        HCCL_E_INTERNAL);
-            f.match = it->second;
-            succ[f.match].push_back(id);
+            CHK_PRT_RET(f.item->key >= identities || f.item->seq >= w->recordSeq[f.item->key],
+                        HCCL_ERROR("[schedule] a notify wait has no matching record"), HCCL_E_INTERNAL);
+            f.match = recordAt[first[f.item->key] + f.item->seq];
+            succ[f.match].Add(id);
             f.indeg++;
         }
     }
@@ -109,10 +157,10 @@ HcclResult BuildOrder(World *w, std::vector<Node> &order, u32 &numLevels, CheckR
             numLevels = std::max(numLevels, f.level + 1);
         }
         const u32 out = f.level + (IsDataOp(*f.item) ? 1 : 0);
-        for (int s : succ[id]) {
+        succ[id].Each([&](int s) {
             flat[s].level = std::max(flat[s].level, out);
             if (--flat[s].indeg == 0) ready.push_back(s);
-        }
+        });
     }
     CHK_PRT_RET(head != flat.size(), HCCL_ERROR("[schedule] the recorded handshakes deadlock"), HCCL_E_INTERNAL);
     if (report != nullptr) {
@@ -137,10 +185,10 @@ HcclResult BuildOrder(World *w, std::vector<Node> &order, u32 &numLevels, CheckR
             reach.assign(flat.size(), std::vector<uint64_t>(words, 0));
             for (size_t k = ready.size(); k-- > 0;) {
                 const int id = ready[k];
-                for (int sx : succ[id]) {
+                succ[id].Each([&](int sx) {
                     for (size_t wd = 0; wd < words; ++wd) reach[id][wd] |= reach[sx][wd];
                     if (dataId[sx] >= 0) reach[id][dataId[sx] / 64] |= 1ull << (dataId[sx] % 64);
-                }
+                });
             }
         }
         auto ordered = [&](int a, int b) {   // flat ids of two data steps
@@ -187,7 +235,13 @@ HcclResult BuildOrder(World *w, std::vector<Node> &order, u32 &numLevels, CheckR
             active.push_back(k);
         }
     }
-    std::stable_sort(order.begin(), order.end(), [](const Node &a, const Node &b) { return a.level < b.level; });
+    // by level, steps of one level in the order found above (a counting sort)
+    std::vector<u32> at(numLevels + 1, 0);
+    for (const Node &nd : order) at[nd.level + 1]++;
+    for (u32 l = 0; l < numLevels; ++l) at[l + 1] += at[l];
+    std::vector<Node> sorted(order.size());
+    for (const Node &nd : order) sorted[at[nd.level]++] = nd;
+    order.swap(sorted);
     return HCCL_SUCCESS;
 }
 
@@ -367,7 +421,7 @@ private:
 // One output piece flattened to a fold: source addresses in fold order.
 struct Fold {
     std::vector<u64> src;
-    u64 dst = 0;
+    std::vector<u64> dsts;    // every output piece that holds this value
     u64 bytes = 0;
     bool chain = true;        // false: a tree that no chain reproduces
     bool fits = true;         // false: a tree too large for the tree kernels
@@ -425,21 +479,25 @@ struct InputRanges {
     }
 };
 
+// An input byte as the trace names it: "x<rank>@<offset>", the lowest rank whose input holds the address, as a
+// reader of the trace expects for shared buffers.
+std::string LeafText(u64 addr, const InputRanges &inputs)
+{
+    const InputRanges::Range *best = nullptr;
+    auto it = std::upper_bound(inputs.sorted.begin(), inputs.sorted.end(), addr,
+                               [](u64 v, const InputRanges::Range &x) { return v < x.base; });
+    while (it != inputs.sorted.begin()) {
+        --it;
+        if (it->base + inputs.longest <= addr) break;
+        if (addr < it->base + std::max<u64>(it->size, 1) && (best == nullptr || it->rank < best->rank)) best = &*it;
+    }
+    if (best == nullptr) return "?";
+    return "x" + std::to_string(best->rank) + "@" + std::to_string(addr - best->base);
+}
+
 std::string ExprText(const Tracer &tr, int e, u64 shift, const InputRanges &inputs)
 {
-    if (e == 0) {
-        // the lowest rank whose input holds the address, as a reader of the trace expects for shared buffers
-        const InputRanges::Range *best = nullptr;
-        auto it = std::upper_bound(inputs.sorted.begin(), inputs.sorted.end(), shift,
-                                   [](u64 v, const InputRanges::Range &x) { return v < x.base; });
-        while (it != inputs.sorted.begin()) {
-            --it;
-            if (it->base + inputs.longest <= shift) break;
-            if (shift < it->base + std::max<u64>(it->size, 1) && (best == nullptr || it->rank < best->rank)) best = &*it;
-        }
-        if (best == nullptr) return "?";
-        return "x" + std::to_string(best->rank) + "@" + std::to_string(shift - best->base);
-    }
+    if (e == 0) return LeafText(shift, inputs);
     const Expr &x = tr.At(e);
     return "(" + ExprText(tr, x.src, shift + x.srcShift, inputs) + "+" + ExprText(tr, x.dst, shift + x.dstShift, inputs) +
            ")";
@@ -539,63 +597,140 @@ struct FusedPlan {
     u64 stagingBytes = 0;
 };
 
+// Output pieces beyond which a schedule is run step by step instead of being fused.
+constexpr size_t kMaxFusedPieces = 400000;
+
 bool Overlaps(u64 a, u64 alen, u64 b, u64 blen) { return a < b + blen && b < a + alen; }
 
-// Builds the fused launch plan from the traced outputs.  Returns false when the schedule cannot be fused
-// (a floating-point tree with more than six levels or 64 leaves, a source that is not an input, or an output
-// that overlaps another fold's source); the caller then runs the steps one by one.
-bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &params, int dtype, int op, u32 esz,
-                    FusedPlan &plan, std::string *text)
+// The folds of a traced schedule: one per distinct value among the output pieces.  Returns false when the schedule
+// cannot be fused (a floating-point tree with more than six levels or 64 leaves, or too many pieces).
+bool FoldsFromTrace(const Tracer &tr, const std::vector<OpParam> &params, int dtype, int op, std::vector<Fold> &folds,
+                    std::string *text)
 {
-    std::vector<Fold> folds;
+    // One fold per distinct value: output pieces that hold the same expression (the copies an AllReduce hands to
+    // every rank) are destinations of one fold, flattened once.
+    struct PieceKey {
+        int expr;
+        u64 shift, len;
+        bool operator==(const PieceKey &o) const { return expr == o.expr && shift == o.shift && len == o.len; }
+    };
+    struct PieceHash {
+        size_t operator()(const PieceKey &k) const
+        {
+            u64 h = static_cast<u64>(k.expr) * 0x9E3779B97F4A7C15ull;
+            h ^= (k.shift + 0x9E3779B97F4A7C15ull + (h << 6) + (h >> 2));
+            h ^= (k.len + 0x9E3779B97F4A7C15ull + (h << 6) + (h >> 2));
+            return static_cast<size_t>(h);
+        }
+    };
+    std::unordered_map<PieceKey, size_t, PieceHash> byPiece;
     bool allFit = true;
+    size_t pieces = 0;
     const InputRanges inputs(params);
     for (size_t r = 0; r < params.size(); ++r) {
         const u64 out = reinterpret_cast<u64>(params[r].outputPtr);
         if (params[r].outputSize == 0) continue;
         for (const Sub &s : tr.Lookup(out, params[r].outputSize)) {
             if (s.expr == 0 && s.shift == s.start) continue;  // never written: stays as it is
-            Fold f = Flatten(tr, s.expr, s.shift, dtype, op);
-            f.dst = s.start;
-            f.bytes = s.len;
             if (text) {
                 std::ostringstream os;
                 os << "rank " << r << " out[" << (s.start - out) << "," << s.len << ") = "
                    << ExprText(tr, s.expr, s.shift, inputs) << "\n";
                 *text += os.str();
             }
-            if (!f.fits) allFit = false;
-            folds.push_back(std::move(f));
-            if (folds.size() > 100000) return false;   // more pieces than one pass is worth planning for
+            if (++pieces > kMaxFusedPieces) return false;   // more pieces than one pass is worth planning for
+            auto found = byPiece.emplace(PieceKey{s.expr, s.shift, s.len}, folds.size());
+            if (found.second) {
+                Fold f = Flatten(tr, s.expr, s.shift, dtype, op);
+                f.bytes = s.len;
+                if (!f.fits) allFit = false;
+                folds.push_back(std::move(f));
+            }
+            folds[found.first->second].dsts.push_back(s.start);
         }
     }
-    if (!allFit) return false;
+    g_phase.Lap(" flatten");
+    return allFit;
+}
+
+// The folds of a collective that its executor and template state in closed form, and, with `text`, the trace they
+// stand for: the same lines the recorded steps give when traced.
+void FoldsFromClosedForm(const std::vector<ClosedFold> &closed, const std::vector<OpParam> &params, std::vector<Fold> &folds,
+                         std::string *text)
+{
+    const InputRanges inputs(params);
+    struct Line {
+        u32 rank;
+        u64 offset;
+        size_t fold;
+    };
+    std::vector<Line> lines;
+    folds.reserve(closed.size());
+    for (const ClosedFold &c : closed) {
+        Fold f;
+        f.bytes = c.bytes;
+        for (const ClosedFold::Ref &s : c.src) f.src.push_back(reinterpret_cast<u64>(params[s.rank].inputPtr) + s.offset);
+        for (const ClosedFold::Ref &d : c.dst) {
+            f.dsts.push_back(reinterpret_cast<u64>(params[d.rank].outputPtr) + d.offset);
+            if (text) lines.push_back({d.rank, d.offset, folds.size()});
+        }
+        folds.push_back(std::move(f));
+    }
+    if (text == nullptr) return;
+    std::sort(lines.begin(), lines.end(),
+              [](const Line &a, const Line &b) { return a.rank != b.rank ? a.rank < b.rank : a.offset < b.offset; });
+    for (const Line &l : lines) {
+        const Fold &f = folds[l.fold];
+        std::string expr = LeafText(f.src[0], inputs);
+        for (size_t k = 1; k < f.src.size(); ++k) expr = "(" + LeafText(f.src[k], inputs) + "+" + expr + ")";
+        std::ostringstream os;
+        os << "rank " << l.rank << " out[" << l.offset << "," << f.bytes << ") = " << expr << "\n";
+        *text += os.str();
+    }
+}
+
+// Builds the fused launch plan from the folds.  Returns false when they cannot run as one pass (a source that is
+// not an input, or an output that overlaps another fold's source); the caller then runs the steps one by one.
+bool BuildFusedPlan(const std::vector<OpParam> &params, std::vector<Fold> &folds, u32 esz, FusedPlan &plan)
+{
+    const InputRanges inputs(params);
     // every source must be input data (or an output that the same fold overwrites in place)
     for (const Fold &f : folds) {
         for (u64 a : f.src) {
             if (inputs.Find(a, f.bytes) == nullptr) return false;
         }
     }
-
-    // group folds with the same sources in the same order: one segment, several destinations
-    std::map<std::vector<u64>, std::vector<size_t>> bySrc;
-    for (size_t i = 0; i < folds.size(); ++i) {
-        std::vector<u64> key = folds[i].src;
-        key.push_back(folds[i].bytes);
-        for (u8 b : folds[i].prog) key.push_back(b);  // same sources, different tree: different value
-        bySrc[key].push_back(i);
+    // Different expressions may still read the same sources in the same order (pieces that were reduced by
+    // different steps of equal shape): they become one fold with all the destinations.
+    {
+        std::map<std::vector<u64>, size_t> bySrc;
+        std::vector<Fold> merged;
+        for (Fold &f : folds) {
+            std::vector<u64> key = f.src;
+            key.push_back(f.bytes);
+            for (u8 b : f.prog) key.push_back(b);  // same sources, different tree: different value
+            auto found = bySrc.emplace(std::move(key), merged.size());
+            if (found.second) {
+                merged.push_back(std::move(f));
+            } else {
+                Fold &into = merged[found.first->second];
+                into.dsts.insert(into.dsts.end(), f.dsts.begin(), f.dsts.end());
+            }
+        }
+        folds.swap(merged);
     }
-    // and find groups of N folds over the same N sources where fold j starts from source j and then takes
-    // the others in a common order: the per-rank order of the one-shot templates, computed in one pass
+    g_phase.Lap(" bysrc");
+    // Find groups of N single-destination folds over the same N sources where fold j starts from source j and then
+    // takes the others in a common order: the per-rank order of the one-shot templates, computed in one pass.
     std::map<std::vector<u64>, std::vector<size_t>> bySet;
-    for (auto &kv : bySrc) {
-        if (kv.second.size() != 1) continue;
-        const Fold &f = folds[kv.second[0]];
+    for (size_t i = 0; i < folds.size(); ++i) {
+        const Fold &f = folds[i];
+        if (f.dsts.size() != 1) continue;
         if (!f.chain || !f.prog.empty() || f.src.size() < 2 || f.src.size() > HCCLX_MAX_WIDE_FAN) continue;
         std::vector<u64> key = f.src;
         std::sort(key.begin(), key.end());
         key.push_back(f.bytes);
-        bySet[key].push_back(kv.second[0]);
+        bySet[key].push_back(i);
     }
     std::vector<bool> taken(folds.size(), false);
     std::vector<bool> staged(folds.size(), false);   // written by the second launch: cannot race with what the first reads
@@ -631,7 +766,7 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
                 bool clash = false;
                 for (size_t j = 0; j < n && !clash; ++j) {
                     for (size_t k = 0; k < n && !clash; ++k) {
-                        clash = Overlaps(folds[owner[j]].dst, folds[owner[j]].bytes, base[k], folds[cand].bytes);
+                        clash = Overlaps(folds[owner[j]].dsts[0], folds[owner[j]].bytes, base[k], folds[cand].bytes);
                     }
                 }
                 hcclx_wide_seg_t seg;
@@ -640,13 +775,14 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
                 seg.nsrc = static_cast<uint32_t>(n);
                 seg.ndst = static_cast<uint32_t>(n);
                 for (size_t j = 0; j < n; ++j) {
+                    const Fold &fj = folds[owner[j]];
                     seg.src[j] = reinterpret_cast<const void *>(base[j]);
-                    seg.dst[j] = reinterpret_cast<void *>(folds[owner[j]].dst);
+                    seg.dst[j] = reinterpret_cast<void *>(fj.dsts[0]);
                     taken[owner[j]] = true;
                     if (clash) {
                         seg.dst[j] = reinterpret_cast<void *>(plan.stagingBytes);
-                        plan.stagedCopies.push_back({plan.stagingBytes, folds[owner[j]].dst, folds[owner[j]].bytes});
-                        plan.stagingBytes += (folds[owner[j]].bytes + 255) & ~static_cast<u64>(255);
+                        plan.stagedCopies.push_back({plan.stagingBytes, fj.dsts[0], fj.bytes});
+                        plan.stagingBytes += (fj.bytes + 255) & ~static_cast<u64>(255);
                         staged[owner[j]] = true;
                     }
                 }
@@ -664,7 +800,7 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
             seg.ndst = static_cast<uint32_t>(n);
             for (size_t j = 0; j < n; ++j) {
                 seg.src[j] = reinterpret_cast<const void *>(base[j]);
-                seg.dst[j] = reinterpret_cast<void *>(folds[owner[j]].dst);
+                seg.dst[j] = reinterpret_cast<void *>(folds[owner[j]].dsts[0]);
                 taken[owner[j]] = true;
                 group[owner[j]] = static_cast<int>(plan.selfSegs.size());
             }
@@ -672,11 +808,27 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
             break;
         }
     }
+    g_phase.Lap(" selfgroups");
     // A destination may coincide exactly with a source of its own fold, or of a fold of the same
     // self-first group (every thread reads all sources of an element before it writes any destination):
     // that is an in-place collective.  Any other overlap between what one fold writes and what another
     // reads would be a race inside a single pass.
-    {
+    // Every source lies in a rank's input and every destination in a rank's output: when no output buffer touches
+    // an input buffer there is nothing to look for.
+    bool apart = true;
+    for (size_t r = 0; r < params.size() && apart; ++r) {
+        if (params[r].outputSize == 0) continue;
+        const u64 lo = reinterpret_cast<u64>(params[r].outputPtr);
+        const u64 hi = lo + params[r].outputSize;
+        for (const InputRanges::Range &in : inputs.sorted) {
+            if (in.base >= hi) break;
+            if (in.size != 0 && in.base + in.size > lo) {
+                apart = false;
+                break;
+            }
+        }
+    }
+    if (!apart) {
         struct Read {
             u64 addr;
             u64 bytes;
@@ -691,36 +843,36 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
         std::sort(reads.begin(), reads.end(), [](const Read &x, const Read &y) { return x.addr < y.addr; });
         for (size_t i = 0; i < folds.size(); ++i) {
             if (staged[i]) continue;
-            // reads that can reach into [dst, dst + bytes) start after dst - longest
-            const u64 from = folds[i].dst > longest ? folds[i].dst - longest : 0;
-            auto it = std::lower_bound(reads.begin(), reads.end(), from,
-                                       [](const Read &x, u64 v) { return x.addr < v; });
-            for (; it != reads.end() && it->addr < folds[i].dst + folds[i].bytes; ++it) {
-                if (!Overlaps(folds[i].dst, folds[i].bytes, it->addr, it->bytes)) continue;
-                const size_t j = it->fold;
-                const bool sameUnit = (i == j) || (group[i] != -1 && group[i] == group[j]);
-                if (sameUnit && it->addr == folds[i].dst) continue;
-                return false;
+            for (u64 dst : folds[i].dsts) {
+                // reads that can reach into [dst, dst + bytes) start after dst - longest
+                const u64 from = dst > longest ? dst - longest : 0;
+                auto it = std::lower_bound(reads.begin(), reads.end(), from,
+                                           [](const Read &x, u64 v) { return x.addr < v; });
+                for (; it != reads.end() && it->addr < dst + folds[i].bytes; ++it) {
+                    if (!Overlaps(dst, folds[i].bytes, it->addr, it->bytes)) continue;
+                    const size_t j = it->fold;
+                    const bool sameUnit = (i == j) || (group[i] != -1 && group[i] == group[j]);
+                    if (sameUnit && it->addr == dst) continue;
+                    return false;
+                }
             }
         }
     }
-    for (auto &kv : bySrc) {
-        std::vector<size_t> rest;
-        for (size_t i : kv.second) {
-            if (!taken[i]) rest.push_back(i);
-        }
-        if (!rest.empty() && (folds[rest[0]].src.size() > HCCLX_MAX_FAN || (1u << folds[rest[0]].levels) > HCCLX_MAX_FAN)) {
+    g_phase.Lap(" overlaps");
+    for (size_t i = 0; i < folds.size(); ++i) {
+        if (taken[i]) continue;
+        const Fold &f = folds[i];
+        if (f.src.size() > HCCLX_MAX_FAN || (1u << f.levels) > HCCLX_MAX_FAN) {
             // more ranks than the register-resident kernels take: the wide kernels
-            const Fold &f = folds[rest[0]];
             if (f.src.size() > HCCLX_MAX_WIDE_FAN) return false;
-            for (size_t at = 0; at < rest.size(); at += HCCLX_MAX_WIDE_FAN) {
+            for (size_t at = 0; at < f.dsts.size(); at += HCCLX_MAX_WIDE_FAN) {
                 hcclx_wide_seg_t seg;
                 std::memset(&seg, 0, sizeof(seg));
                 seg.count = f.bytes / esz;
                 seg.nsrc = static_cast<uint32_t>(f.src.size());
                 for (size_t k = 0; k < f.src.size(); ++k) seg.src[k] = reinterpret_cast<const void *>(f.src[k]);
-                for (size_t d = at; d < rest.size() && d < at + HCCLX_MAX_WIDE_FAN; ++d) {
-                    seg.dst[seg.ndst++] = reinterpret_cast<void *>(folds[rest[d]].dst);
+                for (size_t d = at; d < f.dsts.size() && d < at + HCCLX_MAX_WIDE_FAN; ++d) {
+                    seg.dst[seg.ndst++] = reinterpret_cast<void *>(f.dsts[d]);
                 }
                 if (f.chain) {
                     if (!f.prog.empty()) std::memcpy(seg.prog, f.prog.data(), f.prog.size());
@@ -732,14 +884,13 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
             }
             continue;
         }
-        for (size_t at = 0; at < rest.size(); at += HCCLX_MAX_FAN) {
-            const Fold &f = folds[rest[at]];
+        for (size_t at = 0; at < f.dsts.size(); at += HCCLX_MAX_FAN) {
             hcclx_seg_t seg;
             std::memset(&seg, 0, sizeof(seg));
             seg.nsrc = static_cast<uint32_t>(f.src.size());
             for (size_t k = 0; k < f.src.size(); ++k) seg.src[k] = reinterpret_cast<const void *>(f.src[k]);
-            for (size_t d = at; d < rest.size() && d < at + HCCLX_MAX_FAN; ++d) {
-                seg.dst[seg.ndst++] = reinterpret_cast<void *>(folds[rest[d]].dst);
+            for (size_t d = at; d < f.dsts.size() && d < at + HCCLX_MAX_FAN; ++d) {
+                seg.dst[seg.ndst++] = reinterpret_cast<void *>(f.dsts[d]);
             }
             if (f.src.size() == 1) {
                 seg.count = f.bytes;  // a copy: counted in bytes
@@ -755,7 +906,6 @@ bool BuildFusedPlan(World *w, const Tracer &tr, const std::vector<OpParam> &para
             }
         }
     }
-    (void)w;
     return true;
 }
 
@@ -1403,57 +1553,88 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
     }
 
     // expand: every rank's executor + template records its steps
-    static const bool kTiming = std::getenv("HCCL_VRANK_TIMING") != nullptr;
-    auto tnow = [] { return std::chrono::steady_clock::now(); };
-    auto t0 = tnow();
-    auto lap = [&](const char *what) {
-        if (!kTiming) return;
-        auto t1 = tnow();
-        std::fprintf(stderr, "[timing] %-12s %8.3f ms\n", what, std::chrono::duration<double, std::milli>(t1 - t0).count());
-        t0 = t1;
-    };
-    CHK_RET(w->EnsureScratch());
-    w->ResetRecording();
-    for (u32 r = 0; r < n; ++r) {
-        params[r].algName = algName;
-        std::unique_ptr<InsCollAlgBase> exec = CollAlgExecRegistryV2::Instance().GetAlgExec(type, algName);
-        CHK_PRT_RET(exec == nullptr, HCCL_ERROR("[RunCollective] no executor named %s", algName.c_str()),
-                    HCCL_E_NOT_SUPPORT);
-        AlgResourceCtxSerializable resCtx;
-        const u64 threadNum = exec->CalcThreadNum(params[r], r, n);
-        FillResources(w, r, static_cast<u32>(threadNum), resCtx);
-        CHK_RET(exec->Orchestrate(params[r], resCtx));
-    }
-    lap("record");
+    g_phase.Start();
+    auto lap = [](const char *what) { g_phase.Lap(what); };
+    // A fused pass never touches the scratch buffers (their addresses only name intermediate values while the
+    // schedule is traced), so they stand for themselves as address ranges until a schedule has to run step by step.
     std::vector<Node> order;
     u32 numLevels = 0;
-    w->lastCheck = CheckReport();
-    CHK_RET(BuildOrder(w, order, numLevels, w->check ? &w->lastCheck : nullptr));
-    w->lastLevels = numLevels;
-    lap("order");
-
+    bool recordedOnMemory = false;
+    auto expand = [&](bool scratchMemory) -> HcclResult {
+        CHK_RET(w->EnsureScratch(scratchMemory));
+        recordedOnMemory = w->scratchIsMemory;
+        lap("scratch");
+        w->ResetRecording();
+        for (u32 r = 0; r < n; ++r) {
+            params[r].algName = algName;
+            std::unique_ptr<InsCollAlgBase> exec = CollAlgExecRegistryV2::Instance().GetAlgExec(type, algName);
+            CHK_PRT_RET(exec == nullptr, HCCL_ERROR("[RunCollective] no executor named %s", algName.c_str()),
+                        HCCL_E_NOT_SUPPORT);
+            AlgResourceCtxSerializable resCtx;
+            const u64 threadNum = exec->CalcThreadNum(params[r], r, n);
+            FillResources(w, r, static_cast<u32>(threadNum), resCtx);
+            CHK_RET(exec->Orchestrate(params[r], resCtx));
+        }
+        lap("record");
+        CHK_RET(BuildOrder(w, order, numLevels, w->check ? &w->lastCheck : nullptr));
+        w->lastLevels = numLevels;
+        if (g_phase.on) {
+            size_t items = 0;
+            for (auto &perRank : w->threads) {
+                for (auto &t : perRank) items += t->items.size();
+            }
+            std::fprintf(stderr, "[timing] %zu recorded items, %zu data steps, %u levels\n", items, order.size(), numLevels);
+        }
+        lap("order");
+        return HCCL_SUCCESS;
+    };
     const u32 esz = IsDataMove(type) ? 1 : DATATYPE_SIZE_TABLE[dtype];
     const int foldType = IsDataMove(type) ? HCCL_DATA_TYPE_INT8 : dtype;
-    if (fused || w->dryRun || w->traceText || w->check) {
-        Tracer tr;
-        for (const Node &nd : order) {
-            const TaskItem &it = *nd.item;
-            if (it.kind == ItemKind::COPY) {
-                tr.Copy(reinterpret_cast<u64>(it.dst), reinterpret_cast<u64>(it.src), it.bytes);
-            } else {
-                tr.Reduce(reinterpret_cast<u64>(it.dst), reinterpret_cast<u64>(it.src), it.bytes);
-            }
+    std::string *text = (w->traceText || (w->dryRun && !g_phase.on)) ? &w->lastTrace : nullptr;
+    w->lastTrace.clear();
+    w->lastCheck = CheckReport();
+
+    // A template whose steps grow with the cube of the rank count may state its result in closed form: then nothing
+    // is recorded, ordered or traced.  Only among buffers that lie apart (what the steps amount to does not depend
+    // on where they are then), and never when the schedule itself is to be checked.
+    std::vector<Fold> folds;
+    bool haveFolds = false;
+    const bool plain = !w->dryRun && !w->traceText && !w->check;
+    if ((fused || w->dryRun || w->traceText) && !w->check && !IsDataMove(type) &&
+        (w->closedForm == 2 || (w->closedForm == 1 && plain)) && (plain ? separate : BuffersAreSeparate(params))) {
+        std::unique_ptr<InsCollAlgBase> exec = CollAlgExecRegistryV2::Instance().GetAlgExec(type, algName);
+        std::vector<ClosedFold> closed;
+        params[0].algName = algName;
+        if (exec != nullptr && exec->ClosedForm(params[0], n, w->cclBytes, closed)) {
+            FoldsFromClosedForm(closed, params, folds, text);
+            haveFolds = true;
+            lap("closedform");
         }
-        lap("trace");
-        if (w->check) {
-            CheckSemantics(tr, params, w->lastCheck);
-            CHK_PRT_RET(w->lastCheck.races != 0 || w->lastCheck.semanticErrors != 0,
-                        HCCL_ERROR("[schedule check] %s", w->lastCheck.firstProblem.c_str()), HCCL_E_INTERNAL);
+    }
+    if (!haveFolds) CHK_RET(expand(!fused && !w->dryRun));
+
+    if (fused || w->dryRun || w->traceText || w->check) {
+        bool ok = true;
+        if (!haveFolds) {
+            Tracer tr;
+            for (const Node &nd : order) {
+                const TaskItem &it = *nd.item;
+                if (it.kind == ItemKind::COPY) {
+                    tr.Copy(reinterpret_cast<u64>(it.dst), reinterpret_cast<u64>(it.src), it.bytes);
+                } else {
+                    tr.Reduce(reinterpret_cast<u64>(it.dst), reinterpret_cast<u64>(it.src), it.bytes);
+                }
+            }
+            lap("trace");
+            if (w->check) {
+                CheckSemantics(tr, params, w->lastCheck);
+                CHK_PRT_RET(w->lastCheck.races != 0 || w->lastCheck.semanticErrors != 0,
+                            HCCL_ERROR("[schedule check] %s", w->lastCheck.firstProblem.c_str()), HCCL_E_INTERNAL);
+            }
+            ok = FoldsFromTrace(tr, params, foldType, op, folds, text);
         }
         FusedPlan plan;
-        w->lastTrace.clear();
-        const bool ok = BuildFusedPlan(w, tr, params, foldType, op, esz, plan,
-                                       (w->traceText || w->dryRun) ? &w->lastTrace : nullptr);
+        ok = ok && BuildFusedPlan(params, folds, esz, plan);
         lap("fusedplan");
         w->lastFusedSegments =
             static_cast<u32>(plan.chainSegs.size() + plan.selfSegs.size() + plan.copySegs.size() + plan.treeSegs.size() +
@@ -1525,12 +1706,14 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
             lap("tables");
             w->lastWasFused = true;
             const HcclResult res = LaunchAndKeep(w, std::move(c), stream);
+            lap("launch");
             if (res == HCCL_SUCCESS && separate && !stagedOutputs) {
                 KeepShape(w->planCache, shape, std::move(parts), params, true, numLevels, w->lastFusedSegments);
             }
             return res;
         }
     }
+    if (!recordedOnMemory) CHK_RET(expand(true));   // recorded (again) against scratch buffers that exist
     std::vector<HostPart> parts;
     BuildStepParts(order, numLevels, foldType, op, parts);
     CachedPlan c;

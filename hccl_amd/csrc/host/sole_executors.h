@@ -56,6 +56,29 @@ public:
         TemplateDataParams t;
         detail::FillBuffInfo(param, resCtx, t, res);
         InsAlgTemplate alg(param, myRank_, resCtx.subCommRanks);
+        return Loops(alg, t, [&]() { return alg.KernelRun(param, t, res); });
+    }
+    bool ClosedForm(const OpParam &param, u32 rankSize, u64 cclBytes, std::vector<ClosedFold> &out) override
+    {
+        dataType_ = param.DataDes.dataType;
+        dataCount_ = param.DataDes.count;
+        dataTypeSize_ = DATATYPE_SIZE_TABLE[dataType_];
+        TemplateDataParams t;
+        t.buffInfo.hcclBuff.size = cclBytes;
+        t.repeatNum = 1;
+        InsAlgTemplate alg(param, 0, AlgTopoMatch::Match(rankSize));
+        bool all = true;
+        const HcclResult res = Loops(alg, t, [&]() {
+            all = all && alg.ClosedForm(t, dataTypeSize_, out);
+            return HCCL_SUCCESS;
+        });
+        return res == HCCL_SUCCESS && all;
+    }
+
+private:
+    // The chunk loop (:120-185): `body` runs once per chunk with `t` describing it.
+    template <typename F> HcclResult Loops(InsAlgTemplate &alg, TemplateDataParams &t, F &&body)
+    {
         const u64 mult = alg.CalcScratchMultiple(t.buffInfo.inBuffType, t.buffInfo.outBuffType);
         maxTmpMemSize_ = t.buffInfo.hcclBuff.size;
         const u64 maxCount = MaxDataSizePerLoop(maxTmpMemSize_, mult, maxTmpMemSize_) / dataTypeSize_;
@@ -72,7 +95,7 @@ public:
             t.tailSize = t.sliceSize;
             t.inputSliceStride = 0;
             t.outputSliceStride = 0;
-            CHK_RET(alg.KernelRun(param, t, res));
+            CHK_RET(body());
             done += cur;
         }
         return HCCL_SUCCESS;
@@ -102,6 +125,30 @@ public:
         TemplateDataParams t;
         detail::FillBuffInfo(param, resCtx, t, res);
         InsAlgTemplate alg(param, myRank_, resCtx.subCommRanks);
+        return Loops(alg, t, [&]() { return alg.KernelRun(param, t, res); });
+    }
+    bool ClosedForm(const OpParam &param, u32 rankSize, u64 cclBytes, std::vector<ClosedFold> &out) override
+    {
+        dataType_ = param.DataDes.dataType;
+        dataCount_ = param.DataDes.count;
+        dataTypeSize_ = DATATYPE_SIZE_TABLE[dataType_];
+        dataSize_ = dataCount_ * dataTypeSize_;
+        TemplateDataParams t;
+        t.buffInfo.hcclBuff.size = cclBytes;
+        t.repeatNum = 1;
+        InsAlgTemplate alg(param, 0, AlgTopoMatch::Match(rankSize));
+        bool all = true;
+        const HcclResult res = Loops(alg, t, [&]() {
+            all = all && alg.ClosedForm(t, dataTypeSize_, out);
+            return HCCL_SUCCESS;
+        });
+        return res == HCCL_SUCCESS && all;
+    }
+
+private:
+    // The chunk loop (:123-170): `body` runs once per chunk with `t` describing it.
+    template <typename F> HcclResult Loops(InsAlgTemplate &alg, TemplateDataParams &t, F &&body)
+    {
         const u64 mult = alg.CalcScratchMultiple(t.buffInfo.inBuffType, t.buffInfo.outBuffType);
         maxTmpMemSize_ = t.buffInfo.hcclBuff.size - 1 * 1024 * 1024;  // one MiB is kept back (:126-128)
         const u64 maxCount = MaxDataSizePerLoop(maxTmpMemSize_, mult, maxTmpMemSize_) / dataTypeSize_;
@@ -118,7 +165,7 @@ public:
             t.tailSize = t.sliceSize;
             t.inputSliceStride = dataSize_;  // shard k of the input starts k * (recvCount * size) in
             t.outputSliceStride = 0;
-            CHK_RET(alg.KernelRun(param, t, res));
+            CHK_RET(body());
             done += cur;
         }
         return HCCL_SUCCESS;

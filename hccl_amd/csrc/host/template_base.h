@@ -30,6 +30,17 @@ public:
     virtual HcclResult KernelRun(const OpParam &param, const TemplateDataParams &tempAlgParams,
                                  TemplateResource &templateResource) = 0;
 
+    // The net effect of one KernelRun among all ranks, appended to `out`, for templates whose recorded steps grow
+    // with the cube of the rank count: the world then plans from this instead of recording and tracing them.  Only
+    // the offsets, strides and counts of `tempAlgParams` are used.  The default: no closed form (record the steps).
+    virtual bool ClosedForm(const TemplateDataParams &tempAlgParams, u64 dataTypeSize, std::vector<ClosedFold> &out) const
+    {
+        (void)tempAlgParams;
+        (void)dataTypeSize;
+        (void)out;
+        return false;
+    }
+
     virtual void GetNotifyIdxMainToSub(std::vector<u32> &notifyIdxMainToSub)
     {
         // every sub thread is woken on its own notify 0

@@ -1,6 +1,7 @@
 // Virtual-rank world: creation, the recording primitive backend and the rank rendezvous.
 #include "vcomm.h"
 
+#include <algorithm>
 #include <cstring>
 
 #include "hcclx.h"
@@ -14,14 +15,22 @@ namespace {
 std::mutex g_worldsMu;
 std::vector<World *> g_worlds;
 
-u64 ChannelKey(u32 sender, u32 receiver, u32 idx)
-{
-    return (1ull << 63) | (static_cast<u64>(sender) << 40) | (static_cast<u64>(receiver) << 16) | idx;
-}
+// Notify indices a thread or channel may use (the templates stay below 4 * ranks).
+constexpr u32 kMaxNotifyIdx = 4096;
 
-u64 ThreadKey(const VThread *t, u32 idx)
+// The number of the notify identity `idx` of a table (a channel direction or a thread), assigned on first use and
+// kept for the life of the world.
+bool SlotOf(World *w, std::vector<u32> &table, u32 idx, u64 &slot)
 {
-    return (static_cast<u64>(t->rank) << 40) | (static_cast<u64>(t->index) << 16) | idx;
+    if (idx >= kMaxNotifyIdx) return false;
+    if (idx >= table.size()) table.resize(idx + 1, 0);
+    if (table[idx] == 0) {
+        w->recordSeq.push_back(0);
+        w->waitSeq.push_back(0);
+        table[idx] = static_cast<u32>(w->recordSeq.size());
+    }
+    slot = table[idx] - 1;
+    return true;
 }
 
 VThread *AsThread(ThreadHandle h) { return reinterpret_cast<VThread *>(h); }
@@ -69,7 +78,7 @@ int32_t ReduceArgsOk(HcommDataType dt, HcommReduceOp op)
 World::~World()
 {
     for (char *p : cclBuf) {
-        if (p && !dryRun) (void)hipFree(p);
+        if (p && scratchIsMemory) (void)hipFree(p);
     }
     if (!dryRun && (!planCache.lru.empty() || !planCache.retired.empty())) (void)hipDeviceSynchronize();
     for (RetiredPlan &r : planCache.retired) {
@@ -83,28 +92,42 @@ World::~World()
     }
 }
 
-HcclResult World::EnsureScratch()
+// Placeholder scratch addresses: non-canonical, so they can never collide with memory of the process, one
+// non-overlapping terabyte per rank.
+static char *ScratchPlaceholder(u32 rank)
 {
-    for (u32 r = 0; r < rankSize; ++r) {
-        if (cclBuf[r] == nullptr && dryRun) {
-            // never dereferenced: a distinct, non-overlapping address range per rank
-            cclBuf[r] = reinterpret_cast<char *>(0x7000000000000000ull + static_cast<u64>(r) * (1ull << 40));
+    return reinterpret_cast<char *>(0x7000000000000000ull + static_cast<u64>(rank) * (1ull << 40));
+}
+
+HcclResult World::EnsureScratch(bool memory)
+{
+    if (!memory || dryRun) {
+        for (u32 r = 0; r < rankSize; ++r) {
+            if (cclBuf[r] == nullptr) cclBuf[r] = ScratchPlaceholder(r);
         }
-        if (cclBuf[r] == nullptr) {
-            hipError_t e = hipMalloc(reinterpret_cast<void **>(&cclBuf[r]), cclBytes);
-            if (e != hipSuccess) {
-                HCCL_ERROR("scratch buffer of rank %u: %s", r, hipGetErrorString(e));
-                return HCCL_E_MEMORY;
+        return HCCL_SUCCESS;
+    }
+    if (scratchIsMemory) return HCCL_SUCCESS;
+    std::vector<char *> made(rankSize, nullptr);
+    for (u32 r = 0; r < rankSize; ++r) {
+        const hipError_t e = hipMalloc(reinterpret_cast<void **>(&made[r]), cclBytes);
+        if (e != hipSuccess) {
+            HCCL_ERROR("scratch buffer of rank %u: %s", r, hipGetErrorString(e));
+            for (char *p : made) {
+                if (p) (void)hipFree(p);
             }
+            return HCCL_E_MEMORY;
         }
     }
+    cclBuf = made;
+    scratchIsMemory = true;
     return HCCL_SUCCESS;
 }
 
 void World::ResetRecording()
 {
-    recordSeq.clear();
-    waitSeq.clear();
+    std::fill(recordSeq.begin(), recordSeq.end(), 0u);
+    std::fill(waitSeq.begin(), waitSeq.end(), 0u);
     for (auto &perRank : threads) {
         for (auto &t : perRank) t->items.clear();
     }
@@ -125,6 +148,7 @@ HcclResult WorldCreate(u32 rankSize, u64 cclBytes, bool dryRun, std::vector<Hccl
     }
     if (const char *b = std::getenv("HCCL_VRANK_BLOCKING")) w->blocking = (std::atoi(b) != 0);
     if (const char *c = std::getenv("HCCL_VRANK_CHECK")) w->check = (std::atoi(c) != 0);
+    if (const char *c = std::getenv("HCCL_VRANK_CLOSED_FORM")) w->closedForm = std::max(0, std::min(2, std::atoi(c)));
     {
         u8 level = static_cast<u8>(DeterministicEnableLevel::DETERMINISTIC_DISABLE);
         if (const char *d = std::getenv("HCCL_DETERMINISTIC")) {
@@ -317,7 +341,9 @@ int32_t HcommChannelNotifyRecordOnThread(ThreadHandle thread, ChannelHandle chan
     VThread *t = AsThread(thread);
     VChannel *c = AsChannel(channel);
     if (t == nullptr || c == nullptr) return HCCL_E_PTR;
-    return RecordNotify(t, ItemKind::NOTIFY_RECORD, ChannelKey(c->localRank, c->remoteRank, remoteNotifyIdx));
+    u64 slot = 0;
+    if (!SlotOf(t->world, c->notifySlot, remoteNotifyIdx, slot)) return HCCL_E_PARA;
+    return RecordNotify(t, ItemKind::NOTIFY_RECORD, slot);
 }
 
 int32_t HcommChannelNotifyWaitOnThread(ThreadHandle thread, ChannelHandle channel, uint32_t localNotifyIdx,
@@ -327,7 +353,13 @@ int32_t HcommChannelNotifyWaitOnThread(ThreadHandle thread, ChannelHandle channe
     VThread *t = AsThread(thread);
     VChannel *c = AsChannel(channel);
     if (t == nullptr || c == nullptr) return HCCL_E_PTR;
-    return RecordNotify(t, ItemKind::NOTIFY_WAIT, ChannelKey(c->remoteRank, c->localRank, localNotifyIdx));
+    World *w = t->world;
+    if (c->world != w || c->remoteRank >= w->rankSize || c->localRank >= w->rankSize) return HCCL_E_PARA;
+    // the same identity as the record on the sender's side of the link
+    VChannel *sender = w->channels[c->remoteRank][c->localRank].get();
+    u64 slot = 0;
+    if (!SlotOf(w, sender->notifySlot, localNotifyIdx, slot)) return HCCL_E_PARA;
+    return RecordNotify(t, ItemKind::NOTIFY_WAIT, slot);
 }
 
 int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThread, uint32_t dstNotifyIdx)
@@ -335,7 +367,9 @@ int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThr
     VThread *t = AsThread(thread);
     VThread *d = AsThread(dstThread);
     if (t == nullptr || d == nullptr) return HCCL_E_PTR;
-    return RecordNotify(t, ItemKind::NOTIFY_RECORD, ThreadKey(d, dstNotifyIdx));
+    u64 slot = 0;
+    if (!SlotOf(t->world, d->notifySlot, dstNotifyIdx, slot)) return HCCL_E_PARA;
+    return RecordNotify(t, ItemKind::NOTIFY_RECORD, slot);
 }
 
 int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, uint32_t timeout)
@@ -343,7 +377,9 @@ int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, u
     (void)timeout;
     VThread *t = AsThread(thread);
     if (t == nullptr) return HCCL_E_PTR;
-    return RecordNotify(t, ItemKind::NOTIFY_WAIT, ThreadKey(t, notifyIdx));
+    u64 slot = 0;
+    if (!SlotOf(t->world, t->notifySlot, notifyIdx, slot)) return HCCL_E_PARA;
+    return RecordNotify(t, ItemKind::NOTIFY_WAIT, slot);
 }
 
 int32_t HcommBatchTransferOnThread(ThreadHandle thread, ChannelHandle channel,

@@ -36,7 +36,7 @@ struct TaskItem {
     const char *src = nullptr;
     u64 bytes = 0;
     u64 count = 0;
-    u64 key = 0;  // notify identity: who signals whom on which index
+    u64 key = 0;  // notify identity (who signals whom on which index) as a dense number of the world
     u32 seq = 0;  // n-th record / n-th wait on that identity: they pair up in order
 };
 
@@ -47,12 +47,14 @@ struct VThread {
     u32 rank = 0;
     u32 index = 0;
     std::vector<TaskItem> items;
+    std::vector<u32> notifySlot;  // by notify index of this thread: identity number + 1, 0 = none yet
 };
 
 struct VChannel {
     World *world = nullptr;
     u32 localRank = 0;
     u32 remoteRank = 0;
+    std::vector<u32> notifySlot;  // by notify index, for signals from localRank to remoteRank: identity number + 1
 };
 
 enum class ExecMode {
@@ -151,7 +153,8 @@ struct World {
     ExecMode mode = ExecMode::FUSED;
     bool blocking = false;  // a rank's call returns only after the collective was launched
     std::vector<std::unique_ptr<RankComm>> ranks;
-    std::vector<char *> cclBuf;  // per rank, allocated on first use
+    std::vector<char *> cclBuf;  // per rank: an address range of its own; device memory once a schedule runs step by step
+    bool scratchIsMemory = false;
     std::vector<std::vector<std::unique_ptr<VThread>>> threads;    // [rank][thread]
     std::vector<std::vector<std::unique_ptr<VChannel>>> channels;  // [rank][peer]
 
@@ -162,8 +165,8 @@ struct World {
     std::vector<HcclResult> lastResult;
 
     // recording state of the collective being expanded
-    std::unordered_map<u64, u32> recordSeq;
-    std::unordered_map<u64, u32> waitSeq;
+    std::vector<u32> recordSeq;   // by notify identity: records / waits made so far
+    std::vector<u32> waitSeq;
 
     // statistics of the last launched collective, for tests and the benchmark
     std::string lastAlgName;
@@ -175,6 +178,7 @@ struct World {
     std::string lastTrace;  // expression of every output piece, filled when traceText is set
     bool traceText = false;
     bool check = false;     // verify every schedule before it is launched
+    int closedForm = 1;     // templates' closed forms: 0 never used, 1 for plain launches, 2 also when tracing / dry
     CheckReport lastCheck;
 
     PlanCache planCache;
@@ -191,7 +195,7 @@ struct World {
     bool dryRun = false;
 
     ~World();
-    HcclResult EnsureScratch();
+    HcclResult EnsureScratch(bool memory);
     void ResetRecording();
 };
 

@@ -770,3 +770,54 @@ def test_overlapping_buffers_are_planned_for_their_addresses(stream):
             assert_same_bits(recv2[r].get(np.float32), want3[r], T.FP32, f"shared input, rank {r}")
     finally:
         w.close()
+
+
+@pytest.mark.parametrize("kind,n,dtype,op,count", [("all_reduce", 64, T.FP32, T.SUM, 64 * 63 * 3 + 17),
+                                                   ("all_reduce", 32, T.BFP16, T.SUM, 400003),
+                                                   ("all_reduce", 12, T.INT32, T.MAX, 1 << 20),
+                                                   ("reduce_scatter", 64, T.FP32, T.SUM, 5003),
+                                                   ("reduce_scatter", 16, T.FP16, T.PROD, 70001)])
+def test_mesh_chunk_templates_planned_from_their_closed_form(stream, kind, n, dtype, op, count):
+    """Among many ranks the mesh-chunk templates are planned from their closed form (N (N-1) chains, nothing
+    recorded) and run as one fused pass: 64 ranks too.  The result is the oracle's replay of the N^3 steps, and the
+    same collective with the closed form switched off (steps recorded and traced) gives the same bits."""
+    alg = "InsAllReduceMesh1DTwoShotMeshChunk" if kind == "all_reduce" else "InsReduceScatterMesh1DMeshChunk"
+    cmd = api.CMD_ALLREDUCE if kind == "all_reduce" else api.CMD_REDUCE_SCATTER
+    rng = np.random.default_rng(n + count)
+    esz = T.DTYPE_SIZE[dtype]
+    ccl = 8 << 20
+    kindof = "prod" if op == T.PROD else "uniform" if dtype == T.FP32 else "normal"
+    send_count = count if kind == "all_reduce" else count * n
+    xs = [payload(rng, dtype, send_count, kindof) for _ in range(n)]
+    fused16 = dtype in (T.FP16, T.BFP16) and op == T.SUM
+    if kind == "all_reduce":
+        want = (wide_oracle_allreduce(xs, count, dtype, alg, ccl) if fused16 else
+                T.run_allreduce(T.NumericElems(dtype, op), xs, count, esz, alg, ccl_bytes=ccl))
+    else:
+        want = T.run_reduce_scatter(T.NumericElems(dtype, op), xs, count, esz, alg, ccl_bytes=ccl)
+    send = [DevBuf(x) for x in xs]
+    results = []
+    for closed_form in (1, 0):
+        w = api.World(n, ccl_bytes=ccl)
+        try:
+            w.set_algorithm(cmd, alg)
+            w.set_closed_form(closed_form)
+            recv = [DevBuf(nbytes=count * esz) for _ in range(n)]
+            torch.cuda.synchronize()
+            for r in range(n):
+                if kind == "all_reduce":
+                    assert w.all_reduce(r, send[r].ptr, recv[r].ptr, count, dtype, op, stream.cuda_stream) == 0
+                else:
+                    assert w.reduce_scatter(r, send[r].ptr, recv[r].ptr, count, dtype, op, stream.cuda_stream) == 0
+            stream.synchronize()
+            info = w.last_info()
+            assert info.fused == 1 and info.launches <= 2
+            assert (info.levels == 0) == (closed_form == 1)
+            got = [b.get(T.NP_STORAGE[dtype]) for b in recv]
+            for r in range(n):
+                assert_same_bits(got[r], want[r], dtype, f"{alg} rank {r} closed_form={closed_form}")
+                assert recv[r].guard_intact()
+            results.append(info.fusedSegments)
+        finally:
+            w.close()
+    assert results[0] == results[1]

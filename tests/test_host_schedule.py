@@ -551,3 +551,77 @@ def test_one_host_thread_per_rank_meets_at_every_collective():
         assert w.last_info().algName.decode().startswith("InsReduceScatter")
     finally:
         w.close()
+
+
+def traced(n, call, closed_form):
+    """Trace text and op info of one dry collective; `call(world, rank, in, out)` issues a rank's call."""
+    w = api.World(n, ccl_bytes=SMALL_CCL, dry=True)
+    try:
+        w.set_closed_form(closed_form)
+        return call(w), w.last_info()
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("n", [2, 3, 4, 5, 7, 8, 12, 16, 17, 31, 32])
+@pytest.mark.parametrize("kind", ["all_reduce", "reduce_scatter", "reduce_scatter_gather"])
+def test_closed_form_of_a_template_equals_its_recorded_steps(kind, n):
+    """The mesh-chunk templates and the gather-then-fold ReduceScatter state their result directly (N (N-1) chains,
+    N chains) so that a world need not record, order and trace their N^3 steps.  The statement must be exactly what the steps amount to: line for line the same
+    trace -- same pieces, same association order -- for short, ragged, 4 KiB-aligned and multi-chunk operands, every
+    element size, and in place."""
+    alg = {"all_reduce": "InsAllReduceMesh1DTwoShotMeshChunk", "reduce_scatter": "InsReduceScatterMesh1DMeshChunk",
+           "reduce_scatter_gather": "InsReduceScatterAicpuReduceNHR"}[kind]
+    cmd = api.CMD_ALLREDUCE if kind == "all_reduce" else api.CMD_REDUCE_SCATTER
+    ins, outs = fake_ptrs(n)
+    # per-rank received count for ReduceScatter; several executor chunks at the last sizes
+    # (the ReduceScatter template takes N-1 scratch slots per chunk, so its chunks are short among many ranks)
+    counts = [1, max(1, n - 1), n, n * (n - 1) + 1, 4099] + ([70001] if n <= 12 or kind == "all_reduce" else [])
+    counts += [300001] if n <= 8 else []
+    for count in counts:
+        for dtype in (T.INT8, T.FP32, T.FP64):
+            for in_place in (False, True):
+                if kind != "all_reduce" and in_place:
+                    continue   # a ReduceScatter's output is a part of its input: not apart, never in closed form
+                if (dtype != T.FP32 or in_place) and count not in (n, 4099, counts[-1]):
+                    continue
+
+                def call(w):
+                    w.set_algorithm(cmd, alg)
+                    for r in range(n):
+                        dst = ins[r] if in_place else outs[r]
+                        if kind == "all_reduce":
+                            assert w.all_reduce(r, ins[r], dst, count, dtype, T.SUM, FAKE_STREAM) == 0
+                        else:
+                            assert w.reduce_scatter(r, ins[r], dst, count, dtype, T.SUM, FAKE_STREAM) == 0
+                    return w.last_trace()
+
+                recorded, info_r = traced(n, call, 0)
+                closed, info_c = traced(n, call, 2)
+                assert info_r.levels > 0 and info_c.levels == 0, "the closed form was not used"
+                assert closed == recorded, f"{alg} n={n} count={count} dtype={dtype} in_place={in_place}"
+                assert info_c.fused == info_r.fused == 1 and info_c.fusedSegments == info_r.fusedSegments
+
+
+def test_closed_form_among_64_ranks_and_when_it_is_not_used():
+    alg = "InsAllReduceMesh1DTwoShotMeshChunk"
+    n, count = 64, 64 * 63 * 2 + 5
+    ins, outs = fake_ptrs(n)
+
+    def call(w, alg=alg, srcs=ins):
+        w.set_algorithm(api.CMD_ALLREDUCE, alg)
+        for r in range(n):
+            assert w.all_reduce(r, srcs[r], outs[r], count, T.FP32, T.SUM, FAKE_STREAM) == 0
+        return w.last_trace()
+
+    recorded, info_r = traced(n, call, 0)
+    closed, info_c = traced(n, call, 2)
+    assert closed == recorded and info_c.levels == 0 and info_r.levels > 0
+    assert info_c.fused == 1 and info_c.fusedSegments == info_r.fusedSegments == 64 * 63
+    # a template without a closed form records its steps whatever the mode
+    _, info = traced(n, lambda w: call(w, alg="InsAllReduceMesh1DTwoShot"), 2)
+    assert info.levels > 0
+    # two ranks share an input buffer: the buffers do not lie apart, so the steps are recorded
+    shared = [ins[0]] + ins[:-1]
+    _, info = traced(n, lambda w: call(w, srcs=shared), 2)
+    assert info.levels > 0
