@@ -544,6 +544,21 @@ def small_messages_from_cpp():
         return {"error": repr(e)}
 
 
+def planning_from_cpp():
+    """What a collective costs the host the first time (templates run, steps ordered and traced, or the template's
+    closed form; tables built), on other buffers (the first plan moved there) and from then on, for every AllReduce
+    and ReduceScatter template among 8, 16 and 32 ranks: hccl_amd/lib/first_call_virtual_ranks as a child process."""
+    import subprocess
+    exe = os.path.join(ROOT, "hccl_amd", "lib", "first_call_virtual_ranks")
+    if not os.path.exists(exe):
+        return None
+    try:
+        out = subprocess.run([exe, "32"], capture_output=True, text=True, timeout=120)
+        return json.loads(out.stdout) if out.returncode == 0 else {"error": out.stderr[-300:]}
+    except Exception as e:      # an extra, like the small-message timings
+        return {"error": repr(e)}
+
+
 def time_steps(torch, wl, steps, warmup):
     """W untimed steps, then K steps bracketed by synchronisation; events sit on the launch stream."""
     import gc
@@ -643,6 +658,9 @@ def main():
                 size = line["allreduce_12_ranks_sweep"].get(str(row["bytes_per_rank"]), {})
                 if row["ranks"] == 12 and row["case"] in size:
                     size[row["case"]]["us_from_cpp"] = row["us"]
+        planning = planning_from_cpp()
+        if planning is not None:
+            line["planning_from_cpp"] = planning
 
     if not args.no_cpu and hasattr(wl, "cpu_baseline"):
         v1, sample = wl.cpu_baseline(parallel=False)

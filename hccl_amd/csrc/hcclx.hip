@@ -65,12 +65,22 @@ struct Ring {
     std::vector<hipEvent_t> pool;
 };
 
+// Pinned host memory that a plan's table is assembled in before it is copied to the device on a stream of its own
+// and waited for.
+struct PlanStage {
+    std::mutex mu;
+    char *host = nullptr;
+    size_t bytes = 0;
+    hipStream_t stream = nullptr;   // the copies run on a stream of their own: they order with nothing else
+};
+
 struct DeviceSlot {
     std::once_flag once;
     bool ok = false;
     std::string err;
     DeviceCtx ctx;
     Ring ring;
+    PlanStage stage;
 };
 
 DeviceSlot g_slots[kMaxDevices];
@@ -118,6 +128,15 @@ void init_slot(DeviceSlot *s, int dev)
     e = hipMalloc(reinterpret_cast<void **>(&c.d_ring), c.ring_bytes);
     if (e != hipSuccess) {
         s->err = std::string("hipMalloc(descriptor ring): ") + hipGetErrorString(e);
+        return;
+    }
+    // The runtime sets up its path for host-to-device copies above 16 KiB when the first one is made (6-10 ms):
+    // make it here, so that it does not land in the first collective whose table is that large.
+    e = hipStreamCreateWithFlags(&s->stage.stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipMemcpyAsync(c.d_ring, c.h_ring, 64 * 1024, hipMemcpyHostToDevice, s->stage.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(s->stage.stream);
+    if (e != hipSuccess) {
+        s->err = std::string("first table upload: ") + hipGetErrorString(e);
         return;
     }
     // init_slot runs with `dev` current (device_ctx() asks for the current device): this is that device's copy
@@ -963,10 +982,23 @@ static int plan_from(DeviceCtx *ctx, Built &built, hcclx_plan_t **plan)
     }
     p->table_bytes = total;
     if (total != 0) {
-        std::vector<char> host(total);
-        for (size_t i = 0; i < p->batches.size(); ++i) fill_table(p->batches[i], host.data() + p->offsets[i]);
-        hipError_t e = hipMalloc(reinterpret_cast<void **>(&p->d_table), total);
-        if (e == hipSuccess) e = hipMemcpy(p->d_table, host.data(), total, hipMemcpyHostToDevice);
+        PlanStage &stage = g_slots[ctx->device].stage;
+        std::lock_guard<std::mutex> lock(stage.mu);
+        hipError_t e = hipSuccess;
+        if (stage.bytes < total) {
+            if (stage.host) (void)hipHostFree(stage.host);
+            stage.host = nullptr;
+            stage.bytes = 0;
+            const size_t want = std::max<size_t>(total + total / 2, 1u << 20);
+            e = hipHostMalloc(reinterpret_cast<void **>(&stage.host), want, hipHostMallocDefault);
+            if (e == hipSuccess) stage.bytes = want;
+        }
+        if (e == hipSuccess) {
+            for (size_t i = 0; i < p->batches.size(); ++i) fill_table(p->batches[i], stage.host + p->offsets[i]);
+            e = hipMalloc(reinterpret_cast<void **>(&p->d_table), total);
+        }
+        if (e == hipSuccess) e = hipMemcpyAsync(p->d_table, stage.host, total, hipMemcpyHostToDevice, stage.stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(stage.stream);
         if (e != hipSuccess) {
             if (p->d_table) (void)hipFree(p->d_table);
             delete p;
