@@ -1527,6 +1527,15 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
             w->lastPlanCacheHit = 1;
             return LaunchPlans(w, c->plans, stream);
         }
+        // Everything below allocates tables or sends them through the pinned ring: none of it may be recorded into
+        // a graph (the graph would replay a copy from a ring slot that has long been reused).
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &capturing) == hipSuccess &&
+            capturing != hipStreamCaptureStatusNone) {
+            HCCL_ERROR("[RunCollective] %s on a capturing stream has no plan for these buffers yet: run the same "
+                       "collective on the same buffers once before the capture", algName.c_str());
+            return HCCL_E_NOT_SUPPORT;
+        }
         separate = BuffersAreSeparate(params);
         if (ShapePlan *sp = separate ? FindShape(cache, shape) : nullptr) {
             // The same collective on other buffers: the plan it had, with every pointer moved along with its buffer.

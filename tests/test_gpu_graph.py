@@ -140,3 +140,46 @@ def test_data_movement_collectives_captured_from_their_first_call():
     finally:
         w1.close()
         w2.close()
+
+
+def test_a_collective_without_a_plan_for_its_buffers_refuses_to_be_captured():
+    """Planning a collective, or moving a known plan to other buffers, allocates tables or sends them through the
+    pinned ring.  On a capturing stream such a call must say so (HCCL_E_NOT_SUPPORT) before it touches the GPU, and
+    leave the capture usable for the collectives that are warm."""
+    n, count = 8, 6007
+    rng = np.random.default_rng(9)
+    xs = [payload(rng, T.FP32, count, "uniform") for _ in range(n)]
+    w = api.World(n)
+    try:
+        send = [DevBuf(x) for x in xs]
+        recv = [DevBuf(nbytes=count * 4) for _ in range(n)]
+        other = [DevBuf(nbytes=count * 4) for _ in range(n)]
+        s = torch.cuda.Stream()
+
+        def issue(dst, cnt=count):
+            return [w.all_reduce(r, send[r].ptr, dst[r].ptr, cnt, T.FP32, T.SUM, s.cuda_stream) for r in range(n)]
+
+        assert issue(recv) == [0] * n            # warm for (send, recv)
+        s.synchronize()
+        alg = w.last_info().algName.decode()
+        for r in range(n):
+            recv[r].t.fill_(0xA5)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(s):
+            g.capture_begin()
+            assert issue(other) == [0] * (n - 1) + [5]          # known shape, other buffers: would use the ring
+            assert issue(recv, count - 1) == [0] * (n - 1) + [5]   # unknown shape: would plan and allocate
+            assert issue(recv) == [0] * n                       # warm: kernels only
+            g.capture_end()
+        assert w.last_info().planCacheHit == 1
+        g.replay()
+        torch.cuda.synchronize()
+        want = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs, count, 4, alg)
+        for r in range(n):
+            assert_same_bits(recv[r].get(np.float32), want[r], T.FP32, f"rank {r}")
+            assert recv[r].guard_intact() and other[r].guard_intact()
+            assert (other[r].t == 0xA5).all()
+        del g
+    finally:
+        w.close()
