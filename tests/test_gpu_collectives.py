@@ -821,3 +821,51 @@ def test_mesh_chunk_templates_planned_from_their_closed_form(stream, kind, n, dt
         finally:
             w.close()
     assert results[0] == results[1]
+
+
+def test_a_schedule_that_cannot_be_fused_runs_its_steps(stream):
+    """Rank 1 receives into the buffer rank 0 sends from, 64 bytes further on.  One pass over the inputs would overwrite
+    what other workgroups still read, so the world falls back to the recorded steps (the two-shot template reads every
+    input before it writes any output).  A world in FUSED mode has no scratch buffers until then: they are allocated
+    now and the steps are recorded again against them.  (Exactly on top of rank 0's input it would still be one pass:
+    every thread reads its elements before it writes them.)"""
+    n, count, skew = 4, 50021, 64
+    nbytes = count * 4
+    rng = np.random.default_rng(77)
+    xs = [payload(rng, T.FP32, count, "uniform") for _ in range(n)]
+    alg = "InsAllReduceMesh1DTwoShot"
+    w = api.World(n, ccl_bytes=SMALL_CCL)
+    try:
+        w.set_algorithm(api.CMD_ALLREDUCE, alg)
+        send = [DevBuf(nbytes=nbytes + skew) for _ in range(n)]
+        recv = [DevBuf(nbytes=nbytes) for _ in range(n)]
+
+        def upload():
+            for r in range(n):
+                send[r].t[:nbytes] = torch.from_numpy(xs[r].view(np.uint8).copy()).to("cuda:0")
+            torch.cuda.synchronize()
+
+        def call(outs):
+            for r in range(n):
+                assert w.all_reduce(r, send[r].ptr, outs[r], count, T.FP32, T.SUM, stream.cuda_stream) == 0
+            stream.synchronize()
+            return w.last_info()
+
+        want = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), xs, count, 4, alg, ccl_bytes=SMALL_CCL)
+        upload()
+        assert call([b.ptr for b in recv]).fused == 1      # the world has now run without scratch memory
+        upload()
+        info = call([recv[0].ptr, send[0].ptr, recv[2].ptr, recv[3].ptr])
+        assert info.fused == 1 and info.launches == 1      # exactly on top: in place for that output
+        assert_same_bits(send[0].get(np.uint8)[:nbytes].view(np.float32), want[1], T.FP32, "rank 1 on top of rank 0's input")
+        for rep in range(2):
+            upload()
+            info = call([recv[0].ptr, send[0].ptr + skew, recv[2].ptr, recv[3].ptr])
+            assert info.fused == 0 and info.launches >= info.levels > 1 and info.planCacheHit == rep
+            got = [recv[0].get(np.float32), send[0].get(np.uint8)[skew:skew + nbytes].view(np.float32),
+                   recv[2].get(np.float32), recv[3].get(np.float32)]
+            for r in range(n):
+                assert_same_bits(got[r], want[r], T.FP32, f"rank {r} rep {rep}")
+            assert all(b.guard_intact() for b in recv + send)
+    finally:
+        w.close()
