@@ -56,6 +56,7 @@ struct DeviceCtx {
     // AllGather(V) with host tables: from this many bytes of payload on (HCCLX_AGV_PHASED_FROM, 0 = never) the outputs
     // of a run of a source are written one after the other, each workgroup writing one output.
     uint64_t agv_phased_from = 4ull << 20;
+    uint64_t store_through_upto = 320ull << 20;   // fold launches with several destinations that write no more than this store through the L2 (HCCLX_STORE_THROUGH_UPTO)
     // Descriptor ring: tables of one-shot launches are written to pinned host memory and copied to the
     // device ring on the launch stream just before the kernel.
     char *h_ring = nullptr;

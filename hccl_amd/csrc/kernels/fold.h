@@ -52,9 +52,6 @@ __host__ __device__ constexpr uint64_t wide_tile_vecs(int unroll)
 #ifndef HCCLX_NT_LOAD
 #define HCCLX_NT_LOAD 1
 #endif
-#ifndef HCCLX_NT_STORE
-#define HCCLX_NT_STORE 1
-#endif
 __device__ __forceinline__ u32x4 ld16(const char *p)
 {
 #if HCCLX_NT_LOAD
@@ -63,19 +60,34 @@ __device__ __forceinline__ u32x4 ld16(const char *p)
     return *reinterpret_cast<const u32x4_u *>(p);
 #endif
 }
+// How results leave the CU.  Three ways to store, measured on MI355X:
+//   stream   nontemporal: the line is marked for early eviction.  Best where several output streams are written at
+//            once and for the copy kernels (AlltoAllV 154 us against 162 with write-through stores).
+//   plain    an ordinary store: the line stays in the L2 / Infinity Cache -- for a result that the next launch fans
+//            out to its other destinations.
+//   through  agent scope ("sc1"): written through the L2 instead of sitting there as a dirty line that has to be
+//            evicted later.  Best for a single output stream (8 sources of 64 MiB folded into one output: 97.2 us
+//            against 99.5) and for every launch that writes several streams at once below the size where it is
+//            split into fold + fan-out (8 x 32 MiB AllReduce in one pass: 83.8 us against 96.3).
+// The launcher picks per launch (store_policy_for in hcclx.hip); the self-first orders (N outputs from every
+// workgroup) and the V and MoE kernels always stream.
+constexpr uint32_t kStoreStream = 0;
+constexpr uint32_t kStorePlain = 1;
+constexpr uint32_t kStoreThrough = 2;
 __device__ __forceinline__ void st16(char *p, u32x4 v)
 {
-#if HCCLX_NT_STORE
     __builtin_nontemporal_store(v, reinterpret_cast<u32x4_u *>(p));
-#else
-    *reinterpret_cast<u32x4_u *>(p) = v;
-#endif
 }
-// A result that a second launch fans out to its other destinations is stored the ordinary way, so that it is
-// still in the L2 / Infinity Cache when that launch reads it; everything else streams past the caches.
-__device__ __forceinline__ void st16x(char *p, u32x4 v, bool plain)
+__device__ __forceinline__ void st16x(char *p, u32x4 v, uint32_t policy)
 {
-    if (plain) {
+    if (policy == kStoreThrough) {
+        // global_store_dwordx4 takes any byte address, like the compiler's own store of an unaligned vector.  The
+        // compiler does not look inside an asm statement, so the one hazard of this instruction is handled here: a
+        // VALU instruction that overwrites the data registers of a store of more than 8 bytes must come at least two
+        // wait states after it (the compiler keeps that distance for its own stores); hence the s_nop.  Address and
+        // data are VGPRs whose producers the compiler has already waited for, and no scalar operand is read.
+        asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
+    } else if (policy == kStorePlain) {
         *reinterpret_cast<u32x4_u *>(p) = v;
     } else {
         st16(p, v);
@@ -121,7 +133,7 @@ __device__ __forceinline__ void tree_eval(C (&leaf)[MAXN][NE], uint32_t codes)
 
 template <int DT, int OP, int MAXN, int MODE, bool CHECK>
 __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint32_t ndst, uint64_t v0, uint64_t nvec,
-                                          uint32_t head_bytes, bool plain)
+                                          uint32_t head_bytes, uint32_t policy)
 {
     constexpr int UNROLL = fold_unroll(MAXN);
     using V = Vec16<DT>;
@@ -172,7 +184,7 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
             // batch of scalar loads instead of one dependent load per iteration
 #pragma unroll
             for (int d = 0; d < kMaxFan; ++d) {
-                if (d < static_cast<int>(ndst)) st16x(sd.dst[d] + head_bytes + vi * 16, out, plain);
+                if (d < static_cast<int>(ndst)) st16x(sd.dst[d] + head_bytes + vi * 16, out, policy);
             }
         } else if constexpr (MODE == kFoldTree) {
             C val[MAXN][NE];
@@ -186,7 +198,7 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
             // batch of scalar loads instead of one dependent load per iteration
 #pragma unroll
             for (int d = 0; d < kMaxFan; ++d) {
-                if (d < static_cast<int>(ndst)) st16x(sd.dst[d] + head_bytes + vi * 16, out, plain);
+                if (d < static_cast<int>(ndst)) st16x(sd.dst[d] + head_bytes + vi * 16, out, policy);
             }
         } else {
             C val[MAXN][NE];
@@ -207,7 +219,7 @@ __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint3
                             for (int e = 0; e < NE; ++e) acc[e] = V::template combine<OP>(val[k][e], acc[e]);
                         }
                     }
-                    st16(sd.dst[j] + head_bytes + vi * 16, V::pack(acc));
+                    st16(sd.dst[j] + head_bytes + vi * 16, V::pack(acc));   // N output streams at once: streamed
                 }
             }
         }
@@ -330,9 +342,9 @@ __device__ __forceinline__ void locate_tile(const uint64_t *__restrict__ tile_en
 template <int DT, int OP, int MAXN, int MODE>
 __global__ void __launch_bounds__(kFoldThreads)
 k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, uint32_t nseg, uint64_t total_tiles,
-       uint32_t plain_store, uint32_t uniform_tiles)
+       uint32_t store_policy, uint32_t uniform_tiles)
 {
-    const bool plain = plain_store != 0;
+    const uint32_t policy = store_policy;
     constexpr int NE = Vec16<DT>::kElems;   // elements per 16-byte vector
     constexpr uint64_t TV = fold_tile_vecs(MAXN);
     extern __shared__ uint64_t s_end[];  // nseg entries, sized by the launcher
@@ -365,9 +377,9 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
         // they fail the bound check of the checked path like the ones behind its end.
         const uint64_t v0 = tl * TV + threadIdx.x - shift;
         if (tl * TV >= shift && (tl + 1) * TV - shift <= nvec) {
-            fold_tile<DT, OP, MAXN, MODE, false>(sd, nsrc, ndst, v0, nvec, head_bytes, plain);
+            fold_tile<DT, OP, MAXN, MODE, false>(sd, nsrc, ndst, v0, nvec, head_bytes, policy);
         } else {
-            if (nvec != 0) fold_tile<DT, OP, MAXN, MODE, true>(sd, nsrc, ndst, v0, nvec, head_bytes, plain);
+            if (nvec != 0) fold_tile<DT, OP, MAXN, MODE, true>(sd, nsrc, ndst, v0, nvec, head_bytes, policy);
             // the last tile also takes the elements in front of and behind the vector body, one per thread
             if (tl == (nvec + shift) / TV && threadIdx.x < head + rem) {
                 const uint64_t idx = threadIdx.x < head ? threadIdx.x : head + nvec * NE + (threadIdx.x - head);
@@ -382,7 +394,7 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
 // has.  One vector per thread and tile.
 template <int DT, int OP, int U, bool CHECK>
 __device__ __forceinline__ void fold_tile_wide(const SegWide &sd, uint32_t nsrc, uint32_t ndst, uint64_t v0, uint64_t nvec,
-                                               uint32_t head_bytes, bool plain)
+                                               uint32_t head_bytes, uint32_t policy)
 {
     using V = Vec16<DT>;
     using C = typename V::C;
@@ -434,7 +446,7 @@ __device__ __forceinline__ void fold_tile_wide(const SegWide &sd, uint32_t nsrc,
             if (base + d < ndst) {
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    if (ok[u]) st16x(sd.dst[base + d] + off[u], V::pack(acc[u]), plain);
+                    if (ok[u]) st16x(sd.dst[base + d] + off[u], V::pack(acc[u]), policy);
                 }
             }
         }
@@ -475,7 +487,7 @@ __device__ __forceinline__ void wide_subtree(const SegWide &sd, uint64_t off, ui
 // through the two top levels.
 template <int DT, int OP, bool CHECK>
 __device__ __forceinline__ void fold_tile_wide_tree(const SegWide &sd, uint32_t ndst, uint64_t v, uint64_t nvec,
-                                                    uint32_t head_bytes, bool plain)
+                                                    uint32_t head_bytes, uint32_t policy)
 {
     using V = Vec16<DT>;
     using C = typename V::C;
@@ -498,7 +510,7 @@ __device__ __forceinline__ void fold_tile_wide_tree(const SegWide &sd, uint32_t 
     for (uint32_t base = 0; base < ndst; base += kMaxFan) {
 #pragma unroll
         for (int d = 0; d < kMaxFan; ++d) {
-            if (base + d < ndst) st16x(sd.dst[base + d] + off, out, plain);
+            if (base + d < ndst) st16x(sd.dst[base + d] + off, out, policy);
         }
     }
 }
@@ -568,10 +580,10 @@ __device__ __forceinline__ void fold_tile_wide_self(const SegWide &sd, uint32_t 
 template <int DT, int OP, int MODE, int U>
 __global__ void __launch_bounds__(kFoldThreads)
 k_fold_wide(const uint64_t *__restrict__ tile_end, const SegWide *__restrict__ segs, uint32_t nseg, uint64_t total_tiles,
-            uint32_t xcd_remap, uint32_t plain_store, uint32_t uniform_tiles)
+            uint32_t xcd_remap, uint32_t store_policy, uint32_t uniform_tiles)
 {
     constexpr int NE = Vec16<DT>::kElems;
-    const bool plain = plain_store != 0;
+    const uint32_t policy = store_policy;
     static_assert(MODE == kFoldChain || U == 1, "only the chain moves several vectors per thread");
     constexpr uint64_t TV = wide_tile_vecs(U);
     extern __shared__ uint64_t s_end[];
@@ -598,19 +610,19 @@ k_fold_wide(const uint64_t *__restrict__ tile_end, const SegWide *__restrict__ s
         const uint64_t v = tl * TV + threadIdx.x - shift;   // wraps in front of a shifted segment: fails the check
         if (tl * TV >= shift && (tl + 1) * TV - shift <= nvec) {
             if constexpr (MODE == kFoldTree) {
-                fold_tile_wide_tree<DT, OP, false>(sd, ndst, v, nvec, head_bytes, plain);
+                fold_tile_wide_tree<DT, OP, false>(sd, ndst, v, nvec, head_bytes, policy);
             } else if constexpr (MODE == kFoldSelfFirst) {
                 fold_tile_wide_self<DT, OP, false>(sd, nsrc, v, nvec, head_bytes);
             } else {
-                fold_tile_wide<DT, OP, U, false>(sd, nsrc, ndst, v, nvec, head_bytes, plain);
+                fold_tile_wide<DT, OP, U, false>(sd, nsrc, ndst, v, nvec, head_bytes, policy);
             }
         } else {
             if constexpr (MODE == kFoldTree) {
-                fold_tile_wide_tree<DT, OP, true>(sd, ndst, v, nvec, head_bytes, plain);
+                fold_tile_wide_tree<DT, OP, true>(sd, ndst, v, nvec, head_bytes, policy);
             } else if constexpr (MODE == kFoldSelfFirst) {
                 fold_tile_wide_self<DT, OP, true>(sd, nsrc, v, nvec, head_bytes);
             } else {
-                if (nvec != 0) fold_tile_wide<DT, OP, U, true>(sd, nsrc, ndst, v, nvec, head_bytes, plain);
+                if (nvec != 0) fold_tile_wide<DT, OP, U, true>(sd, nsrc, ndst, v, nvec, head_bytes, policy);
             }
             if (tl == (nvec + shift) / TV && threadIdx.x < head + rem) {
                 const uint64_t idx = threadIdx.x < head ? threadIdx.x : head + nvec * NE + (threadIdx.x - head);
@@ -661,7 +673,7 @@ struct FoldLaunch {
     uint32_t grid;
     int wide_unroll;           // the wide chain kernel: vectors per thread (kWideUnrollMany or kWideUnrollOne)
     uint32_t xcd_remap;        // the wide kernels: give each XCD a contiguous eighth of the tiles
-    uint32_t plain_store;      // chain and tree: results are stored the ordinary way (a fan-out launch reads them next)
+    uint32_t store_policy;     // kStoreStream / kStorePlain / kStoreThrough
     uint32_t uniform_tiles;    // non-zero: every segment has this many tiles, tile t belongs to segment t / uniform_tiles
     hipStream_t stream;
 };
