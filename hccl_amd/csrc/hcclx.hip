@@ -361,7 +361,7 @@ struct Batch {
     std::vector<CopyBlock> blocks;   // instead of everything above: a list of blocks for the block copy kernel
     int block_unroll = 2;
     PhasedLaunch phased;         // instead of everything above: jobs of the copy kernel that writes one output at a time
-    uint32_t store_policy = kStoreStream;   // how the fold kernels store (fold.h); kStorePlain: the next batch fans the results out
+    uint32_t store_policy = kStoreStream;   // how the fold kernels store (fold.h)
     size_t nseg() const { return segs.size() + wide.size(); }
     size_t bytes() const
     {
@@ -468,7 +468,7 @@ int tree_levels(uint32_t nsrc, const uint8_t *prog)
     return static_cast<int>(depth[0]);
 }
 
-int build_wide_batches_impl(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, uint32_t plain_store,
+int build_wide_batches_impl(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode,
                             Built *out);
 
 // What the segments of one launch of the register-resident kernels have in common.
@@ -559,8 +559,8 @@ bool make_segdev(const hcclx_seg_t &s, const SegProto &sp, int mode, SegDev *out
 }
 
 // Results that go to several places, from fanout_from bytes of them on: the fold stores each result once (to
-// dst[0], with ordinary stores) and a second launch copies it to the other places, one place at a time in runs
-// that the L2 still holds; segments that only copy go to that second launch whole (their source is the run).
+// dst[0]) and a second launch copies it to the other places, one place at a time in runs whose re-reads the L2
+// serves; segments that only copy go to that second launch whole (their source is the run).
 // Fills `one` (the segments of the first launch, one destination each) and `fan` (what the second launch copies)
 // and returns true; returns false when the launch stays as it is.  max_fan: the segment type's array size.
 template <typename SEG>
@@ -641,7 +641,7 @@ uint32_t store_policy_for(const DeviceCtx *ctx, const SEG *segs, uint32_t nseg, 
     return (most_dst <= 1 || written <= upto) ? kStoreThrough : kStoreStream;
 }
 
-int build_batches_impl(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, uint32_t plain_store, Built *out);
+int build_batches_impl(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, Built *out);
 
 int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, Built *out)
 {
@@ -650,10 +650,10 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
     std::vector<PhasedStream> fan;
     const DeviceCtx *fctx = device_ctx();
     if (!split_fanout(fctx, segs, nseg, dtype_size(dtype), mode, HCCLX_MAX_FAN, &one, &fan)) {
-        return build_batches_impl(segs, nseg, dtype, op, mode, 0, out);
+        return build_batches_impl(segs, nseg, dtype, op, mode, out);
     }
     const uint64_t algo_before = out->algo_bytes;
-    const int rc = build_batches_impl(one.data(), static_cast<uint32_t>(one.size()), dtype, op, mode, 1, out);
+    const int rc = build_batches_impl(one.data(), static_cast<uint32_t>(one.size()), dtype, op, mode, out);
     if (rc != HCCL_SUCCESS) return rc;
     // the algorithmic bytes are those of the segments as the caller gave them, however the work is split
     out->algo_bytes = algo_before;
@@ -664,7 +664,7 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
     return HCCL_SUCCESS;
 }
 
-int build_batches_impl(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, uint32_t plain_store, Built *out)
+int build_batches_impl(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, Built *out)
 {
     if (nseg != 0 && segs == nullptr) return fail(HCCL_E_PTR, "segs is null");
     // Chains over many sources run faster on the wide chain kernel (sources in groups of eight, two vectors per
@@ -690,7 +690,7 @@ int build_batches_impl(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op
                 for (uint32_t k = 0; k < segs[i].ndst; ++k) wide[i].dst[k] = segs[i].dst[k];
                 for (uint32_t k = 1; k < segs[i].nsrc; ++k) wide[i].prog[k] = segs[i].prog[k];   // operand order per step
             }
-            return build_wide_batches_impl(wide.data(), nseg, dtype, op, HCCLX_FOLD_CHAIN, plain_store, out);
+            return build_wide_batches_impl(wide.data(), nseg, dtype, op, HCCLX_FOLD_CHAIN, out);
         }
     }
     SegProto sp;
@@ -702,7 +702,7 @@ int build_batches_impl(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op
     proto.op = op;
     proto.mode = sp.mode;
     proto.maxn = sp.maxn;
-    proto.store_policy = plain_store ? kStorePlain : store_policy_for(device_ctx(), segs, nseg, sp.copy ? 1 : dtype_size(dtype));
+    proto.store_policy = store_policy_for(device_ctx(), segs, nseg, sp.copy ? 1 : dtype_size(dtype));
     Batch cur = proto;
     for (uint32_t i = 0; i < nseg; ++i) {
         const hcclx_seg_t &s = segs[i];
@@ -733,10 +733,10 @@ int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, i
     std::vector<PhasedStream> fan;
     const DeviceCtx *fctx = device_ctx();
     if (!split_fanout(fctx, segs, nseg, dtype_size(dtype), mode, HCCLX_MAX_WIDE_FAN, &one, &fan)) {
-        return build_wide_batches_impl(segs, nseg, dtype, op, mode, 0, out);
+        return build_wide_batches_impl(segs, nseg, dtype, op, mode, out);
     }
     const uint64_t algo_before = out->algo_bytes;
-    const int rc = build_wide_batches_impl(one.data(), static_cast<uint32_t>(one.size()), dtype, op, mode, 1, out);
+    const int rc = build_wide_batches_impl(one.data(), static_cast<uint32_t>(one.size()), dtype, op, mode, out);
     if (rc != HCCL_SUCCESS) return rc;
     out->algo_bytes = algo_before;
     for (uint32_t i = 0; i < nseg; ++i) {
@@ -747,7 +747,7 @@ int build_wide_batches(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, i
 }
 
 // Wide segments: chain order, up to kMaxWideFan sources and destinations, one kernel for every fan-in.
-int build_wide_batches_impl(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, uint32_t plain_store,
+int build_wide_batches_impl(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int op, int mode,
                             Built *out)
 {
     if (nseg != 0 && segs == nullptr) return fail(HCCL_E_PTR, "segs is null");
@@ -799,7 +799,7 @@ int build_wide_batches_impl(const hcclx_wide_seg_t *segs, uint32_t nseg, int dty
     Batch proto;
     proto.dtype = dtype;
     proto.op = op;
-    proto.store_policy = plain_store ? kStorePlain : store_policy_for(device_ctx(), segs, nseg, dtype_size(dtype));
+    proto.store_policy = store_policy_for(device_ctx(), segs, nseg, dtype_size(dtype));
     // a tree over integers equals the chain of its leaves, and so does every self-first order
     proto.mode = (mode != HCCLX_FOLD_CHAIN && is_float_dtype(dtype) && max_src > 1) ? mode : HCCLX_FOLD_CHAIN;
     proto.maxn = kMaxWideFan;

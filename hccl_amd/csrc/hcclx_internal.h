@@ -46,12 +46,12 @@ struct DeviceCtx {
     // With host tables the V kernels launch one workgroup per run of this many consecutive tiles.
     uint32_t v_tiles_per_block = 1;
     // Writing n outputs at once runs HBM a third slower than writing them one after the other (the banks see n
-    // streams of row misses).  A fold whose result goes to several places therefore stores it once, with ordinary
-    // stores, and a second launch copies it to the other places, one place at a time in runs of fanout_run bytes
-    // (HCCLX_FANOUT_RUN) that the L2 still holds: 8 x 64 MiB fp32 AllReduce 204 -> 176 us.  It pays from about
-    // 640 MiB read and written by such folds in one launch (HCCLX_FANOUT_FROM, 0 = never): below that the
-    // Infinity Cache (256 MiB) absorbs enough of the writes for the single pass to win (8 x 32 MiB: 89 against 93 us).
-    uint64_t fanout_from = 640ull << 20;
+    // streams of row misses).  A fold whose result goes to several places therefore stores it once and a second
+    // launch copies it to the other places, one place at a time in runs of fanout_run bytes (HCCLX_FANOUT_RUN)
+    // whose re-reads the L2 serves: 8 x 64 MiB fp32 AllReduce 204 -> 175 us.  It pays from about 560 MiB read
+    // and written by such folds in one launch (HCCLX_FANOUT_FROM, 0 = never): below that the Infinity Cache
+    // (256 MiB) absorbs enough of the writes for the single pass to win (8 x 32 MiB: 84 against 90 us).
+    uint64_t fanout_from = 560ull << 20;
     uint64_t fanout_run = 8ull << 20;
     // AllGather(V) with host tables: from this many bytes of payload on (HCCLX_AGV_PHASED_FROM, 0 = never) the outputs
     // of a run of a source are written one after the other, each workgroup writing one output.

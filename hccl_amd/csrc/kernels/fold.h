@@ -60,20 +60,17 @@ __device__ __forceinline__ u32x4 ld16(const char *p)
     return *reinterpret_cast<const u32x4_u *>(p);
 #endif
 }
-// How results leave the CU.  Three ways to store, measured on MI355X:
-//   stream   nontemporal: the line is marked for early eviction.  Best where several output streams are written at
-//            once and for the copy kernels (AlltoAllV 154 us against 162 with write-through stores).
-//   plain    an ordinary store: the line stays in the L2 / Infinity Cache -- for a result that the next launch fans
-//            out to its other destinations.
+// How results leave the CU.  Two ways to store, measured on MI355X against each other and against ordinary stores:
+//   stream   nontemporal: the line is marked for early eviction.  Best where many large output streams are
+//            written at once (the self-first orders) and for the copy kernels (AlltoAllV 154 us against 162).
 //   through  agent scope ("sc1"): written through the L2 instead of sitting there as a dirty line that has to be
 //            evicted later.  Best for a single output stream (8 sources of 64 MiB folded into one output: 97.2 us
-//            against 99.5) and for every launch that writes several streams at once below the size where it is
-//            split into fold + fan-out (8 x 32 MiB AllReduce in one pass: 83.8 us against 96.3).
-// The launcher picks per launch (store_policy_for in hcclx.hip); the self-first orders (N outputs from every
-// workgroup) and the V and MoE kernels always stream.
+//            against 99.5 streamed and 96.8 ordinary; also when a second launch fans that output out: 174.6 us
+//            against 179.8 with ordinary stores for the 8 x 64 MiB AllReduce) and for every launch that writes
+//            several streams at once below the size where it is split into fold + fan-out (8 x 32 MiB AllReduce
+//            in one pass: 83.8 us against 96.3).
 constexpr uint32_t kStoreStream = 0;
-constexpr uint32_t kStorePlain = 1;
-constexpr uint32_t kStoreThrough = 2;
+constexpr uint32_t kStoreThrough = 1;
 __device__ __forceinline__ void st16(char *p, u32x4 v)
 {
     __builtin_nontemporal_store(v, reinterpret_cast<u32x4_u *>(p));
@@ -87,8 +84,6 @@ __device__ __forceinline__ void st16x(char *p, u32x4 v, uint32_t policy)
         // wait states after it (the compiler keeps that distance for its own stores); hence the s_nop.  Address and
         // data are VGPRs whose producers the compiler has already waited for, and no scalar operand is read.
         asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
-    } else if (policy == kStorePlain) {
-        *reinterpret_cast<u32x4_u *>(p) = v;
     } else {
         st16(p, v);
     }
@@ -673,7 +668,7 @@ struct FoldLaunch {
     uint32_t grid;
     int wide_unroll;           // the wide chain kernel: vectors per thread (kWideUnrollMany or kWideUnrollOne)
     uint32_t xcd_remap;        // the wide kernels: give each XCD a contiguous eighth of the tiles
-    uint32_t store_policy;     // kStoreStream / kStorePlain / kStoreThrough
+    uint32_t store_policy;     // kStoreStream / kStoreThrough
     uint32_t uniform_tiles;    // non-zero: every segment has this many tiles, tile t belongs to segment t / uniform_tiles
     hipStream_t stream;
 };
