@@ -1599,7 +1599,7 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
     };
     const u32 esz = IsDataMove(type) ? 1 : DATATYPE_SIZE_TABLE[dtype];
     const int foldType = IsDataMove(type) ? HCCL_DATA_TYPE_INT8 : dtype;
-    std::string *text = (w->traceText || (w->dryRun && !g_phase.on)) ? &w->lastTrace : nullptr;
+    std::string *text = (w->traceText || w->dryRun) ? &w->lastTrace : nullptr;
     w->lastTrace.clear();
     w->lastCheck = CheckReport();
 
