@@ -73,6 +73,26 @@ HcclResult InsTempAllReduceMesh1DOneShot::KernelRun(const OpParam &param, const 
     return HCCL_SUCCESS;
 }
 
+// What the steps above amount to: rank r's output is its own data with the others' reduced onto it, ranks ascending.
+bool InsTempAllReduceMesh1DOneShot::ClosedForm(const TemplateDataParams &p, u64 esz, std::vector<ClosedFold> &out) const
+{
+    (void)esz;
+    const u32 n = templateRankSize_;
+    if (n < 2) return false;
+    if (p.sliceSize == 0) return true;
+    for (u32 r = 0; r < n; ++r) {
+        ClosedFold f;
+        f.bytes = p.sliceSize;
+        f.src.push_back({r, p.buffInfo.inBuffBaseOff});
+        for (u32 k = 0; k < n; ++k) {
+            if (k != r) f.src.push_back({k, p.buffInfo.inBuffBaseOff});
+        }
+        f.dst.push_back({r, p.buffInfo.outBuffBaseOff});
+        out.push_back(std::move(f));
+    }
+    return true;
+}
+
 // ---------------------------------------------------------------------------------------------------
 // two-shot mesh: scatter slice k of every rank to rank k, reduce there in slot order, gather back
 // ---------------------------------------------------------------------------------------------------
@@ -157,6 +177,25 @@ HcclResult InsTempAllReduceMesh1DTwoShot::KernelRun(const OpParam &param, const 
     }
     CHK_RET(PostSync(res.threads));
     return HCCL_SUCCESS;
+}
+
+// What the steps above amount to: slice k is the ranks' slices k folded in rank order (slot 0 first, the slots
+// after it one by one), and every rank gets it.
+bool InsTempAllReduceMesh1DTwoShot::ClosedForm(const TemplateDataParams &p, u64 esz, std::vector<ClosedFold> &out) const
+{
+    const u32 n = templateRankSize_;
+    if (n < 2) return false;
+    if (p.count == 0) return true;
+    const std::vector<SliceInfo> sl = SplitDataByRank(p.count, n, esz);
+    for (u32 k = 0; k < n; ++k) {
+        if (sl[k].size == 0) continue;
+        ClosedFold f;
+        f.bytes = sl[k].size;
+        for (u32 s = 0; s < n; ++s) f.src.push_back({s, p.buffInfo.inBuffBaseOff + sl[k].offset});
+        for (u32 r = 0; r < n; ++r) f.dst.push_back({r, p.buffInfo.outBuffBaseOff + sl[k].offset});
+        out.push_back(std::move(f));
+    }
+    return true;
 }
 
 // ---------------------------------------------------------------------------------------------------

@@ -31,9 +31,9 @@ namespace ops_hccl {
     }
 
 // scratch multiples: one_shot.cc:42-48 (N), two_shot.cc:20-27 (2), nhr.cc:20-26 (1), aicpu_reduce_nhr.cc:22-28 (N)
-HCCL_DECLARE_TEMPLATE(InsTempAllReduceMesh1DOneShot, "AllReduce mesh 1D one-shot",
+HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempAllReduceMesh1DOneShot, "AllReduce mesh 1D one-shot",
                       (templateRankSize_ > 1 ? templateRankSize_ : 1), templateRankSize_);
-HCCL_DECLARE_TEMPLATE(InsTempAllReduceMesh1DTwoShot, "AllReduce mesh 1D two-shot",
+HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempAllReduceMesh1DTwoShot, "AllReduce mesh 1D two-shot",
                       (templateRankSize_ > 1 ? templateRankSize_ : 1), 2);
 HCCL_DECLARE_TEMPLATE(InsTempAllReduceNHR, "AllReduce NHR", 1, 1);
 HCCL_DECLARE_TEMPLATE(InsTempAllReduceAicpuReduceNHR, "AllReduce NHR gather + local reduce", 1, templateRankSize_);

@@ -6,7 +6,7 @@ namespace ops_hccl {
 
 // scratch multiples: reduce_scatter mesh_1D.cc:59-63 (N), nhr.cc:369-377 (N); all_gather mesh/NHR (N);
 // all_gather_v mesh_1D.cc:48-57 (N in single-op mode); all_to_all_v mesh_1D.cc:66-73 (min(16, N-1)).
-HCCL_DECLARE_TEMPLATE(InsTempReduceScatterMesh1D, "ReduceScatter mesh 1D",
+HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempReduceScatterMesh1D, "ReduceScatter mesh 1D",
                       (templateRankSize_ > 1 ? templateRankSize_ : 1), templateRankSize_);
 HCCL_DECLARE_TEMPLATE(InsTempReduceScatterNHR, "ReduceScatter NHR", 1, templateRankSize_);
 // reduce_scatter aicpu_reduce_nhr.cc:46-50, :242-249: one thread, N scratch slots

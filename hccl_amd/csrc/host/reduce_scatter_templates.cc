@@ -90,6 +90,29 @@ HcclResult InsTempReduceScatterMesh1D::KernelRun(const OpParam &param, const Tem
     return HCCL_SUCCESS;
 }
 
+// What the steps above amount to, for the layout the sole executor passes (one repeat, equal slices, the output not
+// sliced): rank r's output is its own shard r with the other ranks' shards r reduced onto it, ranks ascending.
+bool InsTempReduceScatterMesh1D::ClosedForm(const TemplateDataParams &p, u64 esz, std::vector<ClosedFold> &out) const
+{
+    (void)esz;
+    const u32 n = templateRankSize_;
+    if (n < 2 || p.repeatNum != 1 || p.tailSize != p.sliceSize || p.outputSliceStride != 0) return false;
+    if (p.buffInfo.inBuffType == p.buffInfo.outBuffType) return false;   // the in-scratch variant: record it
+    if (p.sliceSize == 0) return true;
+    for (u32 r = 0; r < n; ++r) {
+        ClosedFold f;
+        f.bytes = p.sliceSize;
+        const u64 inOff = p.buffInfo.inBuffBaseOff + r * p.inputSliceStride;
+        f.src.push_back({r, inOff});
+        for (u32 k = 0; k < n; ++k) {
+            if (k != r) f.src.push_back({k, inOff});
+        }
+        f.dst.push_back({r, p.buffInfo.outBuffBaseOff});
+        out.push_back(std::move(f));
+    }
+    return true;
+}
+
 // One round per shard: every rank puts its copy of shard k into slot <own rank> of its scratch, the NHR
 // all-gather steps spread the slots until every rank holds all N copies, and rank k alone folds them: own
 // input first, then the slots of the other ranks ascending.  N all-gathers move N times the data a

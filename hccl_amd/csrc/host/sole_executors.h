@@ -65,6 +65,9 @@ public:
         dataTypeSize_ = DATATYPE_SIZE_TABLE[dataType_];
         TemplateDataParams t;
         t.buffInfo.hcclBuff.size = cclBytes;
+        t.buffInfo.inBuffType = BufferType::INPUT;
+        t.buffInfo.outBuffType = BufferType::OUTPUT;
+        t.buffInfo.hcclBuffType = BufferType::HCCL_BUFFER;
         t.repeatNum = 1;
         InsAlgTemplate alg(param, 0, AlgTopoMatch::Match(rankSize));
         bool all = true;
@@ -135,6 +138,9 @@ public:
         dataSize_ = dataCount_ * dataTypeSize_;
         TemplateDataParams t;
         t.buffInfo.hcclBuff.size = cclBytes;
+        t.buffInfo.inBuffType = BufferType::INPUT;
+        t.buffInfo.outBuffType = BufferType::OUTPUT;
+        t.buffInfo.hcclBuffType = BufferType::HCCL_BUFFER;
         t.repeatNum = 1;
         InsAlgTemplate alg(param, 0, AlgTopoMatch::Match(rankSize));
         bool all = true;

@@ -772,16 +772,28 @@ def test_overlapping_buffers_are_planned_for_their_addresses(stream):
         w.close()
 
 
+CLOSED_FORM_ALGS = {"all_reduce": "InsAllReduceMesh1DTwoShotMeshChunk", "reduce_scatter": "InsReduceScatterMesh1DMeshChunk",
+                    "reduce_scatter_gather": "InsReduceScatterAicpuReduceNHR", "all_reduce_one_shot": "InsAllReduceMesh1DOneShot",
+                    "all_reduce_two_shot": "InsAllReduceMesh1DTwoShot", "reduce_scatter_mesh": "InsReduceScatterMesh1D"}
+
+
 @pytest.mark.parametrize("kind,n,dtype,op,count", [("all_reduce", 64, T.FP32, T.SUM, 64 * 63 * 3 + 17),
                                                    ("all_reduce", 32, T.BFP16, T.SUM, 400003),
                                                    ("all_reduce", 12, T.INT32, T.MAX, 1 << 20),
                                                    ("reduce_scatter", 64, T.FP32, T.SUM, 5003),
-                                                   ("reduce_scatter", 16, T.FP16, T.PROD, 70001)])
-def test_mesh_chunk_templates_planned_from_their_closed_form(stream, kind, n, dtype, op, count):
-    """Among many ranks the mesh-chunk templates are planned from their closed form (N (N-1) chains, nothing
-    recorded) and run as one fused pass: 64 ranks too.  The result is the oracle's replay of the N^3 steps, and the
-    same collective with the closed form switched off (steps recorded and traced) gives the same bits."""
-    alg = "InsAllReduceMesh1DTwoShotMeshChunk" if kind == "all_reduce" else "InsReduceScatterMesh1DMeshChunk"
+                                                   ("reduce_scatter", 16, T.FP16, T.PROD, 70001),
+                                                   ("reduce_scatter_gather", 12, T.FP64, T.PROD, 30011),
+                                                   ("all_reduce_one_shot", 24, T.FP32, T.SUM, 100003),
+                                                   ("all_reduce_one_shot", 8, T.FP16, T.MAX, 500001),
+                                                   ("all_reduce_two_shot", 48, T.FP32, T.SUM, 300007),
+                                                   ("all_reduce_two_shot", 8, T.BFP16, T.SUM, 1 << 21),
+                                                   ("reduce_scatter_mesh", 32, T.FP32, T.SUM, 40009)])
+def test_templates_planned_from_their_closed_form(stream, kind, n, dtype, op, count):
+    """Templates that state their result in closed form are planned from it (nothing recorded) and run as one fused
+    pass: the 64-rank mesh-chunk AllReduce too (4032 chains).  The result is the oracle's replay of the template's
+    steps, and the same collective with the closed form switched off (steps recorded and traced) gives the same bits."""
+    alg = CLOSED_FORM_ALGS[kind]
+    kind = "all_reduce" if kind.startswith("all_reduce") else "reduce_scatter"
     cmd = api.CMD_ALLREDUCE if kind == "all_reduce" else api.CMD_REDUCE_SCATTER
     rng = np.random.default_rng(n + count)
     esz = T.DTYPE_SIZE[dtype]
@@ -811,7 +823,7 @@ def test_mesh_chunk_templates_planned_from_their_closed_form(stream, kind, n, dt
                     assert w.reduce_scatter(r, send[r].ptr, recv[r].ptr, count, dtype, op, stream.cuda_stream) == 0
             stream.synchronize()
             info = w.last_info()
-            assert info.fused == 1 and info.launches <= 2
+            assert info.fused == 1 and info.launches <= 3
             assert (info.levels == 0) == (closed_form == 1)
             got = [b.get(T.NP_STORAGE[dtype]) for b in recv]
             for r in range(n):

@@ -564,24 +564,28 @@ def traced(n, call, closed_form):
 
 
 @pytest.mark.parametrize("n", [2, 3, 4, 5, 7, 8, 12, 16, 17, 31, 32])
-@pytest.mark.parametrize("kind", ["all_reduce", "reduce_scatter", "reduce_scatter_gather"])
+@pytest.mark.parametrize("kind", ["all_reduce", "reduce_scatter", "reduce_scatter_gather", "all_reduce_one_shot",
+                                  "all_reduce_two_shot", "reduce_scatter_mesh"])
 def test_closed_form_of_a_template_equals_its_recorded_steps(kind, n):
     """The mesh-chunk templates and the gather-then-fold ReduceScatter state their result directly (N (N-1) chains,
-    N chains) so that a world need not record, order and trace their N^3 steps.  The statement must be exactly what the steps amount to: line for line the same
+    N chains) so that a world need not record, order and trace their N^3 steps; the one-shot, two-shot and mesh
+    ReduceScatter templates (N^2 steps, N chains) do the same.  The statement must be exactly what the steps amount to: line for line the same
     trace -- same pieces, same association order -- for short, ragged, 4 KiB-aligned and multi-chunk operands, every
     element size, and in place."""
     alg = {"all_reduce": "InsAllReduceMesh1DTwoShotMeshChunk", "reduce_scatter": "InsReduceScatterMesh1DMeshChunk",
-           "reduce_scatter_gather": "InsReduceScatterAicpuReduceNHR"}[kind]
-    cmd = api.CMD_ALLREDUCE if kind == "all_reduce" else api.CMD_REDUCE_SCATTER
+           "reduce_scatter_gather": "InsReduceScatterAicpuReduceNHR", "all_reduce_one_shot": "InsAllReduceMesh1DOneShot",
+           "all_reduce_two_shot": "InsAllReduceMesh1DTwoShot", "reduce_scatter_mesh": "InsReduceScatterMesh1D"}[kind]
+    reduces_all = kind.startswith("all_reduce")
+    cmd = api.CMD_ALLREDUCE if reduces_all else api.CMD_REDUCE_SCATTER
     ins, outs = fake_ptrs(n)
     # per-rank received count for ReduceScatter; several executor chunks at the last sizes
     # (the ReduceScatter template takes N-1 scratch slots per chunk, so its chunks are short among many ranks)
-    counts = [1, max(1, n - 1), n, n * (n - 1) + 1, 4099] + ([70001] if n <= 12 or kind == "all_reduce" else [])
+    counts = [1, max(1, n - 1), n, n * (n - 1) + 1, 4099] + ([70001] if n <= 12 or reduces_all else [])
     counts += [300001] if n <= 8 else []
     for count in counts:
         for dtype in (T.INT8, T.FP32, T.FP64):
             for in_place in (False, True):
-                if kind != "all_reduce" and in_place:
+                if not reduces_all and in_place:
                     continue   # a ReduceScatter's output is a part of its input: not apart, never in closed form
                 if (dtype != T.FP32 or in_place) and count not in (n, 4099, counts[-1]):
                     continue
@@ -590,7 +594,7 @@ def test_closed_form_of_a_template_equals_its_recorded_steps(kind, n):
                     w.set_algorithm(cmd, alg)
                     for r in range(n):
                         dst = ins[r] if in_place else outs[r]
-                        if kind == "all_reduce":
+                        if reduces_all:
                             assert w.all_reduce(r, ins[r], dst, count, dtype, T.SUM, FAKE_STREAM) == 0
                         else:
                             assert w.reduce_scatter(r, ins[r], dst, count, dtype, T.SUM, FAKE_STREAM) == 0
@@ -619,7 +623,7 @@ def test_closed_form_among_64_ranks_and_when_it_is_not_used():
     assert closed == recorded and info_c.levels == 0 and info_r.levels > 0
     assert info_c.fused == 1 and info_c.fusedSegments == info_r.fusedSegments == 64 * 63
     # a template without a closed form records its steps whatever the mode
-    _, info = traced(n, lambda w: call(w, alg="InsAllReduceMesh1DTwoShot"), 2)
+    _, info = traced(n, lambda w: call(w, alg="InsAllReduceNHR"), 2)
     assert info.levels > 0
     # two ranks share an input buffer: the buffers do not lie apart, so the steps are recorded
     shared = [ins[0]] + ins[:-1]
