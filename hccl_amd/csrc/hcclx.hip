@@ -67,6 +67,7 @@ struct Ring {
 
 // Pinned host memory that a plan's table is assembled in before it is copied to the device on a stream of its own
 // and waited for.
+constexpr size_t kPlanStageBytes = 4u << 20;   // to begin with; a larger table makes it grow
 struct PlanStage {
     std::mutex mu;
     char *host = nullptr;
@@ -134,6 +135,8 @@ void init_slot(DeviceSlot *s, int dev)
     // The runtime sets up its path for host-to-device copies above 16 KiB when the first one is made (6-10 ms):
     // make it here, so that it does not land in the first collective whose table is that large.
     e = hipStreamCreateWithFlags(&s->stage.stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipHostMalloc(reinterpret_cast<void **>(&s->stage.host), kPlanStageBytes, hipHostMallocDefault);
+    if (e == hipSuccess) s->stage.bytes = kPlanStageBytes;
     if (e == hipSuccess) e = hipMemcpyAsync(c.d_ring, c.h_ring, 64 * 1024, hipMemcpyHostToDevice, s->stage.stream);
     if (e == hipSuccess) e = hipStreamSynchronize(s->stage.stream);
     if (e != hipSuccess) {
@@ -1007,7 +1010,7 @@ static int plan_from(DeviceCtx *ctx, Built &built, hcclx_plan_t **plan)
             if (stage.host) (void)hipHostFree(stage.host);
             stage.host = nullptr;
             stage.bytes = 0;
-            const size_t want = std::max<size_t>(total + total / 2, 1u << 20);
+            const size_t want = total + total / 2;
             e = hipHostMalloc(reinterpret_cast<void **>(&stage.host), want, hipHostMallocDefault);
             if (e == hipSuccess) stage.bytes = want;
         }
