@@ -75,8 +75,8 @@ HcclResult hcclxCommGetLastOpInfo(HcclComm comm, hcclxLastOpInfo *info);
 HcclResult hcclxCommSetTrace(HcclComm comm, int on);
 uint64_t hcclxCommGetLastTrace(HcclComm comm, char *buf, uint64_t size);
 
-/* Closed forms.  A template whose steps grow with the cube of the rank count (the mesh-chunk templates) also states
- * what those steps amount to directly; the world then plans from that statement instead of recording, ordering and
+/* Closed forms.  Some templates (mesh-chunk, gather-then-fold ReduceScatter, one-shot, two-shot, mesh ReduceScatter)
+ * also state what their steps amount to directly; the world then plans from that statement instead of recording, ordering and
  * tracing the steps (nothing is recorded: hcclxLastOpInfo.levels is 0).  mode 0 = never, 1 = for plain launches
  * (the default; also HCCL_VRANK_CLOSED_FORM), 2 = also for traced and dry collectives, so that the trace of the
  * closed form can be compared with the trace of the recorded steps.  Never used while the schedule check is on, in
