@@ -183,7 +183,7 @@ HcclResult WorldCreate(u32 rankSize, u64 cclBytes, bool dryRun, std::vector<Hccl
             vt->index = t;
         }
         for (u32 p = 0; p < rankSize; ++p) {
-            w->channels[r].emplace_back(new VChannel{w, r, p});
+            w->channels[r].emplace_back(new VChannel{w, r, p, {}});
         }
         comms.push_back(w->ranks.back().get());
     }
