@@ -106,3 +106,55 @@ def test_random_reduce_scatter(seed):
             assert recv[r].guard_intact() and send[r].guard_intact(), what
     finally:
         w.close()
+
+
+@pytest.mark.parametrize("alg", AR_ALGS)
+@pytest.mark.parametrize("mode", [api.EXEC_FUSED, api.EXEC_STEP])
+def test_random_buffers_in_one_world(alg, mode):
+    """One world, a few shapes, buffers that keep changing (new ones with random alignment, old ones coming back, in
+    place now and then): plans are made, moved to other buffers and replayed in whatever order that gives, and every
+    result is the oracle's."""
+    n = 12 if alg != "InsAllReduceMesh1DOneShot" else 20
+    rng = np.random.default_rng(len(alg) * 10 + mode)
+    s = torch.cuda.Stream()
+    shapes = [(T.FP32, T.SUM, 4099), (T.BFP16, T.SUM, 30011), (T.INT32, T.MAX, 777), (T.FP32, T.MAX, 20000)]
+    seen = {0: 0, 1: 0, 2: 0}
+    w = api.World(n, ccl_bytes=SMALL_CCL)
+    try:
+        w.set_mode(mode)
+        w.set_algorithm(api.CMD_ALLREDUCE, alg)
+        pool = []
+        for it in range(20):
+            dtype, op, count = shapes[int(rng.integers(len(shapes)))]
+            esz = T.DTYPE_SIZE[dtype]
+            known = [p for p in pool if p[0] == (dtype, op, count)]
+            if known and rng.integers(3) == 0:
+                _, send, recv = known[int(rng.integers(len(known)))]
+            else:
+                send = [DevBuf(nbytes=count * esz, offset=int(rng.integers(5)) * esz) for _ in range(n)]
+                recv = send if rng.integers(4) == 0 else [DevBuf(nbytes=count * esz, offset=int(rng.integers(5)) * esz)
+                                                          for _ in range(n)]
+                pool = (pool + [((dtype, op, count), send, recv)])[-6:]
+            xs = [payload(rng, dtype, count, "uniform" if dtype == T.FP32 else "normal") for _ in range(n)]
+            for r in range(n):
+                send[r].t[send[r].offset:send[r].offset + count * esz] = torch.from_numpy(
+                    xs[r].view(np.uint8).reshape(-1).copy()).to("cuda:0")
+            torch.cuda.synchronize()
+            for r in range(n):
+                assert w.all_reduce(r, send[r].ptr, recv[r].ptr, count, dtype, op, s.cuda_stream) == 0
+            s.synchronize()
+            info = w.last_info()
+            seen[info.planCacheHit] += 1
+            if wide_sum(dtype, op, info.fused):
+                outs = T.run_allreduce(T.NumericElems(T.FP32, T.SUM), [T.widen16(x, dtype) for x in xs], count, esz, alg,
+                                       ccl_bytes=SMALL_CCL)
+                want = [T.narrow16(o, dtype) for o in outs]
+            else:
+                want = T.run_allreduce(T.NumericElems(dtype, op), xs, count, esz, alg, ccl_bytes=SMALL_CCL)
+            for r in range(n):
+                assert_same_bits(recv[r].get(T.NP_STORAGE[dtype]), want[r], dtype,
+                                 f"{alg} call {it} rank {r} cache {info.planCacheHit}")
+                assert recv[r].guard_intact()
+        assert seen[0] >= 1 and seen[2] >= 1, seen     # planned at least once, moved at least once
+    finally:
+        w.close()
