@@ -187,6 +187,25 @@ int hcclx_allgatherv(const void *const *send, void *const *recv, const uint64_t 
             std::vector<PhasedLaunch> launches;
             build_phased(streams, ctx->fanout_run, &launches);
             for (const PhasedLaunch &l : launches) {
+                // Among up to 16 ranks a job's places are one offset into every receive buffer, and the jobs of a
+                // launch usually fit the kernel arguments: no table in memory, nothing copied in front of the kernel.
+                if (n <= kPhasedInlineRanks && l.jobs.size() <= kPhasedInlineJobs && l.nd <= n) {
+                    PhasedInline tab;
+                    std::memset(&tab, 0, sizeof(tab));
+                    for (uint32_t d = 0; d < n; ++d) tab.base[d] = ptrs.recv[d];
+                    bool same_offset = true;
+                    for (size_t j = 0; j < l.jobs.size() && same_offset; ++j) {
+                        tab.jobs[j] = l.jobs[j];
+                        const uint64_t off = reinterpret_cast<uint64_t>(l.dsts[j * l.nd]) - reinterpret_cast<uint64_t>(ptrs.recv[0]);
+                        tab.jobs[j].dst0 = off;
+                        for (uint32_t d = 0; d < l.jobs[j].ndst; ++d) same_offset = same_offset && l.dsts[j * l.nd + d] == ptrs.recv[d] + off;
+                    }
+                    if (same_offset) {
+                        hipError_t e = launch_phased_copy_inline(tab, static_cast<uint32_t>(l.jobs.size()), l.slots, l.nd, st);
+                        if (e != hipSuccess) return fail_hip(e, "allgatherv kernel launch");
+                        continue;
+                    }
+                }
                 char *h = nullptr;
                 char *d = nullptr;
                 rc = ring_reserve(ctx, l.bytes(), st, &h, &d);

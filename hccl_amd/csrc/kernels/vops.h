@@ -101,6 +101,14 @@ struct PhasedJob {
     uint32_t ndst;
     uint32_t tiles;
 };
+// The same for an AllGather(V) among up to 16 ranks whose jobs fit the kernel arguments: every place a job goes to
+// is the same offset (the job's dst0) into the ranks' receive buffers, so the launch needs no table in memory.
+constexpr uint32_t kPhasedInlineJobs = 100;
+constexpr uint32_t kPhasedInlineRanks = 16;
+struct PhasedInline {
+    char *base[kPhasedInlineRanks];
+    PhasedJob jobs[kPhasedInlineJobs];
+};
 struct AgvTablesInline {
     uint64_t counts[kMaxVRanks];
     uint64_t displs[kMaxVRanks];
@@ -114,6 +122,7 @@ hipError_t launch_copy_blocks(const CopyBlock *blocks, uint32_t nblocks, uint32_
 // njobs < 65536
 hipError_t launch_phased_copy(const PhasedJob *jobs, char *const *dsts, uint32_t njobs, uint32_t slots, uint32_t nd,
                               hipStream_t stream);
+hipError_t launch_phased_copy_inline(const PhasedInline &tab, uint32_t njobs, uint32_t slots, uint32_t nd, hipStream_t stream);
 // unroll: 1, 2 or 4 vectors per thread and tile; grid = total number of tiles
 hipError_t launch_alltoallv_direct(const VRankPtrs16 &ptrs, const A2avTablesDirect &tabs, uint32_t n, uint32_t esz,
                                    uint32_t grid, int unroll, hipStream_t stream);

@@ -293,6 +293,24 @@ hipError_t launch_copy_blocks(const CopyBlock *blocks, uint32_t nblocks, uint32_
     return hipGetLastError();
 }
 
+__global__ void __launch_bounds__(kThreads) k_phased_copy_inline(PhasedInline tab, uint32_t slots, uint32_t nd)
+{
+    const uint32_t j = blockIdx.y;
+    const uint32_t d = blockIdx.x / slots;
+    const uint64_t tl = blockIdx.x - d * slots;
+    const PhasedJob &job = tab.jobs[j];
+    if (d >= job.ndst || d >= nd || tl >= job.tiles) return;
+    char *dst = tab.base[d] + job.dst0;
+    copy_tile<kPhasedUnroll, true>(job.src, reinterpret_cast<uint64_t>(tab.base[0]) + job.dst0, job.bytes, tl, 1,
+                                   [=](uint32_t) { return dst; });
+}
+
+hipError_t launch_phased_copy_inline(const PhasedInline &tab, uint32_t njobs, uint32_t slots, uint32_t nd, hipStream_t stream)
+{
+    hipLaunchKernelGGL(k_phased_copy_inline, dim3(slots * nd, njobs), dim3(kThreads), 0, stream, tab, slots, nd);
+    return hipGetLastError();
+}
+
 hipError_t launch_phased_copy(const PhasedJob *jobs, char *const *dsts, uint32_t njobs, uint32_t slots, uint32_t nd,
                               hipStream_t stream)
 {
