@@ -198,7 +198,7 @@ class AllGather(Workload):
     """HcclAllGather fp16, 8 ranks x 33,554,432 elements (64 MiB per rank): every block lands in every
     output; each source byte is read once and written eight times."""
     dtype = "u8"
-    kernel = "hcclx::(anonymous namespace)::k_phased_copy"
+    kernel = "hcclx::(anonymous namespace)::k_phased_copy_inline"
     profile = "profiles/k_phased_copy_all_gather_fp16_8x64MiB.txt"
 
     def __init__(self, torch, api, T, n=8, count=32 * 1024 * 1024):
@@ -227,7 +227,7 @@ class AllGatherV(Workload):
     """benchmark configuration 3: HcclAllGatherV fp16, 16 ranks, per-rank counts uniform in [0, 8,388,608] from a
     seed, displacements their prefix sum (so most blocks start at addresses that are only 2-byte aligned)."""
     dtype = "u8"
-    kernel = "hcclx::(anonymous namespace)::k_phased_copy"
+    kernel = "hcclx::(anonymous namespace)::k_phased_copy_inline"
     profile = "profiles/k_phased_copy_all_gather_v_fp16_16_ranks_ragged.txt"
 
     def __init__(self, torch, api, T, n=16, seed=3):
