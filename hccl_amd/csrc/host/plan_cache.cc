@@ -86,46 +86,80 @@ bool BuffersAreSeparate(const std::vector<OpParam> &params)
     return true;
 }
 
-// Moves the pointers of a shape plan's parts from the buffers it was made for to those of `params`.  Pointers
-// outside the ranks' buffers (the scratch buffers of step plans, which belong to the world) stay.
-void Rebase(const ShapePlan &sp, const std::vector<OpParam> &params, std::vector<HostPart> &parts)
+// For every pointer of a shape plan's parts, in the order segments hold them (sources, then destinations), which of
+// the ranks' buffers it points into: 1 + its index in `buffers`, or 0 for a pointer outside them (the scratch
+// buffers of step plans, which belong to the world and stay where they are).
+static void FindOwners(ShapePlan &sp)
 {
-    struct Move {
+    struct Range {
         u64 lo, hi;
-        int64_t delta;
+        uint16_t owner;
     };
-    std::vector<Move> moves;
-    for (size_t r = 0; r < params.size(); ++r) {
-        const ShapePlan::Buffer &in = sp.buffers[2 * r];
-        const ShapePlan::Buffer &out = sp.buffers[2 * r + 1];
-        const u64 newIn = reinterpret_cast<u64>(params[r].inputPtr);
-        const u64 newOut = reinterpret_cast<u64>(params[r].outputPtr);
+    std::vector<Range> ranges;
+    for (size_t b = 0; b < sp.buffers.size(); b += 2) {
+        const ShapePlan::Buffer &in = sp.buffers[b];
+        const ShapePlan::Buffer &out = sp.buffers[b + 1];
         if (in.base == out.base) {   // in place: one buffer, as long as the longer of the two
             const u64 size = std::max(in.size, out.size);
-            if (size) moves.push_back({in.base, in.base + size, static_cast<int64_t>(newIn - in.base)});
+            if (size) ranges.push_back({in.base, in.base + size, static_cast<uint16_t>(b + 1)});
             continue;
         }
-        if (in.size) moves.push_back({in.base, in.base + in.size, static_cast<int64_t>(newIn - in.base)});
-        if (out.size) moves.push_back({out.base, out.base + out.size, static_cast<int64_t>(newOut - out.base)});
+        if (in.size) ranges.push_back({in.base, in.base + in.size, static_cast<uint16_t>(b + 1)});
+        if (out.size) ranges.push_back({out.base, out.base + out.size, static_cast<uint16_t>(b + 2)});
     }
-    std::sort(moves.begin(), moves.end(), [](const Move &a, const Move &b) { return a.lo < b.lo; });
-    auto shift = [&](const void *p) -> void * {
+    std::sort(ranges.begin(), ranges.end(), [](const Range &a, const Range &b) { return a.lo < b.lo; });
+    // Segments of one plan mostly name the ranks in the same order, so the range the pointer at the same place of
+    // the segment before fell into is tried first; the search is for the others.
+    auto rangeOf = [&](const void *p, size_t guess) -> size_t {
         const u64 a = reinterpret_cast<u64>(p);
-        auto it = std::upper_bound(moves.begin(), moves.end(), a, [](u64 v, const Move &m) { return v < m.lo; });
-        if (it == moves.begin()) return const_cast<void *>(p);
+        if (guess < ranges.size() && a >= ranges[guess].lo && a < ranges[guess].hi) return guess;
+        auto it = std::upper_bound(ranges.begin(), ranges.end(), a, [](u64 v, const Range &m) { return v < m.lo; });
+        if (it == ranges.begin()) return ranges.size();
         --it;
-        return a < it->hi ? reinterpret_cast<void *>(a + it->delta) : const_cast<void *>(p);
+        return a < it->hi ? static_cast<size_t>(it - ranges.begin()) : ranges.size();
+    };
+    sp.owners.assign(sp.parts.size(), {});
+    std::vector<size_t> guess(2 * HCCLX_MAX_WIDE_FAN, ranges.size());
+    for (size_t i = 0; i < sp.parts.size(); ++i) {
+        std::vector<uint16_t> &own = sp.owners[i];
+        auto each = [&](const auto &segs) {
+            for (const auto &g : segs) {
+                for (uint32_t k = 0; k < g.nsrc + g.ndst; ++k) {
+                    const void *p = k < g.nsrc ? g.src[k] : g.dst[k - g.nsrc];
+                    size_t &at = guess[k < g.nsrc ? k : HCCLX_MAX_WIDE_FAN + k - g.nsrc];
+                    at = rangeOf(p, at);
+                    own.push_back(at < ranges.size() ? ranges[at].owner : 0);
+                }
+            }
+        };
+        each(sp.parts[i].segs);
+        each(sp.parts[i].wideSegs);
+    }
+}
+
+// Moves the pointers of a shape plan's parts from the buffers it was made for to those of `params`: every pointer
+// goes along with the buffer it points into.
+void Rebase(const ShapePlan &sp, const std::vector<OpParam> &params, std::vector<HostPart> &parts)
+{
+    std::vector<int64_t> delta(1 + sp.buffers.size(), 0);   // by owner; 0 = stays
+    for (size_t r = 0; r < params.size(); ++r) {
+        delta[1 + 2 * r] = static_cast<int64_t>(reinterpret_cast<u64>(params[r].inputPtr) - sp.buffers[2 * r].base);
+        delta[2 + 2 * r] = static_cast<int64_t>(reinterpret_cast<u64>(params[r].outputPtr) - sp.buffers[2 * r + 1].base);
+    }
+    auto shift = [&](const void *p, uint16_t owner) -> void * {
+        return reinterpret_cast<void *>(reinterpret_cast<u64>(p) + static_cast<u64>(delta[owner]));
     };
     parts = sp.parts;
-    for (HostPart &hp : parts) {
-        for (hcclx_seg_t &g : hp.segs) {
-            for (uint32_t k = 0; k < g.nsrc; ++k) g.src[k] = shift(g.src[k]);
-            for (uint32_t k = 0; k < g.ndst; ++k) g.dst[k] = shift(g.dst[k]);
-        }
-        for (hcclx_wide_seg_t &g : hp.wideSegs) {
-            for (uint32_t k = 0; k < g.nsrc; ++k) g.src[k] = shift(g.src[k]);
-            for (uint32_t k = 0; k < g.ndst; ++k) g.dst[k] = shift(g.dst[k]);
-        }
+    for (size_t i = 0; i < parts.size(); ++i) {
+        const uint16_t *own = sp.owners[i].data();
+        auto each = [&](auto &segs) {
+            for (auto &g : segs) {
+                for (uint32_t k = 0; k < g.nsrc; ++k) g.src[k] = shift(g.src[k], *own++);
+                for (uint32_t k = 0; k < g.ndst; ++k) g.dst[k] = shift(g.dst[k], *own++);
+            }
+        };
+        each(parts[i].segs);
+        each(parts[i].wideSegs);
     }
 }
 
@@ -267,6 +301,8 @@ void KeepShape(PlanCache &cache, const std::vector<u64> &shape, std::vector<Host
         sp.buffers.push_back({reinterpret_cast<u64>(p.inputPtr), p.inputSize});
         sp.buffers.push_back({reinterpret_cast<u64>(p.outputPtr), p.outputSize});
     }
+    FindOwners(sp);
+    for (const std::vector<uint16_t> &own : sp.owners) sp.hostBytes += own.size() * sizeof(uint16_t);
     cache.shapeBytes += sp.hostBytes;
     cache.shapes.push_front(std::move(sp));
     cache.shapeIndex.emplace(HashKey(shape), cache.shapes.begin());

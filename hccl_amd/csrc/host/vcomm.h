@@ -115,6 +115,7 @@ struct ShapePlan {
         u64 base, size;
     };
     std::vector<Buffer> buffers;     // the ranks' input and output buffers the parts' pointers refer to (2 per rank)
+    std::vector<std::vector<uint16_t>> owners;   // per part and pointer: 1 + index of its buffer, 0 = none of them
     bool fused = true;
     u32 levels = 0;
     u32 segments = 0;
