@@ -742,11 +742,12 @@ def run_allgatherv(inputs, counts, displs, out_len, fill):
 
 
 def run_alltoallv(inputs, send_counts, sdispls, recv_counts, rdispls, out_lens, fill=0):
-    """out_j[rdispls[j][i] .. +recv_counts[j][i]) = in_i[sdispls[i][j] .. +send_counts[i][j])."""
+    """out_j[rdispls[j][i] .. +recv_counts[j][i]) = in_i[sdispls[i][j] .. +send_counts[i][j]); other positions keep
+    `fill` (one value, or per rank the array that was there before)."""
     n = len(inputs)
     outs = []
     for j in range(n):
-        o = np.full(out_lens[j], fill, dtype=inputs[0].dtype)
+        o = fill[j].copy() if isinstance(fill, list) else np.full(out_lens[j], fill, dtype=inputs[0].dtype)
         for i in range(n):
             c = send_counts[i][j]
             if c != recv_counts[j][i]:
