@@ -16,8 +16,12 @@ def dev_i32(a):
     return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int32)).to(DEV)
 
 
-def route_on_gpu(dests, n, entries, row_elems):
-    d = [dev_i32(x) for x in dests]
+def route_on_gpu(dests, n, entries, row_elems, skew=0):
+    """`skew`: rank i's destination array starts (i * skew) % 4 entries into its allocation, so that some arrays
+    are not 16-byte aligned."""
+    whole = [dev_i32(np.concatenate([np.zeros((i * skew) % 4, dtype=np.int32), np.asarray(x, dtype=np.int32)]))
+             for i, x in enumerate(dests)]
+    d = [w[(i * skew) % 4:] for i, w in enumerate(whole)]
     tabs = [torch.full((n * n,), -1, dtype=torch.int64, device=DEV) for _ in range(4)]
     perm = [torch.full((entries,), 12345, dtype=torch.int32, device=DEV) for _ in range(n)]
     ws = torch.empty(hcclx.moe_workspace_bytes(n, entries), dtype=torch.uint8, device=DEV)
@@ -28,15 +32,19 @@ def route_on_gpu(dests, n, entries, row_elems):
     return tabs, perm
 
 
-@pytest.mark.parametrize("n,entries", [(1, 5), (2, 256), (3, 257), (8, 4096), (8, 70001), (16, 1000), (64, 33333)])
-def test_route_tables_and_stable_permutation(n, entries):
+@pytest.mark.parametrize("n,entries", [(1, 5), (2, 256), (3, 257), (8, 4096), (8, 70001), (16, 1000), (64, 33333),
+                                       (64, 3001), (33, 7942), (16, 16384), (16, 16385), (5, 3), (12, 4099)])
+@pytest.mark.parametrize("skew", [0, 1])
+def test_route_tables_and_stable_permutation(n, entries, skew):
+    """Both routing paths (one launch up to 16384 entries per rank and 262144 in all, three launches beyond), with
+    destination arrays that are and are not 16-byte aligned."""
     rng = np.random.default_rng(n * 1000 + entries)
     p = 1.0 / np.arange(1, n + 1) ** 1.2
     dests = [rng.choice(n, size=entries, p=p / p.sum()) for _ in range(n)]
     dests[0][::7] = -1                      # dropped entries
     if n > 1:
         dests[1][::5] = n
-    tabs, perm = route_on_gpu(dests, n, entries, 24)
+    tabs, perm = route_on_gpu(dests, n, entries, 24, skew)
     sc, sd, rc, rd, perms = T.moe_route(dests, n, 24)
     for got, want in zip(tabs, (sc, sd, rc, rd)):
         assert np.array_equal(got.cpu().numpy().reshape(n, n), np.array(want, dtype=np.int64))
