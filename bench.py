@@ -478,8 +478,13 @@ def sweep_allreduce_12_ranks(torch, api, T, steps):
     stream_obj = torch.cuda.Stream()
     out = {}
     big = 1 << 30
-    ins = [torch.rand(big // 4, device="cuda:0") * 0.2 + 0.9 for _ in range(n)]     # reused at every size
-    outs = [torch.empty(big // 4, device="cuda:0") for _ in range(n)]
+    # One arena for the inputs and one for the outputs, reused at every size.  The ranks' buffers start 1 GiB apart
+    # (what twelve 1 GiB allocations in a row give); at the largest size the collectives are also timed with the
+    # buffers 1 GiB + 8 KiB apart: at strides that are a multiple of 1 GiB the same offset of every buffer falls
+    # into the same HBM channel and bank, which costs the kernels that read and write all buffers at once 10-25 %.
+    stagger = 8192
+    arena_in = torch.rand(n * (big + stagger) // 4, device="cuda:0") * 0.2 + 0.9
+    arena_out = torch.empty(n * (big + stagger) // 4, device="cuda:0")
     for k in range(10):
         nbytes = 4096 * 4 ** k
         count = nbytes // 4
@@ -490,10 +495,13 @@ def sweep_allreduce_12_ranks(torch, api, T, steps):
 
             class Step:
                 stream_obj_ = stream_obj
+                stride = big
 
                 def step(self_inner):
                     for r in range(n):
-                        rc = w.all_reduce(r, ins[r].data_ptr(), outs[r].data_ptr(), count, dt, op, stream_obj.cuda_stream)
+                        rc = w.all_reduce(r, arena_in.data_ptr() + r * self_inner.stride,
+                                          arena_out.data_ptr() + r * self_inner.stride, count, dt, op,
+                                          stream_obj.cuda_stream)
                         assert rc == 0, rc
             st = Step()
             st.stream_obj = stream_obj
@@ -502,6 +510,12 @@ def sweep_allreduce_12_ranks(torch, api, T, steps):
             info = w.last_info()
             row[name] = {"us": round(ms * 1e3, 1), "GB/s": round(2 * n * nbytes / (ms * 1e-3) / 1e9, 1),
                          "fused": bool(info.fused), "launches": info.launches}
+            if nbytes == big:
+                st.stride = big + stagger
+                _, ms = time_steps(torch, st, reps, 2)
+                row[name]["us_buffers_1GiB_plus_8KiB_apart"] = round(ms * 1e3, 1)
+                row[name]["GB/s_buffers_1GiB_plus_8KiB_apart"] = round(2 * n * nbytes / (ms * 1e-3) / 1e9, 1)
+                st.stride = big
             if nbytes <= (1 << 20):
                 # launch-bound sizes: the warm collective captured 20 times into one HIP graph, so that the
                 # twelve host calls per collective drop out of the replayed time
@@ -524,7 +538,7 @@ def sweep_allreduce_12_ranks(torch, api, T, steps):
                 del g
             w.close()
         out["%d" % nbytes] = row
-    del ins, outs
+    del arena_in, arena_out
     torch.cuda.empty_cache()
     return out
 
