@@ -73,11 +73,10 @@ HcclResult InsTempAllReduceMesh1DOneShot::KernelRun(const OpParam &param, const 
     return HCCL_SUCCESS;
 }
 
-// What the steps above amount to: rank r's output is its own data with the others' reduced onto it, ranks ascending.
-bool InsTempAllReduceMesh1DOneShot::ClosedForm(const TemplateDataParams &p, u64 esz, std::vector<ClosedFold> &out) const
+// Every rank's output is its own data with the others' reduced onto it, ranks ascending: what the steps of the
+// one-shot mesh template, and of the gather-then-fold NHR template, amount to.
+static bool OwnDataThenTheOthersAscending(u32 n, const TemplateDataParams &p, std::vector<ClosedFold> &out)
 {
-    (void)esz;
-    const u32 n = templateRankSize_;
     if (n < 2) return false;
     if (p.sliceSize == 0) return true;
     for (u32 r = 0; r < n; ++r) {
@@ -91,6 +90,12 @@ bool InsTempAllReduceMesh1DOneShot::ClosedForm(const TemplateDataParams &p, u64 
         out.push_back(std::move(f));
     }
     return true;
+}
+
+bool InsTempAllReduceMesh1DOneShot::ClosedForm(const TemplateDataParams &p, u64 esz, std::vector<ClosedFold> &out) const
+{
+    (void)esz;
+    return OwnDataThenTheOthersAscending(templateRankSize_, p, out);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -305,6 +310,13 @@ HcclResult InsTempAllReduceAicpuReduceNHR::KernelRun(const OpParam &param, const
         CHK_RET(LocalReduce(th, DataSlice(ccl, base + k * sliceSize, sliceSize, count), dst, dataType_, reduceOp_));
     }
     return HCCL_SUCCESS;
+}
+
+// The slots are folded in the one-shot template's order (own data, then the others ascending).
+bool InsTempAllReduceAicpuReduceNHR::ClosedForm(const TemplateDataParams &p, u64 esz, std::vector<ClosedFold> &out) const
+{
+    (void)esz;
+    return OwnDataThenTheOthersAscending(templateRankSize_, p, out);
 }
 
 // ---------------------------------------------------------------------------------------------------

@@ -36,7 +36,8 @@ HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempAllReduceMesh1DOneShot, "AllReduce
 HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempAllReduceMesh1DTwoShot, "AllReduce mesh 1D two-shot",
                       (templateRankSize_ > 1 ? templateRankSize_ : 1), 2);
 HCCL_DECLARE_TEMPLATE(InsTempAllReduceNHR, "AllReduce NHR", 1, 1);
-HCCL_DECLARE_TEMPLATE(InsTempAllReduceAicpuReduceNHR, "AllReduce NHR gather + local reduce", 1, templateRankSize_);
+HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempAllReduceAicpuReduceNHR, "AllReduce NHR gather + local reduce", 1,
+                                       templateRankSize_);
 HCCL_DECLARE_TEMPLATE(InsTempAllReduceRing, "AllReduce ring", 1, 1);
 HCCL_DECLARE_TEMPLATE(InsTempAllReduceRHD, "AllReduce recursive halving-doubling", 1, 1);
 
