@@ -12,7 +12,7 @@ HCCL_DECLARE_TEMPLATE(InsTempReduceScatterNHR, "ReduceScatter NHR", 1, templateR
 // reduce_scatter aicpu_reduce_nhr.cc:46-50, :242-249: one thread, N scratch slots
 HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempReduceScatterAicpuReduceNHR, "ReduceScatter NHR gather + local reduce", 1, templateRankSize_);
 // reduce_scatter_v mesh_1D.cc:26-48: N-1 threads (the main thread sends too), N scratch slots
-HCCL_DECLARE_TEMPLATE(InsTempReduceScatterVMesh1D, "ReduceScatterV mesh 1D",
+HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempReduceScatterVMesh1D, "ReduceScatterV mesh 1D",
                       (templateRankSize_ > 1 ? templateRankSize_ - 1 : 1), templateRankSize_);
 // mesh-chunk templates (mesh_chunk_templates.cc): reduce_scatter meshchunk.cc:25-52 (N-1 threads, N-1 scratch
 // multiple); all_reduce two_shot_mesh_chunk.cc:17-38 (N threads, scratch multiple 2)

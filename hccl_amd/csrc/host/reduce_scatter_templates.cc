@@ -322,6 +322,29 @@ HcclResult InsTempReduceScatterVMesh1D::KernelRun(const OpParam &param, const Te
     return HCCL_SUCCESS;
 }
 
+// What the steps above amount to for one repeat: rank r's output is its own part r with the other ranks' parts r
+// reduced onto it, ranks ascending; a rank whose part is empty in this loop gets nothing.
+bool InsTempReduceScatterVMesh1D::ClosedForm(const TemplateDataParams &p, u64 esz, std::vector<ClosedFold> &out) const
+{
+    (void)esz;
+    const u32 n = templateRankSize_;
+    if (n < 2 || p.repeatNum != 1 || p.allRankSliceSize.size() != n || p.allRankDispls.size() != n) return false;
+    if (p.buffInfo.inBuffType == p.buffInfo.outBuffType) return false;
+    for (u32 r = 0; r < n; ++r) {
+        if (p.allRankSliceSize[r] == 0) continue;
+        ClosedFold f;
+        f.bytes = p.allRankSliceSize[r];
+        const u64 inOff = p.buffInfo.inBuffBaseOff + p.allRankDispls[r];
+        f.src.push_back({r, inOff});
+        for (u32 k = 0; k < n; ++k) {
+            if (k != r) f.src.push_back({k, inOff});
+        }
+        f.dst.push_back({r, p.buffInfo.outBuffBaseOff});
+        out.push_back(std::move(f));
+    }
+    return true;
+}
+
 // Strictly deterministic ReduceScatter: every rank sends shard k of its input to rank k (an all-to-all into
 // scratch slots), and rank k folds the N blocks in a tree that is the same on every rank: while more than one
 // block remains, with M the largest power of two below the number of blocks, block v >= M is folded into block

@@ -301,13 +301,40 @@ public:
         TemplateResource res;
         TemplateDataParams t;
         detail::FillBuffInfo(param, resCtx, t, res);
+        InsAlgTemplate alg(param, myRank_, resCtx.subCommRanks);
+        return Loops(param, alg, t, [&]() { return alg.KernelRun(param, t, res); });
+    }
+    bool ClosedForm(const OpParam &param, u32 rankSize, u64 cclBytes, std::vector<ClosedFold> &out) override
+    {
+        rankSize_ = rankSize;
+        dataType_ = param.vDataDes.dataType;
+        dataTypeSize_ = DATATYPE_SIZE_TABLE[dataType_];
+        TemplateDataParams t;
+        t.buffInfo.hcclBuff.size = cclBytes;
+        t.buffInfo.inBuffType = BufferType::INPUT;
+        t.buffInfo.outBuffType = BufferType::OUTPUT;
+        t.buffInfo.hcclBuffType = BufferType::HCCL_BUFFER;
+        InsAlgTemplate alg(param, 0, AlgTopoMatch::Match(rankSize));
+        bool all = true;
+        const HcclResult res = Loops(param, alg, t, [&]() {
+            all = all && alg.ClosedForm(t, dataTypeSize_, out);
+            return HCCL_SUCCESS;
+        });
+        return res == HCCL_SUCCESS && all;
+    }
+
+private:
+    // The chunk loop (sole_executor.cc:133-166): `body` runs once per chunk with `t` describing it.
+    template <typename F> HcclResult Loops(const OpParam &param, InsAlgTemplate &alg, TemplateDataParams &t, F &&body)
+    {
         t.repeatNum = 1;
         t.inputRepeatStride = 0;
         t.outputRepeatStride = 0;
         const std::vector<u64> &counts = param.vDataDes.counts;
+        CHK_PRT_RET(counts.size() != rankSize_ || param.vDataDes.displs.size() != rankSize_,
+                    HCCL_ERROR("[ReduceScatterV executor] count tables do not match the rank size"), HCCL_E_PARA);
         t.allRankDispls = param.vDataDes.displs;
         for (u64 &d : t.allRankDispls) d *= dataTypeSize_;
-        InsAlgTemplate alg(param, myRank_, resCtx.subCommRanks);
         const u64 mult = alg.CalcScratchMultiple(t.buffInfo.inBuffType, t.buffInfo.outBuffType);
         maxTmpMemSize_ = t.buffInfo.hcclBuff.size;
         const u64 maxCount = MaxDataSizePerLoop(maxTmpMemSize_, mult, UB_MAX_DATA_SIZE) / dataTypeSize_;
@@ -330,7 +357,7 @@ public:
             t.buffInfo.outBuffBaseOff = processed * dataTypeSize_;
             t.buffInfo.hcclBuffBaseOff = 0;
             t.outputSliceStride = maxCount * dataTypeSize_;
-            CHK_RET(alg.KernelRun(param, t, res));
+            CHK_RET(body());
             processed += largest;
         }
         return HCCL_SUCCESS;

@@ -608,6 +608,37 @@ def test_closed_form_of_a_template_equals_its_recorded_steps(kind, n):
                 assert info_c.fused == info_r.fused == 1 and info_c.fusedSegments == info_r.fusedSegments
 
 
+@pytest.mark.parametrize("n", [2, 3, 5, 8, 12, 17, 32, 64])
+def test_closed_form_of_reduce_scatter_v_equals_its_recorded_steps(n):
+    """The ragged mesh ReduceScatter states its result too: per executor loop, every rank whose part has not run out
+    gets its part of its own input with the other ranks' reduced onto it, ranks ascending.  Ragged parts with zeros,
+    parts at scattered places of the input, one and several executor loops, three element sizes."""
+    rng = np.random.default_rng(n)
+    ins, outs = fake_ptrs(n)
+    for top in (7, 3000, 40000 if n <= 17 else 9000):
+        counts = [int(c) for c in rng.integers(0, top, size=n)]
+        counts[int(rng.integers(n))] = 0
+        counts[int(rng.integers(n))] = top              # at least one part, and the longest takes several loops
+        displs, at = [0] * n, 3
+        for i in rng.permutation(n):
+            displs[i] = at
+            at += counts[i] + int(rng.integers(5))
+        for dtype in (T.INT8, T.FP32, T.INT64):
+            if dtype != T.FP32 and top != 3000:
+                continue
+
+            def call(w):
+                for r in range(n):
+                    assert w.reduce_scatter_v(r, ins[r], counts, displs, outs[r], counts[r], dtype, T.SUM, FAKE_STREAM) == 0
+                return w.last_trace()
+
+            recorded, info_r = traced(n, call, 0)
+            closed, info_c = traced(n, call, 2)
+            assert info_r.levels > 0 and info_c.levels == 0, "the closed form was not used"
+            assert closed == recorded, f"n={n} counts={counts} displs={displs} dtype={dtype}"
+            assert info_c.fused == info_r.fused == 1 and info_c.fusedSegments == info_r.fusedSegments
+
+
 def test_closed_form_among_64_ranks_and_when_it_is_not_used():
     alg = "InsAllReduceMesh1DTwoShotMeshChunk"
     n, count = 64, 64 * 63 * 2 + 5
