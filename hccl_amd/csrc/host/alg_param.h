@@ -225,6 +225,9 @@ struct ClosedFold {
     std::vector<Ref> src;
     std::vector<Ref> dst;
     u64 bytes = 0;
+    // true: the value accumulated so far is the source operand of every step and src[k] the destination operand
+    // (a ring: the partial result arrives and is reduced onto the rank's own data)
+    bool accIsSource = false;
 };
 
 u32 GetNHRStepNum(u32 rankSize);

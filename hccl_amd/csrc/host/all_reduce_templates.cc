@@ -368,6 +368,26 @@ HcclResult InsTempAllReduceRing::KernelRun(const OpParam &param, const TemplateD
                      DataSlice(p.buffInfo.outputPtr, p.buffInfo.outBuffBaseOff, p.sliceSize, p.count));
 }
 
+// What the two laps amount to: slice c starts as rank c's data, goes round the ring once with every rank's data
+// reduced in as it passes (the partial result arrives and is the source operand), and ends up on every rank.
+bool InsTempAllReduceRing::ClosedForm(const TemplateDataParams &p, u64 esz, std::vector<ClosedFold> &out) const
+{
+    const u32 n = templateRankSize_;
+    if (n < 2) return false;
+    if (p.count == 0) return true;
+    const std::vector<SliceInfo> sl = SplitDataByRank(p.count, n, esz);
+    for (u32 c = 0; c < n; ++c) {
+        if (sl[c].size == 0) continue;
+        ClosedFold f;
+        f.bytes = sl[c].size;
+        f.accIsSource = true;
+        for (u32 k = 0; k < n; ++k) f.src.push_back({(c + k) % n, p.buffInfo.inBuffBaseOff + sl[c].offset});
+        for (u32 r = 0; r < n; ++r) f.dst.push_back({r, p.buffInfo.outBuffBaseOff + sl[c].offset});
+        out.push_back(std::move(f));
+    }
+    return true;
+}
+
 // ---------------------------------------------------------------------------------------------------
 // recursive halving-doubling (from the documentation), any rank count
 // ---------------------------------------------------------------------------------------------------

@@ -306,7 +306,7 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
         std::vector<ClosedFold> closed;
         params[0].algName = algName;
         if (exec != nullptr && exec->ClosedForm(params[0], n, w->cclBytes, closed)) {
-            FoldsFromClosedForm(closed, params, folds, text);
+            FoldsFromClosedForm(closed, params, dtype, op, folds, text);
             haveFolds = true;
             lap("closedform");
         }

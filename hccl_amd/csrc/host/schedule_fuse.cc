@@ -185,10 +185,12 @@ bool FoldsFromTrace(const Tracer &tr, const std::vector<OpParam> &params, int dt
 
 // The folds of a collective that its executor and template state in closed form, and, with `text`, the trace they
 // stand for: the same lines the recorded steps give when traced.
-void FoldsFromClosedForm(const std::vector<ClosedFold> &closed, const std::vector<OpParam> &params, std::vector<Fold> &folds,
-                         std::string *text)
+void FoldsFromClosedForm(const std::vector<ClosedFold> &closed, const std::vector<OpParam> &params, int dtype, int op,
+                         std::vector<Fold> &folds, std::string *text)
 {
     const InputRanges inputs(params);
+    // which operand the accumulated value is only shows in the bits of floating-point MAX and MIN (as in Flatten)
+    const bool orderShows = IsFloatType(dtype) && op != HCCL_REDUCE_SUM && op != HCCL_REDUCE_PROD;
     struct Line {
         u32 rank;
         u64 offset;
@@ -200,6 +202,10 @@ void FoldsFromClosedForm(const std::vector<ClosedFold> &closed, const std::vecto
         Fold f;
         f.bytes = c.bytes;
         for (const ClosedFold::Ref &s : c.src) f.src.push_back(reinterpret_cast<u64>(params[s.rank].inputPtr) + s.offset);
+        if (c.accIsSource && orderShows && c.src.size() > 1) {
+            f.prog.assign(c.src.size(), 1);
+            f.prog[0] = 0;
+        }
         for (const ClosedFold::Ref &d : c.dst) {
             f.dsts.push_back(reinterpret_cast<u64>(params[d.rank].outputPtr) + d.offset);
             if (text) lines.push_back({d.rank, d.offset, folds.size()});
@@ -212,7 +218,10 @@ void FoldsFromClosedForm(const std::vector<ClosedFold> &closed, const std::vecto
     for (const Line &l : lines) {
         const Fold &f = folds[l.fold];
         std::string expr = LeafText(f.src[0], inputs);
-        for (size_t k = 1; k < f.src.size(); ++k) expr = "(" + LeafText(f.src[k], inputs) + "+" + expr + ")";
+        const bool accFirst = closed[l.fold].accIsSource;
+        for (size_t k = 1; k < f.src.size(); ++k) {
+            expr = accFirst ? "(" + expr + "+" + LeafText(f.src[k], inputs) + ")" : "(" + LeafText(f.src[k], inputs) + "+" + expr + ")";
+        }
         std::ostringstream os;
         os << "rank " << l.rank << " out[" << l.offset << "," << f.bytes << ") = " << expr << "\n";
         *text += os.str();

@@ -253,8 +253,8 @@ bool FoldsFromTrace(const Tracer &tr, const std::vector<OpParam> &params, int dt
                     std::string *text);
 // The folds of a collective that its executor and template state in closed form, and, with `text`, the trace they
 // stand for.
-void FoldsFromClosedForm(const std::vector<ClosedFold> &closed, const std::vector<OpParam> &params, std::vector<Fold> &folds,
-                         std::string *text);
+void FoldsFromClosedForm(const std::vector<ClosedFold> &closed, const std::vector<OpParam> &params, int dtype, int op,
+                         std::vector<Fold> &folds, std::string *text);
 // The fused launch lists of the folds; false when they cannot run as one pass.
 bool BuildFusedPlan(const std::vector<OpParam> &params, std::vector<Fold> &folds, u32 esz, FusedPlan &plan);
 // Every output piece against the contract of the collective.

@@ -775,7 +775,7 @@ def test_overlapping_buffers_are_planned_for_their_addresses(stream):
 CLOSED_FORM_ALGS = {"all_reduce": "InsAllReduceMesh1DTwoShotMeshChunk", "reduce_scatter": "InsReduceScatterMesh1DMeshChunk",
                     "reduce_scatter_gather": "InsReduceScatterAicpuReduceNHR", "all_reduce_one_shot": "InsAllReduceMesh1DOneShot",
                     "all_reduce_two_shot": "InsAllReduceMesh1DTwoShot", "reduce_scatter_mesh": "InsReduceScatterMesh1D",
-                    "all_reduce_gather": "InsAllReduceAicpuReduceNHR"}
+                    "all_reduce_gather": "InsAllReduceAicpuReduceNHR", "all_reduce_ring": "InsAllReduceRing"}
 
 
 @pytest.mark.parametrize("kind,n,dtype,op,count", [("all_reduce", 64, T.FP32, T.SUM, 64 * 63 * 3 + 17),
@@ -790,7 +790,10 @@ CLOSED_FORM_ALGS = {"all_reduce": "InsAllReduceMesh1DTwoShotMeshChunk", "reduce_
                                                    ("all_reduce_two_shot", 8, T.BFP16, T.SUM, 1 << 21),
                                                    ("reduce_scatter_mesh", 32, T.FP32, T.SUM, 40009),
                                                    ("all_reduce_gather", 12, T.FP32, T.PROD, 200003),
-                                                   ("all_reduce_gather", 40, T.INT64, T.SUM, 30011)])
+                                                   ("all_reduce_gather", 40, T.INT64, T.SUM, 30011),
+                                                   ("all_reduce_ring", 20, T.FP32, T.MAX, 150001),
+                                                   ("all_reduce_ring", 8, T.BFP16, T.SUM, 1 << 20),
+                                                   ("all_reduce_ring", 64, T.FP32, T.SUM, 37)])
 def test_templates_planned_from_their_closed_form(stream, kind, n, dtype, op, count):
     """Templates that state their result in closed form are planned from it (nothing recorded) and run as one fused
     pass: the 64-rank mesh-chunk AllReduce too (4032 chains).  The result is the oracle's replay of the template's

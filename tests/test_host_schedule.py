@@ -565,7 +565,7 @@ def traced(n, call, closed_form):
 
 @pytest.mark.parametrize("n", [2, 3, 4, 5, 7, 8, 12, 16, 17, 31, 32])
 @pytest.mark.parametrize("kind", ["all_reduce", "reduce_scatter", "reduce_scatter_gather", "all_reduce_one_shot",
-                                  "all_reduce_two_shot", "reduce_scatter_mesh", "all_reduce_gather"])
+                                  "all_reduce_two_shot", "reduce_scatter_mesh", "all_reduce_gather", "all_reduce_ring"])
 def test_closed_form_of_a_template_equals_its_recorded_steps(kind, n):
     """The mesh-chunk templates and the gather-then-fold ReduceScatter state their result directly (N (N-1) chains,
     N chains) so that a world need not record, order and trace their N^3 steps; the one-shot, two-shot and mesh
@@ -575,7 +575,7 @@ def test_closed_form_of_a_template_equals_its_recorded_steps(kind, n):
     alg = {"all_reduce": "InsAllReduceMesh1DTwoShotMeshChunk", "reduce_scatter": "InsReduceScatterMesh1DMeshChunk",
            "reduce_scatter_gather": "InsReduceScatterAicpuReduceNHR", "all_reduce_one_shot": "InsAllReduceMesh1DOneShot",
            "all_reduce_two_shot": "InsAllReduceMesh1DTwoShot", "reduce_scatter_mesh": "InsReduceScatterMesh1D",
-           "all_reduce_gather": "InsAllReduceAicpuReduceNHR"}[kind]
+           "all_reduce_gather": "InsAllReduceAicpuReduceNHR", "all_reduce_ring": "InsAllReduceRing"}[kind]
     reduces_all = kind.startswith("all_reduce")
     cmd = api.CMD_ALLREDUCE if reduces_all else api.CMD_REDUCE_SCATTER
     ins, outs = fake_ptrs(n)
