@@ -228,6 +228,14 @@ struct ClosedFold {
     // true: the value accumulated so far is the source operand of every step and src[k] the destination operand
     // (a ring: the partial result arrives and is reduced onto the rank's own data)
     bool accIsSource = false;
+    // A tree instead of a chain: its inner nodes over src[] as leaves, children before parents, the root last.  A
+    // child c < src.size() is leaf c, any other is inner node c - src.size().  Every node is one reduce step,
+    // value = value(srcChild) (+) value(dstChild).  Empty: the chain of src.
+    struct Step {
+        u32 srcChild;
+        u32 dstChild;
+    };
+    std::vector<Step> tree;
 };
 
 u32 GetNHRStepNum(u32 rankSize);

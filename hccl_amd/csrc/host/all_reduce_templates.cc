@@ -267,6 +267,52 @@ HcclResult InsTempAllReduceNHR::KernelRun(const OpParam &param, const TemplateDa
                      DataSlice(p.buffInfo.outputPtr, p.buffInfo.outBuffBaseOff, p.sliceSize, p.count));
 }
 
+// What the steps above amount to: the reduce-scatter rounds replayed on what every rank holds of every slice (whose
+// data, in which tree), then the all-gather rounds; every rank must end up with the same value of every slice.
+bool InsTempAllReduceNHR::ClosedForm(const TemplateDataParams &p, u64 esz, std::vector<ClosedFold> &out) const
+{
+    const u32 n = templateRankSize_;
+    if (n < 2) return false;
+    if (p.count == 0) return true;
+    const std::vector<SliceInfo> sl = SplitDataByRank(p.count, n, esz);
+    std::vector<SliceValues> slice(n, SliceValues(n));
+    std::vector<std::vector<NHRStepInfo>> steps(n);
+    for (int gather = 0; gather < 2; ++gather) {
+        for (u32 r = 0; r < n; ++r) {
+            if (gather) {
+                GetNHRAllGatherSteps(n, r, steps[r]);
+            } else {
+                GetNHRReduceScatterSteps(n, r, steps[r]);
+            }
+        }
+        for (size_t s = 0; s < steps[0].size(); ++s) {
+            for (u32 r = 0; r < n; ++r) {
+                const NHRStepInfo &st = steps[r][s];
+                for (u32 i = 0; i < st.nSlices; ++i) {
+                    if (gather) {
+                        slice[st.txSliceIdxs[i]].Copy(st.toRank, r);
+                    } else {
+                        slice[st.txSliceIdxs[i]].Reduce(st.toRank, r);
+                    }
+                }
+            }
+            for (SliceValues &v : slice) v.EndRound();
+        }
+    }
+    for (u32 k = 0; k < n; ++k) {
+        if (sl[k].size == 0) continue;
+        ClosedFold f;
+        slice[k].Emit(0, p.buffInfo.inBuffBaseOff + sl[k].offset, f);
+        f.bytes = sl[k].size;
+        for (u32 r = 0; r < n; ++r) {
+            if (!slice[k].Same(0, r)) return false;
+            f.dst.push_back({r, p.buffInfo.outBuffBaseOff + sl[k].offset});
+        }
+        out.push_back(std::move(f));
+    }
+    return true;
+}
+
 // ---------------------------------------------------------------------------------------------------
 // CPU-reduce NHR: all-gather the whole inputs into scratch slots with NHR steps, then fold the slots
 // into the output, own data first (the reference runs this fold on the CPU for PROD and 64-bit types)
@@ -493,6 +539,57 @@ HcclResult InsTempAllReduceRHD::KernelRun(const OpParam &param, const TemplateDa
         }
     }
     return LocalCopy(th, whole, DataSlice(p.buffInfo.outputPtr, p.buffInfo.outBuffBaseOff, p.sliceSize, p.count));
+}
+
+// What the steps above amount to: the fold of the odd ranks and the halving rounds replayed on what every rank holds
+// of every slice; the doubling rounds and the way back to the folded ranks hand every finished slice to everybody.
+bool InsTempAllReduceRHD::ClosedForm(const TemplateDataParams &p, u64 esz, std::vector<ClosedFold> &out) const
+{
+    const u32 n = templateRankSize_;
+    if (n < 2) return false;
+    if (p.count == 0) return true;
+    u32 extra = 0;
+    std::vector<u32> block;
+    RhdBlock(n, extra, block);
+    const u32 p2 = static_cast<u32>(block.size());
+    const std::vector<SliceInfo> sl = SplitDataByRank(p.count, p2, esz);
+    std::vector<SliceValues> slice(p2, SliceValues(n));
+    for (u32 i = 0; i < extra; ++i) {
+        for (SliceValues &v : slice) v.Reduce(2 * i, 2 * i + 1);
+    }
+    for (SliceValues &v : slice) v.EndRound();
+    u32 steps = 0;
+    while ((1u << steps) < p2) ++steps;
+    std::vector<u32> lo(p2, 0), hi(p2, p2);   // slice range every block rank still owns
+    for (u32 s = 0; s < steps; ++s) {
+        for (u32 b = 0; b < p2; ++b) {
+            const u32 mid = (lo[b] + hi[b]) / 2;
+            const bool upper = (b >> s) & 1;
+            const u32 partner = block[b ^ (1u << s)];
+            for (u32 k = upper ? lo[b] : mid; k < (upper ? mid : hi[b]); ++k) slice[k].Reduce(partner, block[b]);
+            if (upper) {
+                lo[b] = mid;
+            } else {
+                hi[b] = mid;
+            }
+        }
+        for (SliceValues &v : slice) v.EndRound();
+    }
+    std::vector<u32> owner(p2, 0);
+    for (u32 b = 0; b < p2; ++b) {
+        if (hi[b] != lo[b] + 1) return false;
+        owner[lo[b]] = block[b];
+    }
+    for (u32 k = 0; k < p2; ++k) {
+        if (sl[k].size == 0) continue;
+        ClosedFold f;
+        slice[k].Emit(owner[k], p.buffInfo.inBuffBaseOff + sl[k].offset, f);
+        if (f.src.size() != n) return false;
+        f.bytes = sl[k].size;
+        for (u32 r = 0; r < n; ++r) f.dst.push_back({r, p.buffInfo.outBuffBaseOff + sl[k].offset});
+        out.push_back(std::move(f));
+    }
+    return true;
 }
 
 }  // namespace ops_hccl

@@ -35,11 +35,11 @@ HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempAllReduceMesh1DOneShot, "AllReduce
                       (templateRankSize_ > 1 ? templateRankSize_ : 1), templateRankSize_);
 HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempAllReduceMesh1DTwoShot, "AllReduce mesh 1D two-shot",
                       (templateRankSize_ > 1 ? templateRankSize_ : 1), 2);
-HCCL_DECLARE_TEMPLATE(InsTempAllReduceNHR, "AllReduce NHR", 1, 1);
+HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempAllReduceNHR, "AllReduce NHR", 1, 1);
 HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempAllReduceAicpuReduceNHR, "AllReduce NHR gather + local reduce", 1,
                                        templateRankSize_);
 HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempAllReduceRing, "AllReduce ring", 1, 1);
-HCCL_DECLARE_TEMPLATE(InsTempAllReduceRHD, "AllReduce recursive halving-doubling", 1, 1);
+HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempAllReduceRHD, "AllReduce recursive halving-doubling", 1, 1);
 
 // Block of ranks that runs halving-doubling when n is not a power of two: the even rank of each of the
 // first `extra` pairs, then every rank from 2 * extra on (RHD.md:17).

@@ -8,7 +8,7 @@ namespace ops_hccl {
 // all_gather_v mesh_1D.cc:48-57 (N in single-op mode); all_to_all_v mesh_1D.cc:66-73 (min(16, N-1)).
 HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempReduceScatterMesh1D, "ReduceScatter mesh 1D",
                       (templateRankSize_ > 1 ? templateRankSize_ : 1), templateRankSize_);
-HCCL_DECLARE_TEMPLATE(InsTempReduceScatterNHR, "ReduceScatter NHR", 1, templateRankSize_);
+HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempReduceScatterNHR, "ReduceScatter NHR", 1, templateRankSize_);
 // reduce_scatter aicpu_reduce_nhr.cc:46-50, :242-249: one thread, N scratch slots
 HCCL_DECLARE_TEMPLATE_WITH_CLOSED_FORM(InsTempReduceScatterAicpuReduceNHR, "ReduceScatter NHR gather + local reduce", 1, templateRankSize_);
 // reduce_scatter_v mesh_1D.cc:26-48: N-1 threads (the main thread sends too), N scratch slots
@@ -39,6 +39,7 @@ public:
     HcclResult KernelRun(const OpParam &param, const TemplateDataParams &tempAlgParams,
                          TemplateResource &templateResource) override;
     void SetMemBlockInfo(const MemBlockInfo &info) { memBlockInfo_ = info; }
+    bool ClosedForm(const TemplateDataParams &tempAlgParams, u64 dataTypeSize, std::vector<ClosedFold> &out) const override;
 
 protected:
     // the peers in the order their shards are sent: ranks me+1, me+2, ... (:200-240)

@@ -262,6 +262,37 @@ HcclResult InsTempReduceScatterNHR::KernelRun(const OpParam &param, const Templa
                      DataSlice(p.buffInfo.outputPtr, p.buffInfo.outBuffBaseOff + me * p.outputSliceStride, size));
 }
 
+// What the steps above amount to: the rounds replayed on what every rank holds of every shard; rank r's output is
+// what it ends up holding of shard r.
+bool InsTempReduceScatterNHR::ClosedForm(const TemplateDataParams &p, u64 esz, std::vector<ClosedFold> &out) const
+{
+    (void)esz;
+    const u32 n = templateRankSize_;
+    if (n < 2 || p.buffInfo.inBuffType == p.buffInfo.outBuffType) return false;
+    if (p.sliceSize == 0 && p.tailSize == 0) return true;
+    std::vector<SliceValues> shard(n, SliceValues(n));
+    std::vector<std::vector<NHRStepInfo>> steps(n);
+    for (u32 r = 0; r < n; ++r) GetNHRReduceScatterSteps(n, r, steps[r]);
+    for (size_t s = 0; s < steps[0].size(); ++s) {
+        for (u32 r = 0; r < n; ++r) {
+            const NHRStepInfo &st = steps[r][s];
+            for (u32 i = 0; i < st.nSlices; ++i) shard[st.txSliceIdxs[i]].Reduce(st.toRank, r);
+        }
+        for (SliceValues &v : shard) v.EndRound();
+    }
+    for (u32 r = 0; r < n; ++r) {
+        const u64 size = (r == n - 1 && p.tailSize > 0) ? p.tailSize : p.sliceSize;
+        if (size == 0) continue;
+        ClosedFold f;
+        shard[r].Emit(r, p.buffInfo.inBuffBaseOff + r * p.inputSliceStride, f);
+        if (f.src.size() != n) return false;   // rank r must hold all of shard r
+        f.bytes = size;
+        f.dst.push_back({r, p.buffInfo.outBuffBaseOff + r * p.outputSliceStride});
+        out.push_back(std::move(f));
+    }
+    return true;
+}
+
 // Ragged mesh ReduceScatter: rank k owns allRankSliceSize[k] bytes at allRankDispls[k] of every input.
 // Every rank writes its part for rank k into slot <own rank> of rank k's scratch (slots are
 // outputSliceStride apart); rank k copies its own part to the output and folds the other slots in,
@@ -430,6 +461,36 @@ HcclResult InsTempReduceScatterOrderPreservedLevel1::KernelRun(const OpParam &pa
                           DataSlice(p.buffInfo.outputPtr, p.buffInfo.outBuffBaseOff, size)));
     }
     return HCCL_SUCCESS;
+}
+
+// What the steps above amount to (whatever order the shards were sent in): every rank's output is the one tree over
+// the ranks' copies of its shard, blocks numbered by the rank they came from.
+bool InsTempReduceScatterOrderPreservedLevel1::ClosedForm(const TemplateDataParams &p, u64 esz,
+                                                          std::vector<ClosedFold> &out) const
+{
+    (void)esz;
+    const u32 n = templateRankSize_;
+    const MemBlockInfo &mb = memBlockInfo_;
+    if (n < 2 || mb.size.size() != n || mb.userInputOffsets.size() != n) return false;
+    if (p.buffInfo.inBuffType == p.buffInfo.outBuffType) return false;
+    SliceValues blocks(n);
+    u32 remaining = n;
+    while (remaining > 1) {
+        u32 m = 1;
+        while (m * 2 < remaining) m *= 2;
+        for (u32 v = m; v < remaining; ++v) blocks.Reduce(v % m, v);
+        blocks.EndRound();
+        remaining = m;
+    }
+    for (u32 r = 0; r < n; ++r) {
+        if (mb.size[r] == 0) continue;
+        ClosedFold f;
+        blocks.Emit(0, mb.userInputOffsets[r], f);
+        f.bytes = mb.size[r];
+        f.dst.push_back({r, p.buffInfo.outBuffBaseOff});
+        out.push_back(std::move(f));
+    }
+    return true;
 }
 
 }  // namespace ops_hccl

@@ -306,8 +306,12 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
         std::vector<ClosedFold> closed;
         params[0].algName = algName;
         if (exec != nullptr && exec->ClosedForm(params[0], n, w->cclBytes, closed)) {
-            FoldsFromClosedForm(closed, params, dtype, op, folds, text);
-            haveFolds = true;
+            if (FoldsFromClosedForm(closed, params, dtype, op, folds, text)) {
+                haveFolds = true;
+            } else {   // a tree that no kernel evaluates: the recorded steps decide how it runs
+                folds.clear();
+                if (text) text->clear();
+            }
             lap("closedform");
         }
     }

@@ -184,8 +184,9 @@ bool FoldsFromTrace(const Tracer &tr, const std::vector<OpParam> &params, int dt
 }
 
 // The folds of a collective that its executor and template state in closed form, and, with `text`, the trace they
-// stand for: the same lines the recorded steps give when traced.
-void FoldsFromClosedForm(const std::vector<ClosedFold> &closed, const std::vector<OpParam> &params, int dtype, int op,
+// stand for: the same lines the recorded steps give when traced.  Returns false when a tree among them cannot be
+// fused (as FoldsFromTrace does); the caller then records the steps.
+bool FoldsFromClosedForm(const std::vector<ClosedFold> &closed, const std::vector<OpParam> &params, int dtype, int op,
                          std::vector<Fold> &folds, std::string *text)
 {
     const InputRanges inputs(params);
@@ -197,35 +198,70 @@ void FoldsFromClosedForm(const std::vector<ClosedFold> &closed, const std::vecto
         size_t fold;
     };
     std::vector<Line> lines;
+    std::vector<std::string> treeText;   // per fold, for trees
+    Tracer tr;                            // holds the reduce steps of the trees; no memory piece is ever written
+    bool allFit = true;
     folds.reserve(closed.size());
     for (const ClosedFold &c : closed) {
         Fold f;
-        f.bytes = c.bytes;
-        for (const ClosedFold::Ref &s : c.src) f.src.push_back(reinterpret_cast<u64>(params[s.rank].inputPtr) + s.offset);
-        if (c.accIsSource && orderShows && c.src.size() > 1) {
-            f.prog.assign(c.src.size(), 1);
-            f.prog[0] = 0;
+        if (c.tree.empty()) {
+            for (const ClosedFold::Ref &s : c.src) f.src.push_back(reinterpret_cast<u64>(params[s.rank].inputPtr) + s.offset);
+            if (c.accIsSource && orderShows && c.src.size() > 1) {
+                f.prog.assign(c.src.size(), 1);
+                f.prog[0] = 0;
+            }
+            if (text) treeText.emplace_back();
+        } else {
+            // the tree as reduce steps over memory as it was (expression 0), then flattened as a traced piece is
+            const size_t leaves = c.src.size();
+            std::vector<int> made;
+            made.reserve(c.tree.size());
+            auto operand = [&](u32 child, int &expr, u64 &shift) {
+                if (child < leaves) {
+                    expr = 0;
+                    shift = reinterpret_cast<u64>(params[c.src[child].rank].inputPtr) + c.src[child].offset;
+                } else {
+                    expr = made[child - leaves];
+                    shift = 0;
+                }
+            };
+            for (const ClosedFold::Step &st : c.tree) {
+                Expr e;
+                operand(st.srcChild, e.src, e.srcShift);
+                operand(st.dstChild, e.dst, e.dstShift);
+                made.push_back(tr.AddExpr(e));
+            }
+            f = Flatten(tr, made.back(), 0, dtype, op);
+            if (!f.fits) allFit = false;
+            if (text) treeText.push_back(ExprText(tr, made.back(), 0, inputs));
         }
+        f.bytes = c.bytes;
         for (const ClosedFold::Ref &d : c.dst) {
             f.dsts.push_back(reinterpret_cast<u64>(params[d.rank].outputPtr) + d.offset);
             if (text) lines.push_back({d.rank, d.offset, folds.size()});
         }
         folds.push_back(std::move(f));
     }
-    if (text == nullptr) return;
+    if (text == nullptr) return allFit;
     std::sort(lines.begin(), lines.end(),
               [](const Line &a, const Line &b) { return a.rank != b.rank ? a.rank < b.rank : a.offset < b.offset; });
     for (const Line &l : lines) {
-        const Fold &f = folds[l.fold];
-        std::string expr = LeafText(f.src[0], inputs);
-        const bool accFirst = closed[l.fold].accIsSource;
-        for (size_t k = 1; k < f.src.size(); ++k) {
-            expr = accFirst ? "(" + expr + "+" + LeafText(f.src[k], inputs) + ")" : "(" + LeafText(f.src[k], inputs) + "+" + expr + ")";
+        const ClosedFold &c = closed[l.fold];
+        std::string expr = treeText[l.fold];
+        if (c.tree.empty()) {
+            auto leaf = [&](size_t k) {
+                return LeafText(reinterpret_cast<u64>(params[c.src[k].rank].inputPtr) + c.src[k].offset, inputs);
+            };
+            expr = leaf(0);
+            for (size_t k = 1; k < c.src.size(); ++k) {
+                expr = c.accIsSource ? "(" + expr + "+" + leaf(k) + ")" : "(" + leaf(k) + "+" + expr + ")";
+            }
         }
         std::ostringstream os;
-        os << "rank " << l.rank << " out[" << l.offset << "," << f.bytes << ") = " << expr << "\n";
+        os << "rank " << l.rank << " out[" << l.offset << "," << c.bytes << ") = " << expr << "\n";
         *text += os.str();
     }
+    return allFit;
 }
 
 // Builds the fused launch plan from the folds.  Returns false when they cannot run as one pass (a source that is

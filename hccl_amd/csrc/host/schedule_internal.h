@@ -150,6 +150,12 @@ public:
     }
 
     const Expr &At(int e) const { return exprs_[e]; }
+    // A reduce step that no memory piece holds yet (closed forms build their trees from these).
+    int AddExpr(const Expr &e)
+    {
+        exprs_.push_back(e);
+        return static_cast<int>(exprs_.size()) - 1;
+    }
 
 private:
     void Split(u64 addr)
@@ -253,7 +259,7 @@ bool FoldsFromTrace(const Tracer &tr, const std::vector<OpParam> &params, int dt
                     std::string *text);
 // The folds of a collective that its executor and template state in closed form, and, with `text`, the trace they
 // stand for.
-void FoldsFromClosedForm(const std::vector<ClosedFold> &closed, const std::vector<OpParam> &params, int dtype, int op,
+bool FoldsFromClosedForm(const std::vector<ClosedFold> &closed, const std::vector<OpParam> &params, int dtype, int op,
                          std::vector<Fold> &folds, std::string *text);
 // The fused launch lists of the folds; false when they cannot run as one pass.
 bool BuildFusedPlan(const std::vector<OpParam> &params, std::vector<Fold> &folds, u32 esz, FusedPlan &plan);

@@ -464,6 +464,34 @@ public:
         TemplateDataParams t;
         detail::FillBuffInfo(param, resCtx, t, res);
         InsAlgTemplate alg(param, myRank_, resCtx.subCommRanks);
+        return Loops(alg, t, [&]() { return alg.KernelRun(param, t, res); });
+    }
+    bool ClosedForm(const OpParam &param, u32 rankSize, u64 cclBytes, std::vector<ClosedFold> &out) override
+    {
+        rankSize_ = rankSize;
+        dataType_ = param.DataDes.dataType;
+        dataTypeSize_ = DATATYPE_SIZE_TABLE[dataType_];
+        dataCount_ = param.DataDes.count;
+        dataSize_ = dataCount_ * dataTypeSize_;
+        TemplateDataParams t;
+        t.buffInfo.hcclBuff.size = cclBytes;
+        t.buffInfo.inBuffType = BufferType::INPUT;
+        t.buffInfo.outBuffType = BufferType::OUTPUT;
+        t.buffInfo.hcclBuffType = BufferType::HCCL_BUFFER;
+        t.repeatNum = 1;
+        InsAlgTemplate alg(param, 0, AlgTopoMatch::Match(rankSize));
+        bool all = true;
+        const HcclResult res = Loops(alg, t, [&]() {
+            all = all && alg.ClosedForm(t, dataTypeSize_, out);
+            return HCCL_SUCCESS;
+        });
+        return res == HCCL_SUCCESS && all;
+    }
+
+private:
+    // The chunk loop: `body` runs once per chunk with `t` and the template's block table describing it.
+    template <typename F> HcclResult Loops(InsAlgTemplate &alg, TemplateDataParams &t, F &&body)
+    {
         const u64 mult = alg.CalcScratchMultiple(t.buffInfo.inBuffType, t.buffInfo.outBuffType);
         maxTmpMemSize_ = t.buffInfo.hcclBuff.size;
         const u64 maxCount = MaxDataSizePerLoop(maxTmpMemSize_, mult, UB_MAX_DATA_SIZE) / dataTypeSize_;
@@ -490,7 +518,7 @@ public:
             t.inputSliceStride = dataSize_;
             t.outputSliceStride = 0;
             alg.SetMemBlockInfo(blocks);
-            CHK_RET(alg.KernelRun(param, t, res));
+            CHK_RET(body());
             done += cur;
         }
         return HCCL_SUCCESS;

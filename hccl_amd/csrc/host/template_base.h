@@ -88,4 +88,30 @@ std::vector<SliceInfo> SplitDataByRank(u64 count, u32 sliceNum, u64 dataTypeSize
 void GetNHRReduceScatterSteps(u32 rankSize, u32 myRankIdx, std::vector<NHRStepInfo> &steps);
 void GetNHRAllGatherSteps(u32 rankSize, u32 myRankIdx, std::vector<NHRStepInfo> &steps);
 
+// What every rank holds of ONE slice while a schedule reduces and copies whole slices from rank to rank: which ranks'
+// data went into it, and in which tree.  For the templates whose result is a tree (log-step schedules) and that
+// state it in closed form: they replay their step tables on these values, N^2 small steps instead of N^2 log N
+// recorded, ordered and traced ones.  The steps of one round read the values from before the round.
+class SliceValues {
+public:
+    explicit SliceValues(u32 ranks);            // every rank holds its own data
+    void Reduce(u32 dstRank, u32 srcRank);      // dst = src (+) dst, when the round ends
+    void Copy(u32 dstRank, u32 srcRank);        // dst = src, when the round ends
+    void EndRound();
+    bool Same(u32 a, u32 b) const { return held_[a] == held_[b]; }
+    // What rank `r` holds, as the sources (every rank's piece at `inOffset`) and the tree of a closed fold.
+    void Emit(u32 r, u64 inOffset, ClosedFold &f) const;
+
+private:
+    struct Node {
+        int src = -1;   // inner node: the two operands of its step
+        int dst = -1;
+        u32 rank = 0;   // leaf: whose data
+    };
+    u32 EmitNode(int node, u64 inOffset, ClosedFold &f) const;
+    std::vector<Node> nodes_;
+    std::vector<int> held_;
+    std::vector<std::pair<u32, int>> staged_;
+};
+
 }  // namespace ops_hccl

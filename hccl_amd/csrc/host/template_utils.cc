@@ -81,4 +81,60 @@ void GetNHRAllGatherSteps(u32 n, u32 me, std::vector<NHRStepInfo> &steps)
     }
 }
 
+SliceValues::SliceValues(u32 ranks)
+{
+    nodes_.resize(ranks);
+    held_.resize(ranks);
+    for (u32 r = 0; r < ranks; ++r) {
+        nodes_[r].rank = r;
+        held_[r] = static_cast<int>(r);
+    }
+}
+
+void SliceValues::Reduce(u32 dstRank, u32 srcRank)
+{
+    Node n;
+    n.src = held_[srcRank];
+    n.dst = held_[dstRank];
+    nodes_.push_back(n);
+    staged_.emplace_back(dstRank, static_cast<int>(nodes_.size()) - 1);
+}
+
+void SliceValues::Copy(u32 dstRank, u32 srcRank) { staged_.emplace_back(dstRank, held_[srcRank]); }
+
+void SliceValues::EndRound()
+{
+    for (const auto &s : staged_) held_[s.first] = s.second;
+    staged_.clear();
+}
+
+// Children first; returns the number the node has in f (a leaf: its place in f.src; an inner node: f.src.size() of
+// the finished fold is not known yet, so inner nodes are numbered from kInner up and renumbered by Emit).
+constexpr u32 kInner = 1u << 30;
+u32 SliceValues::EmitNode(int node, u64 inOffset, ClosedFold &f) const
+{
+    const Node &n = nodes_[node];
+    if (n.src < 0) {
+        f.src.push_back({n.rank, inOffset});
+        return static_cast<u32>(f.src.size()) - 1;
+    }
+    ClosedFold::Step st;
+    st.dstChild = EmitNode(n.dst, inOffset, f);
+    st.srcChild = EmitNode(n.src, inOffset, f);
+    f.tree.push_back(st);
+    return kInner + static_cast<u32>(f.tree.size()) - 1;
+}
+
+void SliceValues::Emit(u32 r, u64 inOffset, ClosedFold &f) const
+{
+    f.src.clear();
+    f.tree.clear();
+    (void)EmitNode(held_[r], inOffset, f);
+    const u32 leaves = static_cast<u32>(f.src.size());
+    for (ClosedFold::Step &st : f.tree) {
+        if (st.srcChild >= kInner) st.srcChild = st.srcChild - kInner + leaves;
+        if (st.dstChild >= kInner) st.dstChild = st.dstChild - kInner + leaves;
+    }
+}
+
 }  // namespace ops_hccl

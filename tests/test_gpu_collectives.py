@@ -775,7 +775,10 @@ def test_overlapping_buffers_are_planned_for_their_addresses(stream):
 CLOSED_FORM_ALGS = {"all_reduce": "InsAllReduceMesh1DTwoShotMeshChunk", "reduce_scatter": "InsReduceScatterMesh1DMeshChunk",
                     "reduce_scatter_gather": "InsReduceScatterAicpuReduceNHR", "all_reduce_one_shot": "InsAllReduceMesh1DOneShot",
                     "all_reduce_two_shot": "InsAllReduceMesh1DTwoShot", "reduce_scatter_mesh": "InsReduceScatterMesh1D",
-                    "all_reduce_gather": "InsAllReduceAicpuReduceNHR", "all_reduce_ring": "InsAllReduceRing"}
+                    "all_reduce_gather": "InsAllReduceAicpuReduceNHR", "all_reduce_ring": "InsAllReduceRing",
+                    "all_reduce_nhr": "InsAllReduceNHR", "reduce_scatter_nhr": "InsReduceScatterNHR",
+                    "all_reduce_rhd": "InsAllReduceRHD", "reduce_scatter_ordered": "ReduceScatterOrderPreserved",
+                    "reduce_scatter_ordered_group": "ReduceScatterOrderPreservedGroup"}
 
 
 @pytest.mark.parametrize("kind,n,dtype,op,count", [("all_reduce", 64, T.FP32, T.SUM, 64 * 63 * 3 + 17),
@@ -793,7 +796,17 @@ CLOSED_FORM_ALGS = {"all_reduce": "InsAllReduceMesh1DTwoShotMeshChunk", "reduce_
                                                    ("all_reduce_gather", 40, T.INT64, T.SUM, 30011),
                                                    ("all_reduce_ring", 20, T.FP32, T.MAX, 150001),
                                                    ("all_reduce_ring", 8, T.BFP16, T.SUM, 1 << 20),
-                                                   ("all_reduce_ring", 64, T.FP32, T.SUM, 37)])
+                                                   ("all_reduce_ring", 64, T.FP32, T.SUM, 37),
+                                                   ("all_reduce_nhr", 24, T.FP32, T.SUM, 200003),
+                                                   ("all_reduce_nhr", 33, T.BFP16, T.SUM, 70001),
+                                                   ("all_reduce_nhr", 5, T.FP64, T.PROD, 1 << 18),
+                                                   ("reduce_scatter_nhr", 12, T.FP32, T.MAX, 30011),
+                                                   ("reduce_scatter_nhr", 64, T.FP16, T.MAX, 2003),
+                                                   ("all_reduce_rhd", 12, T.FP32, T.SUM, 300007),
+                                                   ("all_reduce_rhd", 48, T.BFP16, T.SUM, 90001),
+                                                   ("all_reduce_rhd", 7, T.FP32, T.MIN, 1 << 19),
+                                                   ("reduce_scatter_ordered", 12, T.FP32, T.SUM, 50021),
+                                                   ("reduce_scatter_ordered_group", 40, T.FP32, T.SUM, 9001)])
 def test_templates_planned_from_their_closed_form(stream, kind, n, dtype, op, count):
     """Templates that state their result in closed form are planned from it (nothing recorded) and run as one fused
     pass: the 64-rank mesh-chunk AllReduce too (4032 chains).  The result is the oracle's replay of the template's

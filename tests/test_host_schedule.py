@@ -565,7 +565,9 @@ def traced(n, call, closed_form):
 
 @pytest.mark.parametrize("n", [2, 3, 4, 5, 7, 8, 12, 16, 17, 31, 32])
 @pytest.mark.parametrize("kind", ["all_reduce", "reduce_scatter", "reduce_scatter_gather", "all_reduce_one_shot",
-                                  "all_reduce_two_shot", "reduce_scatter_mesh", "all_reduce_gather", "all_reduce_ring"])
+                                  "all_reduce_two_shot", "reduce_scatter_mesh", "all_reduce_gather", "all_reduce_ring",
+                                  "all_reduce_nhr", "reduce_scatter_nhr", "all_reduce_rhd", "reduce_scatter_ordered",
+                                  "reduce_scatter_ordered_group"])
 def test_closed_form_of_a_template_equals_its_recorded_steps(kind, n):
     """The mesh-chunk templates and the gather-then-fold ReduceScatter state their result directly (N (N-1) chains,
     N chains) so that a world need not record, order and trace their N^3 steps; the one-shot, two-shot and mesh
@@ -575,7 +577,10 @@ def test_closed_form_of_a_template_equals_its_recorded_steps(kind, n):
     alg = {"all_reduce": "InsAllReduceMesh1DTwoShotMeshChunk", "reduce_scatter": "InsReduceScatterMesh1DMeshChunk",
            "reduce_scatter_gather": "InsReduceScatterAicpuReduceNHR", "all_reduce_one_shot": "InsAllReduceMesh1DOneShot",
            "all_reduce_two_shot": "InsAllReduceMesh1DTwoShot", "reduce_scatter_mesh": "InsReduceScatterMesh1D",
-           "all_reduce_gather": "InsAllReduceAicpuReduceNHR", "all_reduce_ring": "InsAllReduceRing"}[kind]
+           "all_reduce_gather": "InsAllReduceAicpuReduceNHR", "all_reduce_ring": "InsAllReduceRing",
+           "all_reduce_nhr": "InsAllReduceNHR", "reduce_scatter_nhr": "InsReduceScatterNHR",
+           "all_reduce_rhd": "InsAllReduceRHD", "reduce_scatter_ordered": "ReduceScatterOrderPreserved",
+           "reduce_scatter_ordered_group": "ReduceScatterOrderPreservedGroup"}[kind]
     reduces_all = kind.startswith("all_reduce")
     cmd = api.CMD_ALLREDUCE if reduces_all else api.CMD_REDUCE_SCATTER
     ins, outs = fake_ptrs(n)
@@ -654,9 +659,12 @@ def test_closed_form_among_64_ranks_and_when_it_is_not_used():
     closed, info_c = traced(n, call, 2)
     assert closed == recorded and info_c.levels == 0 and info_r.levels > 0
     assert info_c.fused == 1 and info_c.fusedSegments == info_r.fusedSegments == 64 * 63
-    # a template without a closed form records its steps whatever the mode
-    _, info = traced(n, lambda w: call(w, alg="InsAllReduceNHR"), 2)
-    assert info.levels > 0
+    # the log-step templates, whose results are trees of six levels here
+    for tree_alg in ("InsAllReduceNHR", "InsAllReduceRHD"):
+        rec, info_rec = traced(n, lambda w: call(w, alg=tree_alg), 0)
+        clo, info_clo = traced(n, lambda w: call(w, alg=tree_alg), 2)
+        assert clo == rec and info_clo.levels == 0 and info_rec.levels > 0, tree_alg
+        assert info_clo.fused == info_rec.fused == 1 and info_clo.fusedSegments == info_rec.fusedSegments
     # two ranks share an input buffer: the buffers do not lie apart, so the steps are recorded
     shared = [ins[0]] + ins[:-1]
     _, info = traced(n, lambda w: call(w, srcs=shared), 2)
