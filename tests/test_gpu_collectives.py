@@ -90,6 +90,33 @@ def test_allreduce_in_place(stream, mode):
         w.close()
 
 
+@pytest.mark.parametrize("alg", AR_ALGS)
+@pytest.mark.parametrize("n,dtype,op,count", [(8, T.FP32, T.SUM, 70001), (20, T.FP32, T.MAX, 30011),
+                                              (33, T.BFP16, T.SUM, 12345)])
+def test_allreduce_in_place_every_template(stream, alg, n, dtype, op, count):
+    """sendBuf == recvBuf on every rank, every template, planned from its closed form and fused into one pass (a
+    destination is then exactly one source of its own fold) -- or, for the self-first orders among more than 16 ranks,
+    staged."""
+    rng = np.random.default_rng(n * 31 + count)
+    xs = [payload(rng, dtype, count, "uniform" if dtype == T.FP32 else "normal") for _ in range(n)]
+    ccl = SMALL_CCL if n <= 20 else T.CCL_BYTES_DEFAULT
+    w = api.World(n, ccl_bytes=ccl)
+    try:
+        w.set_algorithm(api.CMD_ALLREDUCE, alg)
+        got, bufs = run_allreduce(w, stream, xs, count, dtype, op, in_place=True)
+        info = w.last_info()
+        assert info.fused == 1
+        if dtype in (T.FP16, T.BFP16) and op == T.SUM:
+            want = wide_oracle_allreduce(xs, count, dtype, alg, ccl)
+        else:
+            want = T.run_allreduce(T.NumericElems(dtype, op), xs, count, T.DTYPE_SIZE[dtype], alg, ccl_bytes=ccl)
+        for r in range(n):
+            assert_same_bits(got[r], want[r], dtype, f"{alg} n={n} rank {r}")
+            assert bufs[r].guard_intact()
+    finally:
+        w.close()
+
+
 def test_checked_world_verifies_then_launches(stream):
     """With the schedule check on, a collective is verified (no race, right semantics) and then runs as usual."""
     rng = np.random.default_rng(21)
