@@ -707,7 +707,7 @@ def test_ranks_on_different_streams_one_host_thread(stream):
 def test_a_plan_follows_its_collective_to_other_buffers(stream, mode, alg, dtype, op, n, count):
     """The same collective on buffers somewhere else (and differently aligned) is not planned again: the plan of the
     first call is moved there pointer by pointer, gets device tables of its own when the same buffers come a second
-    time, and is replayed from then on.  Every call's result is the oracle's.  Running in place is another shape."""
+    time (large plans: at once), and is replayed from then on.  Every call's result is the oracle's.  Running in place is another shape."""
     rng = np.random.default_rng(count)
     esz = T.DTYPE_SIZE[dtype]
     kind = "prod" if op == T.PROD else "uniform" if dtype == T.FP32 else "normal"
@@ -745,7 +745,10 @@ def test_a_plan_follows_its_collective_to_other_buffers(stream, mode, alg, dtype
         hit0, fused0, launches0 = call(*first, fresh())
         assert hit0 == 0
         assert call(*second, fresh()) == (2, fused0, launches0)    # moved, launched from host tables
-        assert call(*second, fresh()) == (2, fused0, launches0)    # moved, tables now in device memory
+        again = call(*second, fresh())
+        # moved once more, tables now in device memory -- or replayed already: a plan with more than 16 KiB of
+        # segment lists gets its device tables the first time it is moved
+        assert again in ((2, fused0, launches0), (1, fused0, launches0))
         assert call(*second, fresh()) == (1, fused0, launches0)    # replayed
         assert call(*first, fresh()) == (1, fused0, launches0)     # the first plan is still there
         hit, _, _ = call(first[0], first[0], fresh())              # in place: not the same collective
