@@ -342,7 +342,7 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
             ok = FoldsFromTrace(tr, params, foldType, op, folds, text);
         }
         FusedPlan plan;
-        ok = ok && BuildFusedPlan(params, folds, esz, plan);
+        ok = ok && BuildFusedPlan(params, folds, esz, plan, haveFolds);
         lap("fusedplan");
         w->lastFusedSegments =
             static_cast<u32>(plan.chainSegs.size() + plan.selfSegs.size() + plan.copySegs.size() + plan.treeSegs.size() +

@@ -203,6 +203,13 @@ bool FoldsFromClosedForm(const std::vector<ClosedFold> &closed, const std::vecto
     bool allFit = true;
     folds.reserve(closed.size());
     for (const ClosedFold &c : closed) {
+        // the pieces a template names must lie inside the buffers of the call
+        for (const ClosedFold::Ref &s : c.src) {
+            if (s.rank >= params.size() || s.offset + c.bytes > params[s.rank].inputSize) return false;
+        }
+        for (const ClosedFold::Ref &d : c.dst) {
+            if (d.rank >= params.size() || d.offset + c.bytes > params[d.rank].outputSize) return false;
+        }
         Fold f;
         if (c.tree.empty()) {
             for (const ClosedFold::Ref &s : c.src) f.src.push_back(reinterpret_cast<u64>(params[s.rank].inputPtr) + s.offset);
@@ -266,18 +273,21 @@ bool FoldsFromClosedForm(const std::vector<ClosedFold> &closed, const std::vecto
 
 // Builds the fused launch plan from the folds.  Returns false when they cannot run as one pass (a source that is
 // not an input, or an output that overlaps another fold's source); the caller then runs the steps one by one.
-bool BuildFusedPlan(const std::vector<OpParam> &params, std::vector<Fold> &folds, u32 esz, FusedPlan &plan)
+bool BuildFusedPlan(const std::vector<OpParam> &params, std::vector<Fold> &folds, u32 esz, FusedPlan &plan, bool stated)
 {
     const InputRanges inputs(params);
-    // every source must be input data (or an output that the same fold overwrites in place)
+    // every source must be input data (or an output that the same fold overwrites in place); the sources of folds
+    // stated in closed form are pieces of the inputs by construction
     for (const Fold &f : folds) {
+        if (stated) break;
         for (u64 a : f.src) {
             if (inputs.Find(a, f.bytes) == nullptr) return false;
         }
     }
     // Different expressions may still read the same sources in the same order (pieces that were reduced by
-    // different steps of equal shape): they become one fold with all the destinations.
-    {
+    // different steps of equal shape): they become one fold with all the destinations.  (A closed form names every
+    // value once.)
+    if (!stated) {
         std::map<std::vector<u64>, size_t> bySrc;
         std::vector<Fold> merged;
         for (Fold &f : folds) {

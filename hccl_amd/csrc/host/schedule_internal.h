@@ -261,8 +261,10 @@ bool FoldsFromTrace(const Tracer &tr, const std::vector<OpParam> &params, int dt
 // stand for.
 bool FoldsFromClosedForm(const std::vector<ClosedFold> &closed, const std::vector<OpParam> &params, int dtype, int op,
                          std::vector<Fold> &folds, std::string *text);
-// The fused launch lists of the folds; false when they cannot run as one pass.
-bool BuildFusedPlan(const std::vector<OpParam> &params, std::vector<Fold> &folds, u32 esz, FusedPlan &plan);
+// The fused launch lists of the folds; false when they cannot run as one pass.  `stated`: the folds come from a
+// closed form (their sources are input pieces and no two of them are the same value).
+bool BuildFusedPlan(const std::vector<OpParam> &params, std::vector<Fold> &folds, u32 esz, FusedPlan &plan,
+                    bool stated = false);
 // Every output piece against the contract of the collective.
 void CheckSemantics(const Tracer &tr, const std::vector<OpParam> &params, CheckReport &rep);
 
