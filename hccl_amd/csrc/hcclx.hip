@@ -830,6 +830,8 @@ int build_wide_batches_impl(const hcclx_wide_seg_t *segs, uint32_t nseg, int dty
     }
     const int ne = 16 / esz;
     Batch cur = proto;
+    cur.wide.reserve(nseg < static_cast<uint32_t>(kMaxWideSegsPerLaunch) ? nseg : kMaxWideSegsPerLaunch);
+    cur.tile_end.reserve(cur.wide.capacity());
     for (uint32_t i = 0; i < nseg; ++i) {
         const hcclx_wide_seg_t &s = segs[i];
         if (s.count == 0) continue;
@@ -869,6 +871,8 @@ int build_wide_batches_impl(const hcclx_wide_seg_t *segs, uint32_t nseg, int dty
             if (static_cast<int>(cur.wide.size()) == kMaxWideSegsPerLaunch) {
                 out->batches.push_back(std::move(cur));
                 cur = proto;
+                cur.wide.reserve(kMaxWideSegsPerLaunch);
+                cur.tile_end.reserve(kMaxWideSegsPerLaunch);
             }
             cur.total_tiles += tiles;
             cur.tile_end.push_back(cur.total_tiles);
