@@ -149,6 +149,24 @@ HcclResult ForgetfulPair::KernelRun(const OpParam &param, const TemplateDataPara
                        param.DataDes.dataType, param.reduceType);
 }
 
+// "Overreaching": the one-shot template with a closed form that names a piece beyond the end of the input.
+class OverreachingOneShot : public InsTempAllReduceMesh1DOneShot {
+public:
+    using InsTempAllReduceMesh1DOneShot::InsTempAllReduceMesh1DOneShot;
+    bool ClosedForm(const TemplateDataParams &p, u64, std::vector<ClosedFold> &out) const override
+    {
+        ClosedFold f;
+        f.bytes = p.sliceSize;
+        f.src.push_back({0, p.buffInfo.inBuffBaseOff + 64});
+        f.src.push_back({1, p.buffInfo.inBuffBaseOff});
+        f.dst.push_back({0, p.buffInfo.outBuffBaseOff});
+        out.push_back(f);
+        return true;
+    }
+};
+
+REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_ALLREDUCE, TestOverreachingOneShot, InsV2AllReduceSoleExecutor, TopoMatch1D,
+                 OverreachingOneShot);
 REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_ALLREDUCE, TestRacyOneShot, InsV2AllReduceSoleExecutor, TopoMatch1D, RacyOneShot);
 REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_ALLREDUCE, TestForgetfulPair, InsV2AllReduceSoleExecutor, TopoMatch1D, ForgetfulPair);
 '''
@@ -196,6 +214,26 @@ def test_a_wrong_template_is_caught_by_the_semantics_check(plugin):
         assert [w.all_reduce(r, ins[r], outs[r], 1000, T.FP32, T.SUM, FAKE_STREAM) for r in range(4)][-1] == 0
     finally:
         w.close()
+
+
+def test_a_closed_form_that_reaches_beyond_the_buffers_is_not_used(plugin):
+    """A template may state its result in closed form; a statement that names bytes outside the call's buffers is
+    dropped and the recorded steps are planned instead (here they are the one-shot template's)."""
+    def trace(alg, closed_form):
+        w = api.World(4, ccl_bytes=SMALL_CCL, dry=True)
+        try:
+            w.set_closed_form(closed_form)
+            w.set_algorithm(api.CMD_ALLREDUCE, alg)
+            ins, outs = fake_ptrs(4)
+            for r in range(4):
+                assert w.all_reduce(r, ins[r], outs[r], 1000, T.FP32, T.SUM, FAKE_STREAM) == 0
+            return w.last_trace(), w.last_info().levels
+        finally:
+            w.close()
+
+    want, _ = trace("InsAllReduceMesh1DOneShot", 0)
+    got, levels = trace("TestOverreachingOneShot", 2)
+    assert levels > 0 and got == want
 
 
 def run_ar(n, count, dtype, op):
