@@ -150,6 +150,94 @@ k_moe_perm(MoeConstPtrs dest, MoePtrs perm, uint32_t n, uint32_t entries, uint32
     }
 }
 
+// The scan and permutation kernels in one launch, for tables small enough that every workgroup can afford to sum
+// its rank's rows of the per-chunk histogram itself (at most kFusedChunks chunks per rank and kFusedCells histogram
+// cells in all): two dependent launches instead of three.  Workgroup (c, i): per destination the entries of rank i
+// in all chunks and in the chunks before c (one wavefront per destination, one lane per chunk), from them the first
+// row of each destination's group, then the permutation of chunk c as in k_moe_perm.  The workgroups of chunk 0
+// write their rank's rows of the count and displacement tables; workgroup (0, 0) also sums every rank's rows and
+// writes rdispls.  base keeps the raw histogram.
+constexpr uint32_t kFusedChunks = 64;
+constexpr uint32_t kFusedCells = 16384;
+
+__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v)
+{
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+    return v;
+}
+
+__global__ void __launch_bounds__(kMoeChunk)
+k_moe_scan_perm(MoeConstPtrs dest, MoePtrs perm, uint32_t n, uint32_t entries, uint32_t chunks, uint64_t row_elems,
+                const uint32_t *base, uint64_t *send_counts, uint64_t *sdispls, uint64_t *recv_counts, uint64_t *rdispls)
+{
+    __shared__ uint32_t s_total[kMoeMaxRanks];
+    __shared__ uint32_t s_before[kMoeMaxRanks];
+    __shared__ uint32_t s_start[kMoeMaxRanks];
+    __shared__ uint32_t s_cnt[4][kMoeMaxRanks];
+    __shared__ uint32_t s_all[kMoeMaxRanks * kMoeMaxRanks];   // workgroup (0, 0): entries of rank i for destination j
+    const uint32_t c = blockIdx.x;
+    const uint32_t i = blockIdx.y;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63;
+    for (uint32_t d = wave; d < n; d += 4) {
+        const uint32_t v = lane < chunks ? base[(static_cast<uint64_t>(i) * n + d) * chunks + lane] : 0;
+        const uint32_t total = wave_sum_u32(v);
+        const uint32_t before = wave_sum_u32(lane < c ? v : 0);
+        if (lane == 0) {
+            s_total[d] = total;
+            s_before[d] = before;
+        }
+    }
+    if (c == 0 && i == 0) {
+        for (uint32_t cell = threadIdx.x; cell < n * n; cell += kMoeChunk) {
+            uint32_t t = 0;
+            for (uint32_t k = 0; k < chunks; ++k) t += base[static_cast<uint64_t>(cell) * chunks + k];
+            s_all[cell] = t;
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const uint32_t t = lane < n ? s_total[lane] : 0;
+        const uint32_t incl = wave_scan_u32(t);
+        s_start[lane] = incl - t;
+        if (c == 0 && lane < n) {
+            send_counts[i * n + lane] = static_cast<uint64_t>(t) * row_elems;
+            sdispls[i * n + lane] = static_cast<uint64_t>(incl - t) * row_elems;
+            recv_counts[lane * n + i] = static_cast<uint64_t>(t) * row_elems;
+        }
+    }
+    if (c == 0 && i == 0 && threadIdx.x < n) {
+        const uint32_t j = threadIdx.x;
+        uint64_t run = 0;
+        for (uint32_t r = 0; r < n; ++r) {
+            rdispls[j * n + r] = run * row_elems;
+            run += s_all[r * n + j];
+        }
+    }
+    const uint32_t e = c * kMoeChunk + threadIdx.x;
+    int32_t d = -1;
+    if (e < entries) d = static_cast<const int32_t *>(dest.p[i])[e];
+    const bool valid = d >= 0 && static_cast<uint32_t>(d) < n;
+    uint32_t rank = 0;
+    const unsigned long long below = (1ull << lane) - 1ull;
+    for (uint32_t dd = 0; dd < n; ++dd) {
+        const unsigned long long m = __ballot(valid && static_cast<uint32_t>(d) == dd);
+        if (valid && static_cast<uint32_t>(d) == dd) rank = __popcll(m & below);
+        if (lane == 0) s_cnt[wave][dd] = __popcll(m);
+    }
+    __syncthreads();
+    if (e < entries) {
+        uint32_t out = kDropped;
+        if (valid) {
+            uint32_t off = rank;
+            for (uint32_t w = 0; w < wave; ++w) off += s_cnt[w][d];
+            out = s_start[d] + s_before[d] + off;
+        }
+        static_cast<uint32_t *>(perm.p[i])[e] = out;
+    }
+}
+
 // Row gather / scatter: 512 vectors of 16 bytes per workgroup, rows of vpr vectors.
 //   PACK:    packed[perm[e]] = tokens[e / topk]      (g runs over entries x vpr)
 //   UNPACK:  out[t] = packed[perm[t]]                (topk == 1; g runs over tokens x vpr)
@@ -463,6 +551,13 @@ int hcclx_moe_route(const int32_t *const *dest, uint32_t n, uint32_t entries, ui
     uint32_t *base = static_cast<uint32_t *>(workspace);
     uint32_t *row_start = base + static_cast<uint64_t>(n) * n * chunks;
     hipLaunchKernelGGL(k_moe_hist, dim3(chunks, n), dim3(kMoeChunk), 0, st, d, n, entries, chunks, base);
+    if (chunks <= kFusedChunks && static_cast<uint64_t>(n) * n * chunks <= kFusedCells) {
+        hipLaunchKernelGGL(k_moe_scan_perm, dim3(chunks, n), dim3(kMoeChunk), 0, st, d, as_mutable(p), n, entries, chunks,
+                           row_elems, base, send_counts, sdispls, recv_counts, rdispls);
+        hipError_t fe = hipGetLastError();
+        if (fe != hipSuccess) return fail_hip(fe, "moe routing kernels");
+        return HCCL_SUCCESS;
+    }
     hipLaunchKernelGGL(k_moe_scan, dim3(n), dim3(256), 0, st, n, chunks, row_elems, base, row_start, send_counts, sdispls,
                        recv_counts);
     hipLaunchKernelGGL(k_moe_perm, dim3(chunks, n), dim3(kMoeChunk), 0, st, d, as_mutable(p), n, entries, chunks, base,

@@ -36,8 +36,8 @@ def route_on_gpu(dests, n, entries, row_elems, skew=0):
                                        (64, 3001), (33, 7942), (16, 16384), (16, 16385), (5, 3), (12, 4099)])
 @pytest.mark.parametrize("skew", [0, 1])
 def test_route_tables_and_stable_permutation(n, entries, skew):
-    """Both routing paths (one launch up to 16384 entries per rank and 262144 in all, three launches beyond), with
-    destination arrays that are and are not 16-byte aligned."""
+    """Both routing paths (two launches while a rank has at most 64 chunks of 256 entries and the per-chunk histogram at
+    most 16384 cells, three beyond), with destination arrays that are and are not 16-byte aligned."""
     rng = np.random.default_rng(n * 1000 + entries)
     p = 1.0 / np.arange(1, n + 1) ** 1.2
     dests = [rng.choice(n, size=entries, p=p / p.sum()) for _ in range(n)]
