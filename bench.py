@@ -5,9 +5,14 @@ A step is one pass of the hot path over one batch of synthetic input that is alr
 by default the ReduceScatter SUM bf16 of 8 virtual ranks x 33,554,432 elements (64 MiB per rank), mesh
 template order, each output shard a fused 8-way reduce in one HBM pass.  `value` is the effective HBM
 bandwidth: algorithmic bytes (every input byte read once + every output byte written once) divided by
-the time of a step.  One JSON line is printed.
+the time of a step.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--no-ops]
+Output: the LAST line of stdout is the benchmark line, one compact JSON object (under 2000 bytes: metric, value,
+roofline, cpu_baseline and one percentage per op).  The tables behind it (per-op rows, the 12-rank size sweep,
+small-message and planning times from C++) are printed before it, one JSON object per line, and written to
+gpurun_out/bench_details.json.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--no-ops] [--no-sweep]
 """
 import argparse
 import json
@@ -20,6 +25,8 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+METRIC = "effective HBM GB/s (and % of peak) per op at 64MB/rank, 8 virtual ranks"
+LINE_LIMIT = 2000      # bytes: the benchmark line must survive a reader that keeps the last 2000 characters
 
 
 def profile_traffic(path, allow_missing=False):
@@ -130,7 +137,7 @@ class ReduceScatterMesh(Workload):
     def cpu_baseline(self, parallel):
         """The oracle's restatement of the same template on the same shape, timed on the host."""
         import numpy as np
-        T = self.T
+        from oracle import templates as T     # the only use of the oracle in this script: the thing timed here
         rng = np.random.default_rng(0)
         xs = [T.narrow16(rng.standard_normal(self.n * self.recv, dtype=np.float32), T.BFP16) for _ in range(self.n)]
         best = None
@@ -272,10 +279,13 @@ class AllToAllV(Workload):
         w = 1.0 / np.arange(1, n + 1) ** 1.2
         w /= w.sum()
         tok = np.stack([np.bincount(rng.choice(n, size=tokens, p=w), minlength=n) for _ in range(n)])
-        m = (tok * hidden).tolist()
-        self.v = [T.alltoallvc_to_v(m, r) for r in range(n)]
+        m = tok * hidden
+        # rank r sends row r and receives column r; displacements are the exclusive running sums (what
+        # HcclAlltoAllVC derives from the same matrix)
+        excl = lambda a: [int(x) for x in np.concatenate([[0], np.cumsum(a)[:-1]])]
+        self.v = [([int(x) for x in m[r]], excl(m[r]), [int(x) for x in m[:, r]], excl(m[:, r])) for r in range(n)]
         self.tabs = [[api.u64_table(t) for t in self.v[r]] for r in range(n)]   # converted once
-        self.payload = int(sum(sum(row) for row in m)) * 2
+        self.payload = int(m.sum()) * 2
         self.send = [torch.randint(-32768, 32767, (tokens * hidden,), device="cuda:0", dtype=torch.int16)
                      for _ in range(n)]
         self.recv = [torch.empty(max(1, sum(self.v[j][2])), device="cuda:0", dtype=torch.int16) for j in range(n)]
@@ -375,7 +385,7 @@ class MoeDispatchPack(Workload):
             what = "AlltoAllV back + combine in one pass" if self.combine else "route + pack + AlltoAllV in one pass"
         else:
             what = "moe combine (top-1)" if self.combine else "moe route + pack"
-        return {"algorithm": what, "fused": True, "launches": 1 if self.combine else 4, "plan_cache_hit": False}
+        return {"algorithm": what, "fused": True, "launches": 1 if self.combine else 3, "plan_cache_hit": False}
 
 
 class CopyCalibration(Workload):
@@ -596,6 +606,89 @@ def time_steps(torch, wl, steps, warmup):
     return wall_ms, ev_ms
 
 
+# short names of the workloads for the one-number-per-op summary of the benchmark line
+SHORT = {
+    "reduce_scatter_sum_bf16_mesh_8x64MiB": "rs_bf16_8x64M",
+    "all_reduce_sum_fp32_8x64MiB": "ar_f32_8x64M",
+    "all_gather_fp16_8x64MiB": "ag_f16_8x64M",
+    "all_to_all_v_bf16_moe_8x4096x7168": "a2av_moe_4096",
+    "all_to_all_v_bf16_moe_8x4608x7168": "a2av_moe_4608",
+    "all_gather_v_fp16_16_ranks_ragged": "agv_f16_16r",
+    "all_reduce_sum_fp32_8x4MiB": "ar_f32_8x4M_oneshot",
+    "all_reduce_sum_fp32_8x4MiB_ring": "ar_f32_8x4M_ring",
+    "all_reduce_sum_fp32_8x4MiB_ring_step_by_step": "ar_f32_8x4M_ring_steps",
+    "all_reduce_sum_fp32_8x64MiB_two_shot_step_by_step": "ar_f32_8x64M_steps",
+    "all_reduce_sum_fp32_32x16MiB": "ar_f32_32x16M",
+    "all_reduce_sum_fp32_32x16MiB_nhr": "ar_f32_32x16M_nhr",
+    "all_reduce_max_int32_12x64MiB_nhr": "ar_i32max_12x64M_nhr",
+    "all_reduce_prod_fp32_12x64MiB_aicpu_nhr": "ar_f32prod_12x64M",
+    "reduce_scatter_sum_bf16_mesh_32x32MiB": "rs_bf16_32x32M",
+    "moe_dispatch_pack_bf16_8x4096x7168": "moe_pack",
+    "moe_combine_bf16_8x4096x7168": "moe_combine",
+    "moe_route_dispatch_bf16_8x4096x7168": "moe_route_dispatch",
+    "moe_gather_combine_bf16_8x4096x7168": "moe_gather_combine",
+}
+
+
+def benchmark_line(args, wl, wall_ms, ev_ms, traffic, cpu=None, ops=None, small=None):
+    """The benchmark line as a string: one compact JSON object that stays under LINE_LIMIT bytes.
+
+    wl: what the headline workload is (name, dtype, n, algo_bytes, kernel, profile, info); wall_ms / ev_ms: host clock
+    and HIP-event time per step; traffic: HBM bytes per step from the profile (or None); cpu: the cpu_baseline
+    object; ops: {workload name: percent of the 8 TB/s peak}; small: latency-bound collectives in microseconds,
+    from Python and from C++ side by side."""
+    gbs = wl["algo_bytes"] / (ev_ms * 1e-3) / 1e9
+    line = {
+        "metric": METRIC,
+        "value": round(wl["algo_bytes"] / (wall_ms * 1e-3) / 1e9, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": wl["dtype"],
+        "data": "synthetic",
+        "config": {"workload": wl["name"], "virtual_ranks": wl["n"], "algorithm": wl["info"].get("algorithm"),
+                   "launches": wl["info"].get("launches"), "pct_of_hbm_peak": round(gbs / HBM_PEAK_GBS * 100, 1)},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "algorithmic_bytes": wl["algo_bytes"], "kernel": wl["kernel"], "kernel_us": round(ev_ms * 1e3, 2)},
+    }
+    if cpu is not None:
+        line["cpu_baseline"] = cpu
+    if ops:
+        line["ops_pct_of_peak"] = {SHORT.get(k, k): v for k, v in ops.items()}
+    if small:
+        line["small_us"] = small
+    text = json.dumps(line, separators=(",", ":"))
+    if len(text.encode()) >= LINE_LIMIT:
+        # never let an extra push the figures a reader needs out of its window: drop the extras, longest first
+        for key in ("ops_pct_of_peak", "small_us"):
+            line.pop(key, None)
+            text = json.dumps(line, separators=(",", ":"))
+            if len(text.encode()) < LINE_LIMIT:
+                break
+    assert len(text.encode()) < LINE_LIMIT, "benchmark line too long"
+    return text
+
+
+def emit_details(details):
+    """The tables behind the benchmark line: one JSON object per line on stdout (before the benchmark line) and
+    the whole of it in gpurun_out/bench_details.json when that folder can be written."""
+    for key, val in details.items():
+        print(json.dumps({"detail": key, "data": val}))
+    try:
+        out = os.path.join(ROOT, "gpurun_out")
+        os.makedirs(out, exist_ok=True)
+        with open(os.path.join(out, "bench_details.json"), "w") as f:
+            json.dump(details, f, indent=1)
+    except OSError:
+        pass
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -604,7 +697,7 @@ def main():
         sys.exit(2)
     import torch
     from hccl_amd import api, hcclx
-    from oracle import templates as T   # cpu_baseline leg only
+    from hccl_amd import types as T
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -617,30 +710,12 @@ def main():
 
     wl = makers[args.workload](torch, api, T)
     wall_ms, ev_ms = time_steps(torch, wl, args.steps, args.warmup)
-    gbs = wl.algo_bytes() / (ev_ms * 1e-3) / 1e9
-    line = {
-        "metric": "effective HBM GB/s (and % of peak) per op at 64MB/rank, 8 virtual ranks",
-        "value": round(wl.algo_bytes() / (wall_ms * 1e-3) / 1e9, 1),
-        "unit": "GB/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(wall_ms, 5),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": wl.dtype,
-        "data": "synthetic",
-        "config": dict({"workload": wl.name, "virtual_ranks": wl.n, "algorithmic_bytes": wl.algo_bytes(),
-                        "pct_of_hbm_peak": round(gbs / HBM_PEAK_GBS * 100, 1), "entry": "HcclReduceScatter"
-                        if "reduce_scatter" in wl.name else "Hccl* entry points"}, **wl.info()),
-        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": profile_traffic(wl.profile, args.allow_missing_profile),
-                     "traffic_source": wl.profile,
-                     "algorithmic_bytes": wl.algo_bytes(), "kernel": wl.kernel,
-                     "kernel_us": round(ev_ms * 1e3, 2)},
-    }
+    head = {"name": wl.name, "dtype": wl.dtype, "n": wl.n, "algo_bytes": wl.algo_bytes(), "kernel": wl.kernel,
+            "info": wl.info()}
+    traffic = profile_traffic(wl.profile, args.allow_missing_profile)
+    details = {"headline": dict(head, wall_ms=wall_ms, event_ms=ev_ms, traffic_source=wl.profile)}
 
+    ops_pct, small = None, None
     if not args.no_ops:
         ops = {}
         for name, make in WORKLOADS.items():
@@ -662,28 +737,42 @@ def main():
                 w2.world.close()
                 del w2
                 torch.cuda.empty_cache()
-        line["ops"] = ops
+        details["ops"] = ops
+        ops_pct = {k: v["pct_of_peak"] for k, v in ops.items()}
     if not args.no_ops and not args.no_sweep:
-        line["allreduce_12_ranks_sweep"] = sweep_allreduce_12_ranks(torch, api, T, args.steps)
+        sweep = sweep_allreduce_12_ranks(torch, api, T, args.steps)
+        details["allreduce_12_ranks_sweep"] = sweep
         cpp = small_messages_from_cpp()
         if cpp is not None:
-            line["small_messages_from_cpp"] = cpp
+            details["small_messages_from_cpp"] = cpp
             for row in cpp.get("rows", []):
-                size = line["allreduce_12_ranks_sweep"].get(str(row["bytes_per_rank"]), {})
+                size = sweep.get(str(row["bytes_per_rank"]), {})
                 if row["ranks"] == 12 and row["case"] in size:
                     size[row["case"]]["us_from_cpp"] = row["us"]
+            # benchmark configuration 1 (8 x 4 MiB fp32) is bound by launch latency: microseconds per collective
+            # issued from Python (twelve ctypes calls around a 10 us kernel) next to the same collective from C++
+            small = {}
+            for key, case, wname in (("ar_f32_8x4M_oneshot", "fp32_sum_default", "all_reduce_sum_fp32_8x4MiB"),
+                                     ("ar_f32_8x4M_ring", "fp32_sum_ring", "all_reduce_sum_fp32_8x4MiB_ring")):
+                row = [r for r in cpp.get("rows", []) if r["case"] == case and r["ranks"] == 8
+                       and r["bytes_per_rank"] == 4 << 20]
+                if row and wname in details.get("ops", {}):
+                    small[key] = {"py": details["ops"][wname]["us"], "cpp": row[0]["us"]}
         planning = planning_from_cpp()
         if planning is not None:
-            line["planning_from_cpp"] = planning
+            details["planning_from_cpp"] = planning
 
+    cpu = None
     if not args.no_cpu and hasattr(wl, "cpu_baseline"):
         v1, sample = wl.cpu_baseline(parallel=False)
         vp, _ = wl.cpu_baseline(parallel=True)
-        line["cpu_baseline"] = {"value": round(v1, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-                                "sample": sample,
-                                "all_cores": {"value": round(vp, 3),
-                                              "cores": int(os.environ.get("OMP_NUM_THREADS") or os.cpu_count())}}
-    print(json.dumps(line))
+        cores = int(os.environ.get("OMP_NUM_THREADS") or os.cpu_count())
+        cpu = {"value": round(v1, 3), "unit": "GB/s", "cores": 1, "kind": "port", "sample": sample,
+               "all_cores": {"value": round(vp, 3), "cores": cores}}
+        details["cpu_baseline"] = cpu
+    emit_details(details)
+    sys.stdout.flush()
+    print(benchmark_line(args, head, wall_ms, ev_ms, traffic, cpu, ops_pct, small))
 
 
 if __name__ == "__main__":

@@ -977,6 +977,8 @@ int hcclx_init(void) { return device_ctx() ? HCCL_SUCCESS : HCCL_E_RUNTIME; }
 
 const char *hcclx_last_error(void) { return g_err.c_str(); }
 
+uint64_t hcclx_kernels_launched(void) { return hcclx::kernels_launched(); }
+
 uint32_t hcclx_dtype_size(int dtype) { return static_cast<uint32_t>(dtype_size(dtype)); }
 
 static int launch_built(DeviceCtx *ctx, const Built &built, hipStream_t st)
@@ -1086,7 +1088,7 @@ int hcclx_fold_static(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op,
         TablePiece piece;
         const uint32_t n = static_cast<uint32_t>(bytes - off < kPutBytes ? bytes - off : kPutBytes);
         std::memcpy(&piece, table + off, n);
-        hipLaunchKernelGGL(k_put_table, dim3(1), dim3(256), 0, st, piece, ctx->static_table + off, n);
+        HCCLX_LAUNCH(k_put_table, dim3(1), dim3(256), 0, st, piece, ctx->static_table + off, n);
         const hipError_t pe = hipGetLastError();
         if (pe != hipSuccess) return fail_hip(pe, "launch table upload");
     }

@@ -5,6 +5,7 @@
 #include <string>
 #include <vector>
 #include "hccl_types.h"
+#include "kernels/launch.h"
 
 namespace hcclx {
 

@@ -480,16 +480,16 @@ hipError_t launch_gather_long(int kind, dim3 grid, hipStream_t st, const MoeCons
                               uint32_t esz, const uint64_t *sdispls, const uint64_t *rdispls)
 {
     if (kind == HCCL_DATA_TYPE_FP32) {
-        hipLaunchKernelGGL(k_moe_gather_long<HCCL_DATA_TYPE_FP32>, grid, dim3(256), 0, st, rows, dest, perm, out, n, topk,
+        HCCLX_LAUNCH(k_moe_gather_long<HCCL_DATA_TYPE_FP32>, grid, dim3(256), 0, st, rows, dest, perm, out, n, topk,
                            vpr, runs, esz, sdispls, rdispls);
     } else if (kind == HCCL_DATA_TYPE_FP16) {
-        hipLaunchKernelGGL(k_moe_gather_long<HCCL_DATA_TYPE_FP16>, grid, dim3(256), 0, st, rows, dest, perm, out, n, topk,
+        HCCLX_LAUNCH(k_moe_gather_long<HCCL_DATA_TYPE_FP16>, grid, dim3(256), 0, st, rows, dest, perm, out, n, topk,
                            vpr, runs, esz, sdispls, rdispls);
     } else if (kind == HCCL_DATA_TYPE_BFP16) {
-        hipLaunchKernelGGL(k_moe_gather_long<HCCL_DATA_TYPE_BFP16>, grid, dim3(256), 0, st, rows, dest, perm, out, n, topk,
+        HCCLX_LAUNCH(k_moe_gather_long<HCCL_DATA_TYPE_BFP16>, grid, dim3(256), 0, st, rows, dest, perm, out, n, topk,
                            vpr, runs, esz, sdispls, rdispls);
     } else {
-        hipLaunchKernelGGL(k_moe_gather_long<HCCL_DATA_TYPE_INT8>, grid, dim3(256), 0, st, rows, dest, perm, out, n, topk,
+        HCCLX_LAUNCH(k_moe_gather_long<HCCL_DATA_TYPE_INT8>, grid, dim3(256), 0, st, rows, dest, perm, out, n, topk,
                            vpr, runs, esz, sdispls, rdispls);
     }
     return hipGetLastError();
@@ -550,17 +550,17 @@ int hcclx_moe_route(const int32_t *const *dest, uint32_t n, uint32_t entries, ui
     const uint32_t chunks = chunks_of(entries);
     uint32_t *base = static_cast<uint32_t *>(workspace);
     uint32_t *row_start = base + static_cast<uint64_t>(n) * n * chunks;
-    hipLaunchKernelGGL(k_moe_hist, dim3(chunks, n), dim3(kMoeChunk), 0, st, d, n, entries, chunks, base);
+    HCCLX_LAUNCH(k_moe_hist, dim3(chunks, n), dim3(kMoeChunk), 0, st, d, n, entries, chunks, base);
     if (chunks <= kFusedChunks && static_cast<uint64_t>(n) * n * chunks <= kFusedCells) {
-        hipLaunchKernelGGL(k_moe_scan_perm, dim3(chunks, n), dim3(kMoeChunk), 0, st, d, as_mutable(p), n, entries, chunks,
+        HCCLX_LAUNCH(k_moe_scan_perm, dim3(chunks, n), dim3(kMoeChunk), 0, st, d, as_mutable(p), n, entries, chunks,
                            row_elems, base, send_counts, sdispls, recv_counts, rdispls);
         hipError_t fe = hipGetLastError();
         if (fe != hipSuccess) return fail_hip(fe, "moe routing kernels");
         return HCCL_SUCCESS;
     }
-    hipLaunchKernelGGL(k_moe_scan, dim3(n), dim3(256), 0, st, n, chunks, row_elems, base, row_start, send_counts, sdispls,
+    HCCLX_LAUNCH(k_moe_scan, dim3(n), dim3(256), 0, st, n, chunks, row_elems, base, row_start, send_counts, sdispls,
                        recv_counts);
-    hipLaunchKernelGGL(k_moe_perm, dim3(chunks, n), dim3(kMoeChunk), 0, st, d, as_mutable(p), n, entries, chunks, base,
+    HCCLX_LAUNCH(k_moe_perm, dim3(chunks, n), dim3(kMoeChunk), 0, st, d, as_mutable(p), n, entries, chunks, base,
                        row_start, send_counts, rdispls);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail_hip(e, "moe routing kernels");
@@ -586,7 +586,7 @@ int hcclx_moe_pack(const void *const *tokens, const uint32_t *const *perm, uint3
     const uint32_t vpr = static_cast<uint32_t>(row_bytes / 16);
     const uint64_t blocks = (static_cast<uint64_t>(entries) * vpr + 511) / 512;
     if (blocks > 0x7fffffffull) return fail(HCCL_E_PARA, "too much data for one launch");
-    hipLaunchKernelGGL(k_moe_rows<true>, dim3(static_cast<uint32_t>(blocks), n), dim3(256), 0, static_cast<hipStream_t>(stream),
+    HCCLX_LAUNCH(k_moe_rows<true>, dim3(static_cast<uint32_t>(blocks), n), dim3(256), 0, static_cast<hipStream_t>(stream),
                        s, p, as_mutable(o), entries, topk, vpr);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail_hip(e, "moe pack kernel");
@@ -620,18 +620,18 @@ int hcclx_moe_combine(const void *const *packed, const uint32_t *const *perm, ui
     if (topk == 1) {
         const uint64_t blocks = (static_cast<uint64_t>(tokens) * vpr + 511) / 512;
         if (blocks > 0x7fffffffull) return fail(HCCL_E_PARA, "too much data for one launch");
-        hipLaunchKernelGGL(k_moe_rows<false>, dim3(static_cast<uint32_t>(blocks), n), dim3(256), 0, st, s, p, as_mutable(o),
+        HCCLX_LAUNCH(k_moe_rows<false>, dim3(static_cast<uint32_t>(blocks), n), dim3(256), 0, st, s, p, as_mutable(o),
                            tokens, 1u, vpr);
     } else {
         const uint64_t blocks = (static_cast<uint64_t>(tokens) * vpr + 255) / 256;
         if (blocks > 0x7fffffffull) return fail(HCCL_E_PARA, "too much data for one launch");
         const dim3 grid(static_cast<uint32_t>(blocks), n);
         if (dtype == HCCL_DATA_TYPE_FP32) {
-            hipLaunchKernelGGL(k_moe_combine<HCCL_DATA_TYPE_FP32>, grid, dim3(256), 0, st, s, p, as_mutable(o), tokens, topk, vpr);
+            HCCLX_LAUNCH(k_moe_combine<HCCL_DATA_TYPE_FP32>, grid, dim3(256), 0, st, s, p, as_mutable(o), tokens, topk, vpr);
         } else if (dtype == HCCL_DATA_TYPE_FP16) {
-            hipLaunchKernelGGL(k_moe_combine<HCCL_DATA_TYPE_FP16>, grid, dim3(256), 0, st, s, p, as_mutable(o), tokens, topk, vpr);
+            HCCLX_LAUNCH(k_moe_combine<HCCL_DATA_TYPE_FP16>, grid, dim3(256), 0, st, s, p, as_mutable(o), tokens, topk, vpr);
         } else {
-            hipLaunchKernelGGL(k_moe_combine<HCCL_DATA_TYPE_BFP16>, grid, dim3(256), 0, st, s, p, as_mutable(o), tokens, topk, vpr);
+            HCCLX_LAUNCH(k_moe_combine<HCCL_DATA_TYPE_BFP16>, grid, dim3(256), 0, st, s, p, as_mutable(o), tokens, topk, vpr);
         }
     }
     hipError_t e = hipGetLastError();
@@ -667,7 +667,7 @@ int hcclx_moe_dispatch(const void *const *tokens, const int32_t *const *dest, co
         const RowRuns runs = row_runs(vpr, 512);
         const uint64_t long_blocks = static_cast<uint64_t>(entries) * runs.per_row;
         if (long_blocks > 0x7fffffffull) return fail(HCCL_E_PARA, "too much data for one launch");
-        hipLaunchKernelGGL(k_moe_scatter_long, dim3(static_cast<uint32_t>(long_blocks), n), dim3(256), 0,
+        HCCLX_LAUNCH(k_moe_scatter_long, dim3(static_cast<uint32_t>(long_blocks), n), dim3(256), 0,
                            static_cast<hipStream_t>(stream), s, d, p, as_mutable(o), n, topk, vpr, runs, static_cast<uint32_t>(esz),
                            sdispls, rdispls);
         hipError_t le = hipGetLastError();
@@ -676,7 +676,7 @@ int hcclx_moe_dispatch(const void *const *tokens, const int32_t *const *dest, co
     }
     const uint64_t blocks = (static_cast<uint64_t>(entries) * vpr + 511) / 512;
     if (blocks > 0x7fffffffull) return fail(HCCL_E_PARA, "too much data for one launch");
-    hipLaunchKernelGGL(k_moe_dispatch, dim3(static_cast<uint32_t>(blocks), n), dim3(256), 0, static_cast<hipStream_t>(stream), s, d,
+    HCCLX_LAUNCH(k_moe_dispatch, dim3(static_cast<uint32_t>(blocks), n), dim3(256), 0, static_cast<hipStream_t>(stream), s, d,
                        p, as_mutable(o), n, entries, topk, vpr, static_cast<uint32_t>(esz), sdispls, rdispls);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail_hip(e, "moe dispatch kernel");
@@ -725,16 +725,16 @@ int hcclx_moe_gather_combine(const void *const *expert, const int32_t *const *de
     if (blocks > 0x7fffffffull) return fail(HCCL_E_PARA, "too much data for one launch");
     const dim3 grid(static_cast<uint32_t>(blocks), n);
     if (kind == HCCL_DATA_TYPE_FP32) {
-        hipLaunchKernelGGL(k_moe_gather_combine<HCCL_DATA_TYPE_FP32>, grid, dim3(256), 0, st, s, d, p, as_mutable(o), n, tokens, topk,
+        HCCLX_LAUNCH(k_moe_gather_combine<HCCL_DATA_TYPE_FP32>, grid, dim3(256), 0, st, s, d, p, as_mutable(o), n, tokens, topk,
                            vpr, static_cast<uint32_t>(esz), sdispls, rdispls);
     } else if (kind == HCCL_DATA_TYPE_FP16) {
-        hipLaunchKernelGGL(k_moe_gather_combine<HCCL_DATA_TYPE_FP16>, grid, dim3(256), 0, st, s, d, p, as_mutable(o), n, tokens, topk,
+        HCCLX_LAUNCH(k_moe_gather_combine<HCCL_DATA_TYPE_FP16>, grid, dim3(256), 0, st, s, d, p, as_mutable(o), n, tokens, topk,
                            vpr, static_cast<uint32_t>(esz), sdispls, rdispls);
     } else if (kind == HCCL_DATA_TYPE_BFP16) {
-        hipLaunchKernelGGL(k_moe_gather_combine<HCCL_DATA_TYPE_BFP16>, grid, dim3(256), 0, st, s, d, p, as_mutable(o), n, tokens, topk,
+        HCCLX_LAUNCH(k_moe_gather_combine<HCCL_DATA_TYPE_BFP16>, grid, dim3(256), 0, st, s, d, p, as_mutable(o), n, tokens, topk,
                            vpr, static_cast<uint32_t>(esz), sdispls, rdispls);
     } else {
-        hipLaunchKernelGGL(k_moe_gather_combine<HCCL_DATA_TYPE_INT8>, grid, dim3(256), 0, st, s, d, p, as_mutable(o), n, tokens, topk,
+        HCCLX_LAUNCH(k_moe_gather_combine<HCCL_DATA_TYPE_INT8>, grid, dim3(256), 0, st, s, d, p, as_mutable(o), n, tokens, topk,
                            vpr, static_cast<uint32_t>(esz), sdispls, rdispls);
     }
     hipError_t e = hipGetLastError();

@@ -181,25 +181,23 @@ HcclResult CreatePlans(const std::vector<HostPart> &parts, std::vector<hcclx_pla
 // The same parts launched once, their tables travelling through the descriptor ring: no allocation, no plan kept.
 HcclResult LaunchParts(World *w, const std::vector<HostPart> &parts, void *stream)
 {
-    w->lastLaunches = 0;
+    (void)w;
     for (const HostPart &hp : parts) {
         const int rc = hp.wide ? hcclx_fold_wide(hp.wideSegs.data(), static_cast<uint32_t>(hp.wideSegs.size()), hp.dtype, hp.op,
                                                  hp.mode, stream)
                                : hcclx_fold(hp.segs.data(), static_cast<uint32_t>(hp.segs.size()), hp.dtype, hp.op, hp.mode,
                                             stream);
         if (rc != HCCL_SUCCESS) return static_cast<HcclResult>(rc);
-        w->lastLaunches++;
     }
     return HCCL_SUCCESS;
 }
 
 HcclResult LaunchPlans(World *w, const std::vector<hcclx_plan *> &plans, void *stream)
 {
-    w->lastLaunches = 0;
+    (void)w;
     for (hcclx_plan *p : plans) {
         const int rc = hcclx_plan_launch(p, stream);
         if (rc != HCCL_SUCCESS) return static_cast<HcclResult>(rc);
-        w->lastLaunches++;
     }
     return HCCL_SUCCESS;
 }

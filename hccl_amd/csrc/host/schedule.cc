@@ -81,7 +81,6 @@ HcclResult LaunchDataMove(World *w, const std::vector<OpParam> &params, void *st
         recv[r] = params[r].outputPtr;
     }
     const HcclCMDType t = params[0].opType;
-    w->lastLaunches = 1;
     if (t == HcclCMDType::HCCL_CMD_ALLGATHER || t == HcclCMDType::HCCL_CMD_ALLGATHER_V) {
         std::vector<u64> counts(n);
         std::vector<u64> displs(n);
@@ -140,10 +139,17 @@ HcclResult JoinStreams(const std::vector<OpParam> &params, hipStream_t launch, b
 
 HcclResult RunCollective(World *w, std::vector<OpParam> &params)
 {
-    if (w->dryRun) return RunCollectiveOnStream(w, params);
+    if (w->dryRun) {
+        w->lastLaunches = 0;
+        return RunCollectiveOnStream(w, params);
+    }
     hipStream_t launch = static_cast<hipStream_t>(params[w->rankSize - 1].stream);
     CHK_RET(JoinStreams(params, launch, true));
+    // everything a collective launches is launched by this host thread: the kernels it took are the difference
+    // of the library's per-thread count (a fold whose result fans out is two, a large ragged gather several)
+    const uint64_t kernelsBefore = hcclx_kernels_launched();
     const HcclResult res = RunCollectiveOnStream(w, params);
+    w->lastLaunches = static_cast<u32>(hcclx_kernels_launched() - kernelsBefore);
     CHK_RET(JoinStreams(params, launch, false));
     return res;
 }

@@ -12,6 +12,7 @@
 #pragma once
 #include "elem.h"
 #include "segtab.h"
+#include "launch.h"
 
 namespace hcclx {
 

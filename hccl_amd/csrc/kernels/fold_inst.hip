@@ -10,7 +10,7 @@ namespace hcclx {
 template <int DT, int OP, int MAXN, int MODE>
 static hipError_t launch_one(const FoldLaunch &l)
 {
-    hipLaunchKernelGGL((k_fold<DT, OP, MAXN, MODE>), dim3(l.grid), dim3(kFoldThreads), l.nseg * sizeof(uint64_t), l.stream,
+    HCCLX_LAUNCH((k_fold<DT, OP, MAXN, MODE>), dim3(l.grid), dim3(kFoldThreads), l.nseg * sizeof(uint64_t), l.stream,
                        l.tile_end, static_cast<const SegDev *>(l.segs), l.nseg, l.total_tiles, l.store_policy, l.uniform_tiles);
     return hipGetLastError();
 }
@@ -18,7 +18,7 @@ static hipError_t launch_one(const FoldLaunch &l)
 template <int DT, int OP, int MODE, int U>
 static hipError_t launch_wide_u(const FoldLaunch &l)
 {
-    hipLaunchKernelGGL((k_fold_wide<DT, OP, MODE, U>), dim3(l.grid), dim3(kFoldThreads), l.nseg * sizeof(uint64_t), l.stream,
+    HCCLX_LAUNCH((k_fold_wide<DT, OP, MODE, U>), dim3(l.grid), dim3(kFoldThreads), l.nseg * sizeof(uint64_t), l.stream,
                        l.tile_end, static_cast<const SegWide *>(l.segs), l.nseg, l.total_tiles, l.xcd_remap, l.store_policy, l.uniform_tiles);
     return hipGetLastError();
 }

@@ -276,7 +276,7 @@ hipError_t launch_alltoallv(const VRankPtrs &ptrs, const uint64_t *send_counts, 
 {
     const size_t lds = (static_cast<size_t>(n) * n + 4) * sizeof(uint64_t);
     const A2avTablesPtr tabs{send_counts, sdispls, rdispls};
-    hipLaunchKernelGGL((k_alltoallv<VRankPtrs, A2avTablesPtr>), dim3(grid), dim3(kThreads), lds, stream, ptrs, tabs, n,
+    HCCLX_LAUNCH((k_alltoallv<VRankPtrs, A2avTablesPtr>), dim3(grid), dim3(kThreads), lds, stream, ptrs, tabs, n,
                        esz, tiles_per_block);
     return hipGetLastError();
 }
@@ -284,11 +284,11 @@ hipError_t launch_alltoallv(const VRankPtrs &ptrs, const uint64_t *send_counts, 
 hipError_t launch_copy_blocks(const CopyBlock *blocks, uint32_t nblocks, uint32_t grid, int unroll, hipStream_t stream)
 {
     if (unroll == 1) {
-        hipLaunchKernelGGL((k_copy_blocks<1>), dim3(grid), dim3(kThreads), 0, stream, blocks, nblocks);
+        HCCLX_LAUNCH((k_copy_blocks<1>), dim3(grid), dim3(kThreads), 0, stream, blocks, nblocks);
     } else if (unroll == 2) {
-        hipLaunchKernelGGL((k_copy_blocks<2>), dim3(grid), dim3(kThreads), 0, stream, blocks, nblocks);
+        HCCLX_LAUNCH((k_copy_blocks<2>), dim3(grid), dim3(kThreads), 0, stream, blocks, nblocks);
     } else {
-        hipLaunchKernelGGL((k_copy_blocks<4>), dim3(grid), dim3(kThreads), 0, stream, blocks, nblocks);
+        HCCLX_LAUNCH((k_copy_blocks<4>), dim3(grid), dim3(kThreads), 0, stream, blocks, nblocks);
     }
     return hipGetLastError();
 }
@@ -307,14 +307,14 @@ __global__ void __launch_bounds__(kThreads) k_phased_copy_inline(PhasedInline ta
 
 hipError_t launch_phased_copy_inline(const PhasedInline &tab, uint32_t njobs, uint32_t slots, uint32_t nd, hipStream_t stream)
 {
-    hipLaunchKernelGGL(k_phased_copy_inline, dim3(slots * nd, njobs), dim3(kThreads), 0, stream, tab, slots, nd);
+    HCCLX_LAUNCH(k_phased_copy_inline, dim3(slots * nd, njobs), dim3(kThreads), 0, stream, tab, slots, nd);
     return hipGetLastError();
 }
 
 hipError_t launch_phased_copy(const PhasedJob *jobs, char *const *dsts, uint32_t njobs, uint32_t slots, uint32_t nd,
                               hipStream_t stream)
 {
-    hipLaunchKernelGGL(k_phased_copy, dim3(slots * nd, njobs), dim3(kThreads), 0, stream, jobs, dsts, slots, nd);
+    HCCLX_LAUNCH(k_phased_copy, dim3(slots * nd, njobs), dim3(kThreads), 0, stream, jobs, dsts, slots, nd);
     return hipGetLastError();
 }
 
@@ -322,11 +322,11 @@ hipError_t launch_alltoallv_direct(const VRankPtrs16 &ptrs, const A2avTablesDire
                                    uint32_t grid, int unroll, hipStream_t stream)
 {
     if (unroll == 1) {
-        hipLaunchKernelGGL((k_alltoallv_direct<1>), dim3(grid), dim3(kThreads), 0, stream, ptrs, tabs, n, esz);
+        HCCLX_LAUNCH((k_alltoallv_direct<1>), dim3(grid), dim3(kThreads), 0, stream, ptrs, tabs, n, esz);
     } else if (unroll == 2) {
-        hipLaunchKernelGGL((k_alltoallv_direct<2>), dim3(grid), dim3(kThreads), 0, stream, ptrs, tabs, n, esz);
+        HCCLX_LAUNCH((k_alltoallv_direct<2>), dim3(grid), dim3(kThreads), 0, stream, ptrs, tabs, n, esz);
     } else {
-        hipLaunchKernelGGL((k_alltoallv_direct<4>), dim3(grid), dim3(kThreads), 0, stream, ptrs, tabs, n, esz);
+        HCCLX_LAUNCH((k_alltoallv_direct<4>), dim3(grid), dim3(kThreads), 0, stream, ptrs, tabs, n, esz);
     }
     return hipGetLastError();
 }
@@ -347,7 +347,7 @@ k_displs_from_counts(const uint64_t *__restrict__ counts, uint32_t n, uint64_t *
 hipError_t launch_displs_from_counts(const uint64_t *counts, uint32_t rows, uint32_t n, uint64_t *displs, uint64_t *totals,
                                      hipStream_t stream)
 {
-    hipLaunchKernelGGL(k_displs_from_counts, dim3(rows), dim3(64), 0, stream, counts, n, displs, totals);
+    HCCLX_LAUNCH(k_displs_from_counts, dim3(rows), dim3(64), 0, stream, counts, n, displs, totals);
     return hipGetLastError();
 }
 
@@ -356,7 +356,7 @@ hipError_t launch_allgatherv(const VRankPtrs &ptrs, const uint64_t *counts, cons
 {
     const size_t lds = (static_cast<size_t>(n) + 4) * sizeof(uint64_t);
     const AgvTablesPtr tabs{counts, displs};
-    hipLaunchKernelGGL((k_allgatherv<AgvTablesPtr>), dim3(grid), dim3(kThreads), lds, stream, ptrs, tabs, n, esz,
+    HCCLX_LAUNCH((k_allgatherv<AgvTablesPtr>), dim3(grid), dim3(kThreads), lds, stream, ptrs, tabs, n, esz,
                        tiles_per_block);
     return hipGetLastError();
 }
@@ -365,7 +365,7 @@ hipError_t launch_allgatherv_inline(const VRankPtrs &ptrs, const AgvTablesInline
                                     uint32_t grid, uint32_t tiles_per_block, hipStream_t stream)
 {
     const size_t lds = (static_cast<size_t>(n) + 4) * sizeof(uint64_t);
-    hipLaunchKernelGGL((k_allgatherv<AgvTablesInline>), dim3(grid), dim3(kThreads), lds, stream, ptrs, tabs, n, esz,
+    HCCLX_LAUNCH((k_allgatherv<AgvTablesInline>), dim3(grid), dim3(kThreads), lds, stream, ptrs, tabs, n, esz,
                        tiles_per_block);
     return hipGetLastError();
 }

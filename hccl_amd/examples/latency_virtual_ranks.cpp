@@ -1,6 +1,7 @@
 // Time per warm HcclAllReduce for small messages, from C++: one host thread issues every rank's call, no HIP graph.
-// Cases: 8 ranks fp32 SUM with the selector's choice, and 12 ranks int32 MAX / fp32 PROD through the NHR,
-// halving-doubling and CPU-reduce NHR templates.
+// Cases: 8 ranks fp32 SUM with the selector's choice and through the ring template, 4 KiB ... 4 MiB per rank (the
+// largest is the 8 x 1,048,576-element AllReduce), and 12 ranks int32 MAX / fp32 PROD through the NHR,
+// halving-doubling and CPU-reduce NHR templates, 4 KiB ... 1 MiB per rank.
 // Prints one JSON object: per (case, bytes per rank) the microseconds per collective on the GPU timeline
 // ("us": events around `reps` collectives, i.e. the sustained rate) and the host time spent issuing one collective
 // ("host_us": all ranks' calls, nothing waited for).
@@ -41,7 +42,6 @@ int main(int argc, char **argv)
         std::fprintf(stderr, "usage: %s [reps > 0]\n", argv[0]);
         return 2;
     }
-    const size_t max_bytes = 1u << 20;
     hipStream_t stream;
     CHECK_HIP(hipStreamCreate(&stream));
     hipEvent_t t0, t1;
@@ -53,19 +53,22 @@ int main(int argc, char **argv)
         HcclDataType dtype;
         HcclReduceOp op;
         const char *alg;   // nullptr: the selector decides
+        size_t max_bytes;
     };
     const Case cases[] = {
-        {"fp32_sum_default", 8, HCCL_DATA_TYPE_FP32, HCCL_REDUCE_SUM, nullptr},
-        {"fp32_sum_default", 12, HCCL_DATA_TYPE_FP32, HCCL_REDUCE_SUM, nullptr},
-        {"int32_max_nhr", 12, HCCL_DATA_TYPE_INT32, HCCL_REDUCE_MAX, "InsAllReduceNHR"},
-        {"int32_max_rhd", 12, HCCL_DATA_TYPE_INT32, HCCL_REDUCE_MAX, "InsAllReduceRHD"},
-        {"fp32_prod_aicpu_nhr", 12, HCCL_DATA_TYPE_FP32, HCCL_REDUCE_PROD, "InsAllReduceAicpuReduceNHR"},
-        {"fp32_prod_rhd", 12, HCCL_DATA_TYPE_FP32, HCCL_REDUCE_PROD, "InsAllReduceRHD"},
+        {"fp32_sum_default", 8, HCCL_DATA_TYPE_FP32, HCCL_REDUCE_SUM, nullptr, 4u << 20},
+        {"fp32_sum_ring", 8, HCCL_DATA_TYPE_FP32, HCCL_REDUCE_SUM, "InsAllReduceRing", 4u << 20},
+        {"fp32_sum_default", 12, HCCL_DATA_TYPE_FP32, HCCL_REDUCE_SUM, nullptr, 1u << 20},
+        {"int32_max_nhr", 12, HCCL_DATA_TYPE_INT32, HCCL_REDUCE_MAX, "InsAllReduceNHR", 1u << 20},
+        {"int32_max_rhd", 12, HCCL_DATA_TYPE_INT32, HCCL_REDUCE_MAX, "InsAllReduceRHD", 1u << 20},
+        {"fp32_prod_aicpu_nhr", 12, HCCL_DATA_TYPE_FP32, HCCL_REDUCE_PROD, "InsAllReduceAicpuReduceNHR", 1u << 20},
+        {"fp32_prod_rhd", 12, HCCL_DATA_TYPE_FP32, HCCL_REDUCE_PROD, "InsAllReduceRHD", 1u << 20},
     };
     std::printf("{\"reps\": %d, \"op\": \"HcclAllReduce\", \"rows\": [", reps);
     bool first = true;
     for (const Case &c : cases) {
         const uint32_t n = c.ranks;
+        const size_t max_bytes = c.max_bytes;
         std::vector<HcclComm> comm(n);
         CHECK_HCCL(HcclCommInitAll(n, nullptr, comm.data()));
         if (c.alg) CHECK_HCCL(hcclxCommSetAlgorithm(comm[0], HCCLX_CMD_ALLREDUCE, c.alg));

@@ -43,3 +43,12 @@ _SIZES = [1, 2, 4, 2, 4, 8, 8, 1, 2, 4, 8, 2, 16, 2, 1, 1, 1, 1]
 
 def dtype_size(dt):
     return _SIZES[int(dt)]
+
+
+# the enumerators under their short names, so that `from hccl_amd import types as T; T.BFP16, T.SUM` reads like the
+# C header's HCCL_DATA_TYPE_BFP16 / HCCL_REDUCE_SUM
+INT8, INT16, INT32, FP16, FP32, INT64, UINT64, UINT8, UINT16, UINT32, FP64, BFP16, INT128 = (
+    int(DataType.INT8), int(DataType.INT16), int(DataType.INT32), int(DataType.FP16), int(DataType.FP32),
+    int(DataType.INT64), int(DataType.UINT64), int(DataType.UINT8), int(DataType.UINT16), int(DataType.UINT32),
+    int(DataType.FP64), int(DataType.BFP16), int(DataType.INT128))
+SUM, PROD, MAX, MIN = int(ReduceOp.SUM), int(ReduceOp.PROD), int(ReduceOp.MAX), int(ReduceOp.MIN)

@@ -61,7 +61,8 @@ HcclResult hcclxCommSetTopo(HcclComm comm, uint32_t levels, int level0Shape, uin
 typedef struct {
     char algName[64];
     uint32_t levels;        /* dependency levels of the recorded schedule */
-    uint32_t launches;      /* kernel launches made */
+    uint32_t launches;      /* GPU kernels the collective launched (a fold whose result fans out to many
+                               places is two: the fold, then the copy to the other outputs) */
     uint32_t fusedSegments; /* segments of the fused plan */
     int fused;              /* 1 = ran as fused passes, 0 = step by step */
     int planCacheHit;

@@ -87,6 +87,11 @@ int hcclx_init(void);
 /* Text of the last error raised on this thread ("" if none). */
 const char *hcclx_last_error(void);
 
+/* Number of GPU kernels the calling host thread has launched through this library so far (a running count; take
+ * the difference around a call to learn how many kernels it made -- a fold whose result fans out to many places is
+ * two, a large AllGatherV one per length class of its runs).  No counterpart in the reference. */
+uint64_t hcclx_kernels_launched(void);
+
 /* Size in bytes of an HcclDataType (0 if unknown).  DATATYPE_SIZE_TABLE, alg_param.h:43-45. */
 uint32_t hcclx_dtype_size(int dtype);
 
