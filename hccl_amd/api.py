@@ -11,6 +11,7 @@ CMD_ALLREDUCE, CMD_ALLGATHER, CMD_REDUCE_SCATTER, CMD_ALLTOALLV, CMD_ALLTOALLVC,
     2, 6, 7, 8, 9, 10, 16
 CMD_REDUCE_SCATTER_V = 17
 SHAPE_CLOS, SHAPE_MESH_1D = 0, 1
+LINK_HCCS, LINK_ROCE, LINK_PCIE = 0, 1, 2
 
 
 class LastOpInfo(ctypes.Structure):
@@ -42,6 +43,7 @@ def lib():
             "hcclxCommSetBlocking": [vp, ci],
             "hcclxCommSetAlgorithm": [vp, ci, ctypes.c_char_p],
             "hcclxCommSetTopo": [vp, u32, ci, u32],
+            "hcclxCommSetLinkProtocol": [vp, ci],
             "hcclxCommGetLastOpInfo": [vp, ctypes.POINTER(LastOpInfo)],
             "hcclxCommSetTrace": [vp, ci],
             "hcclxCommSetCheck": [vp, ci],
@@ -107,6 +109,10 @@ class World:
 
     def set_topo(self, levels=1, shape=SHAPE_MESH_1D, devices_per_server=0):
         check(lib().hcclxCommSetTopo(self.comms[0], levels, shape, devices_per_server))
+
+    def set_link_protocol(self, protocol):
+        """LINK_PCIE puts the templates that have a read mode into it (the receiver fetches); the values stay the same."""
+        check(lib().hcclxCommSetLinkProtocol(self.comms[0], int(protocol)))
 
     def set_trace(self, on):
         check(lib().hcclxCommSetTrace(self.comms[0], 1 if on else 0))

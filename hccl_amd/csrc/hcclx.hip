@@ -75,6 +75,17 @@ struct PlanStage {
     hipStream_t stream = nullptr;   // the copies run on a stream of their own: they order with nothing else
 };
 
+// Who used the fixed launch table of hcclx_fold_static last.  Calls on one stream follow each other by stream order;
+// a call on another stream first waits for the event recorded behind the previous call's fold kernel, so that the
+// table is never rewritten under a kernel that still reads it.  The event is made once per device: nothing is
+// allocated per call.
+struct StaticTableUse {
+    std::mutex mu;                  // one host thread at a time issues "upload the table, launch the fold"
+    hipEvent_t done = nullptr;      // recorded behind the last fold that read the table
+    hipStream_t last = nullptr;
+    bool recorded = false;
+};
+
 struct DeviceSlot {
     std::once_flag once;
     bool ok = false;
@@ -82,6 +93,7 @@ struct DeviceSlot {
     DeviceCtx ctx;
     Ring ring;
     PlanStage stage;
+    StaticTableUse static_use;
 };
 
 DeviceSlot g_slots[kMaxDevices];
@@ -116,7 +128,9 @@ void init_slot(DeviceSlot *s, int dev)
     }
     if (const char *v = std::getenv("HCCLX_FANOUT_FROM")) c.fanout_from = std::strtoull(v, nullptr, 10);
     if (const char *v = std::getenv("HCCLX_FANOUT_RUN")) {
-        const uint64_t b = std::strtoull(v, nullptr, 10);
+        // between 64 KiB and 1 GiB: a run is one job of a launch, and its tile count has to stay within the length
+        // classes the launches are grouped by
+        const uint64_t b = std::min<uint64_t>(std::strtoull(v, nullptr, 10), 1ull << 30);
         if (b >= 65536) c.fanout_run = b & ~static_cast<uint64_t>(4095);
     }
     if (const char *v = std::getenv("HCCLX_AGV_PHASED_FROM")) c.agv_phased_from = std::strtoull(v, nullptr, 10);
@@ -147,6 +161,11 @@ void init_slot(DeviceSlot *s, int dev)
     e = hipGetSymbolAddress(reinterpret_cast<void **>(&c.static_table), HIP_SYMBOL(scratch));
     if (e != hipSuccess || c.static_table == nullptr) {
         s->err = std::string("hipGetSymbolAddress(launch table): ") + hipGetErrorString(e);
+        return;
+    }
+    e = hipEventCreateWithFlags(&s->static_use.done, hipEventDisableTiming);
+    if (e != hipSuccess) {
+        s->err = std::string("hipEventCreate(launch table): ") + hipGetErrorString(e);
         return;
     }
     s->ok = true;
@@ -266,6 +285,7 @@ void build_phased(std::vector<PhasedStream> &streams, uint64_t run_bytes, std::v
     };
     // runs of equal length per stream, a multiple of the tile size; then launches by length class (powers of four)
     constexpr uint64_t kTile = 256ull * 16 * kPhasedUnroll;
+    run_bytes = std::min<uint64_t>(std::max<uint64_t>(run_bytes, kTile), 1ull << 30);   // every run falls into a class below
     std::vector<Run> runs;
     for (const PhasedStream &st : joined) {
         const uint64_t n = (st.bytes + run_bytes - 1) / run_bytes;
@@ -297,7 +317,7 @@ void build_phased(std::vector<PhasedStream> &streams, uint64_t run_bytes, std::v
         for (const Run &r : runs) {
             int c = 0;
             for (uint32_t t = r.tiles; t > 1; t = (t + 3) / 4) ++c;
-            if (c != cls) continue;
+            if (std::min(c, 15) != cls) continue;
             const uint32_t nd = static_cast<uint32_t>(r.st->dst.size());
             const uint64_t grid_x = (static_cast<uint64_t>(std::max(cur.slots, r.tiles)) + 7) * std::max(cur.nd, nd);
             if (cur.jobs.size() == kMaxJobs || grid_x > 0x7fffffffull ||
@@ -1083,6 +1103,22 @@ int hcclx_fold_static(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op,
     }
     if (total > 0x7fffffffull) return fail(HCCL_E_PARA, "too much data for one launch");
     hipStream_t st = static_cast<hipStream_t>(stream);
+    // One table per GPU: the upload and the fold of a call are issued as a unit, and a call on another stream than
+    // the previous one waits for that one's fold.  While `st` is being captured into a graph neither the wait nor
+    // the record is issued (an event recorded in a capture would draw every later waiter into that capture): the
+    // replays of a captured call are the caller's to order against other users of the table.
+    StaticTableUse &use = g_slots[ctx->device].static_use;
+    std::lock_guard<std::mutex> use_lock(use.mu);
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &capturing) != hipSuccess) {
+        (void)hipGetLastError();
+        capturing = hipStreamCaptureStatusNone;
+    }
+    const bool ordered = capturing == hipStreamCaptureStatusNone;
+    if (ordered && use.recorded && use.last != st) {
+        const hipError_t we = hipStreamWaitEvent(st, use.done, 0);
+        if (we != hipSuccess) return fail_hip(we, "hipStreamWaitEvent(launch table)");
+    }
     // the table travels in kernel arguments, piece by piece; the fold kernel follows on the same stream
     for (size_t off = 0; off < bytes; off += kPutBytes) {
         TablePiece piece;
@@ -1110,6 +1146,12 @@ int hcclx_fold_static(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op,
         e = dispatch_fold(dtype, op, sp.maxn, sp.mode, l);
     }
     if (e != hipSuccess) return fail_hip(e, "fold kernel launch");
+    if (ordered) {
+        e = hipEventRecord(use.done, st);
+        if (e != hipSuccess) return fail_hip(e, "hipEventRecord(launch table)");
+        use.last = st;
+        use.recorded = true;
+    }
     return HCCL_SUCCESS;
 }
 

@@ -1,5 +1,7 @@
 #include "alg_data_trans_wrapper.h"
 
+#include <cstdlib>
+
 #include "hcomm_primitives.h"
 
 namespace ops_hccl {
@@ -8,6 +10,30 @@ namespace {
 constexpr u32 kTimeout = CUSTOM_TIMEOUT;
 
 HcclResult R(int32_t rc) { return static_cast<HcclResult>(rc); }
+
+// Every wait of a verb takes the process-wide time-out when the backend exports the *WithDefaultTimeout form and
+// falls back to the explicit one otherwise (wrapper.cc:22-31 over hcomm_primitives_dl.cc:155-173).  This backend
+// exports both; HCCL_VRANK_NO_DEFAULT_TIMEOUT=1 takes the fallback, so that both routes stay exercised.
+bool UseDefaultTimeout()
+{
+    static const bool on = [] {
+        const char *v = std::getenv("HCCL_VRANK_NO_DEFAULT_TIMEOUT");
+        return !(v != nullptr && v[0] == '1');
+    }();
+    return on;
+}
+
+HcclResult WaitChannel(const ThreadHandle &thread, const ChannelInfo &ch, u32 idx)
+{
+    if (UseDefaultTimeout()) return R(HcommChannelNotifyWaitOnThreadWithDefaultTimeout(thread, ch.handle, idx));
+    return R(HcommChannelNotifyWaitOnThread(thread, ch.handle, idx, kTimeout));
+}
+
+HcclResult WaitThread(const ThreadHandle &thread, u32 idx)
+{
+    if (UseDefaultTimeout()) return R(HcommThreadNotifyWaitOnThreadWithDefaultTimeout(thread, idx));
+    return R(HcommThreadNotifyWaitOnThread(thread, idx, kTimeout));
+}
 
 // LocalReduce routes 64-bit types and PROD to the CPU loop AicpuReduce, everything else to the inline
 // reduce of the transport (wrapper.cc:837-841).  Both are the same fold kernel here, so the two routes
@@ -54,18 +80,25 @@ HcclResult LocalCopy(const ThreadHandle &thread, const DataSlice &srcSlice, cons
 HcclResult LocalReduce(const ThreadHandle &thread, const DataSlice &srcSlice, const DataSlice &dstSlice,
                        HcclDataType dataType, HcclReduceOp reduceOp)
 {
-    if (NeedsAicpuReduce(dataType, reduceOp)) {
-        CHK_PRT_RET(srcSlice.size_ != dstSlice.size_, HCCL_ERROR("AicpuReduce: slice sizes differ"), HCCL_E_INTERNAL);
-        CHK_PRT_RET(!AicpuReduceSupports(dataType), HCCL_ERROR("AicpuReduce: DataType[%d] not support", dataType),
-                    HCCL_E_INTERNAL);
-        const u64 count = srcSlice.size_ / DATATYPE_SIZE_TABLE[dataType];
-        return R(HcommLocalReduceOnThread(thread, GetSliceAddr(dstSlice), GetSliceAddr(srcSlice), count, dataType,
-                                          reduceOp));
-    }
+    if (NeedsAicpuReduce(dataType, reduceOp)) return AicpuReduce(thread, srcSlice, dstSlice, dataType, reduceOp);
     if (srcSlice.size_ == 0) return HCCL_SUCCESS;
     CHK_PRT_RET(srcSlice.size_ != dstSlice.size_, HCCL_ERROR("LocalReduce: slice sizes differ"), HCCL_E_INTERNAL);
     return R(HcommLocalReduceOnThread(thread, GetSliceAddr(dstSlice), GetSliceAddr(srcSlice), srcSlice.count_,
                                       dataType, reduceOp));
+}
+
+// The CPU reduce of the reference (wrapper.cc:1165-1210): equal byte sizes, seven element types, anything else is
+// HCCL_E_INTERNAL.  The reference runs the loop on the host at once and ignores `thread`; here the step is recorded
+// on `thread` like every other reduce and becomes part of the launch.
+HcclResult AicpuReduce(const ThreadHandle &thread, const DataSlice &srcSlice, const DataSlice &dstSlice,
+                       HcclDataType dataType, HcclReduceOp reduceOp)
+{
+    CHK_PRT_RET(srcSlice.size_ != dstSlice.size_, HCCL_ERROR("AicpuReduce: slice sizes differ"), HCCL_E_INTERNAL);
+    CHK_PRT_RET(!AicpuReduceSupports(dataType), HCCL_ERROR("AicpuReduce: DataType[%d] not support", dataType),
+                HCCL_E_INTERNAL);
+    const u64 count = srcSlice.size_ / DATATYPE_SIZE_TABLE[dataType];
+    return R(HcommLocalReduceOnThread(thread, GetSliceAddr(dstSlice), GetSliceAddr(srcSlice), count, dataType,
+                                      reduceOp));
 }
 
 bool IsContinuousSlice(const DataSlice &nxtSlice, const DataSlice &currSlice)
@@ -104,7 +137,7 @@ HcclResult LocalCopySlices(const ThreadHandle &thread, const std::vector<DataSli
 HcclResult SendWrite(const DataInfo &sendInfo, const ThreadHandle &thread)
 {
     const ChannelInfo &ch = sendInfo.channel_;
-    CHK_RET(HcommChannelNotifyWaitOnThread(thread, ch.handle, NOTIFY_IDX_ACK, kTimeout));
+    CHK_RET(WaitChannel(thread, ch, NOTIFY_IDX_ACK));
     for (size_t i = 0; i < sendInfo.slices_.srcSlices_.size(); ++i) {
         const DataSlice &s = sendInfo.slices_.srcSlices_[i];
         const DataSlice &d = sendInfo.slices_.dstSlices_[i];
@@ -118,7 +151,7 @@ HcclResult RecvWrite(const DataInfo &recvInfo, const ThreadHandle &thread)
 {
     const ChannelInfo &ch = recvInfo.channel_;
     CHK_RET(HcommChannelNotifyRecordOnThread(thread, ch.handle, NOTIFY_IDX_ACK));
-    return R(HcommChannelNotifyWaitOnThread(thread, ch.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+    return WaitChannel(thread, ch, NOTIFY_IDX_DATA_SIGNAL);
 }
 
 HcclResult SendRecvWrite(const SendRecvInfo &info, const ThreadHandle &thread)
@@ -128,13 +161,13 @@ HcclResult SendRecvWrite(const SendRecvInfo &info, const ThreadHandle &thread)
     const ChannelInfo &tx = info.sendRecvChannels_.txChannel_;
     const ChannelInfo &rx = info.sendRecvChannels_.rxChannel_;
     CHK_RET(HcommChannelNotifyRecordOnThread(thread, rx.handle, NOTIFY_IDX_ACK));
-    CHK_RET(HcommChannelNotifyWaitOnThread(thread, tx.handle, NOTIFY_IDX_ACK, kTimeout));
+    CHK_RET(WaitChannel(thread, tx, NOTIFY_IDX_ACK));
     for (size_t i = 0; i < src.size(); ++i) {
         if (src[i].size_ == 0) continue;
         CHK_RET(HcommWriteOnThread(thread, tx.handle, GetSliceAddr(dst[i]), GetSliceAddr(src[i]), src[i].size_));
     }
     CHK_RET(HcommChannelNotifyRecordOnThread(thread, tx.handle, NOTIFY_IDX_DATA_SIGNAL));
-    return R(HcommChannelNotifyWaitOnThread(thread, rx.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+    return WaitChannel(thread, rx, NOTIFY_IDX_DATA_SIGNAL);
 }
 
 HcclResult SendRecvWriteReduce(const SendRecvReduceInfo &info, const ThreadHandle &thread)
@@ -144,7 +177,7 @@ HcclResult SendRecvWriteReduce(const SendRecvReduceInfo &info, const ThreadHandl
     const ChannelInfo &tx = info.sendRecvChannels_.txChannel_;
     const ChannelInfo &rx = info.sendRecvChannels_.rxChannel_;
     CHK_RET(HcommChannelNotifyRecordOnThread(thread, rx.handle, NOTIFY_IDX_ACK));
-    CHK_RET(HcommChannelNotifyWaitOnThread(thread, tx.handle, NOTIFY_IDX_ACK, kTimeout));
+    CHK_RET(WaitChannel(thread, tx, NOTIFY_IDX_ACK));
     for (size_t i = 0; i < src.size(); ++i) {
         if (src[i].size_ == 0) continue;
         CHK_RET(CheckReduceSlices(src[i], dst[i], info.dataType_));
@@ -152,22 +185,70 @@ HcclResult SendRecvWriteReduce(const SendRecvReduceInfo &info, const ThreadHandl
                                          info.dataType_, info.reduceType_));
     }
     CHK_RET(HcommChannelNotifyRecordOnThread(thread, tx.handle, NOTIFY_IDX_DATA_SIGNAL));
-    return R(HcommChannelNotifyWaitOnThread(thread, rx.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+    return WaitChannel(thread, rx, NOTIFY_IDX_DATA_SIGNAL);
+}
+
+// One side of SendRecvWriteReduce each: the sender waits for the receiver's ACK, write-reduces its slices into the
+// receiver's buffer and signals; the receiver only shakes hands (wrapper.cc:389-435, :468-477).
+HcclResult SendWriteReduce(const DataReduceInfo &sendInfo, const ThreadHandle &thread)
+{
+    const ChannelInfo &ch = sendInfo.channel_;
+    CHK_RET(WaitChannel(thread, ch, NOTIFY_IDX_ACK));
+    for (size_t i = 0; i < sendInfo.slices_.srcSlices_.size(); ++i) {
+        const DataSlice &s = sendInfo.slices_.srcSlices_[i];
+        const DataSlice &d = sendInfo.slices_.dstSlices_[i];
+        if (s.size_ == 0) continue;
+        CHK_RET(CheckReduceSlices(s, d, sendInfo.dataType_));
+        CHK_RET(HcommWriteReduceOnThread(thread, ch.handle, GetSliceAddr(d), GetSliceAddr(s), s.count_, sendInfo.dataType_,
+                                         sendInfo.reduceType_));
+    }
+    return R(HcommChannelNotifyRecordOnThread(thread, ch.handle, NOTIFY_IDX_DATA_SIGNAL));
+}
+
+HcclResult RecvWriteReduce(const DataReduceInfo &recvInfo, const ThreadHandle &thread)
+{
+    const ChannelInfo &ch = recvInfo.channel_;
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, ch.handle, NOTIFY_IDX_ACK));
+    return WaitChannel(thread, ch, NOTIFY_IDX_DATA_SIGNAL);
 }
 
 // ---- read family: the owner says "my data is ready" (ACK), the reader reads and says "I am done"
+
+// One side of SendRecvReadReduce each: the owner of the data announces it and waits until it has been read; the
+// reader read-reduces the owner's slices into its own buffer (wrapper.cc:638-695).
+HcclResult SendReadReduce(const DataReduceInfo &sendInfo, const ThreadHandle &thread)
+{
+    const ChannelInfo &ch = sendInfo.channel_;
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, ch.handle, NOTIFY_IDX_ACK));
+    return WaitChannel(thread, ch, NOTIFY_IDX_DATA_SIGNAL);
+}
+
+HcclResult RecvReadReduce(const DataReduceInfo &recvInfo, const ThreadHandle &thread)
+{
+    const ChannelInfo &ch = recvInfo.channel_;
+    CHK_RET(WaitChannel(thread, ch, NOTIFY_IDX_ACK));
+    for (size_t i = 0; i < recvInfo.slices_.srcSlices_.size(); ++i) {
+        const DataSlice &s = recvInfo.slices_.srcSlices_[i];
+        const DataSlice &d = recvInfo.slices_.dstSlices_[i];
+        if (s.size_ == 0) continue;
+        CHK_RET(CheckReduceSlices(s, d, recvInfo.dataType_));
+        CHK_RET(HcommReadReduceOnThread(thread, ch.handle, GetSliceAddr(d), GetSliceAddr(s), s.count_, recvInfo.dataType_,
+                                        recvInfo.reduceType_));
+    }
+    return R(HcommChannelNotifyRecordOnThread(thread, ch.handle, NOTIFY_IDX_DATA_SIGNAL));
+}
 
 HcclResult SendRead(const DataInfo &sendInfo, const ThreadHandle &thread)
 {
     const ChannelInfo &ch = sendInfo.channel_;
     CHK_RET(HcommChannelNotifyRecordOnThread(thread, ch.handle, NOTIFY_IDX_ACK));
-    return R(HcommChannelNotifyWaitOnThread(thread, ch.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+    return WaitChannel(thread, ch, NOTIFY_IDX_DATA_SIGNAL);
 }
 
 HcclResult RecvRead(const DataInfo &recvInfo, const ThreadHandle &thread)
 {
     const ChannelInfo &ch = recvInfo.channel_;
-    CHK_RET(HcommChannelNotifyWaitOnThread(thread, ch.handle, NOTIFY_IDX_ACK, kTimeout));
+    CHK_RET(WaitChannel(thread, ch, NOTIFY_IDX_ACK));
     for (size_t i = 0; i < recvInfo.slices_.srcSlices_.size(); ++i) {
         const DataSlice &s = recvInfo.slices_.srcSlices_[i];
         const DataSlice &d = recvInfo.slices_.dstSlices_[i];
@@ -184,13 +265,13 @@ HcclResult SendRecvRead(const SendRecvInfo &info, const ThreadHandle &thread)
     const ChannelInfo &tx = info.sendRecvChannels_.txChannel_;
     const ChannelInfo &rx = info.sendRecvChannels_.rxChannel_;
     CHK_RET(HcommChannelNotifyRecordOnThread(thread, tx.handle, NOTIFY_IDX_ACK));
-    CHK_RET(HcommChannelNotifyWaitOnThread(thread, rx.handle, NOTIFY_IDX_ACK, kTimeout));
+    CHK_RET(WaitChannel(thread, rx, NOTIFY_IDX_ACK));
     for (size_t i = 0; i < src.size(); ++i) {
         if (src[i].size_ == 0) continue;
         CHK_RET(HcommReadOnThread(thread, rx.handle, GetSliceAddr(dst[i]), GetSliceAddr(src[i]), src[i].size_));
     }
     CHK_RET(HcommChannelNotifyRecordOnThread(thread, rx.handle, NOTIFY_IDX_DATA_SIGNAL));
-    return R(HcommChannelNotifyWaitOnThread(thread, tx.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+    return WaitChannel(thread, tx, NOTIFY_IDX_DATA_SIGNAL);
 }
 
 HcclResult SendRecvReadReduce(const SendRecvReduceInfo &info, const ThreadHandle &thread)
@@ -200,7 +281,7 @@ HcclResult SendRecvReadReduce(const SendRecvReduceInfo &info, const ThreadHandle
     const ChannelInfo &tx = info.sendRecvChannels_.txChannel_;
     const ChannelInfo &rx = info.sendRecvChannels_.rxChannel_;
     CHK_RET(HcommChannelNotifyRecordOnThread(thread, tx.handle, NOTIFY_IDX_ACK));
-    CHK_RET(HcommChannelNotifyWaitOnThread(thread, rx.handle, NOTIFY_IDX_ACK, kTimeout));
+    CHK_RET(WaitChannel(thread, rx, NOTIFY_IDX_ACK));
     for (size_t i = 0; i < src.size(); ++i) {
         if (src[i].size_ == 0) continue;
         CHK_RET(CheckReduceSlices(src[i], dst[i], info.dataType_));
@@ -208,7 +289,7 @@ HcclResult SendRecvReadReduce(const SendRecvReduceInfo &info, const ThreadHandle
                                         info.dataType_, info.reduceType_));
     }
     CHK_RET(HcommChannelNotifyRecordOnThread(thread, rx.handle, NOTIFY_IDX_DATA_SIGNAL));
-    return R(HcommChannelNotifyWaitOnThread(thread, tx.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+    return WaitChannel(thread, tx, NOTIFY_IDX_DATA_SIGNAL);
 }
 
 // ---- batch verbs: every slice of the call in one descriptor array (wrapper.cc:99-125), between the handshakes of
@@ -248,7 +329,7 @@ HcclResult RunBatch(const ThreadHandle &thread, const ChannelInfo &ch, const std
 HcclResult SendBatchWrite(const DataInfo &sendInfo, const ThreadHandle &thread)
 {
     const ChannelInfo &ch = sendInfo.channel_;
-    CHK_RET(HcommChannelNotifyWaitOnThread(thread, ch.handle, NOTIFY_IDX_ACK, kTimeout));
+    CHK_RET(WaitChannel(thread, ch, NOTIFY_IDX_ACK));
     CHK_RET(RunBatch(thread, ch, sendInfo.slices_.srcSlices_, sendInfo.slices_.dstSlices_, HCCL_HCOMM_TRANSFER_TYPE_WRITE,
                      false, HCCL_DATA_TYPE_INT8, HCCL_REDUCE_SUM));
     return R(HcommChannelNotifyRecordOnThread(thread, ch.handle, NOTIFY_IDX_DATA_SIGNAL));
@@ -259,11 +340,11 @@ HcclResult SendRecvBatchWrite(const SendRecvInfo &info, const ThreadHandle &thre
     const ChannelInfo &tx = info.sendRecvChannels_.txChannel_;
     const ChannelInfo &rx = info.sendRecvChannels_.rxChannel_;
     CHK_RET(HcommChannelNotifyRecordOnThread(thread, rx.handle, NOTIFY_IDX_ACK));
-    CHK_RET(HcommChannelNotifyWaitOnThread(thread, tx.handle, NOTIFY_IDX_ACK, kTimeout));
+    CHK_RET(WaitChannel(thread, tx, NOTIFY_IDX_ACK));
     CHK_RET(RunBatch(thread, tx, info.sendRecvSlices_.txSlicesList_.srcSlices_, info.sendRecvSlices_.txSlicesList_.dstSlices_,
                      HCCL_HCOMM_TRANSFER_TYPE_WRITE, false, HCCL_DATA_TYPE_INT8, HCCL_REDUCE_SUM));
     CHK_RET(HcommChannelNotifyRecordOnThread(thread, tx.handle, NOTIFY_IDX_DATA_SIGNAL));
-    return R(HcommChannelNotifyWaitOnThread(thread, rx.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+    return WaitChannel(thread, rx, NOTIFY_IDX_DATA_SIGNAL);
 }
 
 HcclResult SendRecvBatchWriteReduce(const SendRecvReduceInfo &info, const ThreadHandle &thread)
@@ -271,17 +352,17 @@ HcclResult SendRecvBatchWriteReduce(const SendRecvReduceInfo &info, const Thread
     const ChannelInfo &tx = info.sendRecvChannels_.txChannel_;
     const ChannelInfo &rx = info.sendRecvChannels_.rxChannel_;
     CHK_RET(HcommChannelNotifyRecordOnThread(thread, rx.handle, NOTIFY_IDX_ACK));
-    CHK_RET(HcommChannelNotifyWaitOnThread(thread, tx.handle, NOTIFY_IDX_ACK, kTimeout));
+    CHK_RET(WaitChannel(thread, tx, NOTIFY_IDX_ACK));
     CHK_RET(RunBatch(thread, tx, info.sendRecvSlices_.txSlicesList_.srcSlices_, info.sendRecvSlices_.txSlicesList_.dstSlices_,
                      HCCL_HCOMM_TRANSFER_TYPE_WRITE_REDUCE, true, info.dataType_, info.reduceType_));
     CHK_RET(HcommChannelNotifyRecordOnThread(thread, tx.handle, NOTIFY_IDX_DATA_SIGNAL));
-    return R(HcommChannelNotifyWaitOnThread(thread, rx.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+    return WaitChannel(thread, rx, NOTIFY_IDX_DATA_SIGNAL);
 }
 
 HcclResult RecvBatchRead(const DataInfo &recvInfo, const ThreadHandle &thread)
 {
     const ChannelInfo &ch = recvInfo.channel_;
-    CHK_RET(HcommChannelNotifyWaitOnThread(thread, ch.handle, NOTIFY_IDX_ACK, kTimeout));
+    CHK_RET(WaitChannel(thread, ch, NOTIFY_IDX_ACK));
     CHK_RET(RunBatch(thread, ch, recvInfo.slices_.srcSlices_, recvInfo.slices_.dstSlices_, HCCL_HCOMM_TRANSFER_TYPE_READ,
                      false, HCCL_DATA_TYPE_INT8, HCCL_REDUCE_SUM));
     return R(HcommChannelNotifyRecordOnThread(thread, ch.handle, NOTIFY_IDX_DATA_SIGNAL));
@@ -292,12 +373,48 @@ HcclResult SendRecvBatchRead(const SendRecvInfo &info, const ThreadHandle &threa
     const ChannelInfo &tx = info.sendRecvChannels_.txChannel_;
     const ChannelInfo &rx = info.sendRecvChannels_.rxChannel_;
     CHK_RET(HcommChannelNotifyRecordOnThread(thread, tx.handle, NOTIFY_IDX_ACK));
-    CHK_RET(HcommChannelNotifyWaitOnThread(thread, rx.handle, NOTIFY_IDX_ACK, kTimeout));
+    CHK_RET(WaitChannel(thread, rx, NOTIFY_IDX_ACK));
     CHK_RET(RunBatch(thread, rx, info.sendRecvSlices_.rxSlicesList_.srcSlices_, info.sendRecvSlices_.rxSlicesList_.dstSlices_,
                      HCCL_HCOMM_TRANSFER_TYPE_READ, false, HCCL_DATA_TYPE_INT8, HCCL_REDUCE_SUM));
     CHK_RET(HcommChannelNotifyRecordOnThread(thread, rx.handle, NOTIFY_IDX_DATA_SIGNAL));
-    return R(HcommChannelNotifyWaitOnThread(thread, tx.handle, NOTIFY_IDX_DATA_SIGNAL, kTimeout));
+    return WaitChannel(thread, tx, NOTIFY_IDX_DATA_SIGNAL);
 }
+
+// The one-sided reduce verbs and the two-sided read-reduce in their batch form (wrapper.cc:437-466, :697-726,
+// :784-813): the same handshakes around one descriptor array.
+HcclResult SendBatchWriteReduce(const DataReduceInfo &sendInfo, const ThreadHandle &thread)
+{
+    const ChannelInfo &ch = sendInfo.channel_;
+    CHK_RET(WaitChannel(thread, ch, NOTIFY_IDX_ACK));
+    CHK_RET(RunBatch(thread, ch, sendInfo.slices_.srcSlices_, sendInfo.slices_.dstSlices_,
+                     HCCL_HCOMM_TRANSFER_TYPE_WRITE_REDUCE, true, sendInfo.dataType_, sendInfo.reduceType_));
+    return R(HcommChannelNotifyRecordOnThread(thread, ch.handle, NOTIFY_IDX_DATA_SIGNAL));
+}
+
+HcclResult RecvBatchReadReduce(const DataReduceInfo &recvInfo, const ThreadHandle &thread)
+{
+    const ChannelInfo &ch = recvInfo.channel_;
+    CHK_RET(WaitChannel(thread, ch, NOTIFY_IDX_ACK));
+    CHK_RET(RunBatch(thread, ch, recvInfo.slices_.srcSlices_, recvInfo.slices_.dstSlices_,
+                     HCCL_HCOMM_TRANSFER_TYPE_READ_REDUCE, true, recvInfo.dataType_, recvInfo.reduceType_));
+    return R(HcommChannelNotifyRecordOnThread(thread, ch.handle, NOTIFY_IDX_DATA_SIGNAL));
+}
+
+HcclResult SendRecvBatchReadReduce(const SendRecvReduceInfo &info, const ThreadHandle &thread)
+{
+    const ChannelInfo &tx = info.sendRecvChannels_.txChannel_;
+    const ChannelInfo &rx = info.sendRecvChannels_.rxChannel_;
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, tx.handle, NOTIFY_IDX_ACK));
+    CHK_RET(WaitChannel(thread, rx, NOTIFY_IDX_ACK));
+    CHK_RET(RunBatch(thread, rx, info.sendRecvSlices_.rxSlicesList_.srcSlices_, info.sendRecvSlices_.rxSlicesList_.dstSlices_,
+                     HCCL_HCOMM_TRANSFER_TYPE_READ_REDUCE, true, info.dataType_, info.reduceType_));
+    CHK_RET(HcommChannelNotifyRecordOnThread(thread, rx.handle, NOTIFY_IDX_DATA_SIGNAL));
+    return WaitChannel(thread, tx, NOTIFY_IDX_DATA_SIGNAL);
+}
+
+// Whether HcommBatchTransferOnThread is there (wrapper.cc:244-247; in the reference the answer comes from dlsym):
+// this backend always has it.
+bool IsHcommBatchTransferOnThreadSupported() { return true; }
 
 // ---- main thread <-> sub threads
 
@@ -312,7 +429,7 @@ HcclResult PreSyncInterThreads(const ThreadHandle &mainThread, const std::vector
         CHK_RET(HcommThreadNotifyRecordOnThread(mainThread, subThreads[i], notifyIdxMainToSub[i]));
     }
     for (size_t i = 0; i < subThreads.size(); ++i) {
-        CHK_RET(HcommThreadNotifyWaitOnThread(subThreads[i], notifyIdxMainToSub[i], kTimeout));
+        CHK_RET(WaitThread(subThreads[i], notifyIdxMainToSub[i]));
     }
     return HCCL_SUCCESS;
 }
@@ -325,7 +442,7 @@ HcclResult PostSyncInterThreads(const ThreadHandle &mainThread, const std::vecto
     CHK_PRT_RET(subThreads.size() != notifyIdxSubToMain.size(), HCCL_ERROR("PostSyncInterThreads: size mismatch"),
                 HCCL_E_INTERNAL);
     for (size_t i = 0; i < subThreads.size(); ++i) {
-        CHK_RET(HcommThreadNotifyWaitOnThread(mainThread, notifyIdxSubToMain[i], kTimeout));
+        CHK_RET(WaitThread(mainThread, notifyIdxSubToMain[i]));
     }
     for (size_t i = 0; i < subThreads.size(); ++i) {
         CHK_RET(HcommThreadNotifyRecordOnThread(subThreads[i], mainThread, notifyIdxSubToMain[i]));

@@ -18,9 +18,21 @@ struct HcclMem {
     u64 size = 0;
 };
 
+// What a link is made of.  The reference takes the enumeration from the transport library; the templates only ask
+// one question of it: a PCIe link is driven in read mode (the receiver fetches), every other one in write mode
+// (src/ops/op_common/template/alg_v2_template_base.cc:91-101).
+enum class CommProtocol : u32 {
+    COMM_PROTOCOL_HCCS = 0,
+    COMM_PROTOCOL_ROCE = 1,
+    COMM_PROTOCOL_PCIE = 2,
+    COMM_PROTOCOL_SIO = 3,
+    COMM_PROTOCOL_RESERVED = 0xFFFFFFFFu
+};
+
 struct ChannelInfo {
     bool isValid = false;
     u32 remoteRank = INVALID_VALUE_RANKID;
+    CommProtocol protocol = CommProtocol::COMM_PROTOCOL_RESERVED;
     u32 notifyNum = 0;
     u32 portGroupSize = 1;
     ChannelHandle handle = 0;

@@ -86,7 +86,8 @@ HcclResult InsTempAllGatherNHR::KernelRun(const OpParam &param, const TemplateDa
                 rxDst.emplace_back(ccl, base + p.sliceSize * rx, sizeOf(rx), sizeOf(rx) / esz);
             }
             SendRecvInfo info{{send, recv}, {{txSrc, txDst}, {rxSrc, rxDst}}};
-            CHK_RET(SendRecvWrite(info, th));
+            // over PCIe links the receiver fetches (ins_temp_all_gather_nhr.cc:119, :320-328)
+            CHK_RET(IsPcieProtocol(res.channels) ? SendRecvRead(info, th) : SendRecvBatchWrite(info, th));
         }
     }
     for (u32 k = 0; k < n; ++k) {  // PostLocalCopy

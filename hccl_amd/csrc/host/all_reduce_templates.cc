@@ -240,6 +240,9 @@ HcclResult InsTempAllReduceNHR::KernelRun(const OpParam &param, const TemplateDa
     void *ccl = p.buffInfo.hcclBuff.addr;
     const u64 base = p.buffInfo.hcclBuffBaseOff;
 
+    // over PCIe links the receiver fetches (read mode): the same slices at the same offsets, the other verb
+    // (ins_temp_all_reduce_nhr.cc:105-106, :231-239, :292-300)
+    const bool dmaRead = IsPcieProtocol(res.channels);
     CHK_RET(LocalCopy(th, DataSlice(p.buffInfo.inputPtr, p.buffInfo.inBuffBaseOff, p.sliceSize, p.count),
                       DataSlice(ccl, base, p.sliceSize, p.count)));
     if (templateRankSize_ > 1) {
@@ -251,7 +254,7 @@ HcclResult InsTempAllReduceNHR::KernelRun(const OpParam &param, const TemplateDa
             StepSlices s;
             BuildSameOffsetStep(st, sl, ccl, base, send, recv, s);
             SendRecvReduceInfo info{{send, recv}, {{s.txSrc, s.txDst}, {s.rxSrc, s.rxDst}}, dataType_, reduceOp_};
-            CHK_RET(SendRecvBatchWriteReduce(info, th));
+            CHK_RET(dmaRead ? SendRecvReadReduce(info, th) : SendRecvBatchWriteReduce(info, th));
         }
         GetNHRAllGatherSteps(templateRankSize_, me, steps);
         for (const NHRStepInfo &st : steps) {
@@ -260,7 +263,7 @@ HcclResult InsTempAllReduceNHR::KernelRun(const OpParam &param, const TemplateDa
             StepSlices s;
             BuildSameOffsetStep(st, sl, ccl, base, send, recv, s);
             SendRecvInfo info{{send, recv}, {{s.txSrc, s.txDst}, {s.rxSrc, s.rxDst}}};
-            CHK_RET(SendRecvWrite(info, th));
+            CHK_RET(dmaRead ? SendRecvRead(info, th) : SendRecvWrite(info, th));
         }
     }
     return LocalCopy(th, DataSlice(ccl, base, p.sliceSize, p.count),

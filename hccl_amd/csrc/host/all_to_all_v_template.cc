@@ -1,9 +1,10 @@
 // AlltoAllV mesh template, restated from the reference
-// (src/ops/all_to_all_v/template/aicpu/ins_temp_all_to_all_v_mesh_1D.cc:75-440), write mode, one channel
-// per peer: the block for rank j is packed into a slot of rank j's scratch buffer, rank j unpacks it to
-// rdispls[i] of its output; the own block is copied directly.  Peers are visited in rounds of at most 16,
-// left and right neighbours at growing distance, and each pair of ranks agrees on its slots through the
-// distance between them.
+// (src/ops/all_to_all_v/template/aicpu/ins_temp_all_to_all_v_mesh_1D.cc:75-440), one channel per peer.
+// Write mode: the block for rank j is packed into a slot of rank j's scratch buffer, rank j unpacks it to
+// rdispls[i] of its output.  Read mode (PCIe links, :137-139, :194-206, :291-294, :343-359): the block for rank j is
+// packed into a slot of the sender's OWN scratch buffer and rank j fetches it straight into its output.  The own
+// block is copied directly in both.  Peers are visited in rounds of at most 16, left and right neighbours at
+// growing distance, and each pair of ranks agrees on its slots through the distance between them.
 #include <algorithm>
 
 #include "data_move_templates.h"
@@ -56,6 +57,20 @@ HcclResult InsTempAlltoAllVMesh1D::KernelRun(const OpParam &param, const Templat
     const u32 commLoops = conc ? (templateRankSize_ - 1 + conc - 1) / conc : 0;
     u32 remain = templateRankSize_ - 1;
 
+    const bool dmaRead = IsPcieProtocol(res.channels);
+    // PreCopy (:412-423): the block for `remote` into the slot of the own scratch buffer that `remote` reads
+    auto preCopy = [&](u32 remote) -> HcclResult {
+        if (p.sendCounts[remote] == 0) return HCCL_SUCCESS;
+        u32 mySlot = 0;
+        u32 remoteSlot = 0;
+        CalcCclBuffIdx(remote, mySlot, remoteSlot);
+        const u64 sendSize = p.sendCounts[remote] * esz;
+        return LocalCopy(threads[mySlot + 1],
+                         DataSlice(p.buffInfo.inputPtr, p.sdispls[remote] * esz, sendSize, p.sendCounts[remote]),
+                         DataSlice(p.buffInfo.hcclBuff.addr, mySlot * p.inputSliceStride + p.buffInfo.hcclBuffBaseOff,
+                                   sendSize, p.sendCounts[remote]));
+    };
+
     CHK_RET(PreSync(threads));
     if (commLoops == 0 && p.sendCounts[me] > 0) {  // a single rank still moves its own block
         CHK_RET(LocalCopy(threads[0],
@@ -66,6 +81,15 @@ HcclResult InsTempAlltoAllVMesh1D::KernelRun(const OpParam &param, const Templat
     std::vector<u32> commRanks;
     for (u32 round = 0; round < commLoops && remain > 0; ++round) {
         CalcCommRankSetForOneLoop(round, remain, commRanks);
+        if (dmaRead && round == 0) {
+            // the first round packs all its blocks before anything else, then joins the threads so that the own
+            // block's copy does not run beside them (:194-203)
+            for (u32 remote : commRanks) CHK_RET(preCopy(remote));
+            if (threads.size() > 1) {
+                CHK_RET(PostSync(threads));
+                CHK_RET(PreSync(threads));
+            }
+        }
         if (round == 0 && p.sendCounts[me] > 0) {  // LocalCopyForMyRank
             CHK_RET(LocalCopy(threads[0],
                               DataSlice(p.buffInfo.inputPtr, p.sdispls[me] * esz, p.sendCounts[me] * esz,
@@ -82,6 +106,7 @@ HcclResult InsTempAlltoAllVMesh1D::KernelRun(const OpParam &param, const Templat
             u32 remoteSlot = 0;
             CalcCclBuffIdx(remote, mySlot, remoteSlot);
             const ThreadHandle th = threads[mySlot + 1];
+            if (dmaRead && round != 0) CHK_RET(preCopy(remote));   // :291-294
             const u64 sendSize = p.sendCounts[remote] * esz;
             const u64 recvSize = p.recvCounts[remote] * esz;
             DataSlice txSrc(p.buffInfo.inputPtr, p.sdispls[remote] * esz, sendSize, p.sendCounts[remote]);
@@ -90,6 +115,17 @@ HcclResult InsTempAlltoAllVMesh1D::KernelRun(const OpParam &param, const Templat
             DataSlice rxSrc(link.remoteCclMem.addr, remoteSlot * p.inputSliceStride + p.buffInfo.hcclBuffBaseOff,
                             recvSize, p.recvCounts[remote]);
             DataSlice rxDst(p.buffInfo.outputPtr, p.rdispls[remote] * esz, recvSize, p.recvCounts[remote]);
+            if (dmaRead) {   // RunSendRecv, read branch (:343-359): the peer's slot straight into the output
+                if (sendSize > 0 && recvSize > 0) {
+                    SendRecvInfo info{{link, link}, {{{txSrc}, {txDst}}, {{rxSrc}, {rxDst}}}, dataType_};
+                    CHK_RET(SendRecvRead(info, th));
+                } else if (sendSize > 0) {
+                    CHK_RET(SendRead(DataInfo(link, {{txSrc}, {txDst}}, dataType_), th));
+                } else if (recvSize > 0) {
+                    CHK_RET(RecvRead(DataInfo(link, {{rxSrc}, {rxDst}}, dataType_), th));
+                }
+                continue;
+            }
             if (sendSize > 0 && recvSize > 0) {
                 SendRecvInfo info{{link, link}, {{{txSrc}, {txDst}}, {{rxSrc}, {rxDst}}}, dataType_};
                 CHK_RET(SendRecvWrite(info, th));

@@ -213,6 +213,15 @@ HcclResult hcclxCommSetTopo(HcclComm comm, uint32_t levels, int level0Shape, uin
     return HCCL_SUCCESS;
 }
 
+HcclResult hcclxCommSetLinkProtocol(HcclComm comm, int protocol)
+{
+    RankComm *rc = AsRankComm(comm);
+    CHK_PTR_NULL(rc);
+    if (protocol < HCCLX_LINK_HCCS || protocol > HCCLX_LINK_PCIE) return HCCL_E_PARA;
+    SetWorldLinkProtocol(rc->world, static_cast<CommProtocol>(protocol));
+    return HCCL_SUCCESS;
+}
+
 HcclResult hcclxCommGetLastOpInfo(HcclComm comm, hcclxLastOpInfo *info)
 {
     RankComm *rc = AsRankComm(comm);

@@ -88,8 +88,10 @@ bool BuffersAreSeparate(const std::vector<OpParam> &params)
 
 // For every pointer of a shape plan's parts, in the order segments hold them (sources, then destinations), which of
 // the ranks' buffers it points into: 1 + its index in `buffers`, or 0 for a pointer outside them (the scratch
-// buffers of step plans, which belong to the world and stay where they are).
-static void FindOwners(ShapePlan &sp)
+// buffers of step plans, which belong to the world and stay where they are).  False when the plan cannot be moved
+// with its buffers: a run that starts in a buffer and ends beyond it (it would straddle two buffers that only
+// happened to lie back to back), or a run of a fused plan, which has no scratch buffers, that lies in none.
+static bool FindOwners(ShapePlan &sp)
 {
     struct Range {
         u64 lo, hi;
@@ -120,8 +122,10 @@ static void FindOwners(ShapePlan &sp)
     };
     sp.owners.assign(sp.parts.size(), {});
     std::vector<size_t> guess(2 * HCCLX_MAX_WIDE_FAN, ranges.size());
+    bool movable = true;
     for (size_t i = 0; i < sp.parts.size(); ++i) {
         std::vector<uint16_t> &own = sp.owners[i];
+        const u64 esz = hcclx_dtype_size(sp.parts[i].dtype);
         auto each = [&](const auto &segs) {
             for (const auto &g : segs) {
                 for (uint32_t k = 0; k < g.nsrc + g.ndst; ++k) {
@@ -129,12 +133,19 @@ static void FindOwners(ShapePlan &sp)
                     size_t &at = guess[k < g.nsrc ? k : HCCLX_MAX_WIDE_FAN + k - g.nsrc];
                     at = rangeOf(p, at);
                     own.push_back(at < ranges.size() ? ranges[at].owner : 0);
+                    if (g.count == 0) continue;
+                    if (at < ranges.size()) {
+                        if (reinterpret_cast<u64>(p) + g.count * esz > ranges[at].hi) movable = false;
+                    } else if (sp.fused) {
+                        movable = false;
+                    }
                 }
             }
         };
         each(sp.parts[i].segs);
         each(sp.parts[i].wideSegs);
     }
+    return movable;
 }
 
 // Moves the pointers of a shape plan's parts from the buffers it was made for to those of `params`: every pointer
@@ -299,7 +310,7 @@ void KeepShape(PlanCache &cache, const std::vector<u64> &shape, std::vector<Host
         sp.buffers.push_back({reinterpret_cast<u64>(p.inputPtr), p.inputSize});
         sp.buffers.push_back({reinterpret_cast<u64>(p.outputPtr), p.outputSize});
     }
-    FindOwners(sp);
+    if (!FindOwners(sp)) return;   // planned for its addresses only
     for (const std::vector<uint16_t> &own : sp.owners) sp.hostBytes += own.size() * sizeof(uint16_t);
     cache.shapeBytes += sp.hostBytes;
     cache.shapes.push_front(std::move(sp));

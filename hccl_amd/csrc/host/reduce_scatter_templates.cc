@@ -164,7 +164,8 @@ HcclResult InsTempReduceScatterAicpuReduceNHR::KernelRun(const OpParam &param, c
                 }
             }
             SendRecvInfo info{{send, recv}, {{txSrc, txDst}, {rxSrc, rxDst}}};
-            CHK_RET(SendRecvWrite(info, th));
+            // over PCIe links the receiver fetches (:62-63, :239-247)
+            CHK_RET(IsPcieProtocol(res.channels) ? SendRecvRead(info, th) : SendRecvWrite(info, th));
         }
         CHK_RET(HcommBatchModeEnd(param.algTag.c_str()));  // :66-70: the CPU fold needs the data to have landed
         CHK_RET(HcommBatchModeStart(param.algTag.c_str()));
@@ -207,7 +208,9 @@ bool InsTempReduceScatterAicpuReduceNHR::ClosedForm(const TemplateDataParams &p,
 
 // Shards are copied into scratch slots (slot k = shard k), the NHR reduce-scatter steps fold them across
 // ranks, and the own slot is copied out.  The slices a rank sends in step 0 go straight from its input
-// (ins_temp_reduce_scatter_nhr.cc:98-101, :329-332), so they are not pre-copied.
+// (ins_temp_reduce_scatter_nhr.cc:98-101, :329-332), so they are not pre-copied -- in write mode.  Over PCIe links
+// the receiver fetches (read mode, :91-92, :353-363): every shard is pre-copied, because a peer can only read
+// what lies in the scratch buffer.
 HcclResult InsTempReduceScatterNHR::KernelRun(const OpParam &param, const TemplateDataParams &p,
                                               TemplateResource &res)
 {
@@ -222,10 +225,11 @@ HcclResult InsTempReduceScatterNHR::KernelRun(const OpParam &param, const Templa
     void *ccl = p.buffInfo.hcclBuff.addr;
     auto sizeOf = [&](u32 idx) { return (idx == n - 1 && p.tailSize > 0) ? p.tailSize : p.sliceSize; };
 
+    const bool dmaRead = IsPcieProtocol(res.channels);
     std::vector<NHRStepInfo> steps;
     if (n > 1) GetNHRReduceScatterSteps(n, me, steps);
     std::vector<bool> sentInStep0(n, false);
-    if (!steps.empty()) {
+    if (!steps.empty() && !dmaRead) {
         for (u32 idx : steps[0].txSliceIdxs) sentInStep0[idx] = true;
     }
     for (u32 k = 0; k < n; ++k) {
@@ -244,7 +248,7 @@ HcclResult InsTempReduceScatterNHR::KernelRun(const OpParam &param, const Templa
             const u32 rx = st.rxSliceIdxs[i];
             const u64 txOff = p.buffInfo.hcclBuffBaseOff + p.sliceSize * tx;
             const u64 rxOff = p.buffInfo.hcclBuffBaseOff + p.sliceSize * rx;
-            if (s == 0) {
+            if (s == 0 && !dmaRead) {
                 txSrc.emplace_back(p.buffInfo.inputPtr, p.buffInfo.inBuffBaseOff + p.inputSliceStride * tx, sizeOf(tx),
                                    sizeOf(tx) / esz);
             } else {
@@ -255,7 +259,7 @@ HcclResult InsTempReduceScatterNHR::KernelRun(const OpParam &param, const Templa
             rxDst.emplace_back(ccl, rxOff, sizeOf(rx), sizeOf(rx) / esz);
         }
         SendRecvReduceInfo info{{send, recv}, {{txSrc, txDst}, {rxSrc, rxDst}}, dataType_, reduceOp_};
-        CHK_RET(SendRecvBatchWriteReduce(info, th));
+        CHK_RET(dmaRead ? SendRecvReadReduce(info, th) : SendRecvBatchWriteReduce(info, th));
     }
     const u64 size = sizeOf(me);
     return LocalCopy(th, DataSlice(ccl, p.buffInfo.hcclBuffBaseOff + p.sliceSize * me, size),

@@ -37,6 +37,12 @@ void SetWorldTopo(World *w, u32 levels, Level0Shape shape, u32 devicesPerServer)
     w->devicesPerServer = devicesPerServer;
 }
 
+void SetWorldLinkProtocol(World *w, CommProtocol protocol)
+{
+    std::lock_guard<std::mutex> lock(w->mu);
+    w->linkProtocol = protocol;
+}
+
 using namespace sched;
 
 namespace {
@@ -213,6 +219,7 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
         PlanCache &cache = w->planCache;
         shape = ShapeKey(params, algName, w->cclBytes);
         shape.push_back(fused ? 1 : 0);
+        shape.push_back(static_cast<u64>(w->linkProtocol));   // read and write mode record different steps
         key = PlanKey(shape, params);
         if (!cache.retired.empty()) ReapRetired(cache, false);
         if (CachedPlan *c = FindPlan(cache, key)) {

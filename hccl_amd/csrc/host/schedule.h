@@ -27,5 +27,7 @@ std::string GetForcedAlgorithm(World *w, HcclCMDType type);
 // Topology the selectors see; default: one level, 1-D mesh.
 struct TopoInfoWithNetLayerDetails;
 void SetWorldTopo(World *w, u32 levels, Level0Shape shape, u32 devicesPerServer);
+// What the channels handed to the templates report as their link; PCIe puts the templates that have one into read mode.
+void SetWorldLinkProtocol(World *w, CommProtocol protocol);
 
 }  // namespace ops_hccl

@@ -54,6 +54,16 @@ public:
     }
 
 protected:
+    // True when a link of this rank is PCIe: the templates that have a read mode then let the receiver fetch
+    // (alg_v2_template_base.cc:91-101).
+    static bool IsPcieProtocol(const std::map<u32, std::vector<ChannelInfo>> &channels)
+    {
+        for (const auto &kv : channels) {
+            if (!kv.second.empty() && kv.second[0].protocol == CommProtocol::COMM_PROTOCOL_PCIE) return true;
+        }
+        return false;
+    }
+
     HcclResult PreSync(const std::vector<ThreadHandle> &threads)
     {
         if (threads.size() <= 1) return HCCL_SUCCESS;

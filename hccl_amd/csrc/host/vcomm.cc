@@ -1,6 +1,8 @@
 // Virtual-rank world: creation, the recording primitive backend and the rank rendezvous.
 #include "vcomm.h"
 
+#include <atomic>
+
 #include <algorithm>
 #include <cstring>
 
@@ -148,6 +150,10 @@ HcclResult WorldCreate(u32 rankSize, u64 cclBytes, bool dryRun, std::vector<Hccl
     }
     if (const char *b = std::getenv("HCCL_VRANK_BLOCKING")) w->blocking = (std::atoi(b) != 0);
     if (const char *c = std::getenv("HCCL_VRANK_CHECK")) w->check = (std::atoi(c) != 0);
+    if (const char *l = std::getenv("HCCL_VRANK_LINK_PROTOCOL")) {
+        if (std::strcmp(l, "pcie") == 0) w->linkProtocol = CommProtocol::COMM_PROTOCOL_PCIE;
+        if (std::strcmp(l, "roce") == 0) w->linkProtocol = CommProtocol::COMM_PROTOCOL_ROCE;
+    }
     if (const char *c = std::getenv("HCCL_VRANK_CLOSED_FORM")) w->closedForm = std::max(0, std::min(2, std::atoi(c)));
     {
         u8 level = static_cast<u8>(DeterministicEnableLevel::DETERMINISTIC_DISABLE);
@@ -246,6 +252,7 @@ void FillResources(World *w, u32 rank, u32 threadNum, AlgResourceCtxSerializable
         ChannelInfo ch;
         ch.isValid = true;
         ch.remoteRank = p;
+        ch.protocol = w->linkProtocol;
         ch.notifyNum = 3;
         ch.portGroupSize = 1;
         ch.handle = reinterpret_cast<ChannelHandle>(w->channels[rank][p].get());
@@ -341,6 +348,7 @@ int32_t HcommChannelNotifyRecordOnThread(ThreadHandle thread, ChannelHandle chan
     VThread *t = AsThread(thread);
     VChannel *c = AsChannel(channel);
     if (t == nullptr || c == nullptr) return HCCL_E_PTR;
+    if (c->world != t->world) return HCCL_E_PARA;   // a handle of another world would index past this world's tables
     u64 slot = 0;
     if (!SlotOf(t->world, c->notifySlot, remoteNotifyIdx, slot)) return HCCL_E_PARA;
     return RecordNotify(t, ItemKind::NOTIFY_RECORD, slot);
@@ -367,6 +375,7 @@ int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThr
     VThread *t = AsThread(thread);
     VThread *d = AsThread(dstThread);
     if (t == nullptr || d == nullptr) return HCCL_E_PTR;
+    if (d->world != t->world) return HCCL_E_PARA;   // as above
     u64 slot = 0;
     if (!SlotOf(t->world, d->notifySlot, dstNotifyIdx, slot)) return HCCL_E_PARA;
     return RecordNotify(t, ItemKind::NOTIFY_RECORD, slot);
@@ -380,6 +389,53 @@ int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, u
     u64 slot = 0;
     if (!SlotOf(t->world, t->notifySlot, notifyIdx, slot)) return HCCL_E_PARA;
     return RecordNotify(t, ItemKind::NOTIFY_WAIT, slot);
+}
+
+// The waits every verb of the reference's wrapper tries first (hcomm_primitives_dl.cc:155-173): the time-out is the
+// process-wide one set with HcommSetNotifyWaitTimeOut.  A recorded wait has no clock, so the value is only kept.
+namespace {
+std::atomic<uint32_t> g_notifyWaitTimeout{0};
+std::atomic<uint32_t> g_threadResAcquireTimeout{0};
+}  // namespace
+
+int32_t HcommSetNotifyWaitTimeOut(uint32_t timeOut)
+{
+    g_notifyWaitTimeout.store(timeOut);
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommThreadResAcquireTimeOut(uint32_t timeOut)
+{
+    g_threadResAcquireTimeout.store(timeOut);
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommThreadNotifyWaitOnThreadWithDefaultTimeout(ThreadHandle thread, uint32_t notifyIdx)
+{
+    return HcommThreadNotifyWaitOnThread(thread, notifyIdx, g_notifyWaitTimeout.load());
+}
+
+int32_t HcommChannelNotifyWaitOnThreadWithDefaultTimeout(ThreadHandle thread, ChannelHandle channel,
+                                                         uint32_t localNotifyIdx)
+{
+    return HcommChannelNotifyWaitOnThread(thread, channel, localNotifyIdx, g_notifyWaitTimeout.load());
+}
+
+int32_t HcommWriteWithNotifyNbiOnThread(ThreadHandle thread, ChannelHandle channel, void *dst, const void *src,
+                                        uint64_t len, uint32_t remoteNotifyIdx)
+{
+    const int32_t rc = HcommWriteOnThread(thread, channel, dst, src, len);
+    if (rc != HCCL_SUCCESS) return rc;
+    return HcommChannelNotifyRecordOnThread(thread, channel, remoteNotifyIdx);
+}
+
+int32_t HcommChannelFenceOnThread(ThreadHandle thread, ChannelHandle channel)
+{
+    // the steps of a thread are recorded, and later ordered, in program order: a fence adds nothing
+    VThread *t = AsThread(thread);
+    VChannel *c = AsChannel(channel);
+    if (t == nullptr || c == nullptr) return HCCL_E_PTR;
+    return c->world == t->world ? HCCL_SUCCESS : HCCL_E_PARA;
 }
 
 int32_t HcommBatchTransferOnThread(ThreadHandle thread, ChannelHandle channel,

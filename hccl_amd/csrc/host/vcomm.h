@@ -188,6 +188,7 @@ struct World {
     std::map<int, std::string> forcedAlg;  // per HcclCMDType; empty = selector decides
     HcclAlgoConfig algoConfig;             // HCCL_ALGO as it was when the world was made
     u32 topoLevels = 1;
+    CommProtocol linkProtocol = CommProtocol::COMM_PROTOCOL_HCCS;   // what every channel of the world reports
     Level0Shape topoShape = Level0Shape::MESH_1D;
     u32 devicesPerServer = 0;
     // A dry world has no GPU behind it: scratch buffers are address ranges that are never touched, and a

@@ -58,6 +58,15 @@ HcclResult hcclxCommSetAlgorithm(HcclComm comm, int cmdType, const char *algName
  * devicesPerServer (0 = all ranks in one server; 1 = single-device servers, which selects the NHR family). */
 HcclResult hcclxCommSetTopo(HcclComm comm, uint32_t levels, int level0Shape, uint32_t devicesPerServer);
 
+/* What the links between the ranks report to the templates.  The NHR templates (AllReduce, ReduceScatter,
+ * AllGather, gather-then-fold ReduceScatter) and the AlltoAllV mesh template drive PCIe links in read mode -- the
+ * receiver fetches -- and every other link in write mode (src/ops/op_common/template/alg_v2_template_base.cc:91-101;
+ * e.g. src/ops/all_reduce/template/aicpu/ins_temp_all_reduce_nhr.cc:105-106, :231-239, :292-300).  Same values either
+ * way; the recorded steps, and so the step-by-step launches, differ.  Default: HCCS (write mode); also
+ * HCCL_VRANK_LINK_PROTOCOL=pcie|roce when the communicator is made. */
+typedef enum { HCCLX_LINK_HCCS = 0, HCCLX_LINK_ROCE = 1, HCCLX_LINK_PCIE = 2 } hcclxLinkProtocol;
+HcclResult hcclxCommSetLinkProtocol(HcclComm comm, int protocol);
+
 typedef struct {
     char algName[64];
     uint32_t levels;        /* dependency levels of the recorded schedule */

@@ -113,8 +113,12 @@ int hcclx_fold_wide(const hcclx_wide_seg_t *segs, uint32_t nseg, int dtype, int 
  * hipHostMalloc or copy, also on its first use (hcclx_init() on the device beforehand does the one-time set-up).
  * At most HCCLX_STATIC_MAX_SEGS segments of at most HCCLX_MAX_FAN sources and destinations per call (more:
  * HCCL_E_PARA); always the register-resident kernels, one launch, so large many-destination folds run slower than
- * through hcclx_fold.  Every call on a GPU uses that GPU's one table: calls on the same stream follow each other
- * safely, calls on different streams that may overlap in time race and must be ordered by the caller. */
+ * through hcclx_fold.  Every call on a GPU uses that GPU's one table.  Calls on the same stream follow each other
+ * by stream order; a call on another stream than the previous call's first waits (hipStreamWaitEvent on an event
+ * the library made at set-up, no allocation) for that call's fold kernel, and concurrent host threads take turns,
+ * so eager calls on any mix of streams and threads are safe and merely serialise on the table.  The one case
+ * left to the caller: a call captured into a HIP graph records no such event, so replays of that graph must not
+ * overlap in time with other users of the table (other replays, or eager calls on other streams). */
 #define HCCLX_STATIC_MAX_SEGS 128
 #define HCCLX_STATIC_TABLE_BYTES 40960
 int hcclx_fold_static(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, void *stream);

@@ -44,6 +44,22 @@ int32_t HcommChannelNotifyWaitOnThread(ThreadHandle thread, ChannelHandle channe
 /* Main thread <-> sub thread fan-out / fan-in inside one rank.          hccl_stub.cc:449, :397 */
 int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThread, uint32_t dstNotifyIdx);
 int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, uint32_t timeout);
+/* The process-wide time-outs and the waits that use them.  Every wait of the reference's wrapper goes through the
+ * *WithDefaultTimeout form first and only falls back to the form with an explicit time-out when libhcomm does not
+ * export it (src/common/hcomm_dlsym/hcomm_primitives_dl.h:95-102, hcomm_primitives_dl.cc:131-173;
+ * src/ops/op_common/template/wrapper/alg_data_trans_wrapper.cc:22-31).  Recorded waits have no clock: the values
+ * are kept and returned as success. */
+int32_t HcommSetNotifyWaitTimeOut(uint32_t timeOut);
+int32_t HcommThreadResAcquireTimeOut(uint32_t timeOut);
+int32_t HcommThreadNotifyWaitOnThreadWithDefaultTimeout(ThreadHandle thread, uint32_t notifyIdx);
+int32_t HcommChannelNotifyWaitOnThreadWithDefaultTimeout(ThreadHandle thread, ChannelHandle channel,
+                                                         uint32_t localNotifyIdx);
+/* A write followed by the record of remoteNotifyIdx on the same channel, and a fence that orders the transfers
+ * issued on a channel so far before the later ones (hcomm_primitives_dl.h:103-105).  Steps of one thread are
+ * recorded in program order, so the fence only checks its handles. */
+int32_t HcommWriteWithNotifyNbiOnThread(ThreadHandle thread, ChannelHandle channel, void *dst, const void *src,
+                                        uint64_t len, uint32_t remoteNotifyIdx);
+int32_t HcommChannelFenceOnThread(ThreadHandle thread, ChannelHandle channel);
 /* Several transfers and handshakes on one channel in one call: what every *Batch* verb of the wrapper issues first
  * (src/ops/op_common/template/wrapper/alg_data_trans_wrapper.cc:99-125) and falls back from, slice by slice, when
  * libhcomm does not export it.  The reference resolves the symbol by this name

@@ -839,7 +839,7 @@ CLOSED_FORM_ALGS = {"all_reduce": "InsAllReduceMesh1DTwoShotMeshChunk", "reduce_
                                                    ("reduce_scatter_ordered_group", 40, T.FP32, T.SUM, 9001)])
 def test_templates_planned_from_their_closed_form(stream, kind, n, dtype, op, count):
     """Templates that state their result in closed form are planned from it (nothing recorded) and run as one fused
-    pass: the 64-rank mesh-chunk AllReduce too (4032 chains).  The result is the oracle's replay of the template's
+    pass: the 64-rank mesh-chunk AllReduce too (4032 chains, eight launches of 512 segments).  The result is the oracle's replay of the template's
     steps, and the same collective with the closed form switched off (steps recorded and traced) gives the same bits."""
     alg = CLOSED_FORM_ALGS[kind]
     kind = "all_reduce" if kind.startswith("all_reduce") else "reduce_scatter"
@@ -872,7 +872,8 @@ def test_templates_planned_from_their_closed_form(stream, kind, n, dtype, op, co
                     assert w.reduce_scatter(r, send[r].ptr, recv[r].ptr, count, dtype, op, stream.cuda_stream) == 0
             stream.synchronize()
             info = w.last_info()
-            assert info.fused == 1 and info.launches <= 3
+            # kernels: a launch table holds 512 wide segments, so the 4032 chains of the 64-rank case take eight
+            assert info.fused == 1 and info.launches <= 8, info.launches
             assert (info.levels == 0) == (closed_form == 1)
             got = [b.get(T.NP_STORAGE[dtype]) for b in recv]
             for r in range(n):

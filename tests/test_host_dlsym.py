@@ -45,6 +45,14 @@ struct Table {
     int32_t (*BatchModeStart)(const char *) = nullptr;
     int32_t (*BatchModeEnd)(const char *) = nullptr;
     int32_t (*ThreadJoin)(ThreadHandle, uint32_t) = nullptr;
+    // the process-wide time-out and the waits that use it, which the reference's wrapper tries first
+    // (hcomm_primitives_dl.h:95-105)
+    int32_t (*SetNotifyWaitTimeOut)(uint32_t) = nullptr;
+    int32_t (*ThreadResAcquireTimeOut)(uint32_t) = nullptr;
+    int32_t (*ThreadWaitDefault)(ThreadHandle, uint32_t) = nullptr;
+    int32_t (*ChannelWaitDefault)(ThreadHandle, ChannelHandle, uint32_t) = nullptr;
+    int32_t (*WriteWithNotify)(ThreadHandle, ChannelHandle, void *, const void *, uint64_t, uint32_t) = nullptr;
+    int32_t (*ChannelFence)(ThreadHandle, ChannelHandle) = nullptr;
     int missing = -1;
 };
 Table g;
@@ -79,6 +87,13 @@ extern "C" int LoadPrimitives(const char *path)
     Find(lib, "HcommBatchModeStart", &g.BatchModeStart);
     Find(lib, "HcommBatchModeEnd", &g.BatchModeEnd);
     Find(lib, "HcommThreadJoin", &g.ThreadJoin);
+    Find(lib, "HcommSetNotifyWaitTimeOut", &g.SetNotifyWaitTimeOut);
+    Find(lib, "HcommThreadResAcquireTimeOut", &g.ThreadResAcquireTimeOut);
+    Find(lib, "HcommThreadNotifyWaitOnThreadWithDefaultTimeout", &g.ThreadWaitDefault);
+    Find(lib, "HcommChannelNotifyWaitOnThreadWithDefaultTimeout", &g.ChannelWaitDefault);
+    Find(lib, "HcommWriteWithNotifyNbiOnThread", &g.WriteWithNotify);
+    Find(lib, "HcommChannelFenceOnThread", &g.ChannelFence);
+    if (g.missing == 0 && (g.SetNotifyWaitTimeOut(1800) != 0 || g.ThreadResAcquireTimeOut(1800) != 0)) return -2;
     return g.missing;
 }
 
@@ -101,7 +116,15 @@ HcclResult DlsymOneShot::KernelRun(const OpParam &param, const TemplateDataParam
         if (k == myRank_) continue;
         const ChannelInfo &link = res.channels.at(k)[0];
         if (g.ChannelRecord(t, link.handle, NOTIFY_IDX_ACK) != 0) return HCCL_E_INTERNAL;       // my slot is free
-        if (g.ChannelWait(t, link.handle, NOTIFY_IDX_ACK, 1800) != 0) return HCCL_E_INTERNAL;   // so is the peer's
+        if (g.ChannelWaitDefault(t, link.handle, NOTIFY_IDX_ACK) != 0) return HCCL_E_INTERNAL;   // so is the peer's
+        if (k % 2 == 1) {
+            // odd peers: the write that records its notify, behind a fence; then the wait with the default time-out
+            if (g.ChannelFence(t, link.handle) != 0) return HCCL_E_INTERNAL;
+            if (g.WriteWithNotify(t, link.handle, static_cast<char *>(link.remoteCclMem.addr) + myRank_ * size, in, size,
+                                  NOTIFY_IDX_DATA_SIGNAL) != 0) return HCCL_E_INTERNAL;
+            if (g.ChannelWaitDefault(t, link.handle, NOTIFY_IDX_DATA_SIGNAL) != 0) return HCCL_E_INTERNAL;
+            continue;
+        }
         HcclHcommBatchTransferDesc d[2] = {};
         d[0].transType = HCCL_HCOMM_TRANSFER_TYPE_WRITE;
         d[0].transferInfo.write.len = size;
@@ -152,7 +175,8 @@ def test_every_declared_primitive_is_found_by_name(plugin):
     handle = ctypes.CDLL(_lib.LIB_PATH)
     for name in NAMES:
         assert hasattr(handle, name), name
-    assert "HcommBatchTransferOnThread" in NAMES and len(NAMES) == 14
+    assert "HcommBatchTransferOnThread" in NAMES and "HcommChannelNotifyWaitOnThreadWithDefaultTimeout" in NAMES
+    assert len(NAMES) == 20
 
 
 @pytest.mark.parametrize("n", [2, 3, 5])
