@@ -352,7 +352,36 @@ HcclResult RunCollectiveOnStream(World *w, std::vector<OpParam> &params)
                 CHK_PRT_RET(w->lastCheck.races != 0 || w->lastCheck.semanticErrors != 0,
                             HCCL_ERROR("[schedule check] %s", w->lastCheck.firstProblem.c_str()), HCCL_E_INTERNAL);
             }
-            ok = FoldsFromTrace(tr, params, foldType, op, folds, text);
+            std::string checkedText;
+            std::string *traceOut = text ? text : (w->check ? &checkedText : nullptr);
+            ok = FoldsFromTrace(tr, params, foldType, op, folds, traceOut);
+            // A template that also states its result in closed form is planned from that statement when the check
+            // is off: so the check holds the statement against what the recorded steps amount to, piece by piece
+            // and in the same association order.
+            if (ok && w->check && !IsDataMove(type) && BuffersAreSeparate(params)) {
+                std::unique_ptr<InsCollAlgBase> exec = CollAlgExecRegistryV2::Instance().GetAlgExec(type, algName);
+                std::vector<ClosedFold> closed;
+                std::vector<Fold> stated;
+                std::string statedText;
+                params[0].algName = algName;
+                if (exec != nullptr && exec->ClosedForm(params[0], n, w->cclBytes, closed) &&
+                    FoldsFromClosedForm(closed, params, dtype, op, stated, &statedText) && statedText != *traceOut) {
+                    // the first line that differs names the piece
+                    size_t at = 0;
+                    while (at < statedText.size() && at < traceOut->size() && statedText[at] == (*traceOut)[at]) ++at;
+                    const size_t from = statedText.rfind('\n', at ? at - 1 : 0);
+                    const size_t lineStart = (from == std::string::npos || at == 0) ? 0 : from + 1;
+                    const size_t lineEnd = statedText.find('\n', lineStart);
+                    w->lastCheck.semanticErrors++;
+                    if (w->lastCheck.firstProblem.empty()) {
+                        w->lastCheck.firstProblem = "the template's closed form is not what its recorded steps amount to; it states: " +
+                                                    statedText.substr(lineStart, lineEnd == std::string::npos ? std::string::npos
+                                                                                                             : lineEnd - lineStart);
+                    }
+                    HCCL_ERROR("[schedule check] %s", w->lastCheck.firstProblem.c_str());
+                    return HCCL_E_INTERNAL;
+                }
+            }
         }
         FusedPlan plan;
         ok = ok && BuildFusedPlan(params, folds, esz, plan, haveFolds);

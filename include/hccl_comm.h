@@ -99,8 +99,11 @@ HcclResult hcclxCommSetClosedForm(HcclComm comm, int mode);
  * (2) no two steps that the handshakes leave unordered touch the same bytes with at least one of them writing
  * (check_rank_mem / the task-graph race rules), (3) every output piece is what the collective's contract says:
  * reduced from each rank exactly once at the matching offset, or copied from the right rank and offset
- * (semantics_check/<op>_semantics_checker.cc).  A collective that fails returns HCCL_E_INTERNAL and launches
- * nothing.  Checked collectives bypass the plan cache. */
+ * (semantics_check/<op>_semantics_checker.cc), (4) when the template also states its result in closed form (see
+ * hcclxCommSetClosedForm) and the ranks' buffers lie apart: that statement, piece by piece and in the same
+ * association order, is what the recorded steps amount to -- a closed form is trusted when the check is off, so
+ * this is where a plug-in template's statement is held against its steps.  A collective that fails returns
+ * HCCL_E_INTERNAL and launches nothing.  Checked collectives bypass the plan cache. */
 typedef struct {
     uint32_t steps, levels, copies, reduces;
     uint32_t races;

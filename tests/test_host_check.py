@@ -92,6 +92,8 @@ def test_the_other_collectives_pass_the_check(n):
 
 PLUGIN = r'''
 // Two deliberately broken AllReduce templates, registered from outside the library through the plugin macros.
+#include <algorithm>
+#include "host/all_reduce_templates.h"
 #include "host/data_move_templates.h"
 #include "host/sole_executors.h"
 using namespace ops_hccl;
@@ -165,6 +167,22 @@ public:
     }
 };
 
+// "Misstated": the two-shot template with a closed form that folds every slice in the opposite order: the right
+// contributions, the wrong association.
+class MisstatedTwoShot : public InsTempAllReduceMesh1DTwoShot {
+public:
+    using InsTempAllReduceMesh1DTwoShot::InsTempAllReduceMesh1DTwoShot;
+    bool ClosedForm(const TemplateDataParams &p, u64 esz, std::vector<ClosedFold> &out) const override
+    {
+        const size_t first = out.size();
+        if (!InsTempAllReduceMesh1DTwoShot::ClosedForm(p, esz, out)) return false;
+        for (size_t i = first; i < out.size(); ++i) std::reverse(out[i].src.begin(), out[i].src.end());
+        return true;
+    }
+};
+REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_ALLREDUCE, TestMisstatedTwoShot, InsV2AllReduceSoleExecutor, TopoMatch1D,
+                 MisstatedTwoShot);
+
 REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_ALLREDUCE, TestOverreachingOneShot, InsV2AllReduceSoleExecutor, TopoMatch1D,
                  OverreachingOneShot);
 REGISTER_EXEC_V2(HcclCMDType::HCCL_CMD_ALLREDUCE, TestRacyOneShot, InsV2AllReduceSoleExecutor, TopoMatch1D, RacyOneShot);
@@ -234,6 +252,40 @@ def test_a_closed_form_that_reaches_beyond_the_buffers_is_not_used(plugin):
     want, _ = trace("InsAllReduceMesh1DOneShot", 0)
     got, levels = trace("TestOverreachingOneShot", 2)
     assert levels > 0 and got == want
+
+
+def test_a_closed_form_that_misstates_the_order_is_caught_by_the_check(plugin):
+    """A template's closed form is trusted for plain launches; with the check on it is held against the recorded
+    steps: the same contributions folded in another order are a different result for floats, and are rejected."""
+    n = 4
+    ins, outs = fake_ptrs(n)
+    w = checked_world(n)
+    try:
+        w.set_algorithm(api.CMD_ALLREDUCE, "TestMisstatedTwoShot")
+        rcs = [w.all_reduce(r, ins[r], outs[r], 1000, T.FP32, T.SUM, FAKE_STREAM) for r in range(n)]
+        assert rcs[-1] == 4
+        rep = w.last_check()
+        assert rep.races == 0 and rep.semanticErrors == 1 and b"closed form" in rep.firstProblem, rep.firstProblem
+        assert b"(x0@0+(x1@0+(x2@0+x3@0)))" in rep.firstProblem       # what it states for the first piece
+        # the built-in template states what it does: accepted under the same check
+        w.set_algorithm(api.CMD_ALLREDUCE, "InsAllReduceMesh1DTwoShot")
+        assert [w.all_reduce(r, ins[r], outs[r], 1000, T.FP32, T.SUM, FAKE_STREAM) for r in range(n)][-1] == 0
+        assert w.last_check().semanticErrors == 0
+        # the comparison is of the statement itself, whatever the type: an integer fold would come out the same in
+        # either order, the statement is still not the template's
+        w.set_algorithm(api.CMD_ALLREDUCE, "TestMisstatedTwoShot")
+        assert [w.all_reduce(r, ins[r], outs[r], 1000, T.INT32, T.MAX, FAKE_STREAM) for r in range(n)][-1] == 4
+    finally:
+        w.close()
+    # unchecked and traced from its closed form, the misstatement is what would run
+    w = api.World(n, ccl_bytes=SMALL_CCL, dry=True)
+    try:
+        w.set_closed_form(2)
+        w.set_algorithm(api.CMD_ALLREDUCE, "TestMisstatedTwoShot")
+        assert [w.all_reduce(r, ins[r], outs[r], 1000, T.FP32, T.SUM, FAKE_STREAM) for r in range(n)][-1] == 0
+        assert "(x0@0+(x1@0+(x2@0+x3@0)))" in w.last_trace() and w.last_info().levels == 0
+    finally:
+        w.close()
 
 
 def run_ar(n, count, dtype, op):

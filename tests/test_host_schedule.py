@@ -669,3 +669,71 @@ def test_closed_form_among_64_ranks_and_when_it_is_not_used():
     shared = [ins[0]] + ins[:-1]
     _, info = traced(n, lambda w: call(w, srcs=shared), 2)
     assert info.levels > 0
+
+
+CLOSED_FORM_TEMPLATES = {
+    api.CMD_ALLREDUCE: ["InsAllReduceMesh1DOneShot", "InsAllReduceMesh1DTwoShot", "InsAllReduceNHR",
+                        "InsAllReduceAicpuReduceNHR", "InsAllReduceMesh1DTwoShotMeshChunk", "InsAllReduceRing",
+                        "InsAllReduceRHD"],
+    api.CMD_REDUCE_SCATTER: ["InsReduceScatterMesh1D", "InsReduceScatterNHR", "InsReduceScatterAicpuReduceNHR",
+                             "InsReduceScatterMesh1DMeshChunk", "ReduceScatterOrderPreserved",
+                             "ReduceScatterOrderPreservedGroup"],
+}
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_closed_forms_equal_the_recorded_steps_over_seeded_random_shapes(seed):
+    """A guard against the two statements of a template drifting apart: random communicators of 2..64 ranks, every
+    template that has a closed form, counts drawn around the places where slices, 4 KiB chunk cuts and executor loops
+    change (also with a scratch buffer so small that nearly every count takes several loops), three element sizes,
+    in and out of place.  The trace of the closed form must be the trace of the recorded steps, line for line."""
+    rng = np.random.default_rng(1000 + seed)
+    cases = 0
+    while cases < 64:
+        n = int(rng.choice([2, 3, 4, 5, 6, 7, 8, 9, 11, 12, 13, 16, 17, 20, 24, 31, 32, 33, 40, 48, 63, 64],
+                           p=None))
+        if n > 33 and rng.random() < 0.6:
+            continue                                   # the widest communicators cost the most: fewer of them
+        cmd = api.CMD_ALLREDUCE if rng.random() < 0.55 else api.CMD_REDUCE_SCATTER
+        alg = str(rng.choice(CLOSED_FORM_TEMPLATES[cmd]))
+        dtype = [T.INT8, T.FP32, T.FP64][int(rng.integers(3))]
+        esz = T.DTYPE_SIZE[dtype]
+        ccl = SMALL_CCL if rng.random() < 0.5 else 1024 * 1024 + 128 * 64 + int(rng.integers(0, 4096)) * 8
+        in_place = cmd == api.CMD_ALLREDUCE and rng.random() < 0.3
+        # around a multiple of the rank count, of a 4 KiB chunk per rank, and of what one executor loop holds
+        slot = max(1, (ccl - (1 << 20 if cmd == api.CMD_REDUCE_SCATTER else 0)) // n // 128 * 128 // esz)
+        anchor = int(rng.choice([1, n, n * n, 4096 // esz, n * (4096 // esz), slot, 2 * slot, n * slot // 2 + 1]))
+        count = max(1, anchor + int(rng.integers(-3, 4)))
+        if cmd == api.CMD_REDUCE_SCATTER:
+            count = max(1, count // n) if rng.random() < 0.5 else count
+        if count * esz * (n if cmd == api.CMD_REDUCE_SCATTER else 1) > (6 << 20) or (n > 33 and count * esz > (1 << 20)):
+            continue                                   # keeps a dry case to milliseconds
+        op = T.SUM if rng.random() < 0.7 else T.MAX
+        ins, outs = fake_ptrs(n)
+
+        def call(w):
+            w.set_algorithm(cmd, alg)
+            for r in range(n):
+                dst = ins[r] if in_place else outs[r]
+                if cmd == api.CMD_ALLREDUCE:
+                    assert w.all_reduce(r, ins[r], dst, count, dtype, op, FAKE_STREAM) == 0
+                else:
+                    assert w.reduce_scatter(r, ins[r], dst, count, dtype, op, FAKE_STREAM) == 0
+            return w.last_trace()
+
+        def traced_with(closed_form):
+            w = api.World(n, ccl_bytes=ccl, dry=True)
+            try:
+                w.set_closed_form(closed_form)
+                return call(w), w.last_info()
+            finally:
+                w.close()
+
+        recorded, info_r = traced_with(0)
+        closed, info_c = traced_with(2)
+        what = f"seed={seed} {alg} n={n} count={count} dtype={dtype} op={op} ccl={ccl} in_place={in_place}"
+        assert info_r.levels > 0, what
+        assert info_c.levels == 0, "the closed form was not used: " + what
+        assert closed == recorded, what
+        assert info_c.fused == info_r.fused and info_c.fusedSegments == info_r.fusedSegments, what
+        cases += 1
