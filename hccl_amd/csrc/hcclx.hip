@@ -133,6 +133,16 @@ void init_slot(DeviceSlot *s, int dev)
         const uint64_t b = std::min<uint64_t>(std::strtoull(v, nullptr, 10), 1ull << 30);
         if (b >= 65536) c.fanout_run = b & ~static_cast<uint64_t>(4095);
     }
+    if (const char *v = std::getenv("HCCLX_WAVES_FROM")) c.waves_from = std::strtoull(v, nullptr, 10);
+    if (const char *v = std::getenv("HCCLX_WAVES_MAX_FAN")) {
+        const unsigned long b = std::strtoul(v, nullptr, 10);
+        c.waves_max_fan = b > HCCLX_MAX_FAN ? static_cast<uint32_t>(HCCLX_MAX_FAN) : static_cast<uint32_t>(b);
+    }
+    if (const char *v = std::getenv("HCCLX_WAVES_CHAINS")) c.waves_chains = std::strtoul(v, nullptr, 10) != 0;
+    if (const char *v = std::getenv("HCCLX_WAVES_PIECES")) {
+        const unsigned long b = std::strtoul(v, nullptr, 10);
+        c.waves_pieces = b > kWavePieces ? static_cast<uint32_t>(kWavePieces) : static_cast<uint32_t>(b);
+    }
     if (const char *v = std::getenv("HCCLX_AGV_PHASED_FROM")) c.agv_phased_from = std::strtoull(v, nullptr, 10);
     if (const char *v = std::getenv("HCCLX_STORE_THROUGH_UPTO")) c.store_through_upto = std::strtoull(v, nullptr, 10);
     c.ring_bytes = kSliceBytes * kSlices;
@@ -385,6 +395,8 @@ struct Batch {
     int block_unroll = 2;
     PhasedLaunch phased;         // instead of everything above: jobs of the copy kernel that writes one output at a time
     uint32_t store_policy = kStoreStream;   // how the fold kernels store (fold.h)
+    uint32_t waves = 0;          // non-zero: the one-store-per-wavefront kernel, this many wavefronts per workgroup
+    uint32_t pieces = 1;         // and this many 1 KiB pieces per source and workgroup
     size_t nseg() const { return segs.size() + wide.size(); }
     size_t bytes() const
     {
@@ -500,6 +512,8 @@ struct SegProto {
     int mode = 0;        // the kernel's mode (integers take the chain kernel whatever order is asked for)
     int maxn = 1;        // source slots of the kernel instance
     int esz = 1;
+    uint32_t waves = 0;  // non-zero: tiles are those of the one-store-per-wavefront kernel (pieces x 64 vectors)
+    uint32_t pieces = 1;
 };
 
 // Checks the segments of a call and works out the kernel instance they need.  Allocates nothing unless it fails.
@@ -574,9 +588,10 @@ bool make_segdev(const hcclx_seg_t &s, const SegProto &sp, int mode, SegDev *out
     }
     if (sp.mode == HCCLX_FOLD_TREE && !embed_tree(s, static_cast<uint32_t>(sp.maxn), &sd)) return false;
     const int ne = sp.copy ? 16 : 16 / sp.esz;
+    const uint64_t tile_vecs = sp.waves != 0 ? waves_tile_vecs(static_cast<int>(sp.pieces)) : fold_tile_vecs(sp.maxn);
     sd.head = fold_head_of(sd.count, sp.copy ? 1 : sp.esz, sd.dst[0]);
-    sd.shift = fold_shift_of(sd.head, sp.copy ? 1 : sp.esz, fold_tile_vecs(sp.maxn), sd.dst[0]);
-    *tiles = fold_tiles_of(sd.count, ne, fold_tile_vecs(sp.maxn), sd.head, sd.shift);
+    sd.shift = fold_shift_of(sd.head, sp.copy ? 1 : sp.esz, tile_vecs, sd.dst[0]);
+    *tiles = fold_tiles_of(sd.count, ne, tile_vecs, sd.head, sd.shift);
     *out = sd;
     return true;
 }
@@ -687,12 +702,50 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
     return HCCL_SUCCESS;
 }
 
+// The n orders of a self-first fold take the kernel in which every wavefront issues one store (fold.h) when the
+// launch writes waves_from bytes or more and its widest segment has at most waves_max_fan sources: measured against
+// the register kernel on fp32 PROD, 64 MiB per rank: 4 ranks 78.7 against 93.5 us, 8 ranks 188 against 203; from
+// twelve ranks on its LDS traffic (every wavefront reads every source piece) takes the gain away (12 ranks: 313
+// against 299 us), and below 16 MiB per rank the shorter workgroups of the register kernel win.  Chains whose value
+// goes to several places run on it too when asked for (waves_chains; off: as one pass it measured 189 to 245 us on
+// the 8 x 64 MiB AllReduce against 172 for the fold + fan-out pair).  Returns the number of wavefronts per workgroup
+// (the widest segment's sources or destinations), 0 = the register kernels.
+uint32_t waves_for(const DeviceCtx *ctx, const hcclx_seg_t *segs, uint32_t nseg, int dtype, int mode, uint32_t *pieces)
+{
+    if (ctx == nullptr || ctx->waves_from == 0 || nseg == 0) return 0;
+    if (mode != HCCLX_FOLD_SELF_FIRST && !(mode == HCCLX_FOLD_CHAIN && ctx->waves_chains)) return 0;
+    const uint64_t esz = static_cast<uint64_t>(dtype_size(dtype));
+    uint32_t most_src = 0;
+    uint32_t most_dst = 0;
+    uint64_t written = 0;
+    uint64_t tiles = 0;
+    for (uint32_t i = 0; i < nseg; ++i) {
+        if (segs[i].nsrc == 0 || segs[i].nsrc > HCCLX_MAX_FAN || segs[i].ndst == 0 || segs[i].ndst > HCCLX_MAX_FAN) return 0;
+        most_src = segs[i].nsrc > most_src ? segs[i].nsrc : most_src;
+        most_dst = segs[i].ndst > most_dst ? segs[i].ndst : most_dst;
+        written += segs[i].count * esz * segs[i].ndst;
+        tiles += segs[i].count * esz / 1024 + 2;
+    }
+    const uint32_t widest = most_src > most_dst ? most_src : most_dst;
+    if (most_src < 2 || most_dst < 2 || widest > ctx->waves_max_fan || written < ctx->waves_from || esz == 0) return 0;
+    // pieces per workgroup: four measured best at every width (a workgroup lives a few microseconds: fewer pieces and
+    // its set-up shows, more and the wavefronts issue too many stores in a row again)
+    const uint32_t p = ctx->waves_pieces != 0 ? ctx->waves_pieces : 4u;
+    if (tiles / p > 0x7fffffffull) return 0;   // one workgroup per tile: the grid has to hold them
+    *pieces = p;
+    return widest;
+}
+
 int build_batches_impl(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int mode, Built *out)
 {
     if (nseg != 0 && segs == nullptr) return fail(HCCL_E_PTR, "segs is null");
+    // the order a launch is asked for, and the one its kernel runs: integer folds are association-free
+    const int kernel_mode = (mode != HCCLX_FOLD_CHAIN && !is_float_dtype(dtype)) ? HCCLX_FOLD_CHAIN : mode;
+    uint32_t wave_pieces = 1;
+    const uint32_t waves = waves_for(device_ctx(), segs, nseg, dtype, kernel_mode, &wave_pieces);
     // Chains over many sources run faster on the wide chain kernel (sources in groups of eight, two vectors per
     // thread) than on the kernel that holds every source in registers.
-    if (mode == HCCLX_FOLD_CHAIN && nseg != 0) {
+    if (mode == HCCLX_FOLD_CHAIN && nseg != 0 && waves == 0) {
         const DeviceCtx *ctx = device_ctx();
         uint32_t most = 0;
         uint32_t most_dst = 0;
@@ -719,12 +772,18 @@ int build_batches_impl(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op
     SegProto sp;
     const int rc = check_segs(segs, nseg, dtype, op, mode, &sp);
     if (rc != HCCL_SUCCESS) return rc;
+    if (waves != 0 && !sp.copy && (sp.mode == HCCLX_FOLD_CHAIN || sp.mode == HCCLX_FOLD_SELF_FIRST)) {
+        sp.waves = waves;
+        sp.pieces = wave_pieces;
+    }
     Batch proto;
     proto.copy = sp.copy;
     proto.dtype = dtype;
     proto.op = op;
     proto.mode = sp.mode;
     proto.maxn = sp.maxn;
+    proto.waves = sp.waves;
+    proto.pieces = sp.pieces;
     proto.store_policy = store_policy_for(device_ctx(), segs, nseg, sp.copy ? 1 : dtype_size(dtype));
     Batch cur = proto;
     for (uint32_t i = 0; i < nseg; ++i) {
@@ -971,6 +1030,8 @@ int launch_batch(const DeviceCtx *ctx, const Batch &b, const char *d_table, hipS
     l.xcd_remap = b.xcd_remap;
     l.store_policy = b.store_policy;
     l.uniform_tiles = uniform_tiles_of(b.tile_end.data(), b.tile_end.size());
+    l.waves = b.waves;
+    l.pieces = b.pieces;
     l.stream = stream;
     const hipError_t e = b.copy ? fold_dispatch_copy(l) : dispatch_fold(b.dtype, b.op, b.maxn, b.mode, l);
     if (e != hipSuccess) return fail_hip(e, "fold kernel launch");
@@ -998,6 +1059,32 @@ int hcclx_init(void) { return device_ctx() ? HCCL_SUCCESS : HCCL_E_RUNTIME; }
 const char *hcclx_last_error(void) { return g_err.c_str(); }
 
 uint64_t hcclx_kernels_launched(void) { return hcclx::kernels_launched(); }
+
+int hcclx_tune(const char *name, uint64_t value)
+{
+    DeviceCtx *ctx = device_ctx();
+    if (!ctx) return HCCL_E_RUNTIME;
+    if (name == nullptr) return fail(HCCL_E_PTR, "name is null");
+    const std::string key(name);
+    if (key == "waves_from") {
+        ctx->waves_from = value;
+    } else if (key == "waves_max_fan") {
+        if (value < 2 || value > HCCLX_MAX_FAN) return fail(HCCL_E_PARA, "waves_max_fan outside 2..16");
+        ctx->waves_max_fan = static_cast<uint32_t>(value);
+    } else if (key == "waves_chains") {
+        ctx->waves_chains = value != 0;
+    } else if (key == "waves_pieces") {
+        if (value > static_cast<uint64_t>(kWavePieces)) return fail(HCCL_E_PARA, "waves_pieces beyond " + std::to_string(kWavePieces));
+        ctx->waves_pieces = static_cast<uint32_t>(value);
+    } else if (key == "fanout_from") {
+        ctx->fanout_from = value;
+    } else if (key == "store_through_upto") {
+        ctx->store_through_upto = value;
+    } else {
+        return fail(HCCL_E_PARA, "unknown knob: " + key);
+    }
+    return HCCL_SUCCESS;
+}
 
 uint32_t hcclx_dtype_size(int dtype) { return static_cast<uint32_t>(dtype_size(dtype)); }
 

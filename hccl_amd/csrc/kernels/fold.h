@@ -53,14 +53,25 @@ __host__ __device__ constexpr uint64_t wide_tile_vecs(int unroll)
 #ifndef HCCLX_NT_LOAD
 #define HCCLX_NT_LOAD 1
 #endif
+// Every data pointer of the library is a device pointer into HBM.  A pointer that a kernel fetched from a table has
+// no address space the compiler can see, and a load through it becomes a FLAT instruction, which counts as an LDS
+// operation too (every wait for LDS then also waits for the loads in flight).  These casts say what the pointers
+// are, and the loads and stores become GLOBAL instructions.
+typedef const u32x4_u __attribute__((address_space(1))) *global_cvec_ptr;
+typedef u32x4_u __attribute__((address_space(1))) *global_vec_ptr;
+__device__ __forceinline__ global_cvec_ptr as_global(const char *p) { return (global_cvec_ptr)(p); }
+__device__ __forceinline__ global_vec_ptr as_global(char *p) { return (global_vec_ptr)(p); }
+
 __device__ __forceinline__ u32x4 ld16(const char *p)
 {
 #if HCCLX_NT_LOAD
-    return __builtin_nontemporal_load(reinterpret_cast<const u32x4_u *>(p));
+    return __builtin_nontemporal_load(as_global(p));
 #else
-    return *reinterpret_cast<const u32x4_u *>(p);
+    return *as_global(p);
 #endif
 }
+// an ordinary (cached) load: the next reader of the same bytes finds them in the L2
+__device__ __forceinline__ u32x4 ld16_cached(const char *p) { return *as_global(p); }
 // How results leave the CU.  Two ways to store, measured on MI355X against each other and against ordinary stores:
 //   stream   nontemporal: the line is marked for early eviction.  Best where many large output streams are
 //            written at once (the self-first orders) and for the copy kernels (AlltoAllV 154 us against 162).
@@ -74,7 +85,7 @@ constexpr uint32_t kStoreStream = 0;
 constexpr uint32_t kStoreThrough = 1;
 __device__ __forceinline__ void st16(char *p, u32x4 v)
 {
-    __builtin_nontemporal_store(v, reinterpret_cast<u32x4_u *>(p));
+    __builtin_nontemporal_store(v, as_global(p));
 }
 __device__ __forceinline__ void st16x(char *p, u32x4 v, uint32_t policy)
 {
@@ -385,6 +396,201 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// One store per wavefront.  A wavefront that issues several 16-byte stores per lane in a row writes HBM a fifth
+// slower than wavefronts that issue one each and end (measured on MI355X with plain fills: 12 streams of 1 GiB,
+// every workgroup all 12: 5.6 TB/s; one stream per wavefront: 6.6 to 7.2), and a fold whose results go to n places
+// is half writes.  Here a workgroup has one wavefront per source / destination: wavefront w loads a 1 KiB piece of
+// source w into LDS; after the barrier every wavefront w < ndst reads all pieces, folds them in its own order and
+// stores the piece of destination w: one global load and one global store per wavefront and piece.  A workgroup
+// takes `pieces` pieces in a row (the load of the next is issued before the current one is folded); the LDS holds
+// two pieces per source.  Same results, bit for bit, as the register kernel: the fold order per element is the same.
+// ---------------------------------------------------------------------------------------------------
+constexpr int kWaveLanes = 64;
+constexpr int kWavePieces = 8;   // most pieces per source and workgroup
+__host__ __device__ constexpr uint64_t waves_tile_vecs(int pieces) { return static_cast<uint64_t>(kWaveLanes) * pieces; }
+// LDS bytes of the pieces: two buffers of `waves` pieces
+__host__ __device__ constexpr uint32_t waves_lds_bytes(int waves) { return 2u * waves * kWaveLanes * 16u; }
+
+// The fold of one piece by one wavefront of k_fold_waves.  The LDS traffic of this kernel is what bounds it after
+// HBM (every wavefront reads every source piece: n * n reads of 1 KiB per 2 n KiB moved), so only the pieces that
+// exist are read: four at a time, all four before the first is combined so that the reads overlap.  Within a group
+// a missing source is read from the group's first slot and dropped by a select: as a branch around each step the
+// test keeps the compiler from overlapping the steps with the reads.
+template <int DT, int OP, int MODE>
+__device__ __forceinline__ void waves_fold(const u32x4 *buf, uint32_t nsrc, uint32_t w, uint32_t lane, uint32_t flips,
+                                           typename Vec16<DT>::C (&acc)[Vec16<DT>::NE])
+{
+    using V = Vec16<DT>;
+    using C = typename V::C;
+    constexpr int NE = V::NE;
+    constexpr int G = 4;
+    // self-first: the wavefront's own source starts the fold (its index is not a compile-time constant: one more
+    // read instead of a register picked at run time); the chain starts from the first source, read with group 0
+    if constexpr (MODE != kFoldChain) V::unpack(buf[w * kWaveLanes + lane], acc);
+#pragma unroll
+    for (int base = 0; base < kMaxFan; base += G) {
+        if (base < static_cast<int>(nsrc)) {
+            u32x4 raw[G];
+#pragma unroll
+            for (int k = 0; k < G; ++k) {
+                const uint32_t slot = static_cast<uint32_t>(base + k) < nsrc ? static_cast<uint32_t>(base + k) : static_cast<uint32_t>(base);
+                raw[k] = buf[slot * kWaveLanes + lane];
+            }
+#pragma unroll
+            for (int k = 0; k < G; ++k) {
+                const int at = base + k;
+                C x[NE];
+                V::unpack(raw[k], x);
+                if (MODE == kFoldChain && at == 0) {
+#pragma unroll
+                    for (int e = 0; e < NE; ++e) acc[e] = x[e];
+                    continue;
+                }
+                const bool take = at < static_cast<int>(nsrc) && (MODE == kFoldChain || at != static_cast<int>(w));
+                const bool flip = MODE == kFoldChain && OperandOrderMatters<DT, OP>::value && ((flips >> at) & 1u);
+#pragma unroll
+                for (int e = 0; e < NE; ++e) {
+                    C r = V::template combine<OP>(x[e], acc[e]);
+                    if (OperandOrderMatters<DT, OP>::value && MODE == kFoldChain) {
+                        const C r2 = V::template combine<OP>(acc[e], x[e]);
+                        r = flip ? r2 : r;
+                    }
+                    acc[e] = take ? r : acc[e];
+                }
+            }
+        }
+    }
+}
+
+// The same fold for a source count the compiler knows: straight-line code, no test per source.  Measured on the
+// twelve orders of a 12-rank AllReduce: 263 us against 271 with the tests (64 MiB per rank).
+template <int DT, int OP, int MODE, int N>
+__device__ __forceinline__ void waves_fold_fixed(const u32x4 *buf, uint32_t w, uint32_t lane, uint32_t flips,
+                                                 typename Vec16<DT>::C (&acc)[Vec16<DT>::NE])
+{
+    using V = Vec16<DT>;
+    using C = typename V::C;
+    constexpr int NE = V::NE;
+    constexpr int G = 4;
+    static_assert(N % G == 0, "whole groups");
+    if constexpr (MODE != kFoldChain) V::unpack(buf[w * kWaveLanes + lane], acc);
+#pragma unroll
+    for (int base = 0; base < N; base += G) {
+        u32x4 raw[G];
+#pragma unroll
+        for (int k = 0; k < G; ++k) raw[k] = buf[(base + k) * kWaveLanes + lane];
+#pragma unroll
+        for (int k = 0; k < G; ++k) {
+            const int at = base + k;
+            C x[NE];
+            V::unpack(raw[k], x);
+            if (MODE == kFoldChain && at == 0) {
+#pragma unroll
+                for (int e = 0; e < NE; ++e) acc[e] = x[e];
+                continue;
+            }
+            const bool flip = MODE == kFoldChain && OperandOrderMatters<DT, OP>::value && ((flips >> at) & 1u);
+#pragma unroll
+            for (int e = 0; e < NE; ++e) {
+                C r = V::template combine<OP>(x[e], acc[e]);
+                if (OperandOrderMatters<DT, OP>::value && MODE == kFoldChain) {
+                    const C r2 = V::template combine<OP>(acc[e], x[e]);
+                    r = flip ? r2 : r;
+                }
+                // self-first: the wavefront's own source has been taken first and is passed over here
+                acc[e] = (MODE == kFoldChain || at != static_cast<int>(w)) ? r : acc[e];
+            }
+        }
+    }
+}
+
+template <int DT, int OP, int MODE>
+__global__ void __launch_bounds__(kMaxFan * kWaveLanes)
+k_fold_waves(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, uint32_t nseg, uint32_t pieces,
+             uint32_t store_policy, uint32_t uniform_tiles)
+{
+    static_assert(MODE == kFoldChain || MODE == kFoldSelfFirst, "trees stay on the register kernel");
+    using V = Vec16<DT>;
+    using C = typename V::C;
+    constexpr int NE = V::NE;
+    constexpr int NV = Vec16<DT>::kElems;   // elements per 16-byte vector
+    extern __shared__ u32x4 s_piece[];      // [2][waves][64], then the staged tile prefix when it is searched in LDS
+    const uint32_t waves = blockDim.x / kWaveLanes;
+    const uint32_t w = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveLanes);
+    const uint32_t lane = threadIdx.x % kWaveLanes;
+    uint32_t s = 0;
+    uint64_t tl = blockIdx.x;
+    if (nseg != 1) {   // a single segment (the n orders of an AllReduce): the tile number is the tile in the segment
+        const uint64_t *s_end = reinterpret_cast<const uint64_t *>(s_piece + 2 * waves * kWaveLanes);
+        const bool direct = nseg <= kFoldDirectSegs || uniform_tiles != 0;
+        if (!direct) {
+            uint64_t *stage = reinterpret_cast<uint64_t *>(s_piece + 2 * waves * kWaveLanes);
+            for (uint32_t i = threadIdx.x; i < nseg; i += blockDim.x) stage[i] = tile_end[i];
+            __syncthreads();
+        }
+        locate_tile(tile_end, s_end, nseg, direct, uniform_tiles, blockIdx.x, &s, &tl);
+    }
+    const SegDev &sd = segs[s];
+    // the pointers are fetched whether or not this wavefront has a source / destination (the arrays hold kMaxFan
+    // entries and a workgroup at most as many wavefronts)
+    const char *src_base = sd.src[w];
+    char *dst_base = sd.dst[w];
+    const uint32_t nsrc = sd.nsrc;
+    const uint32_t ndst = sd.ndst;
+    const uint32_t head = sd.head;
+    const uint32_t shift = sd.shift;
+    const uint64_t count = sd.count;
+    const uint32_t flips = sd.tree_codes;
+    const uint64_t body = count - head;
+    const uint64_t nvec = body / NV;
+    const uint32_t rem = static_cast<uint32_t>(body % NV);
+    const uint32_t head_bytes = head * (16 / NV);
+    const uint64_t TV = waves_tile_vecs(static_cast<int>(pieces));
+    const bool loads = w < nsrc;
+    const bool stores = w < ndst;
+    // vectors in front of a shifted segment wrap below zero and fail the bound check like those behind its end; a
+    // lane outside the segment loads the segment's first vector and stores nothing
+    const uint64_t v_first = tl * TV + lane - shift;
+    const char *src = src_base + head_bytes;
+    char *dst = dst_base + head_bytes;
+    // the load of the next piece is issued before the current one is folded
+    u32x4 next = {0, 0, 0, 0};
+    if (loads && nvec != 0) next = ld16(src + (v_first < nvec ? v_first : 0) * 16);
+    if (nvec != 0) {
+#pragma unroll 1
+        for (uint32_t i = 0; i < pieces; ++i) {
+            const uint64_t v = v_first + static_cast<uint64_t>(i) * kWaveLanes;
+            // the whole piece lies outside the segment (the tile grid is rounded up): every wavefront sees the same
+            if (tl * TV + static_cast<uint64_t>(i) * kWaveLanes >= nvec + shift) break;
+            u32x4 *buf = s_piece + (i & 1u) * waves * kWaveLanes;
+            if (loads) {
+                buf[w * kWaveLanes + lane] = next;
+                const uint64_t vn = v + kWaveLanes;
+                if (i + 1 < pieces) next = ld16(src + (vn < nvec ? vn : 0) * 16);
+            }
+            __syncthreads();
+            if (stores && v < nvec) {
+                C acc[NE];
+                switch (nsrc) {
+                    case 4: waves_fold_fixed<DT, OP, MODE, 4>(buf, w, lane, flips, acc); break;
+                    case 8: waves_fold_fixed<DT, OP, MODE, 8>(buf, w, lane, flips, acc); break;
+                    case 12: waves_fold_fixed<DT, OP, MODE, 12>(buf, w, lane, flips, acc); break;
+                    case 16: waves_fold_fixed<DT, OP, MODE, 16>(buf, w, lane, flips, acc); break;
+                    default: waves_fold<DT, OP, MODE>(buf, nsrc, w, lane, flips, acc); break;
+                }
+                st16x(dst + v * 16, V::pack(acc), store_policy);
+            }
+        }
+    }
+    // the last tile (the one that holds vector nvec + shift; said without a division, which takes hundreds of cycles
+    // for 64-bit operands) also takes the elements in front of and behind the vector body, one per thread
+    if (tl * TV <= nvec + shift && nvec + shift < (tl + 1) * TV && threadIdx.x < head + rem) {
+        const uint64_t idx = threadIdx.x < head ? threadIdx.x : head + nvec * NV + (threadIdx.x - head);
+        fold_tail<DT, OP, kMaxFan, MODE>(sd, nsrc, ndst, idx);
+    }
+}
+
 // More than kMaxFan sources or destinations, chain order: the sources are walked in groups of kMaxFan,
 // each group loaded before it is folded in, so the loads in flight per thread stay what the 16-source kernel
 // has.  One vector per thread and tile.
@@ -671,6 +877,8 @@ struct FoldLaunch {
     uint32_t xcd_remap;        // the wide kernels: give each XCD a contiguous eighth of the tiles
     uint32_t store_policy;     // kStoreStream / kStoreThrough
     uint32_t uniform_tiles;    // non-zero: every segment has this many tiles, tile t belongs to segment t / uniform_tiles
+    uint32_t waves = 0;        // non-zero: the one-store-per-wavefront kernel with this many wavefronts per workgroup
+    uint32_t pieces = 1;       // and this many 1 KiB pieces per source and workgroup
     hipStream_t stream;
 };
 

@@ -15,6 +15,20 @@ static hipError_t launch_one(const FoldLaunch &l)
     return hipGetLastError();
 }
 
+template <int DT, int OP, int MODE>
+static hipError_t launch_waves(const FoldLaunch &l)
+{
+    if constexpr (MODE == kFoldChain || MODE == kFoldSelfFirst) {
+        const bool direct = l.nseg <= kFoldDirectSegs || l.uniform_tiles != 0;
+        const size_t lds = waves_lds_bytes(static_cast<int>(l.waves)) + (direct ? 0 : l.nseg * sizeof(uint64_t));
+        HCCLX_LAUNCH((k_fold_waves<DT, OP, MODE>), dim3(static_cast<uint32_t>(l.total_tiles)), dim3(l.waves * kWaveLanes), lds,
+                     l.stream, l.tile_end, static_cast<const SegDev *>(l.segs), l.nseg, l.pieces, l.store_policy, l.uniform_tiles);
+        return hipGetLastError();
+    } else {
+        return hipErrorInvalidValue;
+    }
+}
+
 template <int DT, int OP, int MODE, int U>
 static hipError_t launch_wide_u(const FoldLaunch &l)
 {
@@ -46,6 +60,7 @@ hipError_t fold_dispatch_copy(const FoldLaunch &l)
 template <int OP, int MODE>
 static hipError_t by_fan(int maxn, const FoldLaunch &l)
 {
+    if (l.waves != 0 && maxn <= kMaxFan) return launch_waves<HCCLX_DT, OP, MODE>(l);
     switch (maxn) {
         case 2: return launch_one<HCCLX_DT, OP, 2, MODE>(l);
         case 4: return launch_one<HCCLX_DT, OP, 4, MODE>(l);

@@ -21,7 +21,10 @@ constexpr uint32_t kMaxVRanks = 64;
 constexpr int kA2avUnroll = HCCLX_A2AV_UNROLL;
 constexpr int kAgvUnroll = HCCLX_AGV_UNROLL;
 // The copies that write one output at a time (large AllGatherV, fan-out of a fold's result): 8 KiB tiles.
-constexpr int kPhasedUnroll = 2;
+#ifndef HCCLX_PHASED_UNROLL
+#define HCCLX_PHASED_UNROLL 2
+#endif
+constexpr int kPhasedUnroll = HCCLX_PHASED_UNROLL;
 
 // Tiles of a block of `bytes` bytes whose first destination byte sits at address `dst`.  Stores are
 // aligned: the bytes before the first 16-byte boundary of dst (head) and after the last whole vector

@@ -81,7 +81,7 @@ template <bool kCached>
 __device__ __forceinline__ u32x4 ld16c(const char *p)
 {
     if constexpr (kCached) {
-        return *reinterpret_cast<const u32x4_u *>(p);
+        return ld16_cached(p);
     } else {
         return ld16(p);
     }

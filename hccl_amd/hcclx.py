@@ -51,6 +51,21 @@ def init():
     check(_lib.load().hcclx_init())
 
 
+def tune(name, value):
+    """Sets a launch-policy knob of the current device (hcclx_tune); plans made before keep their kernels."""
+    L = _lib.load()
+    L.hcclx_tune.argtypes = [ctypes.c_char_p, ctypes.c_uint64]
+    L.hcclx_tune.restype = ctypes.c_int
+    check(L.hcclx_tune(name.encode(), int(value)))
+
+
+def kernels_launched():
+    """Kernels the calling thread has launched through the library so far."""
+    L = _lib.load()
+    L.hcclx_kernels_launched.restype = ctypes.c_uint64
+    return int(L.hcclx_kernels_launched())
+
+
 def fold(segs, dtype, op=0, mode=FOLD_CHAIN, stream=0):
     arr, n = make_segs(segs)
     check(_lib.load().hcclx_fold(arr, n, int(dtype), int(op), int(mode), ctypes.c_void_p(stream)))

@@ -87,6 +87,18 @@ int hcclx_init(void);
 /* Text of the last error raised on this thread ("" if none). */
 const char *hcclx_last_error(void);
 
+/* Sets one of the launch-policy knobs of the current device at run time (the same knobs the HCCLX_* environment
+ * variables set when the device context is made; name = the variable's name without the prefix, lower case):
+ *   "waves_from"      bytes written from which self-first folds take the one-store-per-wavefront kernel (0 = never)
+ *   "waves_max_fan"   widest segment (sources / destinations) that kernel is used for (2..16)
+ *   "waves_chains"    non-zero: chains whose value goes to several places take it too
+ *   "waves_pieces"    1 KiB pieces per source and workgroup (0 = the default)
+ *   "fanout_from"     bytes read and written from which a fold with several destinations is split into fold + fan-out
+ *   "store_through_upto"  bytes written up to which multi-destination folds store through the L2
+ * Plans made before the call keep the kernels they were made for.  Returns HCCL_E_PARA for an unknown name or a
+ * value out of range.  No counterpart in the reference. */
+int hcclx_tune(const char *name, uint64_t value);
+
 /* Number of GPU kernels the calling host thread has launched through this library so far (a running count; take
  * the difference around a call to learn how many kernels it made -- a fold whose result fans out to many places is
  * two, a large AllGatherV one per length class of its runs).  No counterpart in the reference. */
