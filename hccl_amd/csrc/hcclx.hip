@@ -397,6 +397,7 @@ struct Batch {
     uint32_t store_policy = kStoreStream;   // how the fold kernels store (fold.h)
     uint32_t waves = 0;          // non-zero: the one-store-per-wavefront kernel, this many wavefronts per workgroup
     uint32_t pieces = 1;         // and this many 1 KiB pieces per source and workgroup
+    uint32_t waves_fixed = 0;    // and, when every segment has the same number of sources, that number
     size_t nseg() const { return segs.size() + wide.size(); }
     size_t bytes() const
     {
@@ -702,14 +703,19 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
     return HCCL_SUCCESS;
 }
 
-// The n orders of a self-first fold take the kernel in which every wavefront issues one store (fold.h) when the
-// launch writes waves_from bytes or more and its widest segment has at most waves_max_fan sources: measured against
-// the register kernel on fp32 PROD, 64 MiB per rank: 4 ranks 78.7 against 93.5 us, 8 ranks 188 against 203; from
-// twelve ranks on its LDS traffic (every wavefront reads every source piece) takes the gain away (12 ranks: 313
-// against 299 us), and below 16 MiB per rank the shorter workgroups of the register kernel win.  Chains whose value
-// goes to several places run on it too when asked for (waves_chains; off: as one pass it measured 189 to 245 us on
-// the 8 x 64 MiB AllReduce against 172 for the fold + fan-out pair).  Returns the number of wavefronts per workgroup
-// (the widest segment's sources or destinations), 0 = the register kernels.
+// The n orders of a self-first fold take the kernel in which every wavefront issues one store (fold.h) when all
+// segments have the same number of ranks, at most waves_max_fan, and the launch writes waves_from bytes or more.
+// Measured against the register kernel on fp32 PROD (us, register : wavefronts): 4 ranks x 64 MiB 97.7 : 77.4,
+// 8 x 64 MiB 210 : 175, 12 x 64 MiB 281 : 270, 12 x 256 MiB 1183 : 1056, 16 x 256 MiB 1582 : 1445, and at
+// 256 KiB per rank 5.0-5.6 : 3.5 among 7 to 12 ranks (a shorter prologue).  Where the register kernel measured
+// better it stays: two ranks below 32 MiB per rank (no difference), seven and eight ranks between 3 and 12 MiB per
+// rank (8 x 4 MiB: 10.6 : 12.1).  Pieces per workgroup: two up to eight ranks and for small launches, else four,
+// and eight between 2 and 12 MiB per rank (12 x 8 MiB: 35.6 / 36.4 / 32.3 us with 2 / 4 / 8 pieces).  Launches
+// whose segments differ in their number of ranks run on the instance that reads the count per segment, which only
+// wins up to eight ranks.  Chains whose value goes to several places run on this kernel only when asked for
+// (waves_chains; as one pass the 8 x 64 MiB AllReduce measured 189 to 245 us against 172 for fold + fan-out).
+// Returns the number of wavefronts per workgroup (the widest segment's sources or destinations), 0 = the register
+// kernels.
 uint32_t waves_for(const DeviceCtx *ctx, const hcclx_seg_t *segs, uint32_t nseg, int dtype, int mode, uint32_t *pieces)
 {
     if (ctx == nullptr || ctx->waves_from == 0 || nseg == 0) return 0;
@@ -717,20 +723,31 @@ uint32_t waves_for(const DeviceCtx *ctx, const hcclx_seg_t *segs, uint32_t nseg,
     const uint64_t esz = static_cast<uint64_t>(dtype_size(dtype));
     uint32_t most_src = 0;
     uint32_t most_dst = 0;
+    uint32_t least_src = ~0u;
     uint64_t written = 0;
     uint64_t tiles = 0;
     for (uint32_t i = 0; i < nseg; ++i) {
         if (segs[i].nsrc == 0 || segs[i].nsrc > HCCLX_MAX_FAN || segs[i].ndst == 0 || segs[i].ndst > HCCLX_MAX_FAN) return 0;
+        if (segs[i].count == 0) continue;
         most_src = segs[i].nsrc > most_src ? segs[i].nsrc : most_src;
+        least_src = segs[i].nsrc < least_src ? segs[i].nsrc : least_src;
         most_dst = segs[i].ndst > most_dst ? segs[i].ndst : most_dst;
         written += segs[i].count * esz * segs[i].ndst;
         tiles += segs[i].count * esz / 1024 + 2;
     }
     const uint32_t widest = most_src > most_dst ? most_src : most_dst;
     if (most_src < 2 || most_dst < 2 || widest > ctx->waves_max_fan || written < ctx->waves_from || esz == 0) return 0;
-    // pieces per workgroup: four measured best at every width (a workgroup lives a few microseconds: fewer pieces and
-    // its set-up shows, more and the wavefronts issue too many stores in a row again)
-    const uint32_t p = ctx->waves_pieces != 0 ? ctx->waves_pieces : 4u;
+    const bool same = least_src == most_src;
+    if (!same && widest > 8) return 0;
+    const uint64_t per_place = written / most_dst;
+    uint32_t p = ctx->waves_pieces;
+    if (p == 0) {   // the shipped policy; a forced piece count takes every launch that passed the tests above
+        if (mode == HCCLX_FOLD_SELF_FIRST) {
+            if (widest == 2 && per_place < (32ull << 20)) return 0;
+            if ((widest == 7 || widest == 8) && per_place >= (3ull << 20) && per_place < (12ull << 20)) return 0;
+        }
+        p = (widest <= 8 || per_place < (2ull << 20)) ? 2u : per_place < (12ull << 20) ? 8u : 4u;
+    }
     if (tiles / p > 0x7fffffffull) return 0;   // one workgroup per tile: the grid has to hold them
     *pieces = p;
     return widest;
@@ -784,6 +801,17 @@ int build_batches_impl(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op
     proto.maxn = sp.maxn;
     proto.waves = sp.waves;
     proto.pieces = sp.pieces;
+    if (sp.waves != 0) {
+        // the kernel instance compiled for one source count takes launches whose segments all have it
+        uint32_t common = 0;
+        bool same = true;
+        for (uint32_t i = 0; i < nseg; ++i) {
+            if (segs[i].count == 0) continue;
+            if (common == 0) common = segs[i].nsrc;
+            same = same && segs[i].nsrc == common;
+        }
+        proto.waves_fixed = same ? common : 0;
+    }
     proto.store_policy = store_policy_for(device_ctx(), segs, nseg, sp.copy ? 1 : dtype_size(dtype));
     Batch cur = proto;
     for (uint32_t i = 0; i < nseg; ++i) {
@@ -1032,6 +1060,7 @@ int launch_batch(const DeviceCtx *ctx, const Batch &b, const char *d_table, hipS
     l.uniform_tiles = uniform_tiles_of(b.tile_end.data(), b.tile_end.size());
     l.waves = b.waves;
     l.pieces = b.pieces;
+    l.waves_fixed = b.waves_fixed;
     l.stream = stream;
     const hipError_t e = b.copy ? fold_dispatch_copy(l) : dispatch_fold(b.dtype, b.op, b.maxn, b.mode, l);
     if (e != hipSuccess) return fail_hip(e, "fold kernel launch");

@@ -58,11 +58,11 @@ struct DeviceCtx {
     // of a run of a source are written one after the other, each workgroup writing one output.
     uint64_t agv_phased_from = 4ull << 20;
     // The n orders of a self-first fold among up to waves_max_fan ranks (HCCLX_WAVES_MAX_FAN) take the kernel with one
-    // wavefront per source / destination, in which every wavefront issues a single store per piece, from this many
-    // bytes written by the launch (HCCLX_WAVES_FROM, 0 = never); waves_chains (HCCLX_WAVES_CHAINS): also chains whose
-    // value goes to several places; waves_pieces (HCCLX_WAVES_PIECES): 1 KiB pieces per source and workgroup, 0 = 4.
-    uint64_t waves_from = 128ull << 20;
-    uint32_t waves_max_fan = 8;
+    // store per wavefront when the launch writes waves_from bytes or more (HCCLX_WAVES_FROM, 0 = never); waves_chains
+    // (HCCLX_WAVES_CHAINS): also chains whose value goes to several places; waves_pieces (HCCLX_WAVES_PIECES): 1 KiB
+    // pieces per source and workgroup, 0 = chosen per launch (2, 4 or 8).
+    uint64_t waves_from = 1ull << 20;
+    uint32_t waves_max_fan = 16;
     bool waves_chains = false;
     uint32_t waves_pieces = 0;
     uint64_t store_through_upto = 320ull << 20;   // fold launches with several destinations that write no more than this store through the L2 (HCCLX_STORE_THROUGH_UPTO)

@@ -15,15 +15,42 @@ static hipError_t launch_one(const FoldLaunch &l)
     return hipGetLastError();
 }
 
+template <int DT, int OP, int MODE, int NFIX>
+static hipError_t launch_waves_n(const FoldLaunch &l)
+{
+    const bool direct = l.nseg <= kFoldDirectSegs || l.uniform_tiles != 0;
+    const size_t lds = waves_lds_bytes(static_cast<int>(l.waves)) + (direct ? 0 : l.nseg * sizeof(uint64_t));
+    HCCLX_LAUNCH((k_fold_waves<DT, OP, MODE, NFIX>), dim3(static_cast<uint32_t>(l.total_tiles)), dim3(l.waves * kWaveLanes), lds,
+                 l.stream, l.tile_end, static_cast<const SegDev *>(l.segs), l.nseg, l.pieces, l.store_policy, l.uniform_tiles);
+    return hipGetLastError();
+}
+
+// The self-first orders get an instance per rank count up to twelve (the widest the launch policy takes by itself);
+// chains, and wider or mixed launches, run on the instance that reads the count per segment.
 template <int DT, int OP, int MODE>
 static hipError_t launch_waves(const FoldLaunch &l)
 {
-    if constexpr (MODE == kFoldChain || MODE == kFoldSelfFirst) {
-        const bool direct = l.nseg <= kFoldDirectSegs || l.uniform_tiles != 0;
-        const size_t lds = waves_lds_bytes(static_cast<int>(l.waves)) + (direct ? 0 : l.nseg * sizeof(uint64_t));
-        HCCLX_LAUNCH((k_fold_waves<DT, OP, MODE>), dim3(static_cast<uint32_t>(l.total_tiles)), dim3(l.waves * kWaveLanes), lds,
-                     l.stream, l.tile_end, static_cast<const SegDev *>(l.segs), l.nseg, l.pieces, l.store_policy, l.uniform_tiles);
-        return hipGetLastError();
+    if constexpr (MODE == kFoldSelfFirst) {
+        switch (l.waves_fixed) {
+            case 2: return launch_waves_n<DT, OP, MODE, 2>(l);
+            case 3: return launch_waves_n<DT, OP, MODE, 3>(l);
+            case 4: return launch_waves_n<DT, OP, MODE, 4>(l);
+            case 5: return launch_waves_n<DT, OP, MODE, 5>(l);
+            case 6: return launch_waves_n<DT, OP, MODE, 6>(l);
+            case 7: return launch_waves_n<DT, OP, MODE, 7>(l);
+            case 8: return launch_waves_n<DT, OP, MODE, 8>(l);
+            case 9: return launch_waves_n<DT, OP, MODE, 9>(l);
+            case 10: return launch_waves_n<DT, OP, MODE, 10>(l);
+            case 11: return launch_waves_n<DT, OP, MODE, 11>(l);
+            case 12: return launch_waves_n<DT, OP, MODE, 12>(l);
+            case 13: return launch_waves_n<DT, OP, MODE, 13>(l);
+            case 14: return launch_waves_n<DT, OP, MODE, 14>(l);
+            case 15: return launch_waves_n<DT, OP, MODE, 15>(l);
+            case 16: return launch_waves_n<DT, OP, MODE, 16>(l);
+            default: return launch_waves_n<DT, OP, MODE, 0>(l);
+        }
+    } else if constexpr (MODE == kFoldChain) {
+        return launch_waves_n<DT, OP, MODE, 0>(l);
     } else {
         return hipErrorInvalidValue;
     }

@@ -92,7 +92,8 @@ const char *hcclx_last_error(void);
  *   "waves_from"      bytes written from which self-first folds take the one-store-per-wavefront kernel (0 = never)
  *   "waves_max_fan"   widest segment (sources / destinations) that kernel is used for (2..16)
  *   "waves_chains"    non-zero: chains whose value goes to several places take it too
- *   "waves_pieces"    1 KiB pieces per source and workgroup (0 = the default)
+ *   "waves_pieces"    1 KiB pieces per source and workgroup (0 = chosen per launch; another value also takes the
+ *                     launches for which the register kernel is otherwise kept)
  *   "fanout_from"     bytes read and written from which a fold with several destinations is split into fold + fan-out
  *   "store_through_upto"  bytes written up to which multi-destination folds store through the L2
  * Plans made before the call keep the kernels they were made for.  Returns HCCL_E_PARA for an unknown name or a

@@ -13,7 +13,7 @@ from gpu_util import DevBuf, assert_same_bits, fold_oracle, fused_is_wide, paylo
 
 pytestmark = pytest.mark.gpu
 
-DEFAULTS = {"waves_from": 128 << 20, "waves_max_fan": 8, "waves_chains": 0, "waves_pieces": 0}
+DEFAULTS = {"waves_from": 1 << 20, "waves_max_fan": 16, "waves_chains": 0, "waves_pieces": 0}
 
 
 @pytest.fixture()
@@ -120,8 +120,7 @@ def test_chains_to_several_places_on_the_wavefront_kernel(waves_everywhere, nsrc
 
 
 def test_in_place_self_first_and_the_default_policy(waves_everywhere):
-    """sendBuf == recvBuf on every rank (each destination is one of the sources), then the policy as shipped: the
-    wavefront kernel is taken for self-first folds among at most eight ranks that write 128 MiB or more."""
+    """sendBuf == recvBuf on every rank (each destination is one of the sources); the knobs refuse values out of range."""
     rng = np.random.default_rng(5)
     n, nsrc = 100003, 8
     xs = [payload(rng, T.FP32, n, "uniform") for _ in range(nsrc)]
@@ -136,6 +135,29 @@ def test_in_place_self_first_and_the_default_policy(waves_everywhere):
         hcclx.tune("waves_max_fan", 17)
     with pytest.raises(HcclError):
         hcclx.tune("no_such_knob", 1)
+
+
+def test_self_first_segments_of_different_widths_in_one_launch(waves_everywhere):
+    """Segments of 3, 8 and 5 ranks in one launch: the kernel instance that reads the rank count per segment."""
+    rng = np.random.default_rng(21)
+    segs, checks, outs_all, alive = [], [], [], []
+    for nsrc, n in ((3, 4099), (8, 70001), (5, 13)):
+        xs = [payload(rng, T.FP32, n, "prod") for _ in range(nsrc)]
+        bufs = [DevBuf(x, offset=(k % 2) * 4) for k, x in enumerate(xs)]
+        outs = [DevBuf(nbytes=xs[0].nbytes, offset=(k % 3) * 4) for k in range(nsrc)]
+        segs.append((n, [b.ptr for b in bufs], [o.ptr for o in outs]))
+        checks.append((xs, outs))
+        outs_all += outs
+        alive.append(bufs)
+    got, ref = fold_both(segs, T.FP32, T.PROD, hcclx.FOLD_SELF_FIRST, outs_all)
+    at = 0
+    for xs, outs in checks:
+        for r in range(len(xs)):
+            order = [r] + [k for k in range(len(xs)) if k != r]
+            want = fold_oracle(xs, T.FP32, T.PROD, order, wide=False)
+            assert_same_bits(got[at + r], want, T.FP32, f"{len(xs)} ranks, rank {r}")
+            assert_same_bits(ref[at + r], want, T.FP32, f"register kernel, {len(xs)} ranks, rank {r}")
+        at += len(xs)
 
 
 def test_prod_allreduce_of_four_ranks_takes_the_wavefront_kernel_by_default():
