@@ -453,12 +453,12 @@ WORKLOADS = {
         profile="profiles/k_fold_wide_k_phased_copy_all_reduce_nhr_int32_max_12x64MiB.txt"),
     "all_reduce_prod_fp32_12x64MiB_aicpu_nhr": lambda *a: AllReduce(
         *a, n=12, count=16 * 1024 * 1024, op=a[2].PROD, alg="InsAllReduceAicpuReduceNHR",
-        kernel="hcclx::k_fold<4, 1, 16, 1>",
-        profile="profiles/k_fold_self_first_all_reduce_aicpu_nhr_fp32_prod_12x64MiB.txt"),
+        kernel="hcclx::k_fold_waves<4, 1, 1, 12>",
+        profile="profiles/k_fold_waves_all_reduce_aicpu_nhr_fp32_prod_12x64MiB.txt"),
     # the same template among 8 ranks: eight orders from one pass, on the kernel that gives every wavefront one store
     "all_reduce_prod_fp32_8x64MiB_aicpu_nhr": lambda *a: AllReduce(
         *a, n=8, count=16 * 1024 * 1024, op=a[2].PROD, alg="InsAllReduceAicpuReduceNHR",
-        kernel="hcclx::k_fold_waves<4, 1, 1>",
+        kernel="hcclx::k_fold_waves<4, 1, 1, 8>",
         profile="profiles/k_fold_waves_all_reduce_aicpu_nhr_fp32_prod_8x64MiB.txt"),
     "reduce_scatter_sum_bf16_mesh_32x32MiB": lambda *a: ReduceScatterMesh(*a, n=32, recv=512 * 1024),
     "moe_dispatch_pack_bf16_8x4096x7168": lambda *a: MoeDispatchPack(*a),
@@ -475,8 +475,8 @@ EXTRA_WORKLOADS = {
         profile="profiles/k_fold_wide_k_phased_copy_all_reduce_nhr_int32_max_12x1GiB.txt"),
     "all_reduce_prod_fp32_12x1GiB_aicpu_nhr": lambda *a: AllReduce(
         *a, n=12, count=256 * 1024 * 1024, op=a[2].PROD, alg="InsAllReduceAicpuReduceNHR",
-        kernel="hcclx::k_fold<4, 1, 16, 1>",
-        profile="profiles/k_fold_self_first_all_reduce_aicpu_nhr_fp32_prod_12x1GiB.txt"),
+        kernel="hcclx::k_fold_waves<4, 1, 1, 12>",
+        profile="profiles/k_fold_waves_all_reduce_aicpu_nhr_fp32_prod_12x1GiB.txt"),
 }
 
 
