@@ -521,13 +521,15 @@ def sweep_allreduce_12_ranks(torch, api, T, steps):
             st = Step()
             st.stream_obj = stream_obj
             reps = max(3, min(steps, (1 << 32) // max(nbytes * n, 1)))
-            _, ms = time_steps(torch, st, reps, 2)
+            # bandwidth-bound sizes are run in like the rows of the per-op table (see time_steps)
+            busy = OPS_BUSY_MS if nbytes >= (1 << 24) else 0.0
+            _, ms = time_steps(torch, st, reps, 2, busy_ms=busy)
             info = w.last_info()
             row[name] = {"us": round(ms * 1e3, 1), "GB/s": round(2 * n * nbytes / (ms * 1e-3) / 1e9, 1),
                          "fused": bool(info.fused), "launches": info.launches}
             if nbytes == big:
                 st.stride = big + stagger
-                _, ms = time_steps(torch, st, reps, 2)
+                _, ms = time_steps(torch, st, reps, 2, busy_ms=busy)
                 row[name]["us_buffers_1GiB_plus_8KiB_apart"] = round(ms * 1e3, 1)
                 row[name]["GB/s_buffers_1GiB_plus_8KiB_apart"] = round(2 * n * nbytes / (ms * 1e-3) / 1e9, 1)
                 st.stride = big
@@ -600,18 +602,18 @@ def time_steps(torch, wl, steps, warmup, busy_ms=0.0):
     fold: 265 us per launch, then up to 330, then back to 270 over forty launches); a table row of 25 steps would
     report that transient instead of the kernel."""
     import gc
+    gc.collect()
+    gc.disable()   # a full collection of the interpreter's heap would show up as a 40 ms step, or as an idle gap
     torch.cuda.synchronize()
     for _ in range(warmup):
         wl.step()
     torch.cuda.synchronize()
-    if busy_ms > 0:
+    if busy_ms > 0:   # flows into the timed steps with no more than one synchronisation between them
         t_busy = time.perf_counter()
         while (time.perf_counter() - t_busy) * 1e3 < busy_ms:
             for _ in range(10):
                 wl.step()
             torch.cuda.synchronize()
-    gc.collect()
-    gc.disable()   # a full collection of the interpreter's heap would show up as a 40 ms step
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
