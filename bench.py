@@ -328,9 +328,9 @@ class MoeDispatchPack(Workload):
         self.name = ("moe_combine_bf16_%dx%dx%d" if combine else "moe_dispatch_pack_bf16_%dx%dx%d") % (n, tokens, hidden)
         if one_pass:
             self.name = ("moe_gather_combine_bf16_%dx%dx%d" if combine else "moe_route_dispatch_bf16_%dx%dx%d") % (n, tokens, hidden)
-            self.kernel = "k_moe_gather_long" if combine else "k_moe_scatter_long"
+            self.kernel = "k_moe_gather_long" if combine else "k_moe_scatter_rows<2>"
             self.profile = "profiles/%s_bf16_%dx%dx%d.txt" % ("k_moe_gather_long_combine" if combine
-                                                              else "k_moe_scatter_long_dispatch", n, tokens, hidden)
+                                                              else "k_moe_scatter_rows_dispatch", n, tokens, hidden)
         self.tokens, self.hidden = tokens, hidden
         rng = np.random.default_rng(seed)
         w = 1.0 / np.arange(1, n + 1) ** 1.2

@@ -144,6 +144,7 @@ void init_slot(DeviceSlot *s, int dev)
         c.waves_pieces = b > kWavePieces ? static_cast<uint32_t>(kWavePieces) : static_cast<uint32_t>(b);
     }
     if (const char *v = std::getenv("HCCLX_AGV_PHASED_FROM")) c.agv_phased_from = std::strtoull(v, nullptr, 10);
+    if (const char *v = std::getenv("HCCLX_MOE_SCATTER_ROWS")) c.moe_scatter_rows = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
     if (const char *v = std::getenv("HCCLX_STORE_THROUGH_UPTO")) c.store_through_upto = std::strtoull(v, nullptr, 10);
     c.ring_bytes = kSliceBytes * kSlices;
     e = hipHostMalloc(reinterpret_cast<void **>(&c.h_ring), c.ring_bytes, hipHostMallocDefault);
@@ -1107,6 +1108,9 @@ int hcclx_tune(const char *name, uint64_t value)
         ctx->waves_pieces = static_cast<uint32_t>(value);
     } else if (key == "fanout_from") {
         ctx->fanout_from = value;
+    } else if (key == "moe_scatter_rows") {
+        if (value != 1 && value != 2) return fail(HCCL_E_PARA, "moe_scatter_rows is 1 or 2");
+        ctx->moe_scatter_rows = static_cast<uint32_t>(value);
     } else if (key == "store_through_upto") {
         ctx->store_through_upto = value;
     } else {

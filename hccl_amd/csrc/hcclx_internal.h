@@ -65,6 +65,7 @@ struct DeviceCtx {
     uint32_t waves_max_fan = 16;
     bool waves_chains = false;
     uint32_t waves_pieces = 0;
+    uint32_t moe_scatter_rows = 2;          // MoE dispatch of long rows: entries per workgroup, 1 or 2 (HCCLX_MOE_SCATTER_ROWS)
     uint64_t store_through_upto = 320ull << 20;   // fold launches with several destinations that write no more than this store through the L2 (HCCLX_STORE_THROUGH_UPTO)
     // Descriptor ring: tables of one-shot launches are written to pinned host memory and copied to the
     // device ring on the launch stream just before the kernel.
