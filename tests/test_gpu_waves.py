@@ -160,6 +160,32 @@ def test_self_first_segments_of_different_widths_in_one_launch(waves_everywhere)
         at += len(xs)
 
 
+@pytest.mark.parametrize("ragged", [True, False])
+def test_many_segments_in_one_launch(waves_everywhere, ragged):
+    """150 segments of four ranks cut from four inputs: ragged lengths (more than 64 segments: the tile prefix is staged
+    in LDS and searched there) and equal lengths (a tile's segment follows from a division)."""
+    rng = np.random.default_rng(31 + ragged)
+    nsrc = 4
+    counts = [int(c) for c in (rng.integers(1, 3000, 150) if ragged else [1536] * 150)]
+    total = sum(counts)
+    xs = [payload(rng, T.FP32, total, "prod") for _ in range(nsrc)]
+    bufs = [DevBuf(x) for x in xs]
+    outs = [DevBuf(nbytes=xs[0].nbytes) for _ in range(nsrc)]
+    segs, off = [], 0
+    for c in counts:
+        segs.append((c, [b.ptr + off * 4 for b in bufs], [o.ptr + off * 4 for o in outs]))
+        off += c
+    hcclx.tune("waves_pieces", 2)
+    before = hcclx.kernels_launched()
+    got, ref = fold_both(segs, T.FP32, T.PROD, hcclx.FOLD_SELF_FIRST, outs)
+    assert hcclx.kernels_launched() - before == 2
+    for r in range(nsrc):
+        order = [r] + [k for k in range(nsrc) if k != r]
+        want = fold_oracle(xs, T.FP32, T.PROD, order, wide=False)
+        assert_same_bits(got[r], want, T.FP32, f"rank {r}")
+        assert_same_bits(ref[r], want, T.FP32, f"register kernel, rank {r}")
+
+
 def test_prod_allreduce_of_four_ranks_takes_the_wavefront_kernel_by_default():
     """HcclAllReduce fp32 PROD among four ranks at 32 MiB per rank (the CPU-reduce NHR template: four outputs in four
     orders, 128 MiB written) with the shipped policy, sampled against the oracle; the same collective with the kernel
