@@ -710,8 +710,10 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
 // 8 x 64 MiB 210 : 175, 12 x 64 MiB 281 : 270, 12 x 256 MiB 1183 : 1056, 16 x 256 MiB 1582 : 1445, and at
 // 256 KiB per rank 5.0-5.6 : 3.5 among 7 to 12 ranks (a shorter prologue).  Where the register kernel measured
 // better it stays: two ranks below 32 MiB per rank (no difference), seven and eight ranks between 3 and 12 MiB per
-// rank (8 x 4 MiB: 10.6 : 12.1).  Pieces per workgroup: two up to eight ranks and for small launches, else four,
-// and eight between 2 and 12 MiB per rank (12 x 8 MiB: 35.6 / 36.4 / 32.3 us with 2 / 4 / 8 pieces).  Launches
+// rank (8 x 4 MiB: 10.6 : 12.1).  Pieces per workgroup: two for small launches and up to four ranks; five to eight
+// ranks four below 32 MiB per rank (8 x 16 MiB: 47.9 / 43.0 us with 2 / 4) and two from there on (8 x 64 MiB:
+// 168.8 / 182.6); nine and more eight below 12 MiB per rank (12 x 8 MiB: 35.6 / 36.4 / 32.3 us with 2 / 4 / 8) and
+// four from there on (12 x 64 MiB: 268.7 / 260.6 / 281.7).  Launches
 // whose segments differ in their number of ranks run on the instance that reads the count per segment, which only
 // wins up to eight ranks.  Chains whose value goes to several places run on this kernel only when asked for
 // (waves_chains; as one pass the 8 x 64 MiB AllReduce measured 189 to 245 us against 172 for fold + fan-out).
@@ -747,7 +749,13 @@ uint32_t waves_for(const DeviceCtx *ctx, const hcclx_seg_t *segs, uint32_t nseg,
             if (widest == 2 && per_place < (32ull << 20)) return 0;
             if ((widest == 7 || widest == 8) && per_place >= (3ull << 20) && per_place < (12ull << 20)) return 0;
         }
-        p = (widest <= 8 || per_place < (2ull << 20)) ? 2u : per_place < (12ull << 20) ? 8u : 4u;
+        if (per_place < (2ull << 20) || widest <= 4) {
+            p = 2;
+        } else if (widest <= 8) {
+            p = per_place < (32ull << 20) ? 4u : 2u;
+        } else {
+            p = per_place < (12ull << 20) ? 8u : 4u;
+        }
     }
     if (tiles / p > 0x7fffffffull) return 0;   // one workgroup per tile: the grid has to hold them
     *pieces = p;
