@@ -90,6 +90,17 @@ int main(int argc, char **argv)
                 if (all_ranks()) return 1;   // the first call plans the launch
             }
             CHECK_HIP(hipStreamSynchronize(stream));
+            if (bytes >= (1u << 20)) {
+                // sizes whose kernel outweighs the launch: 20 ms of the same collective first, so that the figure is
+                // that of a busy GPU and not of the clock transient after an idle period
+                const auto r0 = std::chrono::steady_clock::now();
+                while (std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - r0).count() < 20.0) {
+                    for (int k = 0; k < 20; ++k) {
+                        if (all_ranks()) return 1;
+                    }
+                    CHECK_HIP(hipStreamSynchronize(stream));
+                }
+            }
             CHECK_HIP(hipEventRecord(t0, stream));
             const auto h0 = std::chrono::steady_clock::now();
             for (int k = 0; k < reps; ++k) {
