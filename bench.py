@@ -455,6 +455,16 @@ WORKLOADS = {
         *a, n=12, count=16 * 1024 * 1024, op=a[2].PROD, alg="InsAllReduceAicpuReduceNHR",
         kernel="hcclx::k_fold_waves<4, 1, 1, 12>",
         profile="profiles/k_fold_waves_all_reduce_aicpu_nhr_fp32_prod_12x64MiB.txt"),
+    # benchmark configuration 5 names the halving-doubling template: the same two collectives through it (for fp32 its
+    # schedule is a tree per slice, folded by the tree kernel, then handed out one output at a time)
+    "all_reduce_max_int32_12x64MiB_rhd": lambda *a: AllReduce(
+        *a, n=12, count=16 * 1024 * 1024, dtype=a[2].INT32, op=a[2].MAX, alg="InsAllReduceRHD",
+        kernel="hcclx::k_fold_wide<2, 2, 0, 4> + k_phased_copy",
+        profile="profiles/k_fold_wide_k_phased_copy_all_reduce_rhd_int32_max_12x64MiB.txt"),
+    "all_reduce_prod_fp32_12x64MiB_rhd": lambda *a: AllReduce(
+        *a, n=12, count=16 * 1024 * 1024, op=a[2].PROD, alg="InsAllReduceRHD",
+        kernel="hcclx::k_fold<4, 1, 16, 2> + k_phased_copy",
+        profile="profiles/k_fold_tree_k_phased_copy_all_reduce_rhd_fp32_prod_12x64MiB.txt"),
     # the same template among 8 ranks: eight orders from one pass, on the kernel that gives every wavefront one store
     "all_reduce_prod_fp32_8x64MiB_aicpu_nhr": lambda *a: AllReduce(
         *a, n=8, count=16 * 1024 * 1024, op=a[2].PROD, alg="InsAllReduceAicpuReduceNHR",
@@ -645,6 +655,8 @@ SHORT = {
     "all_reduce_max_int32_12x64MiB_nhr": "ar_i32max_12x64M_nhr",
     "all_reduce_prod_fp32_12x64MiB_aicpu_nhr": "ar_f32prod_12x64M",
     "all_reduce_prod_fp32_8x64MiB_aicpu_nhr": "ar_f32prod_8x64M",
+    "all_reduce_max_int32_12x64MiB_rhd": "ar_i32max_12x64M_rhd",
+    "all_reduce_prod_fp32_12x64MiB_rhd": "ar_f32prod_12x64M_rhd",
     "reduce_scatter_sum_bf16_mesh_32x32MiB": "rs_bf16_32x32M",
     "moe_dispatch_pack_bf16_8x4096x7168": "moe_pack",
     "moe_combine_bf16_8x4096x7168": "moe_combine",
