@@ -590,7 +590,7 @@ bool make_segdev(const hcclx_seg_t &s, const SegProto &sp, int mode, SegDev *out
     }
     if (sp.mode == HCCLX_FOLD_TREE && !embed_tree(s, static_cast<uint32_t>(sp.maxn), &sd)) return false;
     const int ne = sp.copy ? 16 : 16 / sp.esz;
-    const uint64_t tile_vecs = sp.waves != 0 ? waves_tile_vecs(static_cast<int>(sp.pieces)) : fold_tile_vecs(sp.maxn);
+    const uint64_t tile_vecs = sp.waves != 0 ? waves_tile_vecs(static_cast<int>(sp.pieces)) : fold_tile_vecs(sp.maxn, sp.mode);
     sd.head = fold_head_of(sd.count, sp.copy ? 1 : sp.esz, sd.dst[0]);
     sd.shift = fold_shift_of(sd.head, sp.copy ? 1 : sp.esz, tile_vecs, sd.dst[0]);
     *tiles = fold_tiles_of(sd.count, ne, tile_vecs, sd.head, sd.shift);

@@ -34,14 +34,20 @@ constexpr int kWideGroup = 8;
 constexpr int kWideUnrollMany = 2;   // several destinations
 constexpr int kWideUnrollOne = 4;    // one destination
 constexpr uint32_t kFoldDirectSegs = 64;   // up to this many segments the tile prefix is searched in place
-__host__ __device__ constexpr int fold_unroll(int maxn)
+#ifndef HCCLX_TREE16_UNROLL
+#define HCCLX_TREE16_UNROLL 1   // vectors per thread of the tree over up to 16 leaf slots
+#endif
+static_assert(kFoldTree == 2, "fold_unroll names the tree mode by its number");
+// mode: a FoldMode (segtab.h)
+__host__ __device__ constexpr int fold_unroll(int maxn, int mode)
 {
     constexpr int u[5] = {HCCLX_FOLD_UNROLLS};
+    if (mode == 2 /* kFoldTree */ && maxn > 8) return HCCLX_TREE16_UNROLL;
     return maxn <= 1 ? u[0] : maxn <= 2 ? u[1] : maxn <= 4 ? u[2] : maxn <= 8 ? u[3] : u[4];
 }
-__host__ __device__ constexpr uint64_t fold_tile_vecs(int maxn)
+__host__ __device__ constexpr uint64_t fold_tile_vecs(int maxn, int mode)
 {
-    return static_cast<uint64_t>(kFoldThreads) * fold_unroll(maxn);
+    return static_cast<uint64_t>(kFoldThreads) * fold_unroll(maxn, mode);
 }
 // Tiles of the wide kernels: `unroll` vectors per thread (the chain: kWideUnrollMany or kWideUnrollOne; the
 // self-first and tree orders: 1).
@@ -142,7 +148,7 @@ template <int DT, int OP, int MAXN, int MODE, bool CHECK>
 __device__ __forceinline__ void fold_tile(const SegDev &sd, uint32_t nsrc, uint32_t ndst, uint64_t v0, uint64_t nvec,
                                           uint32_t head_bytes, uint32_t policy)
 {
-    constexpr int UNROLL = fold_unroll(MAXN);
+    constexpr int UNROLL = fold_unroll(MAXN, MODE);
     using V = Vec16<DT>;
     using C = typename V::C;
     constexpr int NE = V::NE;
@@ -353,7 +359,7 @@ k_fold(const uint64_t *__restrict__ tile_end, const SegDev *__restrict__ segs, u
 {
     const uint32_t policy = store_policy;
     constexpr int NE = Vec16<DT>::kElems;   // elements per 16-byte vector
-    constexpr uint64_t TV = fold_tile_vecs(MAXN);
+    constexpr uint64_t TV = fold_tile_vecs(MAXN, MODE);
     extern __shared__ uint64_t s_end[];  // nseg entries, sized by the launcher
     // Few segments: the prefix is searched where it lies (every index is wave-uniform, so these are scalar
     // loads that hit the constant cache after the first workgroup); staging it in LDS would cost a barrier
