@@ -9,8 +9,8 @@ the time of a step.
 
 Output: the LAST line of stdout is the benchmark line, one compact JSON object (under 2000 bytes: metric, value,
 roofline, cpu_baseline and one percentage per op).  The tables behind it (per-op rows, the 12-rank size sweep,
-small-message and planning times from C++) are printed before it, one JSON object per line, and written to
-gpurun_out/bench_details.json.
+small-message and planning times from C++) are printed before it, one JSON object per line, and written to the
+file DETAILS_FILE names.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--no-ops] [--no-sweep]
 """
@@ -710,15 +710,17 @@ def benchmark_line(args, wl, wall_ms, ev_ms, traffic, cpu=None, ops=None, small=
     return text
 
 
+DETAILS_FILE = os.path.join(ROOT, "gpurun_out", "bench_details.json")
+
+
 def emit_details(details):
     """The tables behind the benchmark line: one JSON object per line on stdout (before the benchmark line) and
-    the whole of it in gpurun_out/bench_details.json when that folder can be written."""
+    the whole of it in DETAILS_FILE when its folder can be written."""
     for key, val in details.items():
         print(json.dumps({"detail": key, "data": val}))
     try:
-        out = os.path.join(ROOT, "gpurun_out")
-        os.makedirs(out, exist_ok=True)
-        with open(os.path.join(out, "bench_details.json"), "w") as f:
+        os.makedirs(os.path.dirname(DETAILS_FILE), exist_ok=True)
+        with open(DETAILS_FILE, "w") as f:
             json.dump(details, f, indent=1)
     except OSError:
         pass
