@@ -97,8 +97,9 @@ const char *hcclx_last_error(void);
  *   "fanout_from"     bytes read and written from which a fold with several destinations is split into fold + fan-out
  *   "store_through_upto"  bytes written up to which multi-destination folds store through the L2
  *   "moe_scatter_rows"  entries per workgroup of the MoE dispatch of long rows (1 or 2)
- * Plans made before the call keep the kernels they were made for.  Returns HCCL_E_PARA for an unknown name or a
- * value out of range.  No counterpart in the reference. */
+ * Plans made before the call keep the kernels they were made for.  The knobs are plain fields of the device's
+ * context: set them while no other thread is planning a launch on that device.  Returns HCCL_E_PARA for an unknown
+ * name or a value out of range.  No counterpart in the reference. */
 int hcclx_tune(const char *name, uint64_t value);
 
 /* Number of GPU kernels the calling host thread has launched through this library so far (a running count; take
