@@ -708,7 +708,8 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
 // segments have the same number of ranks, at most waves_max_fan, and the launch writes waves_from bytes or more.
 // Measured against the register kernel on fp32 PROD (us, register : wavefronts): 4 ranks x 64 MiB 97.7 : 77.4,
 // 8 x 64 MiB 210 : 175, 12 x 64 MiB 281 : 270, 12 x 256 MiB 1183 : 1056, 16 x 256 MiB 1582 : 1445, and at
-// 256 KiB per rank 5.0-5.6 : 3.5 among 7 to 12 ranks (a shorter prologue).  Where the register kernel measured
+// 256 KiB per rank and below 4.6-5.6 : 3.2-3.5 among 8 to 12 ranks (at 4 KiB per rank: 4 ranks 3.9 : 3.1, 16 ranks
+// 5.3 : 3.9; the register kernel's threads each walk all the sources, here the wavefronts share them).  Where the register kernel measured
 // better it stays: two ranks below 32 MiB per rank (no difference), seven and eight ranks between 3 and 12 MiB per
 // rank (8 x 4 MiB: 10.6 : 12.1).  Pieces per workgroup: two for small launches and up to four ranks; five to eight
 // ranks four below 32 MiB per rank (8 x 16 MiB: 47.9 / 43.0 us with 2 / 4) and two from there on (8 x 64 MiB:

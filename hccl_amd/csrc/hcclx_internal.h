@@ -61,7 +61,7 @@ struct DeviceCtx {
     // store per wavefront when the launch writes waves_from bytes or more (HCCLX_WAVES_FROM, 0 = never); waves_chains
     // (HCCLX_WAVES_CHAINS): also chains whose value goes to several places; waves_pieces (HCCLX_WAVES_PIECES): 1 KiB
     // pieces per source and workgroup, 0 = chosen per launch (2, 4 or 8).
-    uint64_t waves_from = 1ull << 20;
+    uint64_t waves_from = 1;
     uint32_t waves_max_fan = 16;
     bool waves_chains = false;
     uint32_t waves_pieces = 0;

@@ -13,7 +13,7 @@ from gpu_util import DevBuf, assert_same_bits, fold_oracle, fused_is_wide, paylo
 
 pytestmark = pytest.mark.gpu
 
-DEFAULTS = {"waves_from": 1 << 20, "waves_max_fan": 16, "waves_chains": 0, "waves_pieces": 0}
+DEFAULTS = {"waves_from": 1, "waves_max_fan": 16, "waves_chains": 0, "waves_pieces": 0}
 
 
 @pytest.fixture()
