@@ -716,14 +716,17 @@ int build_batches(const hcclx_seg_t *segs, uint32_t nseg, int dtype, int op, int
 // 168.8 / 182.6); nine and more eight below 12 MiB per rank (12 x 8 MiB: 35.6 / 36.4 / 32.3 us with 2 / 4 / 8) and
 // four from there on (12 x 64 MiB: 268.7 / 260.6 / 281.7).  Launches
 // whose segments differ in their number of ranks run on the instance that reads the count per segment, which only
-// wins up to eight ranks.  Chains whose value goes to several places run on this kernel only when asked for
-// (waves_chains; as one pass the 8 x 64 MiB AllReduce measured 189 to 245 us against 172 for fold + fan-out).
+// wins up to eight ranks.  Chains whose value goes to several places (integer one-shot AllReduce, two-shot, NHR of
+// integers) take this kernel up to 256 KiB per place, where its prologue is the shorter one (12 ranks: 3.4-3.6
+// against 3.9-4.3 us for one segment, 5.0-6.2 against 5.9-6.8 for twelve slices; from 1 MiB per place on the register
+// kernels win: 4.9 against 5.5), and beyond only when asked for (waves_chains; as one pass the 8 x 64 MiB AllReduce
+// measured 189 to 245 us against 172 for fold + fan-out).
 // Returns the number of wavefronts per workgroup (the widest segment's sources or destinations), 0 = the register
 // kernels.
 uint32_t waves_for(const DeviceCtx *ctx, const hcclx_seg_t *segs, uint32_t nseg, int dtype, int mode, uint32_t *pieces)
 {
     if (ctx == nullptr || ctx->waves_from == 0 || nseg == 0) return 0;
-    if (mode != HCCLX_FOLD_SELF_FIRST && !(mode == HCCLX_FOLD_CHAIN && ctx->waves_chains)) return 0;
+    if (mode != HCCLX_FOLD_SELF_FIRST && mode != HCCLX_FOLD_CHAIN) return 0;
     const uint64_t esz = static_cast<uint64_t>(dtype_size(dtype));
     uint32_t most_src = 0;
     uint32_t most_dst = 0;
@@ -742,8 +745,12 @@ uint32_t waves_for(const DeviceCtx *ctx, const hcclx_seg_t *segs, uint32_t nseg,
     const uint32_t widest = most_src > most_dst ? most_src : most_dst;
     if (most_src < 2 || most_dst < 2 || widest > ctx->waves_max_fan || written < ctx->waves_from || esz == 0) return 0;
     const bool same = least_src == most_src;
-    if (!same && widest > 8) return 0;
     const uint64_t per_place = written / most_dst;
+    if (mode == HCCLX_FOLD_SELF_FIRST) {
+        if (!same && widest > 8) return 0;
+    } else if (!ctx->waves_chains && per_place > (256ull << 10)) {
+        return 0;   // chains to several places: only the small ones by default (see above)
+    }
     uint32_t p = ctx->waves_pieces;
     if (p == 0) {   // the shipped policy; a forced piece count takes every launch that passed the tests above
         if (mode == HCCLX_FOLD_SELF_FIRST) {

@@ -91,7 +91,8 @@ const char *hcclx_last_error(void);
  * variables set when the device context is made; name = the variable's name without the prefix, lower case):
  *   "waves_from"      bytes written from which self-first folds take the one-store-per-wavefront kernel (0 = never)
  *   "waves_max_fan"   widest segment (sources / destinations) that kernel is used for (2..16)
- *   "waves_chains"    non-zero: chains whose value goes to several places take it too
+ *   "waves_chains"    non-zero: chains whose value goes to several places take it at every size (else up to 256 KiB
+ *                     per place)
  *   "waves_pieces"    1 KiB pieces per source and workgroup (0 = chosen per launch; another value also takes the
  *                     launches for which the register kernel is otherwise kept)
  *   "fanout_from"     bytes read and written from which a fold with several destinations is split into fold + fan-out
